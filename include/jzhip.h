@@ -1,0 +1,325 @@
+/*
+ * jzhip.h — C ABI of the MI355X (gfx950) device library behind Juzhen's
+ * Matrix<ROCMfloat>.
+ *
+ * Conventions (all entry points):
+ *   - plain C: device pointers are `float*`, element counts `size_t`, matrix
+ *     dimensions `int`, flags `int` (0/1).  No C++ or torch types cross it.
+ *   - return value: 0 = success, -1 = invalid argument (null pointer,
+ *     non-positive dimension, unsupported flag), otherwise a positive
+ *     hipError_t value.  `jzhip_error_string` turns it into text.
+ *   - matrices are fp32, column-major: element (i,j) of a matrix with
+ *     physical row count `ld` lives at `p[j*ld + i]`.  A "trans" flag means
+ *     the logical matrix is the transpose of the physical one
+ *     (reference: cpp/hipmatrix.cuh:64-66).
+ *   - ordering: every call enqueues on the library's current stream (the
+ *     null stream unless `jzhip_set_stream` was called) and returns without
+ *     synchronising; issue order is execution order, exactly as the
+ *     reference's null-stream launches (cpp/hipkernels.cpp:610-622).  Only
+ *     the memcpy calls and `jzhip_synchronize` block the host.
+ *   - no entry point allocates device memory behind the caller's back except
+ *     `jzhip_malloc` and the one-time lazily created reduction workspace
+ *     (see `jzhip_workspace_bytes`).
+ *
+ * Citations `file:line` refer to the reference tree (anewgithubname/Juzhen).
+ */
+#ifndef JZHIP_H
+#define JZHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ── runtime ─────────────────────────────────────────────────────────── */
+
+/* Replaces Juzhen::RocmRuntimeAvailable (cpp/hipbackend.hpp:10). 1 when a
+ * gfx950 device is usable, else 0. */
+int jzhip_runtime_available(void);
+/* Library ABI version (major*100+minor). */
+int jzhip_version(void);
+/* Text for a return code of this library. Never NULL. */
+const char* jzhip_error_string(int rc);
+/* Number of compute units of the current device (0 on failure). */
+int jzhip_num_compute_units(void);
+
+/* Replaces Juzhen::RocmMalloc / RocmFree (cpp/hipbackend.hpp:12-13,
+ * cpp/hipkernels.cpp:513-533). `count` is in floats; count==0 allocates one. */
+int jzhip_malloc(float** ptr, size_t count);
+int jzhip_free(float* ptr);
+/* Replaces Juzhen::RocmMemcpyH2D/D2H/D2D (cpp/hipbackend.hpp:14-16,
+ * cpp/hipkernels.cpp:535-569). Synchronous with respect to the host, ordered
+ * after all work previously issued on the current stream. */
+int jzhip_memcpy_h2d(float* dst_device, const float* src_host, size_t count);
+int jzhip_memcpy_d2h(float* dst_host, const float* src_device, size_t count);
+int jzhip_memcpy_d2d(float* dst_device, const float* src_device, size_t count);
+
+/* No reference counterpart (the reference uses the null stream only,
+ * cpp/hipkernels.cpp:458-461): select the hipStream_t every later call of
+ * this thread's process enqueues on; NULL restores the null stream. */
+int jzhip_set_stream(void* hip_stream);
+void* jzhip_get_stream(void);
+/* Block until the current stream is idle. */
+int jzhip_synchronize(void);
+/* Bytes of the lazily created reduction workspace (0 before first use). */
+size_t jzhip_workspace_bytes(void);
+
+/* ── random numbers ──────────────────────────────────────────────────── */
+
+/* Replace Juzhen::RocmRandUniform / RocmRandNormal (cpp/hipbackend.hpp:18-20,
+ * cpp/hipkernels.cpp:571-608; rocRAND there, Philox4x32-10 + Box-Muller here).
+ * seed==0 continues the library's running stream; seed!=0 restarts it. */
+int jzhip_rand_uniform(float* dst, size_t count, uint64_t seed);
+int jzhip_rand_normal(float* dst, size_t count, float mean, float stddev,
+                      uint64_t seed);
+
+/* ── flat elementwise ops (operate on `count` contiguous floats) ─────── */
+
+/* Juzhen::RocmFill (cpp/hipbackend.hpp:22). */
+int jzhip_fill(float* dst, size_t count, float value);
+/* Juzhen::RocmExpInplace / RocmLogInplace (cpp/hipbackend.hpp:23-24);
+ * oracle exp/log loops cpp/matrix.hpp:253-279. */
+int jzhip_exp_inplace(float* x, size_t count);
+int jzhip_log_inplace(float* x, size_t count);
+/* Out-of-place forms (one pass instead of the reference's D2D copy + in-place
+ * kernel, cpp/hipmatrix.cpp:338-353). out may equal in. */
+int jzhip_exp(float* out, const float* in, size_t count);
+int jzhip_log(float* out, const float* in, size_t count);
+/* Juzhen::RocmAxpby (cpp/hipbackend.hpp:25-26): out = s1*a + s2*b, same
+ * physical layout for all three; out may alias a or b.
+ * Oracle cpp/core.hpp:414-449. */
+int jzhip_axpby(float* out, const float* a, const float* b, size_t count,
+                float s1, float s2);
+/* Juzhen::RocmAffineInplace (cpp/hipbackend.hpp:27): x = s1*x + a.
+ * Oracle cpp/core.hpp:453-469. */
+int jzhip_affine_inplace(float* x, size_t count, float s1, float a);
+/* One-pass out-of-place form of the above (cpp/hipmatrix.cpp:190-201). */
+int jzhip_affine(float* out, const float* in, size_t count, float s1, float a);
+/* Juzhen::RocmHadamard / RocmHadamardInplace (cpp/hipbackend.hpp:28-31).
+ * Oracle cpp/matrix.hpp:428-474. */
+int jzhip_hadamard(float* out, const float* a, const float* b, size_t count);
+int jzhip_hadamard_inplace(float* x, const float* other, size_t count);
+/* Juzhen::RocmElemInvInplace (cpp/hipbackend.hpp:32): x = l / x. */
+int jzhip_eleminv_inplace(float* x, size_t count, float l);
+/* out = (float)(l / (double)in), the oracle's arithmetic
+ * (cpp/core.hpp:472-482 divides in double, then rounds). out may equal in. */
+int jzhip_eleminv(float* out, const float* in, size_t count, double l);
+/* Juzhen::RocmCopy (cpp/hipbackend.hpp:33). */
+int jzhip_copy(float* dst, const float* src, size_t count);
+/* Juzhen::RocmSquare(Inplace), RocmTanh(Inplace), RocmDTanh(Inplace)
+ * (cpp/hipbackend.hpp:34-39); oracle cpp/matrix.hpp:280-326,407-425. */
+int jzhip_square(float* out, const float* in, size_t count);
+int jzhip_square_inplace(float* x, size_t count);
+int jzhip_tanh(float* out, const float* in, size_t count);
+int jzhip_tanh_inplace(float* x, size_t count);
+int jzhip_dtanh(float* out, const float* in, size_t count);
+int jzhip_dtanh_inplace(float* x, size_t count);
+/* Fixed-function forms of the functors the layers pass to elemwise<F>:
+ * relu / d_relu (ml/util.cuh:74-82), sqrt (cpp/juzhen.hpp:71-79),
+ * clamp (ml/util.cuh:84-89). out may equal in. */
+int jzhip_relu(float* out, const float* in, size_t count);
+int jzhip_drelu(float* out, const float* in, size_t count);
+int jzhip_sqrt(float* out, const float* in, size_t count);
+int jzhip_clamp(float* out, const float* in, size_t count, float lo, float hi);
+/* out = d_relu(pre) * up in one pass: the product every backward() forms as
+ * hadmd(d_relu(Matrix(val)), upstream) (ml/layer.hpp:100,1672-1674,3189). */
+int jzhip_drelu_mul(float* out, const float* pre, const float* up, size_t count);
+/* GELU (exact erf form) and its derivative times an upstream gradient. No
+ * reference counterpart (the reference FFN is ReLU, ml/layer.hpp:3018); used
+ * by the character-LM configuration. */
+int jzhip_gelu(float* out, const float* in, size_t count);
+int jzhip_dgelu_mul(float* out, const float* pre, const float* up, size_t count);
+
+/* ── 2-D elementwise ops honouring transpose flags ───────────────────── */
+
+/* out(i,j) = s1*a(i,j) + s2*b(i,j) over logical rows x cols, each operand
+ * with its own physical leading dimension and transpose flag. This is the
+ * logical-index semantics of the CPU oracle (cpp/core.hpp:414-449) that the
+ * reference's flat RocmAxpby call ignores (cpp/hipmatrix.cpp:154-188).
+ * out may alias a (same ld and flag) for the in-place form. */
+int jzhip_axpby2d(float* out, int ldo, int trans_o,
+                  const float* a, int lda, int trans_a,
+                  const float* b, int ldb, int trans_b,
+                  int rows, int cols, float s1, float s2);
+/* Same for the Hadamard product (oracle cpp/matrix.hpp:428-474). */
+int jzhip_hadamard2d(float* out, int ldo, int trans_o,
+                     const float* a, int lda, int trans_a,
+                     const float* b, int ldb, int trans_b,
+                     int rows, int cols);
+/* dst(dr0+i, dc0+j) = src(sr0+i, sc0+j) for a logical rows x cols block. */
+int jzhip_copy2d(float* dst, int ldd, int trans_d, size_t dr0, size_t dc0,
+                 const float* src, int lds, int trans_s, size_t sr0, size_t sc0,
+                 size_t rows, size_t cols);
+
+/* Juzhen::RocmStackCopyCols / RocmStackCopyRows (cpp/hipbackend.hpp:40-53,
+ * kernels cpp/hipkernels.cpp:116-158; oracle hstack/vstack
+ * cpp/matrix.hpp:93-150). */
+int jzhip_stack_copy_cols(float* dst, size_t dst_numrow, size_t dst_col_offset,
+                          const float* src, size_t src_numrow, size_t src_numcol,
+                          int src_transpose);
+int jzhip_stack_copy_rows(float* dst, size_t dst_numrow, size_t dst_row_offset,
+                          const float* src, size_t src_numrow, size_t src_numcol,
+                          int src_transpose);
+/* Juzhen::RocmSliceExtract / RocmSliceAssign (cpp/hipbackend.hpp:54-72,
+ * kernels cpp/hipkernels.cpp:160-206; oracle slice cpp/core.hpp:353-373). */
+int jzhip_slice_extract(float* dst, size_t dst_numrow,
+                        const float* src, size_t src_numrow, int src_transpose,
+                        size_t rstart, size_t cstart, size_t rows, size_t cols);
+int jzhip_slice_assign(float* dst, size_t dst_numrow, int dst_transpose,
+                       size_t rstart, size_t cstart,
+                       const float* src, size_t src_numrow, int src_transpose,
+                       size_t rows, size_t cols);
+
+/* ── reductions ──────────────────────────────────────────────────────── */
+
+/* Sums over a physical column-major numrow x numcol buffer; replace the
+ * ones-vector GEMV of sum(M,dim) (cpp/hipmatrix.cpp:529-555; oracle
+ * cpp/matrix.hpp:74-91).
+ *   jzhip_sum_cols: out[j] = sum_i a[j*ld+i]   (numcol outputs)
+ *   jzhip_sum_rows: out[i] = sum_j a[j*ld+i]   (numrow outputs) */
+int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, int ld);
+int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, int ld);
+/* out[0] = sqrt(sum x^2): replaces hipblasSnrm2 in norm()
+ * (cpp/hipmatrix.cpp:232-254; oracle cpp/core.hpp:337-344). */
+int jzhip_nrm2(float* out_device, const float* x, size_t count);
+/* out[j] = max_i a[j*ld+i], the functor col_softmax / predict_one_hot pass to
+ * reduce<F> (ml/layer.hpp:2346-2351, ml/util.cuh:260-272). */
+int jzhip_max_cols(float* out, const float* a, int numrow, int numcol, int ld);
+/* out[j] = index (stored as int32) of the first maximum of column j: the
+ * first-maximum rule of std::max_element (ml/util.cuh:104-110,
+ * examples/demo_transformer.cu:350-357). Bit-exact. */
+int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numcol, int ld);
+
+/* ── GEMM family ─────────────────────────────────────────────────────── */
+
+/* Juzhen::RocmGemm (cpp/hipbackend.hpp:77-81, hipBLAS there
+ * cpp/hipmatrix.cpp:605-652): C(m x n) = alpha*op(A)(m x k)*op(B)(k x n)
+ * + beta*C, column-major, fp32 MFMA with fp32 accumulation. Returns -1 for
+ * m,n,k <= 0 or null pointers, as the reference does (:611-612).
+ * Oracle: Matrix::dot -> gemm (cpp/core.hpp:395-411, cpp/cpulinalg.hpp:46-91). */
+int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, int k,
+               int trans_a, int trans_b, int lda, int ldb, int ldc,
+               float alpha, float beta);
+/* Juzhen::RocmGemmNN (cpp/hipbackend.hpp:94-95). */
+int jzhip_gemm_nn(const float* A, const float* B, float* C, int m, int n, int k,
+                  float alpha, float beta);
+/* Juzhen::RocmGemv (cpp/hipbackend.hpp:84-91; oracle cpp/cpulinalg.hpp:96-131):
+ * y = alpha*op(A)*x + beta*y, A physically m x n. */
+int jzhip_gemv(const float* A, const float* x, float* y, int m, int n,
+               int trans_a, int lda, int incx, int incy, float alpha, float beta);
+/* Strided-batched GEMM, the shape contract of the reference's CUDA attention
+ * path (cublasSgemmStridedBatched, ml/layer.hpp:2896-2927): batch b uses
+ * A + b*stride_a, B + b*stride_b, C + b*stride_c. */
+int jzhip_gemm_strided_batched(const float* A, const float* B, float* C,
+                               int m, int n, int k, int trans_a, int trans_b,
+                               int lda, int ldb, int ldc,
+                               long long stride_a, long long stride_b,
+                               long long stride_c, int batch,
+                               float alpha, float beta);
+/* y(rows x cols, column-major, ld=rows) += b[i] broadcast over columns: the
+ * rank-1 product `b * ones(1,N)` the layers use for every bias
+ * (ml/layer.hpp:79,120,2797; CUDA add_bias_kernel ml/layer.hpp:2538-2542). */
+int jzhip_add_bias(float* y, const float* b, int rows, int cols);
+
+/* ── softmax family ──────────────────────────────────────────────────── */
+
+/* Column softmax of a physical numrow x numcol buffer (each contiguous
+ * column is one distribution): out = exp(x-max) * 1/(sum+1e-12), the
+ * arithmetic of col_softmax (ml/layer.hpp:2344-2358). out may equal in. */
+int jzhip_softmax_cols(float* out, const float* in, int numrow, int numcol, int ld);
+/* Row softmax of the same buffer (each physical row, stride ld, is one
+ * distribution): row_softmax = col_softmax(M.T()).T() (ml/layer.hpp:2364-2367). */
+int jzhip_softmax_rows(float* out, const float* in, int numrow, int numcol, int ld);
+/* Attention softmax over `nblk` column-major S x S score blocks stored back
+ * to back, with the score scale and the causal mask fused: x = in*scale,
+ * masked entries (key index > query index) are set to -1e9 before the
+ * softmax exactly as the reference does (host loop ml/layer.hpp:2979-2994,
+ * CUDA causal_mask_kernel :2401-2412, softmax_rows_batched_kernel
+ * :2373-2399), then p = exp(x-max) * 1/(sum+1e-12).
+ *   keys_along_rows == 0: element (query a, key b) of a block at a + b*S —
+ *       the reference's cached_A layout; the softmax runs along a block row.
+ *   keys_along_rows == 1: element (key b, query a) at b + a*S — the
+ *       transposed block; the softmax runs along a contiguous column.
+ * out may equal in. */
+int jzhip_attn_softmax(float* out, const float* in, int S, int nblk,
+                       float scale, int causal, int keys_along_rows);
+/* Softmax backward for the same two layouts: dS = A*(dA - sum_keys A*dA)*scale
+ * (CUDA softmax_backward_rows_kernel ml/layer.hpp:2418-2445; generic form
+ * :3343-3350). dS may equal dA. */
+int jzhip_attn_softmax_bwd(float* dS, const float* A, const float* dA, int S,
+                           int nblk, float scale, int keys_along_rows);
+/* Softmax cross-entropy of logits (K x N, one sample per column) against
+ * integer labels: loss_out[0] = -(1/N) sum_n log softmax(x_n)[label_n] and,
+ * when dlogits != NULL, dlogits = (softmax - onehot)/N: LogisticLayer's
+ * value and gradient (ml/layer.hpp:232-284) without materialising the
+ * one-hot matrix. */
+int jzhip_softmax_xent(float* loss_out, float* dlogits, const float* logits,
+                       const int32_t* labels, int K, int N, int ld);
+
+/* ── LayerNorm ───────────────────────────────────────────────────────── */
+
+/* Per column of x (dim x N): mean, biased variance, inv = 1/sqrt(var+1e-5),
+ * xhat = (x-mean)*inv, y = gamma*xhat + beta; writes y, xhat (dim x N) and
+ * inv_std (N). LayerNorm<D>::forward (ml/layer.hpp:2632-2639; CUDA kernel
+ * :2483-2508). */
+int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const float* x,
+                        const float* gamma, const float* beta, int dim, int N);
+/* dx = inv*(dxh - mean(dxh) - xhat*mean(dxh*xhat)), dxh = gamma*dy
+ * (ml/layer.hpp:2674-2681; CUDA kernel :2512-2534). */
+int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma,
+                        const float* xhat, const float* inv_std, int dim, int N);
+/* dgamma[i] = sum_c dy*xhat, dbeta[i] = sum_c dy in one pass over dy/xhat:
+ * the two sum(...,1) calls of ml/layer.hpp:2683-2686. */
+int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,
+                                const float* xhat, int dim, int N);
+
+/* ── optimisers ──────────────────────────────────────────────────────── */
+
+/* adam_update (ml/util.cuh:166-256): m,v updated in place, g overwritten by
+ * the step alpha*m_hat/(sqrt(v_hat)+eps) with the exact float expression of
+ * the CPU loop (:223-245); `iteration` is the 1-based step counter the
+ * caller keeps in adam_state. */
+int jzhip_adam_update(float* g, float* m, float* v, size_t count, float alpha,
+                      float beta1, float beta2, float eps, int iteration);
+/* Adam step with the weight update fused: w -= step (the `W -= adam_update`
+ * of ml/layer.hpp:108-111), and decoupled weight decay w -= alpha*wd*w when
+ * wd != 0 (AdamW; no reference counterpart). g is left untouched. */
+int jzhip_adamw_step(float* w, const float* g, float* m, float* v, size_t count,
+                     float alpha, float beta1, float beta2, float eps,
+                     float weight_decay, int iteration);
+
+/* ── convolution data movement ───────────────────────────────────────── */
+
+/* Juzhen::RocmIm2col / RocmCol2im (cpp/hipbackend.hpp:99-111; oracle
+ * make_im2col / col2im ml/layer.hpp:1897-1925,1975-1999). Bit-exact. */
+int jzhip_im2col(const float* input, float* col, int C_in, int H_in, int W_in,
+                 int kH, int kW, int pad_h, int pad_w, int stride_h,
+                 int stride_w, int H_out, int W_out, int N);
+int jzhip_col2im(const float* col, float* dx, int C_in, int H_in, int W_in,
+                 int kH, int kW, int pad_h, int pad_w, int stride_h,
+                 int stride_w, int H_out, int W_out, int N);
+/* Juzhen::RocmConvForwardReshapeBias / RocmConvBackwardReshape
+ * (cpp/hipbackend.hpp:113-117; oracle ml/layer.hpp:1942-1973). */
+int jzhip_conv_forward_reshape_bias(const float* y2d, float* out,
+                                    const float* bias, int C_out, int P, int N);
+int jzhip_conv_backward_reshape(const float* t, float* t2d, int C_out, int P,
+                                int N);
+/* Juzhen::RocmConvTransScatter / Gather / Reshape (cpp/hipbackend.hpp:119-136;
+ * oracle ml/layer.hpp:2112-2221). */
+int jzhip_convtrans_scatter(const float* patches, float* out, const float* bias,
+                            int C_out, int H_out, int W_out, int H_in, int W_in,
+                            int kH, int kW, int pad_h, int pad_w, int stride_h,
+                            int stride_w, int N);
+int jzhip_convtrans_gather(const float* t, float* tp, int C_out, int H_out,
+                           int W_out, int H_in, int W_in, int kH, int kW,
+                           int pad_h, int pad_w, int stride_h, int stride_w,
+                           int N);
+int jzhip_convtrans_reshape(const float* src, float* dst, int C, int spatial,
+                            int N, int direction);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JZHIP_H */

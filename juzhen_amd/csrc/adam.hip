@@ -1,0 +1,144 @@
+// Fused Adam / AdamW: one pass over (g, m, v[, w]) instead of the ~12 generic
+// matrix ops and temporaries of adam_update's generic formulation
+// (ml/util.cuh:247-255).  24 bytes per parameter for the update-only form,
+// 28 for the form with the weight update fused (g is not rewritten).
+//
+// The expression is the CPU oracle's fused loop (ml/util.cuh:223-245), which
+// is itself bit-identical to the generic op chain: every product and sum is
+// rounded separately (this file is built with -ffp-contract=off), the "+0.0f"
+// terms come from scale() being add(0, s), the bias corrections are narrowed
+// from double, and the final division is a double reciprocal narrowed to float
+// followed by a float multiply.
+#include "common.hpp"
+
+#include <cmath>
+
+namespace jz {
+namespace {
+
+struct AdamConst {
+    float alpha, beta1, beta2, omb1, omb2, eps, r1, r2, decay;  // decay = 1 - alpha*wd
+    int use_decay;
+};
+
+__device__ __forceinline__ float adam_one(float gi, float& mi_io, float& vi_io, const AdamConst& c) {
+    const float mi = (c.beta1 * mi_io + 0.0f) + (c.omb1 * gi + 0.0f);
+    const float vi = (c.beta2 * vi_io + 0.0f) + (c.omb2 * (gi * gi) + 0.0f);
+    mi_io = mi;
+    vi_io = vi;
+    const float mh = c.r1 * mi + 0.0f;
+    const float vh = c.r2 * vi + 0.0f;
+    const float den = 1.0f * sqrtf(vh) + c.eps;
+    return (c.alpha * mh + 0.0f) * static_cast<float>(1.0 / static_cast<double>(den));
+}
+
+// FUSE_W = false: g <- step.  FUSE_W = true: w <- decay*w - step, g untouched.
+template <bool FUSE_W, bool VEC>
+__global__ __launch_bounds__(kBlock) void adam_kernel(float* w, float* g, float* m, float* v,
+                                                      size_t n, AdamConst c) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if constexpr (VEC) {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride) {
+            float4 gv = reinterpret_cast<const float4*>(g)[i];
+            float4 mv = reinterpret_cast<float4*>(m)[i];
+            float4 vv = reinterpret_cast<float4*>(v)[i];
+            float4 st;
+            st.x = adam_one(gv.x, mv.x, vv.x, c);
+            st.y = adam_one(gv.y, mv.y, vv.y, c);
+            st.z = adam_one(gv.z, mv.z, vv.z, c);
+            st.w = adam_one(gv.w, mv.w, vv.w, c);
+            reinterpret_cast<float4*>(m)[i] = mv;
+            reinterpret_cast<float4*>(v)[i] = vv;
+            if constexpr (FUSE_W) {
+                float4 wv = reinterpret_cast<float4*>(w)[i];
+                if (c.use_decay) {
+                    wv.x *= c.decay; wv.y *= c.decay; wv.z *= c.decay; wv.w *= c.decay;
+                }
+                wv.x = 1.0f * wv.x + -1.0f * st.x;
+                wv.y = 1.0f * wv.y + -1.0f * st.y;
+                wv.z = 1.0f * wv.z + -1.0f * st.z;
+                wv.w = 1.0f * wv.w + -1.0f * st.w;
+                reinterpret_cast<float4*>(w)[i] = wv;
+            } else {
+                reinterpret_cast<float4*>(g)[i] = st;
+            }
+        }
+        for (size_t j = n4 * 4 + tid; j < n; j += stride) {
+            float mi = m[j], vi = v[j];
+            const float st = adam_one(g[j], mi, vi, c);
+            m[j] = mi;
+            v[j] = vi;
+            if constexpr (FUSE_W) {
+                float wj = w[j];
+                if (c.use_decay) wj *= c.decay;
+                w[j] = 1.0f * wj + -1.0f * st;
+            } else {
+                g[j] = st;
+            }
+        }
+    } else {
+        for (size_t j = tid; j < n; j += stride) {
+            float mi = m[j], vi = v[j];
+            const float st = adam_one(g[j], mi, vi, c);
+            m[j] = mi;
+            v[j] = vi;
+            if constexpr (FUSE_W) {
+                float wj = w[j];
+                if (c.use_decay) wj *= c.decay;
+                w[j] = 1.0f * wj + -1.0f * st;
+            } else {
+                g[j] = st;
+            }
+        }
+    }
+}
+
+AdamConst make_const(float alpha, float beta1, float beta2, float eps, float wd, int iteration) {
+    AdamConst c;
+    c.alpha = alpha;
+    c.beta1 = beta1;
+    c.beta2 = beta2;
+    c.omb1 = 1 - beta1;
+    c.omb2 = 1 - beta2;
+    c.eps = eps;
+    // ml/util.cuh:226-227
+    c.r1 = static_cast<float>(1.0 / (1.0 - std::pow(static_cast<double>(beta1), static_cast<double>(iteration))));
+    c.r2 = static_cast<float>(1.0 / (1.0 - std::pow(static_cast<double>(beta2), static_cast<double>(iteration))));
+    c.use_decay = wd != 0.0f;
+    c.decay = 1.0f - alpha * wd;
+    return c;
+}
+
+template <bool FUSE_W>
+int launch_adam(float* w, float* g, float* m, float* v, size_t n, const AdamConst& c) {
+    if (n == 0) return 0;
+    const bool vec = aligned16(g) && aligned16(m) && aligned16(v) && (!FUSE_W || aligned16(w));
+    const unsigned grid = grid_for(vec ? (n + 3) / 4 : n, kBlock, 8);
+    if (vec)
+        adam_kernel<FUSE_W, true><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
+    else
+        adam_kernel<FUSE_W, false><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
+    return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_adam_update(float* g, float* m, float* v, size_t count, float alpha, float beta1,
+                             float beta2, float eps, int iteration) {
+    if (count && (!g || !m || !v)) return -1;
+    if (iteration < 1) return -1;
+    return launch_adam<false>(nullptr, g, m, v, count, make_const(alpha, beta1, beta2, eps, 0.f, iteration));
+}
+
+JZ_API int jzhip_adamw_step(float* w, const float* g, float* m, float* v, size_t count, float alpha,
+                            float beta1, float beta2, float eps, float weight_decay, int iteration) {
+    if (count && (!w || !g || !m || !v)) return -1;
+    if (iteration < 1) return -1;
+    return launch_adam<true>(w, const_cast<float*>(g), m, v, count,
+                             make_const(alpha, beta1, beta2, eps, weight_decay, iteration));
+}

@@ -1,0 +1,119 @@
+// Shared host/device helpers for the gfx950 kernel library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "jzhip.h"
+
+#define JZ_API extern "C" __attribute__((visibility("default")))
+
+namespace jz {
+
+constexpr int kWave = 64;        // CDNA wavefront width
+constexpr int kBlock = 256;      // default workgroup: 4 waves, one per SIMD
+
+// ── host-side runtime state (runtime.hip) ───────────────────────────────
+hipStream_t stream();
+int num_cus();
+// Reads and clears the sticky launch error, like the reference's
+// hipGetLastError() after each launch (cpp/hipkernels.cpp:463-465).
+inline int launch_rc() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : static_cast<int>(e);
+}
+inline int rc_of(hipError_t e) { return e == hipSuccess ? 0 : static_cast<int>(e); }
+// Device scratch for two-phase reductions; created once, never resized.
+// Returns nullptr on allocation failure. Capacity in floats.
+float* workspace();
+constexpr size_t kWorkspaceFloats = size_t(4) << 20;  // 16 MiB
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Grid size for a grid-stride kernel over `work` items with `per_block` items
+// per block per sweep: enough blocks to cover the data, capped at a few
+// resident blocks per CU so that 8 XCDs x 32 CUs stay busy.
+inline unsigned grid_for(size_t work, size_t per_block, int blocks_per_cu = 8) {
+    size_t need = (work + per_block - 1) / per_block;
+    size_t cap = static_cast<size_t>(num_cus()) * blocks_per_cu;
+    if (need < 1) need = 1;
+    return static_cast<unsigned>(need < cap ? need : cap);
+}
+
+// ── wave64 reductions: DPP inside a 16-lane row, bpermute across rows ────
+#ifdef __HIPCC__
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+struct SumOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MaxOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a > b ? a : b; }
+};
+
+// After the call every lane holds the reduction over the whole wavefront.
+template <class Op>
+__device__ __forceinline__ float wave_allreduce(float v, Op op) {
+    v = op(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = op(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = op(v, dpp_mov<0x141>(v));  // row_half_mirror
+    v = op(v, dpp_mov<0x140>(v));  // row_mirror: every lane has its row's value
+    v = op(v, __shfl_xor(v, 16, kWave));
+    v = op(v, __shfl_xor(v, 32, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) { return wave_allreduce(v, SumOp{}); }
+__device__ __forceinline__ float wave_max(float v) { return wave_allreduce(v, MaxOp{}); }
+
+// Block-wide reduction for blocks of NW waves; `smem` holds NW floats.
+// Every thread gets the result.
+template <int NW, class Op>
+__device__ __forceinline__ float block_allreduce(float v, Op op, float* smem, float identity) {
+    v = wave_allreduce(v, op);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();  // protect smem from a previous use
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float r = identity;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) r = op(r, smem[w]);
+    return r;
+}
+
+// Unsigned division by a runtime-uniform divisor via multiply-high.
+// Valid for n < 2^31 and 1 <= d < 2^31.
+struct FastDiv {
+    uint32_t mul;
+    uint32_t shift;
+    uint32_t d;
+};
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv& f) {
+    return f.d == 1 ? n : (__umulhi(n, f.mul) >> f.shift);
+}
+#endif
+
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    if (d == 1) {
+        f.mul = 0;
+        f.shift = 0;
+        return f;
+    }
+    uint32_t l = 0;
+    while ((uint32_t(1) << l) < d) ++l;  // l = ceil(log2 d), 1..31
+    // mul = floor(2^(32+l-1) / d) + 1 truncated to 32 bits works for n < 2^31
+    uint64_t m = ((uint64_t(1) << (32 + l - 1)) / d) + 1;
+    f.mul = static_cast<uint32_t>(m);
+    f.shift = l - 1;
+    return f;
+}
+
+}  // namespace jz

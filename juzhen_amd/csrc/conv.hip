@@ -1,0 +1,265 @@
+// Convolution data movement: im2col, col2im and the channel/space repacking
+// kernels of the ROCm ConvLayer / convtransLayer (ml/layer.hpp:1611-1869).
+// All index maps are integer-exact restatements of the CPU loops
+// (ml/layer.hpp:1897-1999, 2112-2221); values are copied, or summed in the CPU
+// loop's order, so results are bit-identical to the oracle.
+//
+// Three kernels cover the seven entry points:
+//   * patch gather  (im2col; convtrans_gather is the same map with the roles
+//     of the input and output grids exchanged),
+//   * patch scatter-as-gather (col2im; convtrans_scatter is the same map with
+//     a bias as the initial value),
+//   * batched tile transpose (the four reshape kernels are all
+//     (R x C) -> (C x R) per sample, with an optional per-row bias).
+#include "common.hpp"
+
+namespace jz {
+namespace {
+
+struct PatchGeom {
+    int C, H, W;        // image side: channels, height, width
+    int kH, kW;
+    int pad_h, pad_w, stride_h, stride_w;
+    int Hp, Wp;         // patch-grid side (conv output positions)
+    int N;
+    int K;              // C*kH*kW
+    int P;              // Hp*Wp
+    FastDiv dK, dP, dWp, dKK, dkW, dCHW, dHW, dW;
+};
+
+PatchGeom make_geom(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int stride_h,
+                    int stride_w, int Hp, int Wp, int N) {
+    PatchGeom g;
+    g.C = C; g.H = H; g.W = W; g.kH = kH; g.kW = kW;
+    g.pad_h = pad_h; g.pad_w = pad_w; g.stride_h = stride_h; g.stride_w = stride_w;
+    g.Hp = Hp; g.Wp = Wp; g.N = N;
+    g.K = C * kH * kW;
+    g.P = Hp * Wp;
+    g.dK = make_fastdiv(g.K);
+    g.dP = make_fastdiv(g.P);
+    g.dWp = make_fastdiv(Wp);
+    g.dKK = make_fastdiv(kH * kW);
+    g.dkW = make_fastdiv(kW);
+    g.dCHW = make_fastdiv(C * H * W);
+    g.dHW = make_fastdiv(H * W);
+    g.dW = make_fastdiv(W);
+    return g;
+}
+
+// col(K, P*N)[k, c] = image(C*H*W, N)[(ci,ih,iw), n] or 0 in the padding.
+// VEC consecutive k per thread (VEC=4 needs K % 4 == 0 and an aligned col).
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void im2col_kernel(const float* img, float* col, PatchGeom g,
+                                                        FastDiv dKv, size_t total_vec) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    const uint32_t kvec = g.K / VEC;
+    for (size_t t = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; t < total_vec; t += stride) {
+        // t < 2^31 is guaranteed by the launcher
+        const uint32_t tt = static_cast<uint32_t>(t);
+        const uint32_t c = fdiv(tt, dKv);
+        const uint32_t k0 = (tt - c * kvec) * VEC;
+        const uint32_t n = fdiv(c, g.dP);
+        const uint32_t p = c - n * g.P;
+        const uint32_t ph = fdiv(p, g.dWp);
+        const uint32_t pw = p - ph * g.Wp;
+        uint32_t ci = fdiv(k0, g.dKK);
+        const uint32_t rem = k0 - ci * (g.kH * g.kW);
+        uint32_t kh = fdiv(rem, g.dkW);
+        uint32_t kw = rem - kh * g.kW;
+        const int h0 = static_cast<int>(ph) * g.stride_h - g.pad_h;
+        const int w0 = static_cast<int>(pw) * g.stride_w - g.pad_w;
+        const float* src = img + static_cast<size_t>(n) * (g.C * g.H * g.W);
+        float vals[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            const int ih = h0 + static_cast<int>(kh);
+            const int iw = w0 + static_cast<int>(kw);
+            float x = 0.0f;
+            if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+                x = src[(static_cast<size_t>(ci) * g.H + ih) * g.W + iw];
+            vals[v] = x;
+            if (++kw == static_cast<uint32_t>(g.kW)) {
+                kw = 0;
+                if (++kh == static_cast<uint32_t>(g.kH)) {
+                    kh = 0;
+                    ++ci;
+                }
+            }
+        }
+        float* dst = col + static_cast<size_t>(c) * g.K + k0;
+        if constexpr (VEC == 4) {
+            *reinterpret_cast<float4*>(dst) = make_float4(vals[0], vals[1], vals[2], vals[3]);
+        } else {
+            dst[0] = vals[0];
+        }
+    }
+}
+
+// image[(ci,ih,iw), n] = init + sum over patch positions (ph asc, pw asc) of
+// col[k(ci,kh,kw), c(n,ph,pw)] with ih = ph*stride - pad + kh: the gather form
+// of the CPU scatter loop, visiting contributions in the CPU's order
+// (ml/layer.hpp:1979-1995: ph ascending, then pw ascending, i.e. kh and kw
+// descending).  init = bias[ci] (convtrans forward) or 0 (col2im).
+__global__ __launch_bounds__(kBlock) void col2im_kernel(const float* col, float* img,
+                                                        const float* bias, PatchGeom g,
+                                                        size_t total) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    for (size_t t = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; t < total; t += stride) {
+        const uint32_t tt = static_cast<uint32_t>(t);
+        const uint32_t n = fdiv(tt, g.dCHW);
+        const uint32_t r = tt - n * (g.C * g.H * g.W);
+        const uint32_t ci = fdiv(r, g.dHW);
+        const uint32_t rem = r - ci * (g.H * g.W);
+        const uint32_t ih = fdiv(rem, g.dW);
+        const uint32_t iw = rem - ih * g.W;
+        float val = bias ? bias[ci] : 0.0f;
+        const float* base = col + static_cast<size_t>(n) * g.P * g.K + static_cast<size_t>(ci) * g.kH * g.kW;
+        for (int kh = g.kH - 1; kh >= 0; --kh) {
+            const int hn = static_cast<int>(ih) + g.pad_h - kh;
+            if (hn < 0) continue;
+            const int ph = hn / g.stride_h;
+            if (ph * g.stride_h != hn || ph >= g.Hp) continue;
+            for (int kw = g.kW - 1; kw >= 0; --kw) {
+                const int wn = static_cast<int>(iw) + g.pad_w - kw;
+                if (wn < 0) continue;
+                const int pw = wn / g.stride_w;
+                if (pw * g.stride_w != wn || pw >= g.Wp) continue;
+                val += base[static_cast<size_t>(ph * g.Wp + pw) * g.K + kh * g.kW + kw];
+            }
+        }
+        img[t] = val;
+    }
+}
+
+// dst[b] (C x R, ld = C) = transpose(src[b] (R x C, ld = R)) + bias[r]
+constexpr int kT = 32;
+__global__ __launch_bounds__(kT * 8) void transpose_batched_kernel(float* dst, const float* src,
+                                                                   const float* bias, int R, int C,
+                                                                   unsigned tiles_r) {
+    __shared__ float tile[kT][kT + 1];
+    const size_t boff = static_cast<size_t>(blockIdx.y) * R * C;
+    const int r0 = static_cast<int>(blockIdx.x % tiles_r) * kT;
+    const int c0 = static_cast<int>(blockIdx.x / tiles_r) * kT;
+    const int tx = threadIdx.x % kT, ty = threadIdx.x / kT;
+#pragma unroll
+    for (int k = 0; k < kT; k += 8) {
+        const int r = r0 + tx, c = c0 + ty + k;
+        if (r < R && c < C) tile[ty + k][tx] = src[boff + static_cast<size_t>(c) * R + r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kT; k += 8) {
+        const int c = c0 + tx, r = r0 + ty + k;
+        if (r < R && c < C) {
+            float v = tile[tx][ty + k];
+            if (bias) v = v + bias[r];
+            dst[boff + static_cast<size_t>(r) * C + c] = v;
+        }
+    }
+}
+
+int transpose_batched(float* dst, const float* src, const float* bias, int R, int C, int batch) {
+    if (R <= 0 || C <= 0 || batch <= 0 || !dst || !src) return -1;
+    const unsigned tiles_r = (R + kT - 1) / kT, tiles_c = (C + kT - 1) / kT;
+    int done = 0;
+    while (done < batch) {
+        const int nb = (batch - done) < 65535 ? (batch - done) : 65535;
+        const size_t off = static_cast<size_t>(done) * R * C;
+        dim3 grid(tiles_r * tiles_c, nb);
+        transpose_batched_kernel<<<grid, kT * 8, 0, stream()>>>(dst + off, src + off, bias, R, C, tiles_r);
+        done += nb;
+    }
+    return launch_rc();
+}
+
+bool geom_ok(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int stride_h, int stride_w,
+             int Hp, int Wp, int N) {
+    return C > 0 && H > 0 && W > 0 && kH > 0 && kW > 0 && pad_h >= 0 && pad_w >= 0 && stride_h > 0 &&
+           stride_w > 0 && Hp > 0 && Wp > 0 && N > 0;
+}
+
+int gather_patches(const float* img, float* col, const PatchGeom& g) {
+    const size_t total = static_cast<size_t>(g.K) * g.P * g.N;
+    if (total >= (size_t(1) << 31)) return -1;
+    if (static_cast<size_t>(g.C) * g.H * g.W * g.N >= (size_t(1) << 31)) return -1;
+    if (g.K % 4 == 0 && aligned16(col)) {
+        const size_t tv = total / 4;
+        im2col_kernel<4><<<grid_for(tv, kBlock, 8), kBlock, 0, stream()>>>(img, col, g, make_fastdiv(g.K / 4), tv);
+    } else {
+        im2col_kernel<1><<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(img, col, g, g.dK, total);
+    }
+    return launch_rc();
+}
+
+int scatter_patches(const float* col, float* img, const float* bias, const PatchGeom& g) {
+    const size_t total = static_cast<size_t>(g.C) * g.H * g.W * g.N;
+    if (total >= (size_t(1) << 31)) return -1;
+    if (static_cast<size_t>(g.K) * g.P * g.N >= (size_t(1) << 31)) return -1;
+    col2im_kernel<<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(col, img, bias, g, total);
+    return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_im2col(const float* input, float* col, int C_in, int H_in, int W_in, int kH, int kW,
+                        int pad_h, int pad_w, int stride_h, int stride_w, int H_out, int W_out,
+                        int N) {
+    if (!input || !col || !geom_ok(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N))
+        return -1;
+    return gather_patches(input, col,
+                          make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N));
+}
+
+JZ_API int jzhip_col2im(const float* col, float* dx, int C_in, int H_in, int W_in, int kH, int kW,
+                        int pad_h, int pad_w, int stride_h, int stride_w, int H_out, int W_out,
+                        int N) {
+    if (!col || !dx || !geom_ok(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N))
+        return -1;
+    return scatter_patches(col, dx, nullptr,
+                           make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N));
+}
+
+// y2d(C_out, P*N) -> out(C_out*P, N) + bias[co]   (ml/layer.hpp:1959-1973)
+JZ_API int jzhip_conv_forward_reshape_bias(const float* y2d, float* out, const float* bias,
+                                           int C_out, int P, int N) {
+    return transpose_batched(out, y2d, bias, C_out, P, N);
+}
+
+// t(C_out*P, N) -> t2d(C_out, P*N)   (ml/layer.hpp:1942-1957)
+JZ_API int jzhip_conv_backward_reshape(const float* t, float* t2d, int C_out, int P, int N) {
+    return transpose_batched(t2d, t, nullptr, P, C_out, N);
+}
+
+// Transposed convolution: the output image grid (H_out x W_out) is the image
+// side and the input grid (H_in x W_in) is the patch side of the same maps
+// (oh = ih*stride - pad + kh, ml/layer.hpp:2159-2171,2190-2202).
+JZ_API int jzhip_convtrans_scatter(const float* patches, float* out, const float* bias, int C_out,
+                                   int H_out, int W_out, int H_in, int W_in, int kH, int kW,
+                                   int pad_h, int pad_w, int stride_h, int stride_w, int N) {
+    if (!patches || !out || !bias ||
+        !geom_ok(C_out, H_out, W_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_in, W_in, N))
+        return -1;
+    return scatter_patches(patches, out, bias,
+                           make_geom(C_out, H_out, W_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_in, W_in, N));
+}
+
+JZ_API int jzhip_convtrans_gather(const float* t, float* tp, int C_out, int H_out, int W_out,
+                                  int H_in, int W_in, int kH, int kW, int pad_h, int pad_w,
+                                  int stride_h, int stride_w, int N) {
+    if (!t || !tp || !geom_ok(C_out, H_out, W_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_in, W_in, N))
+        return -1;
+    return gather_patches(t, tp,
+                          make_geom(C_out, H_out, W_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_in, W_in, N));
+}
+
+// direction 0: (C*spatial, N) -> (C, spatial*N); direction 1: the inverse
+// (ml/layer.hpp:2112-2126,2206-2221).
+JZ_API int jzhip_convtrans_reshape(const float* src, float* dst, int C, int spatial, int N,
+                                   int direction) {
+    if (direction == 0) return transpose_batched(dst, src, nullptr, spatial, C, N);
+    if (direction == 1) return transpose_batched(dst, src, nullptr, C, spatial, N);
+    return -1;
+}

@@ -1,0 +1,460 @@
+// fp32 GEMM on CDNA4 matrix cores: C = alpha*op(A)*op(B) + beta*C, column-major,
+// all four transpose variants, arbitrary leading dimensions, plus the
+// bandwidth-bound special cases the layers generate (rank-1 products for bias
+// broadcasts, matrix-vector products) and a strided-batched form for attention.
+//
+// Tiled kernel: a workgroup of four wavefronts owns a BM x BN tile of C and
+// walks K in steps of BK=16 through two LDS buffers (global loads for step
+// t+1 are in flight while step t is multiplied).  Both operand tiles are kept
+// in LDS as [k][m] / [k][n] so one v_mfma_f32_32x32x2_f32 operand is a single
+// conflict-free 32-lane row read.  The MFMA is issued with B^T as its first
+// operand and A^T as its second, i.e. it produces C^T tiles: each accumulator
+// register then maps to 32 consecutive rows of one column of C, so the epilogue
+// writes 128-byte contiguous segments of the column-major C.
+#include "common.hpp"
+
+namespace jz {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 16;
+constexpr int kPad = 4;  // keeps 16-byte alignment of LDS rows, skews banks
+
+// Global -> register staging for one operand tile of EXT (BM or BN) x BK.
+// MNC = true : the operand is contiguous along its m/n index (A not
+//              transposed, or B transposed): element (x, k) at p[k*ld + x].
+// MNC = false: contiguous along k (A transposed, or B not transposed):
+//              element (x, k) at p[x*ld + k].
+template <int EXT, bool MNC>
+struct TileLoader {
+    static constexpr int kVecs = EXT * BK / 4;             // float4 per tile
+    static constexpr int kPasses = (kVecs + kBlock - 1) / kBlock;
+    float4 reg[kPasses];
+
+    // FAST: tile fully inside the matrix, ld % 4 == 0, base 16-byte aligned.
+    template <bool FAST>
+    __device__ __forceinline__ void load(const float* __restrict__ p, size_t ld, int x0, int k0,
+                                         int X, int K) {
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const int v = threadIdx.x + ps * kBlock;
+            if (kVecs % kBlock != 0 && v >= kVecs) break;
+            int x, k;
+            if constexpr (MNC) {
+                x = (v % (EXT / 4)) * 4;
+                k = v / (EXT / 4);
+            } else {
+                k = (v % (BK / 4)) * 4;
+                x = v / (BK / 4);
+            }
+            const int gx = x0 + x, gk = k0 + k;
+            if constexpr (FAST) {
+                const float* src = MNC ? p + static_cast<size_t>(gk) * ld + gx
+                                       : p + static_cast<size_t>(gx) * ld + gk;
+                reg[ps] = *reinterpret_cast<const float4*>(src);
+            } else {
+                float t[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int ex = MNC ? gx + e : gx;
+                    const int ek = MNC ? gk : gk + e;
+                    t[e] = (ex < X && ek < K)
+                               ? (MNC ? p[static_cast<size_t>(ek) * ld + ex] : p[static_cast<size_t>(ex) * ld + ek])
+                               : 0.0f;
+                }
+                reg[ps] = make_float4(t[0], t[1], t[2], t[3]);
+            }
+        }
+    }
+
+    // registers -> LDS tile laid out [BK][EXT + kPad]
+    __device__ __forceinline__ void store(float* __restrict__ s) const {
+        constexpr int LD = EXT + kPad;
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const int v = threadIdx.x + ps * kBlock;
+            if (kVecs % kBlock != 0 && v >= kVecs) break;
+            if constexpr (MNC) {
+                const int x = (v % (EXT / 4)) * 4;
+                const int k = v / (EXT / 4);
+                *reinterpret_cast<float4*>(s + k * LD + x) = reg[ps];
+            } else {
+                const int k = (v % (BK / 4)) * 4;
+                const int x = v / (BK / 4);
+                s[(k + 0) * LD + x] = reg[ps].x;
+                s[(k + 1) * LD + x] = reg[ps].y;
+                s[(k + 2) * LD + x] = reg[ps].z;
+                s[(k + 3) * LD + x] = reg[ps].w;
+            }
+        }
+    }
+};
+
+// WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
+template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST>
+__global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
+    size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
+    long long strideB, long long strideC, int tiles_m, int tiles_n) {
+    static_assert(WGM * WGN == kBlock / kWave, "four waves per workgroup");
+    constexpr int BM = WGM * TM * 32;
+    constexpr int BN = WGN * TN * 32;
+    constexpr int LDA_S = BM + kPad;
+    constexpr int LDB_S = BN + kPad;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA_S];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB_S];
+
+    // Tile rasterisation.  Workgroups are dealt round-robin to the 8 XCDs, so
+    // ids congruent mod 8 share an L2; give each XCD a contiguous run of the
+    // tile order, and walk that order in column panels of 8 tile-rows so a
+    // panel's A rows and B columns stay L2-resident.
+    const int ntiles = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        constexpr int kXcd = 8;
+        const int per = ntiles / kXcd;
+        const int rem = ntiles % kXcd;
+        if (per > 0) {
+            const int x = pid % kXcd, l = pid / kXcd;
+            // XCDs with index < rem hold (per+1) tiles
+            pid = x * per + (x < rem ? x : rem) + l;
+        }
+    }
+    constexpr int kGroup = 8;
+    const int group_size = kGroup * tiles_n;
+    const int group = pid / group_size;
+    const int first_m = group * kGroup;
+    const int gm = (tiles_m - first_m) < kGroup ? (tiles_m - first_m) : kGroup;
+    const int tile_m = first_m + (pid % group_size) % gm;
+    const int tile_n = (pid % group_size) / gm;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+
+    const int batch = blockIdx.z;
+    A += batch * strideA;
+    B += batch * strideB;
+    C += batch * strideC;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    TileLoader<BM, !TA> la;
+    TileLoader<BN, TB> lb;
+
+    const int nk = (K + BK - 1) / BK;
+    la.template load<FAST>(A, lda, m0, 0, M, K);
+    lb.template load<FAST>(B, ldb, n0, 0, N, K);
+    la.store(As[0]);
+    lb.store(Bs[0]);
+    __syncthreads();
+
+    int cur = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        if (kt + 1 < nk) {
+            la.template load<FAST>(A, lda, m0, (kt + 1) * BK, M, K);
+            lb.template load<FAST>(B, ldb, n0, (kt + 1) * BK, N, K);
+        }
+        const float* as = As[cur] + wm * (TM * 32) + l32;
+        const float* bs = Bs[cur] + wn * (TN * 32) + l32;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[i] = as[(kk + h) * LDA_S + i * 32];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bf[j] = bs[(kk + h) * LDB_S + j * 32];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            la.store(As[cur ^ 1]);
+            lb.store(Bs[cur ^ 1]);
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    // Epilogue.  Register v of lane (h, l32) holds C(row, col) with
+    // row = l32 and col = 8*(v/4) + 4*h + v%4 inside the 32x32 tile.
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int row = m0 + (wm * TM + i) * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int cbase = n0 + (wn * TN + j) * 32 + 4 * h;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int col = cbase + 8 * (v / 4) + (v % 4);
+                if (FAST || (row < M && col < N)) {
+                    float* dst = C + static_cast<size_t>(col) * ldc + row;
+                    float r = alpha * acc[i][j][v];
+                    if (beta != 0.0f) r += beta * *dst;
+                    *dst = r;
+                }
+            }
+        }
+    }
+}
+
+// ── bandwidth-bound special cases ────────────────────────────────────────
+
+// k == 1: C(i,j) = alpha*a_i*b_j + beta*C(i,j).  a has stride sa, b stride sb.
+__global__ __launch_bounds__(kBlock) void rank1_kernel(float* C, const float* a, size_t sa,
+                                                       const float* b, size_t sb, int M, int N,
+                                                       size_t ldc, float alpha, float beta) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= M) return;
+    const float ai = alpha * a[i * sa];
+    for (int j = blockIdx.y; j < N; j += gridDim.y) {
+        float r = ai * b[j * sb];
+        float* dst = C + static_cast<size_t>(j) * ldc + i;
+        if (beta != 0.0f) r += beta * *dst;
+        *dst = r;
+    }
+}
+
+// y[j] = alpha * <A[:,j], x> + beta*y[j]: one wavefront per column of the
+// physical m x n matrix (op = transpose).
+__global__ __launch_bounds__(kBlock) void gemv_t_kernel(const float* A, const float* x, float* y,
+                                                        int m, int n, size_t lda, size_t incx,
+                                                        size_t incy, float alpha, float beta) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t j = wave0; j < static_cast<size_t>(n); j += nwaves) {
+        const float* col = A + j * lda;
+        float acc = 0.f;
+        for (int i = lane; i < m; i += kWave) acc += col[i] * x[i * incx];
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            float r = alpha * acc;
+            if (beta != 0.0f) r += beta * y[j * incy];
+            y[j * incy] = r;
+        }
+    }
+}
+
+// y[i] = alpha * sum_j A[i,j]*x[j] + beta*y[i] (op = none): lanes along rows,
+// the block's waves split the columns, combined through LDS.  Partial results
+// over column chunks go to part[chunk*m + i].
+__global__ __launch_bounds__(kBlock) void gemv_n_partial_kernel(const float* A, const float* x,
+                                                                float* part, int m, int n,
+                                                                size_t lda, size_t incx,
+                                                                int chunk_len) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = blockIdx.x * kWave + lane;
+    const int c_begin = blockIdx.y * chunk_len;
+    int c_end = c_begin + chunk_len;
+    if (c_end > n) c_end = n;
+    float acc = 0.f;
+    if (row < m)
+        for (int c = c_begin + wave; c < c_end; c += NW) acc += A[static_cast<size_t>(c) * lda + row] * x[c * incx];
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && row < m) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += red[w][lane];
+        part[static_cast<size_t>(blockIdx.y) * m + row] = s;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gemv_n_combine_kernel(float* y, const float* part, int m,
+                                                                int chunks, size_t incy,
+                                                                float alpha, float beta) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= m) return;
+    float acc = 0.f;
+    for (int c = 0; c < chunks; ++c) acc += part[static_cast<size_t>(c) * m + i];
+    float r = alpha * acc;
+    if (beta != 0.0f) r += beta * y[i * incy];
+    y[i * incy] = r;
+}
+
+// y(rows x cols) += b[i]
+__global__ __launch_bounds__(kBlock) void add_bias_kernel(float* y, const float* b, int rows,
+                                                          size_t total4) {
+    // rows % 4 == 0: a float4 never straddles a column
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    const unsigned rows4 = rows / 4;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < total4; i += stride) {
+        const unsigned r4 = static_cast<unsigned>(i % rows4);
+        float4 v = reinterpret_cast<float4*>(y)[i];
+        const float4 bb = reinterpret_cast<const float4*>(b)[r4];
+        v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+        reinterpret_cast<float4*>(y)[i] = v;
+    }
+}
+__global__ __launch_bounds__(kBlock) void add_bias_scalar_kernel(float* y, const float* b, int rows,
+                                                                 size_t total) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride)
+        y[i] += b[i % rows];
+}
+
+// ── dispatch ─────────────────────────────────────────────────────────────
+struct GemmArgs {
+    const float* A;
+    const float* B;
+    float* C;
+    int M, N, K;
+    size_t lda, ldb, ldc;
+    float alpha, beta;
+    long long sA, sB, sC;
+    int batch;
+};
+
+template <int WGM, int WGN, int TM, int TN, bool TA, bool TB>
+int launch_tile(const GemmArgs& g) {
+    constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    const bool fast = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && (g.lda % 4 == 0) &&
+                      (g.ldb % 4 == 0) && aligned16(g.A) && aligned16(g.B) && (g.sA % 4 == 0) &&
+                      (g.sB % 4 == 0);
+    dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, 1, g.batch);
+    if (fast)
+        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true><<<grid, kBlock, 0, stream()>>>(
+            g.A, g.B, g.C, g.M, g.N, g.K, g.lda, g.ldb, g.ldc, g.alpha, g.beta, g.sA, g.sB, g.sC,
+            tiles_m, tiles_n);
+    else
+        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, false><<<grid, kBlock, 0, stream()>>>(
+            g.A, g.B, g.C, g.M, g.N, g.K, g.lda, g.ldb, g.ldc, g.alpha, g.beta, g.sA, g.sB, g.sC,
+            tiles_m, tiles_n);
+    return launch_rc();
+}
+
+template <bool TA, bool TB>
+int launch_shape(const GemmArgs& g) {
+    // Pick the tile that wastes the least work on the ragged edge while
+    // keeping every CU busy.
+    const long long cus = num_cus();
+    auto tiles = [&](int bm, int bn) {
+        return static_cast<long long>((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
+    };
+    if (g.M <= 32) return launch_tile<1, 4, 1, 2, TA, TB>(g);   // 32 x 256
+    if (g.N <= 32) return launch_tile<4, 1, 2, 1, TA, TB>(g);   // 256 x 32
+    if (g.M <= 64) return launch_tile<1, 4, 2, 1, TA, TB>(g);   // 64 x 128
+    if (g.N <= 64) return launch_tile<4, 1, 1, 2, TA, TB>(g);   // 128 x 64
+    if (tiles(128, 128) < cus) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
+    return launch_tile<2, 2, 2, 2, TA, TB>(g);                  // 128 x 128
+}
+
+int gemm_dispatch(const GemmArgs& g, bool ta, bool tb) {
+    if (ta) return tb ? launch_shape<true, true>(g) : launch_shape<true, false>(g);
+    return tb ? launch_shape<false, true>(g) : launch_shape<false, false>(g);
+}
+
+int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda,
+              size_t incx, size_t incy, float alpha, float beta) {
+    hipStream_t s = stream();
+    if (trans) {
+        gemv_t_kernel<<<grid_for(n, kBlock / kWave, 8), kBlock, 0, s>>>(A, x, y, m, n, lda, incx, incy,
+                                                                         alpha, beta);
+        return launch_rc();
+    }
+    const int row_blocks = (m + kWave - 1) / kWave;
+    int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
+    if (chunks > n / 32) chunks = n / 32;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 4096) chunks = 4096;
+    while (chunks > 1 && static_cast<size_t>(chunks) * m > kWorkspaceFloats) --chunks;
+    if (static_cast<size_t>(chunks) * m > kWorkspaceFloats) return -1;
+    const int chunk_len = (n + chunks - 1) / chunks;
+    chunks = (n + chunk_len - 1) / chunk_len;
+    float* part = workspace();
+    if (!part) return -2;
+    gemv_n_partial_kernel<<<dim3(row_blocks, chunks), kBlock, 0, s>>>(A, x, part, m, n, lda, incx, chunk_len);
+    gemv_n_combine_kernel<<<(m + kBlock - 1) / kBlock, kBlock, 0, s>>>(y, part, m, chunks, incy, alpha, beta);
+    return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_gemm_strided_batched(const float* A, const float* B, float* C, int m, int n, int k,
+                                      int trans_a, int trans_b, int lda, int ldb, int ldc,
+                                      long long stride_a, long long stride_b, long long stride_c,
+                                      int batch, float alpha, float beta) {
+    if (m <= 0 || n <= 0 || k <= 0 || batch <= 0) return -1;
+    if (!A || !B || !C) return -1;
+    if (lda < (trans_a ? k : m) || ldb < (trans_b ? n : k) || ldc < m) return -1;
+    if (batch > 65535) return -1;
+    GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
+               static_cast<size_t>(ldc), alpha, beta, stride_a, stride_b, stride_c, batch};
+    return gemm_dispatch(g, trans_a != 0, trans_b != 0);
+}
+
+JZ_API int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, int k, int trans_a,
+                      int trans_b, int lda, int ldb, int ldc, float alpha, float beta) {
+    if (m <= 0 || n <= 0 || k <= 0) return -1;
+    if (!A || !B || !C) return -1;
+    if (lda < (trans_a ? k : m) || ldb < (trans_b ? n : k) || ldc < m) return -1;
+    hipStream_t s = stream();
+    if (k == 1) {
+        // rank-1 update: the layers' broadcast idiom (bias * ones(1,N))
+        const size_t sa = trans_a ? lda : 1;   // op(A)(i,0)
+        const size_t sb = trans_b ? 1 : ldb;   // op(B)(0,j)
+        int gy = n < 1024 ? n : 1024;
+        rank1_kernel<<<dim3((m + kBlock - 1) / kBlock, gy), kBlock, 0, s>>>(C, A, sa, B, sb, m, n, ldc,
+                                                                            alpha, beta);
+        return launch_rc();
+    }
+    if (n == 1) {
+        // C(:,0) = alpha*op(A)*b: op(B)(p,0) has stride 1 (B not transposed) or ldb
+        const size_t incx = trans_b ? ldb : 1;
+        if (!trans_a) return gemv_impl(A, B, C, m, k, false, lda, incx, 1, alpha, beta);
+        return gemv_impl(A, B, C, k, m, true, lda, incx, 1, alpha, beta);
+    }
+    if (m == 1) {
+        // C(0,:) = alpha*a^T*op(B)  ==  op(B)^T a: a gemv on B with the flag flipped
+        const size_t incx = trans_a ? 1 : lda;
+        if (trans_b) return gemv_impl(B, A, C, n, k, false, ldb, incx, ldc, alpha, beta);
+        return gemv_impl(B, A, C, k, n, true, ldb, incx, ldc, alpha, beta);
+    }
+    GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
+               static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
+    return gemm_dispatch(g, trans_a != 0, trans_b != 0);
+}
+
+JZ_API int jzhip_gemm_nn(const float* A, const float* B, float* C, int m, int n, int k, float alpha,
+                         float beta) {
+    return jzhip_gemm(A, B, C, m, n, k, 0, 0, m, k, m, alpha, beta);
+}
+
+JZ_API int jzhip_gemv(const float* A, const float* x, float* y, int m, int n, int trans_a, int lda,
+                      int incx, int incy, float alpha, float beta) {
+    if (m <= 0 || n <= 0 || lda < m) return -1;
+    if (!A || !x || !y) return -1;
+    if (incx <= 0 || incy <= 0) return -1;
+    return gemv_impl(A, x, y, m, n, trans_a != 0, lda, incx, incy, alpha, beta);
+}
+
+JZ_API int jzhip_add_bias(float* y, const float* b, int rows, int cols) {
+    if (rows <= 0 || cols <= 0 || !y || !b) return -1;
+    const size_t total = static_cast<size_t>(rows) * cols;
+    if (rows % 4 == 0 && aligned16(y) && aligned16(b)) {
+        add_bias_kernel<<<grid_for(total / 4, kBlock, 8), kBlock, 0, stream()>>>(y, b, rows, total / 4);
+    } else {
+        add_bias_scalar_kernel<<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(y, b, rows, total);
+    }
+    return launch_rc();
+}

@@ -1,0 +1,295 @@
+// Fused LayerNorm forward / backward over the columns of a (dim x N)
+// column-major activation matrix: one wavefront per token column, the column
+// held in registers between the statistics and the normalisation, so x is read
+// once and y / xhat written once (the reference's generic formulation is ~12
+// matrix ops and four rank-1 GEMMs per call, ml/layer.hpp:2632-2639,2674-2681).
+//
+// Arithmetic mirrors the generic formulation: mean = sum(x)/dim, centred
+// two-pass biased variance, inv = 1.0f/sqrtf(var + 1e-5f).
+#include "common.hpp"
+
+#include <cmath>
+
+namespace jz {
+namespace {
+
+constexpr float kLnEps = 1e-5f;
+
+// NV float4 per lane: dim <= 256*NV, dim % 4 == 0, 16-byte aligned columns.
+template <int NV>
+__global__ __launch_bounds__(kBlock) void ln_fwd_vec_kernel(float* y, float* xhat, float* inv_std,
+                                                            const float* x, const float* gamma,
+                                                            const float* beta, int dim, int N) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    const float invdim = 1.0f / static_cast<float>(dim);
+
+    float4 g[NV], b[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int r = (lane + v * kWave) * 4;
+        if (r < dim) {
+            g[v] = *reinterpret_cast<const float4*>(gamma + r);
+            b[v] = *reinterpret_cast<const float4*>(beta + r);
+        }
+    }
+    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+        const size_t base = col * dim;
+        float4 xv[NV];
+        float s = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                xv[v] = *reinterpret_cast<const float4*>(x + base + r);
+                s += (xv[v].x + xv[v].y) + (xv[v].z + xv[v].w);
+            }
+        }
+        const float mu = wave_sum(s) * invdim;
+        float q = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                xv[v].x -= mu; xv[v].y -= mu; xv[v].z -= mu; xv[v].w -= mu;
+                q += (xv[v].x * xv[v].x + xv[v].y * xv[v].y) + (xv[v].z * xv[v].z + xv[v].w * xv[v].w);
+            }
+        }
+        const float var = wave_sum(q) * invdim;
+        const float inv = 1.0f / sqrtf(var + kLnEps);
+        if (lane == 0) inv_std[col] = inv;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                float4 h, o;
+                h.x = xv[v].x * inv; h.y = xv[v].y * inv; h.z = xv[v].z * inv; h.w = xv[v].w * inv;
+                o.x = g[v].x * h.x + b[v].x; o.y = g[v].y * h.y + b[v].y;
+                o.z = g[v].z * h.z + b[v].z; o.w = g[v].w * h.w + b[v].w;
+                *reinterpret_cast<float4*>(xhat + base + r) = h;
+                *reinterpret_cast<float4*>(y + base + r) = o;
+            }
+        }
+    }
+}
+
+// Any dim / alignment: one wavefront per column, three sweeps (L1/L2 hits).
+__global__ __launch_bounds__(kBlock) void ln_fwd_generic_kernel(float* y, float* xhat,
+                                                                float* inv_std, const float* x,
+                                                                const float* gamma,
+                                                                const float* beta, int dim, int N) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    const float invdim = 1.0f / static_cast<float>(dim);
+    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+        const size_t base = col * dim;
+        float s = 0.f;
+        for (int r = lane; r < dim; r += kWave) s += x[base + r];
+        const float mu = wave_sum(s) * invdim;
+        float q = 0.f;
+        for (int r = lane; r < dim; r += kWave) {
+            const float c = x[base + r] - mu;
+            q += c * c;
+        }
+        const float var = wave_sum(q) * invdim;
+        const float inv = 1.0f / sqrtf(var + kLnEps);
+        if (lane == 0) inv_std[col] = inv;
+        for (int r = lane; r < dim; r += kWave) {
+            const float h = (x[base + r] - mu) * inv;
+            xhat[base + r] = h;
+            y[base + r] = gamma[r] * h + beta[r];
+        }
+    }
+}
+
+template <int NV>
+__global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const float* dy,
+                                                            const float* gamma, const float* xhat,
+                                                            const float* inv_std, int dim, int N) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    const float invdim = 1.0f / static_cast<float>(dim);
+    float4 g[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int r = (lane + v * kWave) * 4;
+        if (r < dim) g[v] = *reinterpret_cast<const float4*>(gamma + r);
+    }
+    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+        const size_t base = col * dim;
+        float4 d[NV], h[NV];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                d[v] = *reinterpret_cast<const float4*>(dy + base + r);
+                h[v] = *reinterpret_cast<const float4*>(xhat + base + r);
+                d[v].x *= g[v].x; d[v].y *= g[v].y; d[v].z *= g[v].z; d[v].w *= g[v].w;
+                s1 += (d[v].x + d[v].y) + (d[v].z + d[v].w);
+                s2 += (d[v].x * h[v].x + d[v].y * h[v].y) + (d[v].z * h[v].z + d[v].w * h[v].w);
+            }
+        }
+        const float m1 = wave_sum(s1) * invdim;
+        const float m2 = wave_sum(s2) * invdim;
+        const float inv = inv_std[col];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                float4 o;
+                o.x = inv * (d[v].x - m1 - h[v].x * m2);
+                o.y = inv * (d[v].y - m1 - h[v].y * m2);
+                o.z = inv * (d[v].z - m1 - h[v].z * m2);
+                o.w = inv * (d[v].w - m1 - h[v].w * m2);
+                *reinterpret_cast<float4*>(dx + base + r) = o;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const float* dy,
+                                                                const float* gamma,
+                                                                const float* xhat,
+                                                                const float* inv_std, int dim,
+                                                                int N) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    const float invdim = 1.0f / static_cast<float>(dim);
+    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+        const size_t base = col * dim;
+        float s1 = 0.f, s2 = 0.f;
+        for (int r = lane; r < dim; r += kWave) {
+            const float d = dy[base + r] * gamma[r];
+            s1 += d;
+            s2 += d * xhat[base + r];
+        }
+        const float m1 = wave_sum(s1) * invdim;
+        const float m2 = wave_sum(s2) * invdim;
+        const float inv = inv_std[col];
+        for (int r = lane; r < dim; r += kWave) {
+            const float d = dy[base + r] * gamma[r];
+            dx[base + r] = inv * (d - m1 - xhat[base + r] * m2);
+        }
+    }
+}
+
+// dgamma / dbeta partials: lanes along rows, waves along column phases of the
+// block's column chunk.  part layout: [chunk][2][dim].
+__global__ __launch_bounds__(kBlock) void ln_param_partial_kernel(float* part, const float* dy,
+                                                                  const float* xhat, int dim, int N,
+                                                                  int chunk_len) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[2][NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = blockIdx.x * kWave + lane;
+    const int chunk = blockIdx.y;
+    const int c_begin = chunk * chunk_len;
+    int c_end = c_begin + chunk_len;
+    if (c_end > N) c_end = N;
+    float ag = 0.f, ab = 0.f;
+    if (row < dim) {
+        for (int c = c_begin + wave; c < c_end; c += NW) {
+            const size_t i = static_cast<size_t>(c) * dim + row;
+            const float d = dy[i];
+            ag += d * xhat[i];
+            ab += d;
+        }
+    }
+    red[0][wave][lane] = ag;
+    red[1][wave][lane] = ab;
+    __syncthreads();
+    if (wave == 0 && row < dim) {
+        float sg = 0.f, sb = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            sg += red[0][w][lane];
+            sb += red[1][w][lane];
+        }
+        part[(static_cast<size_t>(chunk) * 2 + 0) * dim + row] = sg;
+        part[(static_cast<size_t>(chunk) * 2 + 1) * dim + row] = sb;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void ln_param_combine_kernel(float* dgamma, float* dbeta,
+                                                                  const float* part, int dim,
+                                                                  int chunks) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= dim) return;
+    float sg = 0.f, sb = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+        sg += part[(static_cast<size_t>(c) * 2 + 0) * dim + i];
+        sb += part[(static_cast<size_t>(c) * 2 + 1) * dim + i];
+    }
+    dgamma[i] = sg;
+    dbeta[i] = sb;
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const float* x,
+                               const float* gamma, const float* beta, int dim, int N) {
+    if (dim <= 0 || N <= 0 || !y || !xhat || !inv_std || !x || !gamma || !beta) return -1;
+    const bool vec = (dim % 4 == 0) && dim <= 1024 && aligned16(x) && aligned16(y) &&
+                     aligned16(xhat) && aligned16(gamma) && aligned16(beta);
+    const unsigned grid = grid_for(N, kBlock / kWave, 8);
+    hipStream_t s = stream();
+    if (vec && dim <= 256)
+        ln_fwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
+    else if (vec && dim <= 512)
+        ln_fwd_vec_kernel<2><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
+    else if (vec)
+        ln_fwd_vec_kernel<4><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
+    else
+        ln_fwd_generic_kernel<<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
+    return launch_rc();
+}
+
+JZ_API int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma, const float* xhat,
+                               const float* inv_std, int dim, int N) {
+    if (dim <= 0 || N <= 0 || !dx || !dy || !gamma || !xhat || !inv_std) return -1;
+    const bool vec = (dim % 4 == 0) && dim <= 1024 && aligned16(dx) && aligned16(dy) &&
+                     aligned16(xhat) && aligned16(gamma);
+    const unsigned grid = grid_for(N, kBlock / kWave, 8);
+    hipStream_t s = stream();
+    if (vec && dim <= 256)
+        ln_bwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+    else if (vec && dim <= 512)
+        ln_bwd_vec_kernel<2><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+    else if (vec)
+        ln_bwd_vec_kernel<4><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+    else
+        ln_bwd_generic_kernel<<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+    return launch_rc();
+}
+
+JZ_API int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,
+                                       const float* xhat, int dim, int N) {
+    if (dim <= 0 || N <= 0 || !dgamma || !dbeta || !dy || !xhat) return -1;
+    const int row_blocks = (dim + kWave - 1) / kWave;
+    size_t want = static_cast<size_t>(num_cus()) * 4;
+    int chunks = static_cast<int>((want + row_blocks - 1) / row_blocks);
+    if (chunks > N / 16) chunks = N / 16;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 65535) chunks = 65535;
+    while (chunks > 1 && static_cast<size_t>(chunks) * 2 * dim > kWorkspaceFloats) --chunks;
+    if (static_cast<size_t>(chunks) * 2 * dim > kWorkspaceFloats) return -1;
+    const int chunk_len = (N + chunks - 1) / chunks;
+    chunks = (N + chunk_len - 1) / chunk_len;
+    float* part = workspace();
+    if (!part) return -2;
+    hipStream_t s = stream();
+    dim3 grid(row_blocks, chunks);
+    ln_param_partial_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
+    ln_param_combine_kernel<<<(dim + kBlock - 1) / kBlock, kBlock, 0, s>>>(dgamma, dbeta, part, dim,
+                                                                          chunks);
+    return launch_rc();
+}

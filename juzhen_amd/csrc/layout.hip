@@ -1,0 +1,168 @@
+// Two-dimensional elementwise kernels that honour per-operand transpose
+// flags and leading dimensions: the logical-index semantics of the CPU oracle
+// (cpp/core.hpp:414-449, cpp/matrix.hpp:93-150,428-474, cpp/core.hpp:353-373).
+//
+// Everything is expressed in the *output's physical frame*: the output is an
+// R x C column-major block with leading dimension ldo; an operand whose
+// transpose flag differs from the output's is "relatively transposed" and its
+// element (r,c) lives at x[r*ldx + c].  Such operands are staged through a
+// padded LDS tile so that both the global read and the global write are
+// coalesced along the contiguous dimension of their own buffer.
+#include "common.hpp"
+
+namespace jz {
+namespace {
+
+constexpr int kTile = 32;
+constexpr int kRowsPerPass = 8;  // block = 32 x 8 threads, 4 passes per tile
+
+enum : int { kOpCopy = 0, kOpAxpby = 1, kOpHadamard = 2 };
+
+template <int OP>
+__global__ __launch_bounds__(kTile* kRowsPerPass) void ew2d_kernel(
+    float* out, size_t ldo, const float* a, size_t lda, int rel_a, const float* b, size_t ldb,
+    int rel_b, size_t R, size_t C, unsigned tiles_r, float s1, float s2) {
+    __shared__ float ta[kTile][kTile + 1];
+    __shared__ float tb[kTile][kTile + 1];
+    const unsigned tile = blockIdx.x;
+    const size_t r0 = static_cast<size_t>(tile % tiles_r) * kTile;
+    const size_t c0 = static_cast<size_t>(tile / tiles_r) * kTile;
+    const int tx = threadIdx.x % kTile;
+    const int ty = threadIdx.x / kTile;
+
+    if (rel_a) {
+#pragma unroll
+        for (int k = 0; k < kTile; k += kRowsPerPass) {
+            const size_t r = r0 + ty + k, c = c0 + tx;
+            if (r < R && c < C) ta[ty + k][tx] = a[r * lda + c];
+        }
+    }
+    if (OP != kOpCopy && rel_b) {
+#pragma unroll
+        for (int k = 0; k < kTile; k += kRowsPerPass) {
+            const size_t r = r0 + ty + k, c = c0 + tx;
+            if (r < R && c < C) tb[ty + k][tx] = b[r * ldb + c];
+        }
+    }
+    if (rel_a || (OP != kOpCopy && rel_b)) __syncthreads();
+
+#pragma unroll
+    for (int k = 0; k < kTile; k += kRowsPerPass) {
+        const int cl = ty + k;
+        const size_t r = r0 + tx, c = c0 + cl;
+        if (r < R && c < C) {
+            const float va = rel_a ? ta[tx][cl] : a[c * lda + r];
+            float res;
+            if constexpr (OP == kOpCopy) {
+                res = va;
+            } else {
+                const float vb = rel_b ? tb[tx][cl] : b[c * ldb + r];
+                res = (OP == kOpAxpby) ? (s1 * va + s2 * vb) : (va * vb);
+            }
+            out[c * ldo + r] = res;
+        }
+    }
+}
+
+template <int OP>
+int launch2d(float* out, size_t ldo, const float* a, size_t lda, int rel_a, const float* b,
+             size_t ldb, int rel_b, size_t R, size_t C, float s1, float s2) {
+    if (R == 0 || C == 0) return 0;
+    const size_t tiles_r = (R + kTile - 1) / kTile;
+    const size_t tiles_c = (C + kTile - 1) / kTile;
+    if (tiles_r * tiles_c > 0x7fffffffull) return -1;
+    ew2d_kernel<OP><<<static_cast<unsigned>(tiles_r * tiles_c), kTile * kRowsPerPass, 0, stream()>>>(
+        out, ldo, a, lda, rel_a, b, ldb, rel_b, R, C, static_cast<unsigned>(tiles_r), s1, s2);
+    return launch_rc();
+}
+
+// Shared front end of axpby2d / hadamard2d.  rows/cols are logical.
+template <int OP>
+int binary2d(float* out, int ldo, int trans_o, const float* a, int lda, int trans_a,
+             const float* b, int ldb, int trans_b, int rows, int cols, float s1, float s2) {
+    if (rows < 0 || cols < 0) return -1;
+    if (rows == 0 || cols == 0) return 0;
+    if (!out || !a || !b) return -1;
+    // physical extent of the output block
+    const size_t R = trans_o ? cols : rows;
+    const size_t C = trans_o ? rows : cols;
+    if (ldo < static_cast<int>(R)) return -1;
+    const int rel_a = (trans_a != 0) != (trans_o != 0);
+    const int rel_b = (trans_b != 0) != (trans_o != 0);
+    if (lda < static_cast<int>(rel_a ? C : R) || ldb < static_cast<int>(rel_b ? C : R)) return -1;
+    // contiguous, identically laid out operands: flat vectorised kernel
+    if (!rel_a && !rel_b && static_cast<size_t>(ldo) == R && static_cast<size_t>(lda) == R &&
+        static_cast<size_t>(ldb) == R) {
+        return OP == kOpAxpby ? jzhip_axpby(out, a, b, R * C, s1, s2) : jzhip_hadamard(out, a, b, R * C);
+    }
+    return launch2d<OP>(out, ldo, a, lda, rel_a, b, ldb, rel_b, R, C, s1, s2);
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_axpby2d(float* out, int ldo, int trans_o, const float* a, int lda, int trans_a,
+                         const float* b, int ldb, int trans_b, int rows, int cols, float s1,
+                         float s2) {
+    return binary2d<kOpAxpby>(out, ldo, trans_o, a, lda, trans_a, b, ldb, trans_b, rows, cols, s1, s2);
+}
+
+JZ_API int jzhip_hadamard2d(float* out, int ldo, int trans_o, const float* a, int lda, int trans_a,
+                            const float* b, int ldb, int trans_b, int rows, int cols) {
+    return binary2d<kOpHadamard>(out, ldo, trans_o, a, lda, trans_a, b, ldb, trans_b, rows, cols, 1.f,
+                                 1.f);
+}
+
+JZ_API int jzhip_copy2d(float* dst, int ldd, int trans_d, size_t dr0, size_t dc0, const float* src,
+                        int lds, int trans_s, size_t sr0, size_t sc0, size_t rows, size_t cols) {
+    if (rows == 0 || cols == 0) return 0;
+    if (!dst || !src || ldd <= 0 || lds <= 0) return -1;
+    // move to the destination's physical frame
+    const size_t R = trans_d ? cols : rows;
+    const size_t C = trans_d ? rows : cols;
+    float* d0 = dst + (trans_d ? dr0 * ldd + dc0 : dc0 * ldd + dr0);
+    const float* s0 = src + (trans_s ? sr0 * lds + sc0 : sc0 * lds + sr0);
+    const int rel = (trans_s != 0) != (trans_d != 0);
+    if (!rel && static_cast<size_t>(ldd) == R && static_cast<size_t>(lds) == R) {
+        return jzhip_copy(d0, s0, R * C);
+    }
+    return launch2d<kOpCopy>(d0, ldd, s0, lds, rel, nullptr, 0, 0, R, C, 1.f, 0.f);
+}
+
+// hstack/vstack building blocks (cpp/hipmatrix.cpp:447-527): copy the logical
+// content of a possibly transposed source into a column / row offset of a
+// plain column-major destination.
+JZ_API int jzhip_stack_copy_cols(float* dst, size_t dst_numrow, size_t dst_col_offset,
+                                 const float* src, size_t src_numrow, size_t src_numcol,
+                                 int src_transpose) {
+    const size_t rows = src_transpose ? src_numcol : src_numrow;
+    const size_t cols = src_transpose ? src_numrow : src_numcol;
+    return jzhip_copy2d(dst, static_cast<int>(dst_numrow), 0, 0, dst_col_offset, src,
+                        static_cast<int>(src_numrow), src_transpose, 0, 0, rows, cols);
+}
+
+JZ_API int jzhip_stack_copy_rows(float* dst, size_t dst_numrow, size_t dst_row_offset,
+                                 const float* src, size_t src_numrow, size_t src_numcol,
+                                 int src_transpose) {
+    const size_t rows = src_transpose ? src_numcol : src_numrow;
+    const size_t cols = src_transpose ? src_numrow : src_numcol;
+    return jzhip_copy2d(dst, static_cast<int>(dst_numrow), 0, dst_row_offset, 0, src,
+                        static_cast<int>(src_numrow), src_transpose, 0, 0, rows, cols);
+}
+
+// slice get / set (cpp/hipmatrix.cpp:268-324).
+JZ_API int jzhip_slice_extract(float* dst, size_t dst_numrow, const float* src, size_t src_numrow,
+                               int src_transpose, size_t rstart, size_t cstart, size_t rows,
+                               size_t cols) {
+    return jzhip_copy2d(dst, static_cast<int>(dst_numrow), 0, 0, 0, src,
+                        static_cast<int>(src_numrow), src_transpose, rstart, cstart, rows, cols);
+}
+
+JZ_API int jzhip_slice_assign(float* dst, size_t dst_numrow, int dst_transpose, size_t rstart,
+                              size_t cstart, const float* src, size_t src_numrow,
+                              int src_transpose, size_t rows, size_t cols) {
+    return jzhip_copy2d(dst, static_cast<int>(dst_numrow), dst_transpose, rstart, cstart, src,
+                        static_cast<int>(src_numrow), src_transpose, 0, 0, rows, cols);
+}

@@ -1,0 +1,354 @@
+// Fixed-function reductions: column / row sums, Frobenius norm, column max
+// and argmax.  All are HBM-bound single reads of the operand
+// (4*(numrow*numcol + outputs) bytes).  Within a wavefront values are combined
+// with DPP row operations, across waves through LDS, and across workgroups
+// through a two-phase partial buffer, so results are deterministic (no float
+// atomics on global memory).
+#include "common.hpp"
+
+#include <cmath>
+
+namespace jz {
+namespace {
+
+// ── column sums: out[j] = sum_i a[j*ld + i] ──────────────────────────────
+// One wavefront per (column, row-chunk).  VEC=4 uses float4 loads and needs
+// ld % 4 == 0, a 16-byte aligned base and chunk boundaries that are multiples
+// of 4.
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const float* a, int numrow,
+                                                          int numcol, size_t ld, int chunks,
+                                                          int chunk_len) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    const size_t items = static_cast<size_t>(numcol) * chunks;
+    for (size_t it = wave0; it < items; it += nwaves) {
+        const int col = static_cast<int>(it % numcol);
+        const int chunk = static_cast<int>(it / numcol);
+        const int r_begin = chunk * chunk_len;
+        int r_end = r_begin + chunk_len;
+        if (r_end > numrow) r_end = numrow;
+        const float* p = a + static_cast<size_t>(col) * ld;
+        float acc0 = 0.f, acc1 = 0.f;
+        if constexpr (VEC == 4) {
+            const int v_end = r_begin + ((r_end - r_begin) / 4) * 4;
+            int r = r_begin + lane * 4;
+            for (; r + kWave * 4 < v_end; r += 2 * kWave * 4) {
+                const float4 x = *reinterpret_cast<const float4*>(p + r);
+                const float4 y = *reinterpret_cast<const float4*>(p + r + kWave * 4);
+                acc0 += (x.x + x.y) + (x.z + x.w);
+                acc1 += (y.x + y.y) + (y.z + y.w);
+            }
+            for (; r < v_end; r += kWave * 4) {
+                const float4 x = *reinterpret_cast<const float4*>(p + r);
+                acc0 += (x.x + x.y) + (x.z + x.w);
+            }
+            for (int t = v_end + lane; t < r_end; t += kWave) acc1 += p[t];
+        } else {
+            for (int r = r_begin + lane; r < r_end; r += kWave) acc0 += p[r];
+        }
+        const float s = wave_sum(acc0 + acc1);
+        if (lane == 0) out[static_cast<size_t>(chunk) * numcol + col] = s;
+    }
+}
+
+// out[i] = sum_{c<chunks} part[c*n + i]
+__global__ __launch_bounds__(kBlock) void combine_partials_kernel(float* out, const float* part,
+                                                                  int n, int chunks) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    float acc = 0.f;
+    for (int c = 0; c < chunks; ++c) acc += part[static_cast<size_t>(c) * n + i];
+    out[i] = acc;
+}
+
+// ── row sums: out[i] = sum_j a[j*ld + i] ─────────────────────────────────
+// Lanes run along rows (the contiguous dimension); the four waves of a block
+// take interleaved columns of the block's column chunk and are combined
+// through LDS.  VEC rows per lane.
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void sum_rows_kernel(float* out, const float* a, int numrow,
+                                                          int numcol, size_t ld, int chunk_len) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][kWave * VEC];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = (blockIdx.x * kWave + lane) * VEC;
+    const int chunk = blockIdx.y;
+    const int c_begin = chunk * chunk_len;
+    int c_end = c_begin + chunk_len;
+    if (c_end > numcol) c_end = numcol;
+
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+    if (row < numrow) {
+        if constexpr (VEC == 4) {
+            // numrow % 4 == 0 is guaranteed by the launcher
+            int c = c_begin + wave;
+            for (; c + NW < c_end; c += 2 * NW) {
+                const float4 x = *reinterpret_cast<const float4*>(a + static_cast<size_t>(c) * ld + row);
+                const float4 y =
+                    *reinterpret_cast<const float4*>(a + static_cast<size_t>(c + NW) * ld + row);
+                acc[0] += x.x; acc[1] += x.y; acc[2] += x.z; acc[3] += x.w;
+                acc[0] += y.x; acc[1] += y.y; acc[2] += y.z; acc[3] += y.w;
+            }
+            for (; c < c_end; c += NW) {
+                const float4 x = *reinterpret_cast<const float4*>(a + static_cast<size_t>(c) * ld + row);
+                acc[0] += x.x; acc[1] += x.y; acc[2] += x.z; acc[3] += x.w;
+            }
+        } else {
+            for (int c = c_begin + wave; c < c_end; c += NW) acc[0] += a[static_cast<size_t>(c) * ld + row];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) red[wave][lane * VEC + v] = acc[v];
+    __syncthreads();
+    if (wave == 0 && row < numrow) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) s += red[w][lane * VEC + v];
+            out[static_cast<size_t>(chunk) * numrow + row + v] = s;
+        }
+    }
+}
+
+// Row sums of a short, contiguous matrix (numrow <= 64, ld == numrow): the
+// buffer is read as one flat stream; each thread strides by a multiple of
+// numrow so it always lands on the same row, then threads of equal row are
+// combined through LDS.
+__global__ __launch_bounds__(kBlock) void sum_rows_short_kernel(float* part, const float* a,
+                                                                int numrow, size_t total,
+                                                                int active, size_t span) {
+    __shared__ float red[kBlock];
+    const int t = threadIdx.x;
+    const size_t begin = static_cast<size_t>(blockIdx.x) * span;  // multiple of numrow
+    size_t end = begin + span;
+    if (end > total) end = total;
+    float acc0 = 0.f, acc1 = 0.f;
+    if (t < active) {
+        size_t i = begin + t;
+        for (; i + active < end; i += 2 * static_cast<size_t>(active)) {
+            acc0 += a[i];
+            acc1 += a[i + active];
+        }
+        if (i < end) acc0 += a[i];
+    }
+    red[t] = acc0 + acc1;
+    __syncthreads();
+    if (t < numrow) {
+        float s = 0.f;
+        for (int k = t; k < active; k += numrow) s += red[k];
+        part[static_cast<size_t>(blockIdx.x) * numrow + t] = s;
+    }
+}
+
+// ── flat sum of squares (norm) ───────────────────────────────────────────
+__global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(float* part, const float* x, size_t n,
+                                                               int vec_ok) {
+    __shared__ float red[kBlock / kWave];
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    float acc0 = 0.f, acc1 = 0.f;
+    if (vec_ok) {
+        const size_t n4 = n / 4;
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+        size_t i = tid;
+        for (; i + stride < n4; i += 2 * stride) {
+            const float4 p = x4[i], q = x4[i + stride];
+            acc0 += (p.x * p.x + p.y * p.y) + (p.z * p.z + p.w * p.w);
+            acc1 += (q.x * q.x + q.y * q.y) + (q.z * q.z + q.w * q.w);
+        }
+        if (i < n4) {
+            const float4 p = x4[i];
+            acc0 += (p.x * p.x + p.y * p.y) + (p.z * p.z + p.w * p.w);
+        }
+        for (size_t j = n4 * 4 + tid; j < n; j += stride) acc1 += x[j] * x[j];
+    } else {
+        for (size_t i = tid; i < n; i += stride) acc0 += x[i] * x[i];
+    }
+    const float s = block_allreduce<kBlock / kWave>(acc0 + acc1, SumOp{}, red, 0.f);
+    if (threadIdx.x == 0) part[blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(kBlock) void sqrt_sum_kernel(float* out, const float* part, int n) {
+    __shared__ float red[kBlock / kWave];
+    float acc = 0.f;
+    for (int i = threadIdx.x; i < n; i += kBlock) acc += part[i];
+    const float s = block_allreduce<kBlock / kWave>(acc, SumOp{}, red, 0.f);
+    if (threadIdx.x == 0) out[0] = sqrtf(s);
+}
+
+// ── column max / argmax: one wavefront per column ────────────────────────
+template <bool ARG>
+__global__ __launch_bounds__(kBlock) void max_cols_kernel(float* out_val, int32_t* out_idx,
+                                                          const float* a, int numrow, int numcol,
+                                                          size_t ld) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t col = wave0; col < static_cast<size_t>(numcol); col += nwaves) {
+        const float* p = a + col * ld;
+        // std::max_element order: keep the incumbent unless a later element is
+        // strictly greater, so the first maximum wins (ml/util.cuh:104-110)
+        float best = -INFINITY;
+        int bidx = 0x7fffffff;
+        if (lane < numrow) {
+            best = p[lane];
+            bidx = lane;
+        }
+        for (int r = lane + kWave; r < numrow; r += kWave) {
+            const float v = p[r];
+            if (best < v) {
+                best = v;
+                bidx = r;
+            }
+        }
+        if constexpr (ARG) {
+            // butterfly on (value, index): larger value wins, ties -> smaller index
+#pragma unroll
+            for (int off = 1; off < kWave; off <<= 1) {
+                const float ov = __shfl_xor(best, off, kWave);
+                const int oi = __shfl_xor(bidx, off, kWave);
+                if (ov > best || (ov == best && oi < bidx)) {
+                    best = ov;
+                    bidx = oi;
+                }
+            }
+            if (lane == 0) out_idx[col] = bidx;
+        } else {
+            const float m = wave_max(best);
+            if (lane == 0) out_val[col] = m;
+        }
+    }
+}
+
+int pick_chunks(size_t independent, size_t length, size_t min_len) {
+    // enough (independent x chunks) work items to give every SIMD a few waves
+    const size_t want = static_cast<size_t>(num_cus()) * 16;
+    if (independent >= want) return 1;
+    size_t chunks = (want + independent - 1) / independent;
+    const size_t max_chunks = length / min_len;
+    if (chunks > max_chunks) chunks = max_chunks;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 1024) chunks = 1024;
+    return static_cast<int>(chunks);
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow) return -1;
+    if (!out || !a) return -1;
+    const bool vec = aligned16(a) && (ld % 4 == 0);
+    int chunks = pick_chunks(numcol, numrow, 2048);
+    while (chunks > 1 && static_cast<size_t>(chunks) * numcol > kWorkspaceFloats) --chunks;
+    int chunk_len = (numrow + chunks - 1) / chunks;
+    chunk_len = (chunk_len + 3) & ~3;  // keep float4 alignment of chunk starts
+    chunks = (numrow + chunk_len - 1) / chunk_len;
+    float* dst = out;
+    if (chunks > 1) {
+        dst = workspace();
+        if (!dst) return -2;
+    }
+    const size_t items = static_cast<size_t>(numcol) * chunks;
+    const unsigned grid = grid_for(items, kBlock / kWave, 8);
+    hipStream_t s = stream();
+    if (vec)
+        sum_cols_kernel<4><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
+    else
+        sum_cols_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
+    if (chunks > 1) {
+        combine_partials_kernel<<<(numcol + kBlock - 1) / kBlock, kBlock, 0, s>>>(out, dst, numcol,
+                                                                                  chunks);
+    }
+    return launch_rc();
+}
+
+JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow) return -1;
+    if (!out || !a) return -1;
+    hipStream_t s = stream();
+    if (numrow <= kWave && ld == numrow) {
+        // short contiguous matrix: flat stream
+        const size_t total = static_cast<size_t>(numrow) * numcol;
+        const int active = (kBlock / numrow) * numrow;
+        // columns per block so that there are a few blocks per CU
+        size_t blocks = (total + static_cast<size_t>(active) * 16 - 1) / (static_cast<size_t>(active) * 16);
+        const size_t cap = static_cast<size_t>(num_cus()) * 8;
+        if (blocks > cap) blocks = cap;
+        if (blocks < 1) blocks = 1;
+        while (blocks > 1 && blocks * numrow > kWorkspaceFloats) blocks /= 2;
+        size_t cols_per_block = (numcol + blocks - 1) / blocks;
+        blocks = (numcol + cols_per_block - 1) / cols_per_block;
+        const size_t span = cols_per_block * numrow;
+        float* dst = out;
+        if (blocks > 1) {
+            dst = workspace();
+            if (!dst) return -2;
+        }
+        sum_rows_short_kernel<<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(dst, a, numrow, total,
+                                                                              active, span);
+        if (blocks > 1) {
+            combine_partials_kernel<<<(numrow + kBlock - 1) / kBlock, kBlock, 0, s>>>(
+                out, dst, numrow, static_cast<int>(blocks));
+        }
+        return launch_rc();
+    }
+    const bool vec = aligned16(a) && (ld % 4 == 0) && (numrow % 4 == 0);
+    const int rows_per_block = kWave * (vec ? 4 : 1);
+    const int row_blocks = (numrow + rows_per_block - 1) / rows_per_block;
+    int chunks = pick_chunks(row_blocks * (kBlock / kWave), numcol, 64);
+    while (chunks > 1 && static_cast<size_t>(chunks) * numrow > kWorkspaceFloats) --chunks;
+    if (chunks > 65535) chunks = 65535;
+    const int chunk_len = (numcol + chunks - 1) / chunks;
+    chunks = (numcol + chunk_len - 1) / chunk_len;
+    float* dst = out;
+    if (chunks > 1) {
+        dst = workspace();
+        if (!dst) return -2;
+    }
+    dim3 grid(row_blocks, chunks);
+    if (vec)
+        sum_rows_kernel<4><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
+    else
+        sum_rows_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
+    if (chunks > 1) {
+        combine_partials_kernel<<<(numrow + kBlock - 1) / kBlock, kBlock, 0, s>>>(out, dst, numrow,
+                                                                                  chunks);
+    }
+    return launch_rc();
+}
+
+JZ_API int jzhip_nrm2(float* out_device, const float* x, size_t count) {
+    if (!out_device) return -1;
+    if (count == 0) return jzhip_fill(out_device, 1, 0.f);
+    if (!x) return -1;
+    float* part = workspace();
+    if (!part) return -2;
+    const unsigned grid = grid_for(count / 4 + 1, static_cast<size_t>(kBlock) * 2, 4);
+    hipStream_t s = stream();
+    sumsq_partial_kernel<<<grid, kBlock, 0, s>>>(part, x, count, aligned16(x) ? 1 : 0);
+    sqrt_sum_kernel<<<1, kBlock, 0, s>>>(out_device, part, static_cast<int>(grid));
+    return launch_rc();
+}
+
+JZ_API int jzhip_max_cols(float* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
+    const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+    max_cols_kernel<false><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
+    return launch_rc();
+}
+
+JZ_API int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
+    const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+    max_cols_kernel<true><<<grid, kBlock, 0, stream()>>>(nullptr, out, a, numrow, numcol, ld);
+    return launch_rc();
+}

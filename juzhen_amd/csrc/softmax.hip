@@ -1,0 +1,402 @@
+// Single-pass fused softmax kernels.
+//
+// The reference builds a softmax from ~9 generic matrix ops (max reduce,
+// rank-1 broadcast, subtract, exp, ones-GEMV sum, reciprocal, rank-1 broadcast,
+// Hadamard: ml/layer.hpp:2344-2358); here each distribution is read once,
+// kept in registers, and written once: 8 bytes per element.
+//
+// Arithmetic follows the reference expression: m = max(x) (floor -1e30f),
+// e = expf(x - m), p = e * (1.0f / (sum(e) + 1e-12f)).
+#include "common.hpp"
+
+#include <cmath>
+
+namespace jz {
+namespace {
+
+// Optional pre-processing of attention scores: x*scale and the causal mask
+// (key index > query index -> -1e9f, ml/layer.hpp:2979-2994).
+struct ScoreXform {
+    float scale;
+    int causal;
+    int S;  // block edge; 0 = plain softmax
+};
+
+// ── distributions along contiguous columns ───────────────────────────────
+// One wavefront per column, NV values per lane held in registers
+// (numrow <= 64*NV).
+template <int NV>
+__global__ __launch_bounds__(kBlock) void softmax_cols_kernel(float* out, const float* in,
+                                                              int numrow, size_t numcol, size_t ld,
+                                                              ScoreXform xf) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t col = wave0; col < numcol; col += nwaves) {
+        const float* p = in + col * ld;
+        float* q = out + col * ld;
+        const int qidx = xf.S ? static_cast<int>(col % xf.S) : 0;  // query index of this column
+        float x[NV];
+        float m = -1e30f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            if (r < numrow) {
+                float t = p[r];
+                if (xf.S) {
+                    t = t * xf.scale;
+                    if (xf.causal && r > qidx) t = -1e9f;
+                }
+                x[v] = t;
+                m = m > t ? m : t;
+            } else {
+                x[v] = -INFINITY;
+            }
+        }
+        m = wave_max(m);
+        float s = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            x[v] = (r < numrow) ? expf(x[v] - m) : 0.f;
+            s += x[v];
+        }
+        s = wave_sum(s);
+        const float inv = 1.0f / (s + 1e-12f);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            if (r < numrow) q[r] = x[v] * inv;
+        }
+    }
+}
+
+// Long columns (numrow > 1024): one block per column, three sweeps; the
+// second and third hit L2.
+__global__ __launch_bounds__(kBlock) void softmax_cols_long_kernel(float* out, const float* in,
+                                                                   int numrow, size_t numcol,
+                                                                   size_t ld) {
+    __shared__ float red[kBlock / kWave];
+    for (size_t col = blockIdx.x; col < numcol; col += gridDim.x) {
+        const float* p = in + col * ld;
+        float* q = out + col * ld;
+        float m = -1e30f;
+        for (int r = threadIdx.x; r < numrow; r += kBlock) m = m > p[r] ? m : p[r];
+        m = block_allreduce<kBlock / kWave>(m, MaxOp{}, red, -1e30f);
+        float s = 0.f;
+        for (int r = threadIdx.x; r < numrow; r += kBlock) s += expf(p[r] - m);
+        s = block_allreduce<kBlock / kWave>(s, SumOp{}, red, 0.f);
+        const float inv = 1.0f / (s + 1e-12f);
+        for (int r = threadIdx.x; r < numrow; r += kBlock) q[r] = expf(p[r] - m) * inv;
+    }
+}
+
+// ── distributions along rows (stride ld) ─────────────────────────────────
+// A block owns RPB consecutive rows of one matrix (blockIdx.y selects the
+// matrix of a batch); its 256 threads are RPB row lanes x (256/RPB) column
+// phases, so global accesses are coalesced along the rows.  Max and sum are
+// combined across the column phases through LDS.
+template <int RPB>
+__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(float* out, const float* in,
+                                                              int numrow, int numcol, size_t ld,
+                                                              size_t batch_stride, ScoreXform xf) {
+    constexpr int CP = kBlock / RPB;
+    __shared__ float red[CP][RPB];
+    const int rl = threadIdx.x % RPB;
+    const int cp = threadIdx.x / RPB;
+    const int row = blockIdx.x * RPB + rl;
+    const float* p = in + static_cast<size_t>(blockIdx.y) * batch_stride;
+    float* q = out + static_cast<size_t>(blockIdx.y) * batch_stride;
+    const bool live = row < numrow;
+    // with a causal mask only keys <= query (columns <= row) are unmasked;
+    // masked entries contribute expf(-1e9 - m) == 0 exactly and are written as 0
+    const int c_live = (xf.S && xf.causal) ? (row + 1 < numcol ? row + 1 : numcol) : numcol;
+
+    float m = -1e30f;
+    if (live) {
+        for (int c = cp; c < c_live; c += CP) {
+            float t = p[static_cast<size_t>(c) * ld + row];
+            if (xf.S) t = t * xf.scale;
+            m = m > t ? m : t;
+        }
+        if (c_live < numcol) m = m > -1e9f ? m : -1e9f;
+    }
+    red[cp][rl] = m;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < CP; ++k) m = m > red[k][rl] ? m : red[k][rl];
+    __syncthreads();
+
+    float s = 0.f;
+    if (live) {
+        for (int c = cp; c < c_live; c += CP) {
+            float t = p[static_cast<size_t>(c) * ld + row];
+            if (xf.S) t = t * xf.scale;
+            s += expf(t - m);
+        }
+    }
+    red[cp][rl] = s;
+    __syncthreads();
+    s = 0.f;
+#pragma unroll
+    for (int k = 0; k < CP; ++k) s += red[k][rl];
+    const float inv = 1.0f / (s + 1e-12f);
+    if (live) {
+        for (int c = cp; c < numcol; c += CP) {
+            float r = 0.f;
+            if (c < c_live) {
+                float t = p[static_cast<size_t>(c) * ld + row];
+                if (xf.S) t = t * xf.scale;
+                r = expf(t - m) * inv;
+            } else {
+                r = expf(-1e9f - m) * inv;
+            }
+            q[static_cast<size_t>(c) * ld + row] = r;
+        }
+    }
+}
+
+// ── softmax backward: dS = A*(dA - sum_keys(A*dA))*scale ─────────────────
+template <int NV>
+__global__ __launch_bounds__(kBlock) void softmax_bwd_cols_kernel(float* dS, const float* A,
+                                                                  const float* dA, int numrow,
+                                                                  size_t numcol, float scale) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t col = wave0; col < numcol; col += nwaves) {
+        const size_t base = col * numrow;
+        float a[NV], g[NV];
+        float dot = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            a[v] = r < numrow ? A[base + r] : 0.f;
+            g[v] = r < numrow ? dA[base + r] : 0.f;
+            dot += a[v] * g[v];
+        }
+        dot = wave_sum(dot);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            if (r < numrow) dS[base + r] = (a[v] * (g[v] - dot)) * scale;
+        }
+    }
+}
+
+template <int RPB>
+__global__ __launch_bounds__(kBlock) void softmax_bwd_rows_kernel(float* dS, const float* A,
+                                                                  const float* dA, int S,
+                                                                  float scale) {
+    constexpr int CP = kBlock / RPB;
+    __shared__ float red[CP][RPB];
+    const int rl = threadIdx.x % RPB;
+    const int cp = threadIdx.x / RPB;
+    const int row = blockIdx.x * RPB + rl;
+    const size_t off = static_cast<size_t>(blockIdx.y) * S * S;
+    const bool live = row < S;
+    float dot = 0.f;
+    if (live) {
+        for (int c = cp; c < S; c += CP) {
+            const size_t i = off + static_cast<size_t>(c) * S + row;
+            dot += A[i] * dA[i];
+        }
+    }
+    red[cp][rl] = dot;
+    __syncthreads();
+    dot = 0.f;
+#pragma unroll
+    for (int k = 0; k < CP; ++k) dot += red[k][rl];
+    if (live) {
+        for (int c = cp; c < S; c += CP) {
+            const size_t i = off + static_cast<size_t>(c) * S + row;
+            dS[i] = (A[i] * (dA[i] - dot)) * scale;
+        }
+    }
+}
+
+// ── softmax cross-entropy against integer labels ─────────────────────────
+// One wavefront per sample column.  per_sample[n] = x[label] - lse.
+template <int NV>
+__global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, float* dlogits,
+                                                           const float* logits,
+                                                           const int32_t* labels, int K, int N,
+                                                           size_t ld, float inv_n) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+        const float* p = logits + col * ld;
+        const int label = labels[col];
+        float x[NV];
+        float m = -1e30f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            x[v] = r < K ? p[r] : -INFINITY;
+            if (r < K) m = m > x[v] ? m : x[v];
+        }
+        m = wave_max(m);
+        float s = 0.f, picked = 0.f;
+        float e[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = lane + v * kWave;
+            e[v] = r < K ? expf(x[v] - m) : 0.f;
+            s += e[v];
+            if (r == label) picked = x[v];
+        }
+        s = wave_sum(s);
+        picked = wave_sum(picked);
+        if (lane == 0) per_sample[col] = picked - (logf(s) + m);
+        if (dlogits) {
+            // -(y - E/Z)/N with E/Z = e * (float)(1.0/(double)Z)  (ml/layer.hpp:258-261)
+            const float invz = static_cast<float>(1.0 / static_cast<double>(s));
+            float* d = dlogits + col * ld;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const int r = lane + v * kWave;
+                if (r < K) {
+                    const float y = (r == label) ? 1.0f : 0.0f;
+                    d[r] = -(y - e[v] * invz) * inv_n;
+                }
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void neg_mean_kernel(float* out, const float* v, int n,
+                                                          float inv_n) {
+    __shared__ float red[kBlock / kWave];
+    float acc = 0.f;
+    for (int i = threadIdx.x; i < n; i += kBlock) acc += v[i];
+    const float s = block_allreduce<kBlock / kWave>(acc, SumOp{}, red, 0.f);
+    if (threadIdx.x == 0) out[0] = -s * inv_n;
+}
+
+template <template <int> class Launcher, class... Args>
+int dispatch_nv(int numrow, Args... args) {
+    if (numrow <= 64) return Launcher<1>::run(args...);
+    if (numrow <= 128) return Launcher<2>::run(args...);
+    if (numrow <= 256) return Launcher<4>::run(args...);
+    if (numrow <= 512) return Launcher<8>::run(args...);
+    return Launcher<16>::run(args...);
+}
+
+template <int NV>
+struct SoftmaxColsL {
+    static int run(float* out, const float* in, int numrow, size_t numcol, size_t ld, ScoreXform xf) {
+        const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+        softmax_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld, xf);
+        return launch_rc();
+    }
+};
+template <int NV>
+struct SoftmaxBwdColsL {
+    static int run(float* dS, const float* A, const float* dA, int numrow, size_t numcol, float scale) {
+        const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+        softmax_bwd_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(dS, A, dA, numrow, numcol, scale);
+        return launch_rc();
+    }
+};
+template <int NV>
+struct XentL {
+    static int run(float* per_sample, float* dlogits, const float* logits, const int32_t* labels,
+                   int K, int N, size_t ld) {
+        const unsigned grid = grid_for(N, kBlock / kWave, 8);
+        xent_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, labels, K, N,
+                                                            ld, static_cast<float>(1.0 / N));
+        return launch_rc();
+    }
+};
+
+int softmax_cols_impl(float* out, const float* in, int numrow, size_t numcol, size_t ld,
+                      ScoreXform xf) {
+    if (numrow <= 1024) return dispatch_nv<SoftmaxColsL>(numrow, out, in, numrow, numcol, ld, xf);
+    if (xf.S) return -1;
+    const unsigned grid = grid_for(numcol, 1, 8);
+    softmax_cols_long_kernel<<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld);
+    return launch_rc();
+}
+
+int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_t ld, int batch,
+                      size_t batch_stride, ScoreXform xf) {
+    if (batch > 65535) return -1;
+    // small problems: 16-row strips give 4x more blocks than 64-row strips
+    const bool small = static_cast<size_t>((numrow + 63) / 64) * batch < static_cast<size_t>(num_cus()) * 2;
+    if (small) {
+        dim3 grid((numrow + 15) / 16, batch);
+        softmax_rows_kernel<16><<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+    } else {
+        dim3 grid((numrow + 63) / 64, batch);
+        softmax_rows_kernel<64><<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+    }
+    return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_softmax_cols(float* out, const float* in, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !in) return -1;
+    return softmax_cols_impl(out, in, numrow, numcol, ld, ScoreXform{1.f, 0, 0});
+}
+
+JZ_API int jzhip_softmax_rows(float* out, const float* in, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !in) return -1;
+    return softmax_rows_impl(out, in, numrow, numcol, ld, 1, 0, ScoreXform{1.f, 0, 0});
+}
+
+JZ_API int jzhip_attn_softmax(float* out, const float* in, int S, int nblk, float scale,
+                              int causal, int keys_along_rows) {
+    if (S <= 0 || nblk <= 0 || !out || !in) return -1;
+    const ScoreXform xf{scale, causal ? 1 : 0, S};
+    if (keys_along_rows) {
+        return softmax_cols_impl(out, in, S, static_cast<size_t>(S) * nblk, S, xf);
+    }
+    // blocks are independent S x S matrices; split the batch over grid.y
+    int done = 0;
+    while (done < nblk) {
+        const int nb = (nblk - done) < 65535 ? (nblk - done) : 65535;
+        const size_t off = static_cast<size_t>(done) * S * S;
+        int rc = softmax_rows_impl(out + off, in + off, S, S, S, nb, static_cast<size_t>(S) * S, xf);
+        if (rc) return rc;
+        done += nb;
+    }
+    return 0;
+}
+
+JZ_API int jzhip_attn_softmax_bwd(float* dS, const float* A, const float* dA, int S, int nblk,
+                                  float scale, int keys_along_rows) {
+    if (S <= 0 || nblk <= 0 || !dS || !A || !dA) return -1;
+    if (keys_along_rows) {
+        if (S > 1024) return -1;
+        return dispatch_nv<SoftmaxBwdColsL>(S, dS, A, dA, S, static_cast<size_t>(S) * nblk, scale);
+    }
+    int done = 0;
+    while (done < nblk) {
+        const int nb = (nblk - done) < 65535 ? (nblk - done) : 65535;
+        const size_t off = static_cast<size_t>(done) * S * S;
+        dim3 grid((S + 63) / 64, nb);
+        softmax_bwd_rows_kernel<64><<<grid, kBlock, 0, stream()>>>(dS + off, A + off, dA + off, S, scale);
+        int rc = launch_rc();
+        if (rc) return rc;
+        done += nb;
+    }
+    return 0;
+}
+
+JZ_API int jzhip_softmax_xent(float* loss_out, float* dlogits, const float* logits,
+                              const int32_t* labels, int K, int N, int ld) {
+    if (K <= 0 || N <= 0 || ld < K || !loss_out || !logits || !labels) return -1;
+    if (K > 1024) return -1;
+    if (static_cast<size_t>(N) > kWorkspaceFloats) return -1;
+    float* per_sample = workspace();
+    if (!per_sample) return -2;
+    int rc = dispatch_nv<XentL>(K, per_sample, dlogits, logits, labels, K, N, static_cast<size_t>(ld));
+    if (rc) return rc;
+    neg_mean_kernel<<<1, kBlock, 0, stream()>>>(loss_out, per_sample, N, static_cast<float>(1.0 / N));
+    return launch_rc();
+}

@@ -1,0 +1,68 @@
+"""The C-ABI library loads and exports every symbol include/jzhip.h declares,
+and the ctypes table mirrors the header.  No compute calls: runs without a GPU."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "jzhip.h"
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(jzhip_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_reference_device_api():
+    """One entry point per Juzhen::Rocm* function of cpp/hipbackend.hpp:10-136."""
+    names = set(declared_symbols())
+    rocm = ["runtime_available", "malloc", "free", "memcpy_h2d", "memcpy_d2h", "memcpy_d2d", "rand_uniform",
+            "rand_normal", "fill", "exp_inplace", "log_inplace", "axpby", "affine_inplace", "hadamard",
+            "hadamard_inplace", "eleminv_inplace", "copy", "square", "square_inplace", "tanh", "tanh_inplace",
+            "dtanh", "dtanh_inplace", "stack_copy_cols", "stack_copy_rows", "slice_extract", "slice_assign",
+            "gemm", "gemv", "gemm_nn", "im2col", "col2im", "conv_forward_reshape_bias", "conv_backward_reshape",
+            "convtrans_scatter", "convtrans_gather", "convtrans_reshape"]
+    assert len(rocm) == 37
+    for r in rocm:
+        assert "jzhip_" + r in names, r
+
+
+def test_library_exports_every_declared_symbol():
+    from juzhen_amd import capi
+    if not capi.LIB_PATH.exists():
+        pytest.fail(f"{capi.LIB_PATH} not built: run python -m juzhen_amd.build")
+    lib = ctypes.CDLL(str(capi.LIB_PATH))
+    missing = [n for n in declared_symbols() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_ctypes_table_matches_header():
+    from juzhen_amd import capi
+    assert sorted(capi.SIGNATURES) == declared_symbols()
+    # argument counts agree with the prototypes
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    for name, (_, args) in capi.SIGNATURES.items():
+        m = re.search(r"\b" + name + r"\s*\(([^;]*?)\)\s*;", text, flags=re.S)
+        assert m, name
+        params = m.group(1).strip()
+        n = 0 if params in ("", "void") else params.count(",") + 1
+        assert n == len(args), (name, n, len(args))
+
+
+def test_argument_validation_without_gpu():
+    """Null pointers and non-positive sizes are rejected with rc -1 before any launch
+    (cpp/hipmatrix.cpp:611-612,672-674)."""
+    from juzhen_amd import capi
+    lib = capi.load()
+    assert lib.jzhip_gemm(None, None, None, 2, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0) == -1
+    assert lib.jzhip_gemm(None, None, None, 0, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0) == -1
+    assert lib.jzhip_gemv(None, None, None, 2, 2, 0, 2, 1, 1, 1.0, 0.0) == -1
+    assert lib.jzhip_sum_cols(None, None, 4, 4, 4) == -1
+    assert lib.jzhip_im2col(None, None, 1, 4, 4, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    assert lib.jzhip_layernorm_fwd(None, None, None, None, None, None, 8, 8) == -1
+    assert lib.jzhip_adam_update(None, None, None, 4, 1e-3, 0.9, 0.999, 1e-8, 1) == -1
+    assert lib.jzhip_fill(None, 0, 1.0) == 0          # empty input is a no-op
+    assert lib.jzhip_error_string(-1).decode().startswith("jzhip")
+    assert lib.jzhip_version() >= 100

@@ -1,0 +1,636 @@
+"""GPU parity: every C-ABI entry point against the CPU oracle on identical
+seeded inputs.  Tolerances are the ones the task fixes: bit-exact for index
+maps and argmax; relative 1e-5 for elementwise ops; 1e-4 for reductions,
+softmax and LayerNorm; 1e-3 for GEMM.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from util import dev_empty, dptr, hptr, max_rel, rel_err, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+TOL_EW = 1e-5
+TOL_RED = 1e-4
+TOL_GEMM = 1e-3
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ── flat elementwise ─────────────────────────────────────────────────────
+UNARY = [
+    ("exp", "jzo_exp", (), lambda r, n: r.normal(0, 2, n)),
+    ("log", "jzo_log", (), lambda r, n: r.uniform(1e-3, 50, n)),
+    ("tanh", "jzo_tanh", (), lambda r, n: r.normal(0, 2, n)),
+    ("dtanh", "jzo_dtanh", (), lambda r, n: r.normal(0, 2, n)),
+    ("square", "jzo_square", (), lambda r, n: r.normal(0, 3, n)),
+    ("relu", "jzo_relu", (), lambda r, n: r.normal(0, 1, n)),
+    ("drelu", "jzo_drelu", (), lambda r, n: r.normal(0, 1, n)),
+    ("sqrt", "jzo_sqrt", (), lambda r, n: r.uniform(0, 9, n)),
+    ("gelu", "jzo_gelu", (), lambda r, n: r.normal(0, 2, n)),
+]
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 255, 1024, 4099, 1 << 20])
+@pytest.mark.parametrize("name,oname,extra,gen", UNARY, ids=[u[0] for u in UNARY])
+def test_unary(gpu, oracle_lib, name, oname, extra, gen, n):
+    x = gen(rng(n), n).astype(np.float32)
+    ref = np.empty_like(x)
+    getattr(oracle_lib, oname)(hptr(ref), hptr(x), n, *extra)
+    dx = to_dev(x)
+    dy = dev_empty(n)
+    getattr(gpu, name)(dptr(dy), dptr(dx), n, *extra)
+    got = to_host(dy)
+    if name in ("square", "relu", "drelu", "sqrt"):
+        assert np.array_equal(got, ref)
+    elif name == "gelu":
+        # oracle evaluates the closed form in double; the kernel in fp32
+        assert np.max(np.abs(got - ref)) <= 1e-6 + TOL_EW * np.max(np.abs(ref))
+    else:
+        assert max_rel(got, ref, floor=1e-30) <= TOL_EW
+    # in-place form returns the same numbers
+    if name in ("exp", "log", "tanh", "dtanh", "square"):
+        getattr(gpu, name + "_inplace")(dptr(dx), n)
+        assert np.array_equal(to_host(dx), got)
+
+
+@pytest.mark.parametrize("n", [1, 5, 1000, 65537])
+def test_unary_unaligned_pointer(gpu, oracle_lib, n):
+    """Sub-buffer views are not 16-byte aligned: the scalar path must agree."""
+    x = rng(1).normal(0, 1, n + 3).astype(np.float32)
+    dx = to_dev(x)
+    dy = dev_empty(n + 3)
+    gpu.exp(C.c_void_p(dy.data_ptr() + 4), C.c_void_p(dx.data_ptr() + 8), n)
+    ref = np.empty(n, dtype=np.float32)
+    oracle_lib.jzo_exp(hptr(ref), hptr(x[2:2 + n].copy()), n)
+    assert max_rel(to_host(dy)[1:1 + n], ref) <= TOL_EW
+
+
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_affine_eleminv_clamp_fill_copy(gpu, oracle_lib, n):
+    r = rng(n)
+    x = r.normal(0, 2, n).astype(np.float32)
+    x[np.abs(x) < 1e-3] = 0.5
+    dx = to_dev(x)
+    dy = dev_empty(n)
+    ref = np.empty_like(x)
+
+    oracle_lib.jzo_affine(hptr(ref), hptr(x), n, 0.37, -1.25)
+    gpu.affine(dptr(dy), dptr(dx), n, 0.37, -1.25)
+    assert np.array_equal(to_host(dy), ref)
+
+    oracle_lib.jzo_eleminv(hptr(ref), hptr(x), n, 0.1)
+    gpu.eleminv(dptr(dy), dptr(dx), n, 0.1)
+    assert np.array_equal(to_host(dy), ref)
+
+    oracle_lib.jzo_clamp(hptr(ref), hptr(x), n, -0.5, 0.75)
+    gpu.clamp(dptr(dy), dptr(dx), n, -0.5, 0.75)
+    assert np.array_equal(to_host(dy), ref)
+
+    gpu.fill(dptr(dy), n, 3.5)
+    assert np.array_equal(to_host(dy), np.full(n, 3.5, np.float32))
+    gpu.copy(dptr(dy), dptr(dx), n)
+    assert np.array_equal(to_host(dy), x)
+
+    # in-place forms
+    d2 = to_dev(x)
+    gpu.affine_inplace(dptr(d2), n, 2.0, 1.0)
+    oracle_lib.jzo_affine(hptr(ref), hptr(x), n, 2.0, 1.0)
+    assert np.array_equal(to_host(d2), ref)
+    d2 = to_dev(x)
+    gpu.eleminv_inplace(dptr(d2), n, 1.0)
+    oracle_lib.jzo_eleminv(hptr(ref), hptr(x), n, 1.0)
+    assert np.array_equal(to_host(d2), ref)
+
+
+@pytest.mark.parametrize("n", [1, 6, 2048, 77777])
+def test_binary_flat(gpu, oracle_lib, n):
+    r = rng(n + 1)
+    a = r.normal(0, 1, n).astype(np.float32)
+    b = r.normal(0, 1, n).astype(np.float32)
+    da, db, do = to_dev(a), to_dev(b), dev_empty(n)
+    ref = np.empty_like(a)
+    oracle_lib.jzo_axpby2d(hptr(ref), n, 0, hptr(a), n, 0, hptr(b), n, 0, n, 1, 1.5, -0.25)
+    gpu.axpby(dptr(do), dptr(da), dptr(db), n, 1.5, -0.25)
+    assert np.array_equal(to_host(do), ref)
+    oracle_lib.jzo_hadamard2d(hptr(ref), n, 0, hptr(a), n, 0, hptr(b), n, 0, n, 1)
+    gpu.hadamard(dptr(do), dptr(da), dptr(db), n)
+    assert np.array_equal(to_host(do), ref)
+    oracle_lib.jzo_drelu_mul(hptr(ref), hptr(a), hptr(b), n)
+    gpu.drelu_mul(dptr(do), dptr(da), dptr(db), n)
+    assert np.array_equal(to_host(do), ref)
+    oracle_lib.jzo_dgelu_mul(hptr(ref), hptr(a), hptr(b), n)
+    gpu.dgelu_mul(dptr(do), dptr(da), dptr(db), n)
+    assert np.max(np.abs(to_host(do) - ref)) <= 1e-6 + TOL_EW * np.max(np.abs(ref))
+    # aliasing: out == a
+    gpu.hadamard_inplace(dptr(da), dptr(db), n)
+    oracle_lib.jzo_hadamard2d(hptr(ref), n, 0, hptr(a), n, 0, hptr(b), n, 0, n, 1)
+    assert np.array_equal(to_host(da), ref)
+
+
+# ── transpose-aware 2-D ops ──────────────────────────────────────────────
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 5), (33, 65), (128, 96), (257, 1000)])
+@pytest.mark.parametrize("to,ta,tb", [(0, 0, 0), (0, 1, 0), (0, 0, 1), (0, 1, 1), (1, 0, 0), (1, 0, 1), (1, 1, 0)])
+def test_axpby_hadamard_2d(gpu, oracle_lib, rows, cols, to, ta, tb):
+    r = rng(rows * 1000 + cols)
+    a = r.normal(0, 1, rows * cols).astype(np.float32)
+    b = r.normal(0, 1, rows * cols).astype(np.float32)
+    ldo = cols if to else rows
+    lda = cols if ta else rows
+    ldb = cols if tb else rows
+    da, db, do = to_dev(a), to_dev(b), dev_empty(rows * cols)
+    ref = np.empty(rows * cols, np.float32)
+    oracle_lib.jzo_axpby2d(hptr(ref), ldo, to, hptr(a), lda, ta, hptr(b), ldb, tb, rows, cols, 0.5, 2.0)
+    gpu.axpby2d(dptr(do), ldo, to, dptr(da), lda, ta, dptr(db), ldb, tb, rows, cols, 0.5, 2.0)
+    assert np.array_equal(to_host(do), ref)
+    oracle_lib.jzo_hadamard2d(hptr(ref), ldo, to, hptr(a), lda, ta, hptr(b), ldb, tb, rows, cols)
+    gpu.hadamard2d(dptr(do), ldo, to, dptr(da), lda, ta, dptr(db), ldb, tb, rows, cols)
+    assert np.array_equal(to_host(do), ref)
+
+
+@pytest.mark.parametrize("ts", [0, 1])
+@pytest.mark.parametrize("td", [0, 1])
+def test_slice_and_stack(gpu, oracle_lib, ts, td):
+    r = rng(ts * 2 + td)
+    R, Cc = 70, 45            # logical source shape
+    src = r.normal(0, 1, R * Cc).astype(np.float32)
+    lds = Cc if ts else R
+    dsrc = to_dev(src)
+    # extract logical block [5:40, 3:30]
+    rows, cols = 35, 27
+    ref = np.zeros(rows * cols, np.float32)
+    oracle_lib.jzo_copy2d(hptr(ref), rows, 0, 0, 0, hptr(src), lds, ts, 5, 3, rows, cols)
+    dout = dev_empty(rows * cols)
+    gpu.slice_extract(dptr(dout), rows, dptr(dsrc), lds, ts, 5, 3, rows, cols)
+    assert np.array_equal(to_host(dout), ref)
+    # assign it into a destination with its own flag at (2, 4)
+    DR, DC = 50, 40
+    dst0 = r.normal(0, 1, DR * DC).astype(np.float32)
+    ldd = DC if td else DR
+    refd = dst0.copy()
+    oracle_lib.jzo_copy2d(hptr(refd), ldd, td, 2, 4, hptr(ref), rows, 0, 0, 0, rows, cols)
+    ddst = to_dev(dst0)
+    gpu.slice_assign(dptr(ddst), ldd, td, 2, 4, dptr(dout), rows, 0, rows, cols)
+    assert np.array_equal(to_host(ddst), refd)
+    # stack copies: logical source placed at a column / row offset
+    big = np.zeros(R * (Cc + 7), np.float32)
+    refb = big.copy()
+    oracle_lib.jzo_copy2d(hptr(refb), R, 0, 0, 7, hptr(src), lds, ts, 0, 0, R, Cc)
+    dbig = to_dev(big)
+    gpu.stack_copy_cols(dptr(dbig), R, 7, dptr(dsrc), lds, (R * Cc) // lds, ts)
+    assert np.array_equal(to_host(dbig), refb)
+    tall = np.zeros((R + 9) * Cc, np.float32)
+    reft = tall.copy()
+    oracle_lib.jzo_copy2d(hptr(reft), R + 9, 0, 9, 0, hptr(src), lds, ts, 0, 0, R, Cc)
+    dtall = to_dev(tall)
+    gpu.stack_copy_rows(dptr(dtall), R + 9, 9, dptr(dsrc), lds, (R * Cc) // lds, ts)
+    assert np.array_equal(to_host(dtall), reft)
+
+
+# ── reductions ───────────────────────────────────────────────────────────
+SHAPES_RED = [(1, 1), (1, 1000), (1000, 1), (3, 8192), (10, 128), (64, 64), (256, 4096), (257, 33),
+              (512, 16384), (1024, 1024), (100000, 3), (1 << 20, 1)]
+
+
+@pytest.mark.parametrize("numrow,numcol", SHAPES_RED)
+def test_sums(gpu, oracle_lib, numrow, numcol):
+    a = rng(numrow + numcol).normal(0, 1, numrow * numcol).astype(np.float32)
+    da = to_dev(a)
+    # the serial fp32 oracle and a tree reduction differ by rounding only:
+    # compare both against float64 and require the kernel to be no worse than 1e-4
+    A = a.reshape(numcol, numrow).astype(np.float64)  # row j = physical column j
+    for which, exact in (("sum_cols", A.sum(axis=1)), ("sum_rows", A.sum(axis=0))):
+        n_out = exact.size
+        ref = np.empty(n_out, np.float32)
+        oracle_lib.jzo_sum_phys(hptr(ref), hptr(a), numrow, numcol, numrow, 0 if which == "sum_cols" else 1)
+        out = dev_empty(n_out)
+        getattr(gpu, which)(dptr(out), dptr(da), numrow, numcol, numrow)
+        got = to_host(out)
+        scale = np.linalg.norm(np.abs(A).sum(axis=1 if which == "sum_cols" else 0))
+        assert np.linalg.norm(got - exact) <= TOL_RED * scale
+        assert np.linalg.norm(got - ref) <= TOL_RED * scale
+
+
+def test_sum_with_padding_ld(gpu, oracle_lib):
+    numrow, numcol, ld = 37, 50, 48
+    a = rng(5).normal(0, 1, ld * numcol).astype(np.float32)
+    da = to_dev(a)
+    for which, dimp, n_out in (("sum_cols", 0, numcol), ("sum_rows", 1, numrow)):
+        ref = np.empty(n_out, np.float32)
+        oracle_lib.jzo_sum_phys(hptr(ref), hptr(a), numrow, numcol, ld, dimp)
+        out = dev_empty(n_out)
+        getattr(gpu, which)(dptr(out), dptr(da), numrow, numcol, ld)
+        assert rel_err(to_host(out), ref) <= TOL_RED
+
+
+@pytest.mark.parametrize("n", [1, 3, 1000, 65536, 1 << 22])
+def test_nrm2(gpu, oracle_lib, n):
+    x = rng(n).normal(0, 1, n).astype(np.float32)
+    out = dev_empty(1)
+    gpu.nrm2(dptr(out), dptr(to_dev(x)), n)
+    exact = np.linalg.norm(x.astype(np.float64))
+    assert abs(to_host(out)[0] - exact) <= TOL_RED * exact
+    assert abs(oracle_lib.jzo_norm(hptr(x), n) - exact) <= 1e-3 * exact
+
+
+@pytest.mark.parametrize("numrow,numcol", [(1, 5), (10, 128), (256, 16384), (1000, 7), (65, 65)])
+def test_max_argmax_cols(gpu, oracle_lib, numrow, numcol):
+    r = rng(numrow * 7 + numcol)
+    # few distinct values -> many ties, so the first-maximum rule is exercised
+    a = r.integers(-3, 4, numrow * numcol).astype(np.float32)
+    da = to_dev(a)
+    refm = np.empty(numcol, np.float32)
+    refi = np.empty(numcol, np.int32)
+    oracle_lib.jzo_max_cols(hptr(refm), hptr(a), numrow, numcol, numrow)
+    oracle_lib.jzo_argmax_cols(hptr(refi), hptr(a), numrow, numcol, numrow)
+    om = dev_empty(numcol)
+    oi = dev_empty(numcol, np.int32)
+    gpu.max_cols(dptr(om), dptr(da), numrow, numcol, numrow)
+    gpu.argmax_cols(dptr(oi), dptr(da), numrow, numcol, numrow)
+    assert np.array_equal(to_host(om), refm)
+    assert np.array_equal(to_host(oi), refi)
+    assert np.array_equal(refi, a.reshape(numcol, numrow).argmax(axis=1).astype(np.int32))
+
+
+# ── GEMM family ──────────────────────────────────────────────────────────
+def naive_gemm64(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc):
+    """Double-precision reference, the method of tests/testCpuLinalg.cu:54-66."""
+    Am = A.astype(np.float64).reshape(-1, lda).T  # physical (lda x cols)
+    Bm = B.astype(np.float64).reshape(-1, ldb).T
+    opA = Am[:k, :m].T if ta else Am[:m, :k]
+    opB = Bm[:n, :k].T if tb else Bm[:k, :n]
+    C0 = Cm.astype(np.float64).reshape(-1, ldc).T.copy()
+    C0[:m, :n] = alpha * (opA @ opB) + beta * C0[:m, :n]
+    return C0.T.reshape(-1)
+
+
+GEMM_SHAPES = [(1, 1, 1), (2, 2, 2), (3, 5, 7), (1, 40, 33), (40, 1, 33), (17, 19, 1), (64, 64, 64),
+               (128, 128, 16), (129, 127, 17), (33, 300, 9), (300, 33, 70), (256, 512, 128),
+               (32, 1000, 288), (10, 128, 1254), (65, 250, 130)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_variants(gpu, oracle_lib, m, n, k, ta, tb):
+    r = rng(m * 10007 + n * 101 + k)
+    for pad, alpha, beta in ((0, 1.0, 0.0), (3, 0.75, -0.5), (0, 1.0, 1.0)):
+        lda = (k if ta else m) + pad
+        ldb = (n if tb else k) + pad
+        ldc = m + pad
+        A = r.normal(0, 1, lda * (m if ta else k)).astype(np.float32)
+        B = r.normal(0, 1, ldb * (k if tb else n)).astype(np.float32)
+        C0 = r.normal(0, 1, ldc * n).astype(np.float32)
+        exact = naive_gemm64(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C0, ldc)
+        ref = C0.copy()
+        oracle_lib.jzo_gemm(ta, tb, m, n, k, alpha, hptr(A), lda, hptr(B), ldb, beta, hptr(ref), ldc)
+        dC = to_dev(C0)
+        gpu.gemm(dptr(to_dev(A)), dptr(to_dev(B)), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc, alpha, beta)
+        got = to_host(dC)
+        assert rel_err(got, exact) <= TOL_GEMM
+        assert rel_err(got, ref) <= TOL_GEMM
+        if pad:
+            # rows m..ldc-1 of every column must be untouched (tests/testCpuLinalg.cu:152-172)
+            g2 = got.reshape(n, ldc)
+            assert np.array_equal(g2[:, m:], C0.reshape(n, ldc)[:, m:])
+
+
+def test_gemm_known_answer(gpu):
+    """tests/testRocmDeviceProof.cu:36-41: [[1,2],[3,4]]*[[5,6],[7,8]] = [[19,22],[43,50]]."""
+    A = np.array([1, 3, 2, 4], np.float32)  # column-major
+    B = np.array([5, 7, 6, 8], np.float32)
+    dC = dev_empty(4)
+    gpu.gemm_nn(dptr(to_dev(A)), dptr(to_dev(B)), dptr(dC), 2, 2, 2, 1.0, 0.0)
+    assert np.array_equal(to_host(dC), np.array([19, 43, 22, 50], np.float32))
+
+
+def test_gemm_rejects_bad_arguments(gpu):
+    from juzhen_amd import capi
+    lib = capi.load()
+    d = dev_empty(16)
+    assert lib.jzhip_gemm(dptr(d), dptr(d), dptr(d), 0, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0) == -1
+    assert lib.jzhip_gemm(None, dptr(d), dptr(d), 2, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0) == -1
+    assert lib.jzhip_gemv(dptr(d), dptr(d), dptr(d), 2, 2, 0, 2, 0, 1, 1.0, 0.0) == -1
+
+
+@pytest.mark.parametrize("m,n,trans", [(1, 1, 0), (5, 3, 0), (5, 3, 1), (1000, 37, 0), (1000, 37, 1), (64, 5000, 0),
+                                       (64, 5000, 1)])
+def test_gemv(gpu, oracle_lib, m, n, trans):
+    r = rng(m + n)
+    lda = m + 2
+    A = r.normal(0, 1, lda * n).astype(np.float32)
+    lx, ly = (m, n) if trans else (n, m)
+    x = r.normal(0, 1, lx).astype(np.float32)
+    y0 = r.normal(0, 1, ly).astype(np.float32)
+    ref = y0.copy()
+    oracle_lib.jzo_gemv(trans, m, n, 0.5, hptr(A), lda, hptr(x), 1, 2.0, hptr(ref), 1)
+    dy = to_dev(y0)
+    gpu.gemv(dptr(to_dev(A)), dptr(to_dev(x)), dptr(dy), m, n, trans, lda, 1, 1, 0.5, 2.0)
+    assert rel_err(to_host(dy), ref) <= TOL_GEMM
+
+
+@pytest.mark.parametrize("ta,tb", [(1, 0), (0, 1), (0, 0)])
+def test_gemm_strided_batched(gpu, oracle_lib, ta, tb):
+    """Attention-shaped batches: per (head, sequence) S x S scores from d_h x S slices."""
+    r = rng(9)
+    S, dh, dk, batch = 48, 16, 64, 5
+    Q = r.normal(0, 1, dk * S * batch).astype(np.float32)
+    K = r.normal(0, 1, dk * S * batch).astype(np.float32)
+    if (ta, tb) == (1, 0):      # scores = Qi^T Ki
+        m, n, k, lda, ldb, sa, sb = S, S, dh, dk, dk, dk * S, dk * S
+    elif (ta, tb) == (0, 1):    # Hi = Vi * Ai^T with Ai (S x S): here B = K viewed (S x dh)
+        m, n, k, lda, ldb, sa, sb = dh, dh, S, dk, dk, dk * S, dk * S
+        tb = 1
+    else:
+        m, n, k, lda, ldb, sa, sb = dh, S, dh, dk, dk, dk * S, dk * S
+    ldc = m
+    out = np.zeros(m * n * batch, np.float32)
+    for b in range(batch):
+        Cb = np.zeros(m * n, np.float32)
+        oracle_lib.jzo_gemm(ta, tb, m, n, k, 1.0, hptr(Q[b * sa:]), lda, hptr(K[b * sb:]), ldb, 0.0, hptr(Cb), ldc)
+        out[b * m * n:(b + 1) * m * n] = Cb
+    dC = dev_empty(m * n * batch)
+    gpu.gemm_strided_batched(dptr(to_dev(Q)), dptr(to_dev(K)), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc,
+                             sa, sb, m * n, batch, 1.0, 0.0)
+    assert rel_err(to_host(dC), out) <= TOL_GEMM
+
+
+def test_add_bias(gpu):
+    r = rng(3)
+    for rows, cols in ((512, 100), (10, 33), (1, 7)):
+        y = r.normal(0, 1, rows * cols).astype(np.float32)
+        b = r.normal(0, 1, rows).astype(np.float32)
+        dy = to_dev(y)
+        gpu.add_bias(dptr(dy), dptr(to_dev(b)), rows, cols)
+        assert np.array_equal(to_host(dy), (y.reshape(cols, rows) + b[None, :]).reshape(-1))
+
+
+# ── softmax family ───────────────────────────────────────────────────────
+@pytest.mark.parametrize("rows,cols", [(1, 1), (10, 128), (64, 9), (100, 300), (256, 2048), (1024, 64), (3000, 5)])
+def test_softmax_cols_rows(gpu, oracle_lib, rows, cols):
+    x = rng(rows + cols).normal(0, 3, rows * cols).astype(np.float32)
+    dx = to_dev(x)
+    out = dev_empty(rows * cols)
+    ref = np.empty_like(x)
+    oracle_lib.jzo_softmax_cols(hptr(ref), hptr(x), rows, cols, rows)
+    gpu.softmax_cols(dptr(out), dptr(dx), rows, cols, rows)
+    got = to_host(out)
+    assert rel_err(got, ref) <= TOL_RED
+    assert np.allclose(got.reshape(cols, rows).sum(axis=1), 1.0, atol=1e-5)
+    oracle_lib.jzo_softmax_rows(hptr(ref), hptr(x), rows, cols, rows)
+    gpu.softmax_rows(dptr(out), dptr(dx), rows, cols, rows)
+    got = to_host(out)
+    assert rel_err(got, ref) <= TOL_RED
+    assert np.allclose(got.reshape(cols, rows).sum(axis=0), 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("S,nblk", [(8, 3), (64, 4), (100, 2), (256, 6)])
+@pytest.mark.parametrize("causal", [0, 1])
+@pytest.mark.parametrize("kar", [0, 1])
+def test_attn_softmax_fwd_bwd(gpu, oracle_lib, S, nblk, causal, kar):
+    r = rng(S * 10 + nblk + causal)
+    n = S * S * nblk
+    x = r.normal(0, 4, n).astype(np.float32)
+    scale = 1.0 / np.sqrt(np.float32(64))
+    ref = np.empty_like(x)
+    oracle_lib.jzo_attn_softmax(hptr(ref), hptr(x), S, nblk, scale, causal, kar)
+    out = dev_empty(n)
+    gpu.attn_softmax(dptr(out), dptr(to_dev(x)), S, nblk, scale, causal, kar)
+    got = to_host(out)
+    assert rel_err(got, ref) <= TOL_RED
+    if causal:
+        blk = got.reshape(nblk, S, S)  # [b, col, row]
+        qi, ki = (np.arange(S)[:, None], np.arange(S)[None, :]) if kar else (np.arange(S)[None, :], np.arange(S)[:, None])
+        assert np.all(blk[:, ki > qi] == 0.0)
+    dA = r.normal(0, 1, n).astype(np.float32)
+    refd = np.empty_like(x)
+    oracle_lib.jzo_attn_softmax_bwd(hptr(refd), hptr(ref), hptr(dA), S, nblk, scale, kar)
+    dS = dev_empty(n)
+    gpu.attn_softmax_bwd(dptr(dS), dptr(to_dev(ref)), dptr(to_dev(dA)), S, nblk, scale, kar)
+    assert rel_err(to_host(dS), refd) <= TOL_RED
+
+
+@pytest.mark.parametrize("K,N", [(10, 128), (256, 4096), (2, 1), (77, 300)])
+def test_softmax_xent(gpu, oracle_lib, K, N):
+    r = rng(K + N)
+    x = r.normal(0, 2, K * N).astype(np.float32)
+    lab = r.integers(0, K, N).astype(np.int32)
+    refd = np.empty_like(x)
+    ref_loss = oracle_lib.jzo_softmax_xent(hptr(refd), hptr(x), hptr(lab), K, N, K)
+    dl = dev_empty(1)
+    dd = dev_empty(K * N)
+    gpu.softmax_xent(dptr(dl), dptr(dd), dptr(to_dev(x)), dptr(to_dev(lab)), K, N, K)
+    assert abs(to_host(dl)[0] - ref_loss) <= TOL_RED * abs(ref_loss)
+    assert rel_err(to_host(dd), refd) <= TOL_RED
+    # closed form in float64
+    X = x.reshape(N, K).astype(np.float64)
+    lse = np.log(np.exp(X - X.max(1, keepdims=True)).sum(1)) + X.max(1)
+    exact = -(X[np.arange(N), lab] - lse).mean()
+    assert abs(to_host(dl)[0] - exact) <= TOL_RED * abs(exact)
+
+
+# ── LayerNorm ────────────────────────────────────────────────────────────
+@pytest.mark.parametrize("dim,N", [(4, 3), (256, 512), (512, 1024), (1024, 33), (100, 77), (1030, 9), (513, 5)])
+def test_layernorm(gpu, oracle_lib, dim, N):
+    r = rng(dim + N)
+    x = r.normal(0.3, 2, dim * N).astype(np.float32)
+    gamma = r.normal(1, 0.2, dim).astype(np.float32)
+    beta = r.normal(0, 0.2, dim).astype(np.float32)
+    y, xh, inv = (np.empty(dim * N, np.float32), np.empty(dim * N, np.float32), np.empty(N, np.float32))
+    oracle_lib.jzo_layernorm_fwd(hptr(y), hptr(xh), hptr(inv), hptr(x), hptr(gamma), hptr(beta), dim, N)
+    dy_, dxh, dinv = dev_empty(dim * N), dev_empty(dim * N), dev_empty(N)
+    dg, db = to_dev(gamma), to_dev(beta)
+    gpu.layernorm_fwd(dptr(dy_), dptr(dxh), dptr(dinv), dptr(to_dev(x)), dptr(dg), dptr(db), dim, N)
+    assert rel_err(to_host(dy_), y) <= TOL_RED
+    assert rel_err(to_host(dxh), xh) <= TOL_RED
+    assert rel_err(to_host(dinv), inv) <= TOL_RED
+    # float64 closed form
+    X = x.reshape(N, dim).astype(np.float64)
+    mu = X.mean(1, keepdims=True)
+    var = ((X - mu) ** 2).mean(1, keepdims=True)
+    exact = (X - mu) / np.sqrt(var + 1e-5) * gamma + beta
+    assert rel_err(to_host(dy_), exact.reshape(-1)) <= TOL_RED
+
+    g = r.normal(0, 1, dim * N).astype(np.float32)
+    dx = np.empty(dim * N, np.float32)
+    oracle_lib.jzo_layernorm_bwd(hptr(dx), hptr(g), hptr(gamma), hptr(xh), hptr(inv), dim, N)
+    ddx = dev_empty(dim * N)
+    gpu.layernorm_bwd(dptr(ddx), dptr(to_dev(g)), dptr(dg), dptr(to_dev(xh)), dptr(to_dev(inv)), dim, N)
+    assert rel_err(to_host(ddx), dx) <= TOL_RED
+
+    rg, rb = np.empty(dim, np.float32), np.empty(dim, np.float32)
+    oracle_lib.jzo_layernorm_param_grads(hptr(rg), hptr(rb), hptr(g), hptr(xh), dim, N)
+    og, ob = dev_empty(dim), dev_empty(dim)
+    gpu.layernorm_param_grads(dptr(og), dptr(ob), dptr(to_dev(g)), dptr(to_dev(xh)), dim, N)
+    G = g.reshape(N, dim).astype(np.float64)
+    XH = xh.reshape(N, dim).astype(np.float64)
+    sg = np.linalg.norm(np.abs(G * XH).sum(0))
+    sb = np.linalg.norm(np.abs(G).sum(0))
+    assert np.linalg.norm(to_host(og) - (G * XH).sum(0)) <= TOL_RED * sg
+    assert np.linalg.norm(to_host(ob) - G.sum(0)) <= TOL_RED * sb
+    assert np.linalg.norm(to_host(og) - rg) <= TOL_RED * sg
+
+
+# ── Adam ─────────────────────────────────────────────────────────────────
+@pytest.mark.parametrize("n", [1, 5, 4096, 1 << 20])
+def test_adam_bit_exact(gpu, oracle_lib, n):
+    r = rng(n)
+    g0 = r.normal(0, 1, n).astype(np.float32)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    dm, dv = to_dev(m), to_dev(v)
+    for it in range(1, 6):
+        g = (g0 * np.float32(1.0 / it)).astype(np.float32)
+        dg = to_dev(g)
+        oracle_lib.jzo_adam_update(hptr(g), hptr(m), hptr(v), n, 1e-3, 0.9, 0.999, 1e-8, it)
+        gpu.adam_update(dptr(dg), dptr(dm), dptr(dv), n, 1e-3, 0.9, 0.999, 1e-8, it)
+        assert np.array_equal(to_host(dg), g)
+        assert np.array_equal(to_host(dm), m)
+        assert np.array_equal(to_host(dv), v)
+    # step 1 closed form: update = alpha * g/(|g| + eps*...) ~ alpha*sign(g)
+    g = g0.copy()
+    m[:] = 0
+    v[:] = 0
+    oracle_lib.jzo_adam_update(hptr(g), hptr(m), hptr(v), n, 1e-3, 0.9, 0.999, 1e-8, 1)
+    big = np.abs(g0) > 1e-3
+    assert np.allclose(g[big], 1e-3 * np.sign(g0[big]), rtol=1e-4)
+
+
+@pytest.mark.parametrize("wd", [0.0, 0.01])
+def test_adamw_step(gpu, oracle_lib, wd):
+    n = 10007
+    r = rng(11)
+    w = r.normal(0, 1, n).astype(np.float32)
+    g = r.normal(0, 1, n).astype(np.float32)
+    m = r.normal(0, 0.1, n).astype(np.float32)
+    v = r.uniform(0, 0.1, n).astype(np.float32)
+    dw, dg, dm, dv = to_dev(w), to_dev(g), to_dev(m), to_dev(v)
+    oracle_lib.jzo_adamw_step(hptr(w), hptr(g), hptr(m), hptr(v), n, 3e-4, 0.9, 0.999, 1e-8, wd, 7)
+    gpu.adamw_step(dptr(dw), dptr(dg), dptr(dm), dptr(dv), n, 3e-4, 0.9, 0.999, 1e-8, wd, 7)
+    assert np.array_equal(to_host(dw), w)
+    assert np.array_equal(to_host(dm), m)
+    assert np.array_equal(to_host(dv), v)
+    assert np.array_equal(to_host(dg), g)
+
+
+# ── convolution data movement (bit-exact) ────────────────────────────────
+CONV_CASES = [
+    # N, C, H, W, kH, kW, pad, stride
+    (2, 1, 5, 5, 3, 3, 1, 1),
+    (3, 2, 7, 6, 3, 3, 0, 1),
+    (2, 3, 8, 8, 3, 3, 1, 2),
+    (2, 4, 9, 7, 2, 2, 0, 2),
+    (1, 2, 6, 6, 5, 5, 2, 1),
+    (4, 1, 28, 28, 3, 3, 1, 1),
+    (2, 32, 28, 28, 3, 3, 1, 2),
+    (2, 3, 10, 10, 4, 4, 1, 2),
+    (2, 5, 7, 9, 3, 2, 1, 3),
+]
+
+
+def conv_dims(H, W, kH, kW, pad, stride):
+    return (H + 2 * pad - kH) // stride + 1, (W + 2 * pad - kW) // stride + 1
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_im2col_col2im(gpu, oracle_lib, case):
+    N, Cc, H, W, kH, kW, pad, stride = case
+    Ho, Wo = conv_dims(H, W, kH, kW, pad, stride)
+    K, P = Cc * kH * kW, Ho * Wo
+    r = rng(sum(case))
+    x = r.normal(0, 1, Cc * H * W * N).astype(np.float32)
+    col = np.empty(K * P * N, np.float32)
+    args = (Cc, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    oracle_lib.jzo_im2col(hptr(x), hptr(col), *args)
+    dcol = dev_empty(K * P * N)
+    gpu.im2col(dptr(to_dev(x)), dptr(dcol), *args)
+    assert np.array_equal(to_host(dcol), col)
+
+    c2 = r.normal(0, 1, K * P * N).astype(np.float32)
+    dx = np.empty(Cc * H * W * N, np.float32)
+    oracle_lib.jzo_col2im(hptr(c2), hptr(dx), *args)
+    ddx = dev_empty(Cc * H * W * N)
+    gpu.col2im(dptr(to_dev(c2)), dptr(ddx), *args)
+    assert np.array_equal(to_host(ddx), dx)
+    # adjoint identity <im2col(x), c> == <x, col2im(c)>
+    lhs = np.dot(col.astype(np.float64), c2.astype(np.float64))
+    rhs = np.dot(x.astype(np.float64), dx.astype(np.float64))
+    assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs))
+
+
+@pytest.mark.parametrize("C_out,P,N", [(1, 1, 1), (32, 784, 4), (3, 50, 7), (64, 196, 2), (33, 65, 3)])
+def test_conv_reshapes(gpu, oracle_lib, C_out, P, N):
+    r = rng(C_out + P + N)
+    n = C_out * P * N
+    y2d = r.normal(0, 1, n).astype(np.float32)
+    bias = r.normal(0, 1, C_out).astype(np.float32)
+    ref = np.empty(n, np.float32)
+    oracle_lib.jzo_conv_forward_reshape_bias(hptr(y2d), hptr(ref), hptr(bias), C_out, P, N)
+    out = dev_empty(n)
+    gpu.conv_forward_reshape_bias(dptr(to_dev(y2d)), dptr(out), dptr(to_dev(bias)), C_out, P, N)
+    assert np.array_equal(to_host(out), ref)
+    back = np.empty(n, np.float32)
+    oracle_lib.jzo_conv_backward_reshape(hptr(ref), hptr(back), C_out, P, N)
+    dback = dev_empty(n)
+    gpu.conv_backward_reshape(dptr(out), dptr(dback), C_out, P, N)
+    assert np.array_equal(to_host(dback), back)
+    for direction in (0, 1):
+        oracle_lib.jzo_convtrans_reshape(hptr(y2d), hptr(ref), C_out, P, N, direction)
+        gpu.convtrans_reshape(dptr(to_dev(y2d)), dptr(out), C_out, P, N, direction)
+        assert np.array_equal(to_host(out), ref)
+
+
+CT_CASES = [
+    # N, C_out, H_in, W_in, kH, kW, pad, stride
+    (2, 3, 4, 4, 4, 4, 1, 2),
+    (1, 2, 5, 3, 3, 3, 0, 1),
+    (2, 4, 8, 8, 4, 4, 1, 2),
+    (3, 1, 3, 5, 2, 2, 0, 2),
+    (2, 2, 4, 4, 3, 3, 1, 3),
+]
+
+
+@pytest.mark.parametrize("case", CT_CASES)
+def test_convtrans_scatter_gather(gpu, oracle_lib, case):
+    N, Co, Hi, Wi, kH, kW, pad, stride = case
+    Ho = (Hi - 1) * stride - 2 * pad + kH
+    Wo = (Wi - 1) * stride - 2 * pad + kW
+    R, Pin = Co * kH * kW, Hi * Wi
+    r = rng(sum(case))
+    patches = r.normal(0, 1, R * Pin * N).astype(np.float32)
+    bias = r.normal(0, 1, Co).astype(np.float32)
+    args = (Co, Ho, Wo, Hi, Wi, kH, kW, pad, pad, stride, stride, N)
+    ref = np.empty(Co * Ho * Wo * N, np.float32)
+    oracle_lib.jzo_convtrans_scatter(hptr(patches), hptr(ref), hptr(bias), *args)
+    out = dev_empty(ref.size)
+    gpu.convtrans_scatter(dptr(to_dev(patches)), dptr(out), dptr(to_dev(bias)), *args)
+    assert np.array_equal(to_host(out), ref)
+    t = r.normal(0, 1, ref.size).astype(np.float32)
+    tp = np.empty(R * Pin * N, np.float32)
+    oracle_lib.jzo_convtrans_gather(hptr(t), hptr(tp), *args)
+    dtp = dev_empty(tp.size)
+    gpu.convtrans_gather(dptr(to_dev(t)), dptr(dtp), *args)
+    assert np.array_equal(to_host(dtp), tp)
+
+
+# ── random numbers: range / moments only (tests/testRocmCpuParity.cu:214-224) ──
+def test_rand(gpu):
+    n = 1 << 20
+    d = dev_empty(n)
+    gpu.rand_uniform(dptr(d), n, 123)
+    u = to_host(d)
+    assert np.all(np.isfinite(u)) and u.min() >= 0.0 and u.max() < 1.0
+    assert abs(u.mean() - 0.5) < 5e-3 and abs(u.var() - 1 / 12) < 5e-3
+    gpu.rand_normal(dptr(d), n, 1.0, 2.0, 0)
+    z = to_host(d)
+    assert np.all(np.isfinite(z))
+    assert abs(z.mean() - 1.0) < 2e-2 and abs(z.std() - 2.0) < 2e-2
+    # seed != 0 restarts the stream, seed == 0 continues it
+    gpu.rand_uniform(dptr(d), 1000, 123)
+    assert np.array_equal(to_host(d)[:1000], u[:1000])
+    gpu.rand_uniform(dptr(d), 1000, 0)
+    assert not np.array_equal(to_host(d)[:1000], u[:1000])

@@ -1,0 +1,41 @@
+"""Helpers shared by the parity tests (numpy <-> device buffers <-> oracle)."""
+import ctypes as C
+
+import numpy as np
+
+
+def dptr(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def hptr(a):
+    return C.c_void_p(a.ctypes.data)
+
+
+def to_dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def to_host(t):
+    return t.cpu().numpy()
+
+
+def dev_empty(n, dtype=np.float32):
+    import torch
+    return torch.empty(int(n), dtype=torch.float32 if dtype == np.float32 else torch.int32, device="cuda")
+
+
+def rel_err(got, ref):
+    """Relative Frobenius error, the reference tests' norm-based criterion
+    (tests/testRocmCpuParity.cu:20-30)."""
+    got = np.asarray(got, dtype=np.float64).ravel()
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    den = np.linalg.norm(ref)
+    return np.linalg.norm(got - ref) / (den if den > 0 else 1.0)
+
+
+def max_rel(got, ref, floor=1e-30):
+    got = np.asarray(got, dtype=np.float64).ravel()
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
