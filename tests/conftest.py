@@ -27,3 +27,10 @@ def gpu():
     from juzhen_amd import capi
     capi.load()  # raises if libjzhip.so is missing: no fallback
     return capi.jz
+
+
+@pytest.fixture(autouse=True)
+def _release_kept_buffers():
+    yield
+    import util
+    util._KEEP.clear()

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import dev_empty, dptr, hptr, max_rel, rel_err, to_dev, to_host
+from util import dev_empty, dp, dptr, hp, hptr, max_rel, rel_err, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +51,13 @@ def test_unary(gpu, oracle_lib, name, oname, extra, gen, n):
     elif name == "gelu":
         # oracle evaluates the closed form in double; the kernel in fp32
         assert np.max(np.abs(got - ref)) <= 1e-6 + TOL_EW * np.max(np.abs(ref))
+    elif name == "dtanh":
+        # 1 - tanh(x)^2 cancels for |x| > 2, so a 1-ulp difference between the two
+        # tanhf implementations is amplified in the element's own relative error;
+        # the criterion is norm-wise (as in tests/testRocmCpuParity.cu:20-30) plus
+        # an absolute bound of two ulps of the operand tanh(x)^2 ~ 1
+        assert rel_err(got, ref) <= TOL_EW
+        assert np.max(np.abs(got - ref)) <= 2.4e-7
     else:
         assert max_rel(got, ref, floor=1e-30) <= TOL_EW
     # in-place form returns the same numbers
@@ -67,7 +74,7 @@ def test_unary_unaligned_pointer(gpu, oracle_lib, n):
     dy = dev_empty(n + 3)
     gpu.exp(C.c_void_p(dy.data_ptr() + 4), C.c_void_p(dx.data_ptr() + 8), n)
     ref = np.empty(n, dtype=np.float32)
-    oracle_lib.jzo_exp(hptr(ref), hptr(x[2:2 + n].copy()), n)
+    oracle_lib.jzo_exp(hptr(ref), hp(x[2:2 + n].copy()), n)
     assert max_rel(to_host(dy)[1:1 + n], ref) <= TOL_EW
 
 
@@ -232,10 +239,14 @@ def test_sum_with_padding_ld(gpu, oracle_lib):
 def test_nrm2(gpu, oracle_lib, n):
     x = rng(n).normal(0, 1, n).astype(np.float32)
     out = dev_empty(1)
-    gpu.nrm2(dptr(out), dptr(to_dev(x)), n)
+    gpu.nrm2(dptr(out), dp(x), n)
     exact = np.linalg.norm(x.astype(np.float64))
     assert abs(to_host(out)[0] - exact) <= TOL_RED * exact
-    assert abs(oracle_lib.jzo_norm(hptr(x), n) - exact) <= 1e-3 * exact
+    # the oracle's serial fp32 accumulation (cpp/core.hpp:337-344) itself drifts
+    # from the exact value by up to ~n*eps/2; the kernel must be inside that band
+    band = max(TOL_RED, n * 6e-8) * exact
+    assert abs(oracle_lib.jzo_norm(hptr(x), n) - exact) <= band
+    assert abs(to_host(out)[0] - oracle_lib.jzo_norm(hptr(x), n)) <= band
 
 
 @pytest.mark.parametrize("numrow,numcol", [(1, 5), (10, 128), (256, 16384), (1000, 7), (65, 65)])
@@ -289,7 +300,7 @@ def test_gemm_variants(gpu, oracle_lib, m, n, k, ta, tb):
         ref = C0.copy()
         oracle_lib.jzo_gemm(ta, tb, m, n, k, alpha, hptr(A), lda, hptr(B), ldb, beta, hptr(ref), ldc)
         dC = to_dev(C0)
-        gpu.gemm(dptr(to_dev(A)), dptr(to_dev(B)), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc, alpha, beta)
+        gpu.gemm(dp(A), dp(B), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc, alpha, beta)
         got = to_host(dC)
         assert rel_err(got, exact) <= TOL_GEMM
         assert rel_err(got, ref) <= TOL_GEMM
@@ -304,7 +315,7 @@ def test_gemm_known_answer(gpu):
     A = np.array([1, 3, 2, 4], np.float32)  # column-major
     B = np.array([5, 7, 6, 8], np.float32)
     dC = dev_empty(4)
-    gpu.gemm_nn(dptr(to_dev(A)), dptr(to_dev(B)), dptr(dC), 2, 2, 2, 1.0, 0.0)
+    gpu.gemm_nn(dp(A), dp(B), dptr(dC), 2, 2, 2, 1.0, 0.0)
     assert np.array_equal(to_host(dC), np.array([19, 43, 22, 50], np.float32))
 
 
@@ -329,7 +340,7 @@ def test_gemv(gpu, oracle_lib, m, n, trans):
     ref = y0.copy()
     oracle_lib.jzo_gemv(trans, m, n, 0.5, hptr(A), lda, hptr(x), 1, 2.0, hptr(ref), 1)
     dy = to_dev(y0)
-    gpu.gemv(dptr(to_dev(A)), dptr(to_dev(x)), dptr(dy), m, n, trans, lda, 1, 1, 0.5, 2.0)
+    gpu.gemv(dp(A), dp(x), dptr(dy), m, n, trans, lda, 1, 1, 0.5, 2.0)
     assert rel_err(to_host(dy), ref) <= TOL_GEMM
 
 
@@ -351,10 +362,10 @@ def test_gemm_strided_batched(gpu, oracle_lib, ta, tb):
     out = np.zeros(m * n * batch, np.float32)
     for b in range(batch):
         Cb = np.zeros(m * n, np.float32)
-        oracle_lib.jzo_gemm(ta, tb, m, n, k, 1.0, hptr(Q[b * sa:]), lda, hptr(K[b * sb:]), ldb, 0.0, hptr(Cb), ldc)
+        oracle_lib.jzo_gemm(ta, tb, m, n, k, 1.0, hp(Q[b * sa:]), lda, hp(K[b * sb:]), ldb, 0.0, hptr(Cb), ldc)
         out[b * m * n:(b + 1) * m * n] = Cb
     dC = dev_empty(m * n * batch)
-    gpu.gemm_strided_batched(dptr(to_dev(Q)), dptr(to_dev(K)), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc,
+    gpu.gemm_strided_batched(dp(Q), dp(K), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc,
                              sa, sb, m * n, batch, 1.0, 0.0)
     assert rel_err(to_host(dC), out) <= TOL_GEMM
 
@@ -365,7 +376,7 @@ def test_add_bias(gpu):
         y = r.normal(0, 1, rows * cols).astype(np.float32)
         b = r.normal(0, 1, rows).astype(np.float32)
         dy = to_dev(y)
-        gpu.add_bias(dptr(dy), dptr(to_dev(b)), rows, cols)
+        gpu.add_bias(dptr(dy), dp(b), rows, cols)
         assert np.array_equal(to_host(dy), (y.reshape(cols, rows) + b[None, :]).reshape(-1))
 
 
@@ -399,7 +410,7 @@ def test_attn_softmax_fwd_bwd(gpu, oracle_lib, S, nblk, causal, kar):
     ref = np.empty_like(x)
     oracle_lib.jzo_attn_softmax(hptr(ref), hptr(x), S, nblk, scale, causal, kar)
     out = dev_empty(n)
-    gpu.attn_softmax(dptr(out), dptr(to_dev(x)), S, nblk, scale, causal, kar)
+    gpu.attn_softmax(dptr(out), dp(x), S, nblk, scale, causal, kar)
     got = to_host(out)
     assert rel_err(got, ref) <= TOL_RED
     if causal:
@@ -410,7 +421,7 @@ def test_attn_softmax_fwd_bwd(gpu, oracle_lib, S, nblk, causal, kar):
     refd = np.empty_like(x)
     oracle_lib.jzo_attn_softmax_bwd(hptr(refd), hptr(ref), hptr(dA), S, nblk, scale, kar)
     dS = dev_empty(n)
-    gpu.attn_softmax_bwd(dptr(dS), dptr(to_dev(ref)), dptr(to_dev(dA)), S, nblk, scale, kar)
+    gpu.attn_softmax_bwd(dptr(dS), dp(ref), dp(dA), S, nblk, scale, kar)
     assert rel_err(to_host(dS), refd) <= TOL_RED
 
 
@@ -423,14 +434,16 @@ def test_softmax_xent(gpu, oracle_lib, K, N):
     ref_loss = oracle_lib.jzo_softmax_xent(hptr(refd), hptr(x), hptr(lab), K, N, K)
     dl = dev_empty(1)
     dd = dev_empty(K * N)
-    gpu.softmax_xent(dptr(dl), dptr(dd), dptr(to_dev(x)), dptr(to_dev(lab)), K, N, K)
-    assert abs(to_host(dl)[0] - ref_loss) <= TOL_RED * abs(ref_loss)
+    gpu.softmax_xent(dptr(dl), dptr(dd), dp(x), dp(lab), K, N, K)
+    assert abs(to_host(dl)[0] - ref_loss) <= TOL_RED * (abs(ref_loss) + np.abs(x).max())
     assert rel_err(to_host(dd), refd) <= TOL_RED
     # closed form in float64
     X = x.reshape(N, K).astype(np.float64)
     lse = np.log(np.exp(X - X.max(1, keepdims=True)).sum(1)) + X.max(1)
     exact = -(X[np.arange(N), lab] - lse).mean()
-    assert abs(to_host(dl)[0] - exact) <= TOL_RED * abs(exact)
+    # x[label] - lse cancels when the label dominates, so the bound is relative
+    # to the magnitude of the terms that are subtracted
+    assert abs(to_host(dl)[0] - exact) <= TOL_RED * (abs(exact) + np.abs(lse).mean())
 
 
 # ── LayerNorm ────────────────────────────────────────────────────────────
@@ -444,7 +457,7 @@ def test_layernorm(gpu, oracle_lib, dim, N):
     oracle_lib.jzo_layernorm_fwd(hptr(y), hptr(xh), hptr(inv), hptr(x), hptr(gamma), hptr(beta), dim, N)
     dy_, dxh, dinv = dev_empty(dim * N), dev_empty(dim * N), dev_empty(N)
     dg, db = to_dev(gamma), to_dev(beta)
-    gpu.layernorm_fwd(dptr(dy_), dptr(dxh), dptr(dinv), dptr(to_dev(x)), dptr(dg), dptr(db), dim, N)
+    gpu.layernorm_fwd(dptr(dy_), dptr(dxh), dptr(dinv), dp(x), dptr(dg), dptr(db), dim, N)
     assert rel_err(to_host(dy_), y) <= TOL_RED
     assert rel_err(to_host(dxh), xh) <= TOL_RED
     assert rel_err(to_host(dinv), inv) <= TOL_RED
@@ -459,13 +472,13 @@ def test_layernorm(gpu, oracle_lib, dim, N):
     dx = np.empty(dim * N, np.float32)
     oracle_lib.jzo_layernorm_bwd(hptr(dx), hptr(g), hptr(gamma), hptr(xh), hptr(inv), dim, N)
     ddx = dev_empty(dim * N)
-    gpu.layernorm_bwd(dptr(ddx), dptr(to_dev(g)), dptr(dg), dptr(to_dev(xh)), dptr(to_dev(inv)), dim, N)
+    gpu.layernorm_bwd(dptr(ddx), dp(g), dptr(dg), dp(xh), dp(inv), dim, N)
     assert rel_err(to_host(ddx), dx) <= TOL_RED
 
     rg, rb = np.empty(dim, np.float32), np.empty(dim, np.float32)
     oracle_lib.jzo_layernorm_param_grads(hptr(rg), hptr(rb), hptr(g), hptr(xh), dim, N)
     og, ob = dev_empty(dim), dev_empty(dim)
-    gpu.layernorm_param_grads(dptr(og), dptr(ob), dptr(to_dev(g)), dptr(to_dev(xh)), dim, N)
+    gpu.layernorm_param_grads(dptr(og), dptr(ob), dp(g), dp(xh), dim, N)
     G = g.reshape(N, dim).astype(np.float64)
     XH = xh.reshape(N, dim).astype(np.float64)
     sg = np.linalg.norm(np.abs(G * XH).sum(0))
@@ -547,14 +560,14 @@ def test_im2col_col2im(gpu, oracle_lib, case):
     args = (Cc, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
     oracle_lib.jzo_im2col(hptr(x), hptr(col), *args)
     dcol = dev_empty(K * P * N)
-    gpu.im2col(dptr(to_dev(x)), dptr(dcol), *args)
+    gpu.im2col(dp(x), dptr(dcol), *args)
     assert np.array_equal(to_host(dcol), col)
 
     c2 = r.normal(0, 1, K * P * N).astype(np.float32)
     dx = np.empty(Cc * H * W * N, np.float32)
     oracle_lib.jzo_col2im(hptr(c2), hptr(dx), *args)
     ddx = dev_empty(Cc * H * W * N)
-    gpu.col2im(dptr(to_dev(c2)), dptr(ddx), *args)
+    gpu.col2im(dp(c2), dptr(ddx), *args)
     assert np.array_equal(to_host(ddx), dx)
     # adjoint identity <im2col(x), c> == <x, col2im(c)>
     lhs = np.dot(col.astype(np.float64), c2.astype(np.float64))
@@ -571,7 +584,7 @@ def test_conv_reshapes(gpu, oracle_lib, C_out, P, N):
     ref = np.empty(n, np.float32)
     oracle_lib.jzo_conv_forward_reshape_bias(hptr(y2d), hptr(ref), hptr(bias), C_out, P, N)
     out = dev_empty(n)
-    gpu.conv_forward_reshape_bias(dptr(to_dev(y2d)), dptr(out), dptr(to_dev(bias)), C_out, P, N)
+    gpu.conv_forward_reshape_bias(dp(y2d), dptr(out), dp(bias), C_out, P, N)
     assert np.array_equal(to_host(out), ref)
     back = np.empty(n, np.float32)
     oracle_lib.jzo_conv_backward_reshape(hptr(ref), hptr(back), C_out, P, N)
@@ -580,7 +593,7 @@ def test_conv_reshapes(gpu, oracle_lib, C_out, P, N):
     assert np.array_equal(to_host(dback), back)
     for direction in (0, 1):
         oracle_lib.jzo_convtrans_reshape(hptr(y2d), hptr(ref), C_out, P, N, direction)
-        gpu.convtrans_reshape(dptr(to_dev(y2d)), dptr(out), C_out, P, N, direction)
+        gpu.convtrans_reshape(dp(y2d), dptr(out), C_out, P, N, direction)
         assert np.array_equal(to_host(out), ref)
 
 
@@ -607,13 +620,13 @@ def test_convtrans_scatter_gather(gpu, oracle_lib, case):
     ref = np.empty(Co * Ho * Wo * N, np.float32)
     oracle_lib.jzo_convtrans_scatter(hptr(patches), hptr(ref), hptr(bias), *args)
     out = dev_empty(ref.size)
-    gpu.convtrans_scatter(dptr(to_dev(patches)), dptr(out), dptr(to_dev(bias)), *args)
+    gpu.convtrans_scatter(dp(patches), dptr(out), dp(bias), *args)
     assert np.array_equal(to_host(out), ref)
     t = r.normal(0, 1, ref.size).astype(np.float32)
     tp = np.empty(R * Pin * N, np.float32)
     oracle_lib.jzo_convtrans_gather(hptr(t), hptr(tp), *args)
     dtp = dev_empty(tp.size)
-    gpu.convtrans_gather(dptr(to_dev(t)), dptr(dtp), *args)
+    gpu.convtrans_gather(dp(t), dptr(dtp), *args)
     assert np.array_equal(to_host(dtp), tp)
 
 

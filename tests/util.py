@@ -39,3 +39,22 @@ def max_rel(got, ref, floor=1e-30):
     got = np.asarray(got, dtype=np.float64).ravel()
     ref = np.asarray(ref, dtype=np.float64).ravel()
     return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+
+
+# Device copies made through dp() stay alive until the test ends (conftest
+# clears the list), so a raw pointer never outlives its tensor.
+_KEEP = []
+
+
+def dp(a):
+    """Pointer to a device copy of the numpy array `a`."""
+    t = to_dev(a)
+    _KEEP.append(t)
+    return dptr(t)
+
+
+def hp(a):
+    """Pointer to a host array that is kept alive until the test ends."""
+    a = np.ascontiguousarray(a)
+    _KEEP.append(a)
+    return hptr(a)
