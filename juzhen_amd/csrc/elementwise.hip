@@ -33,10 +33,13 @@ struct LogF {
 struct TanhF {
     __device__ float operator()(float x) const { return tanhf(x); }
 };
-struct DTanhF {  // cpp/matrix.hpp:300-302: 1 - tanh(x)*tanh(x)
+struct DTanhF {
+    // cpp/matrix.hpp:300-302 evaluates 1 - tanh(x)*tanh(x) in double and narrows
+    // on store; the subtraction cancels for |x| > 2, so fp32 would lose the
+    // element's relative accuracy.  Same arithmetic here.
     __device__ float operator()(float x) const {
-        float t = tanhf(x);
-        return 1.0f - t * t;
+        const double t = tanh(static_cast<double>(x));
+        return static_cast<float>(1.0 - t * t);
     }
 };
 struct SquareF {

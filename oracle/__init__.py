@@ -115,3 +115,55 @@ def ptr(a: np.ndarray) -> C.c_void_p:
 
 def f32(a) -> np.ndarray:
     return np.ascontiguousarray(a, dtype=np.float32)
+
+
+PP = C.POINTER(C.c_void_p)
+REF_SIGNATURES = {
+    "jzref_init": (None, []),
+    "jzref_dot": (None, [P, P, I, I, I, P, I, I, I]),
+    "jzref_add": (I, [P, P, I, I, I, P, I, I, I, F, F]),
+    "jzref_add_inplace": (None, [P, I, I, I, P, I, I, I, F, F]),
+    "jzref_hadmd": (I, [P, P, I, I, I, P, I, I, I]),
+    "jzref_unary": (I, [I, P, P, I, D, D]),
+    "jzref_chain": (None, [P, P, I, I, P, I]),
+    "jzref_sum": (None, [P, P, I, I, I, I]),
+    "jzref_norm": (F, [P, I]),
+    "jzref_slice": (None, [P, P, I, I, I, I, I, I, I]),
+    "jzref_slice_assign": (None, [P, I, I, I, I, I, I, I, P, I, I, I]),
+    "jzref_stack2": (None, [P, I, P, I, I, I, P, I, I, I]),
+    "jzref_softmax": (None, [P, P, I, I, I, I]),
+    "jzref_max_cols": (None, [P, P, I, I]),
+    "jzref_adam_update": (None, [P, P, P, I, F, F, F, F, I]),
+    "jzref_layernorm_fwd": (None, [P, P, P, P, P, P, I, I]),
+    "jzref_layernorm_bwd": (None, [P, P, P, P, P, P, P, I, I]),
+    "jzref_logistic": (F, [P, P, P, I, I]),
+    "jzref_conv_eval": (None, [P, P, P, P] + [I] * 10),
+    "jzref_conv_backward": (None, [P, P, P, P, P] + [I] * 10),
+    "jzref_convtrans_eval": (None, [P, P, P, P] + [I] * 10),
+    "jzref_convtrans_backward": (None, [P, P, P, P, P] + [I] * 10),
+    "jzref_block_create": (P, [I, I, I, I, I, I, I]),
+    "jzref_block_destroy": (None, [P]),
+    "jzref_block_param": (I, [P, I, P, I]),
+    "jzref_block_set_lr": (None, [P, F]),
+    "jzref_block_eval": (None, [P, P, P]),
+    "jzref_block_backward": (None, [P, P, P, P, I]),
+    "jzref_mlp_step": (F, [I, P, P, PP, PP, PP, PP, PP, PP, P, P, I, F, I]),
+}
+
+_ref = None
+
+
+def load_ref():
+    """The reference CPU path (oracle/_ref/libjzref.so), or None if it was never built."""
+    global _ref
+    if _ref is None:
+        if not REF_LIB.exists():
+            return None
+        lib = C.CDLL(str(REF_LIB))
+        for name, (res, args) in REF_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        lib.jzref_init()
+        _ref = lib
+    return _ref

@@ -149,16 +149,16 @@ JZO_API void jzo_eleminv(float* out, const float* in, size_t n, double l) {
     for (size_t i = 0; i < n; i++) out[i] = (float)(l / in[i]); /* core.hpp:473,480 */
 }
 JZO_API void jzo_exp(float* out, const float* in, size_t n) {
-    for (size_t i = 0; i < n; i++) out[i] = expf(in[i]); /* matrix.hpp:257,265 */
+    for (size_t i = 0; i < n; i++) out[i] = (float)exp((double)in[i]); /* matrix.hpp:257,265: ::exp(double), narrowed on store */
 }
 JZO_API void jzo_log(float* out, const float* in, size_t n) {
-    for (size_t i = 0; i < n; i++) out[i] = logf(in[i]); /* matrix.hpp:275 */
+    for (size_t i = 0; i < n; i++) out[i] = (float)log((double)in[i]); /* matrix.hpp:275 */
 }
 JZO_API void jzo_tanh(float* out, const float* in, size_t n) {
-    for (size_t i = 0; i < n; i++) out[i] = tanhf(in[i]); /* matrix.hpp:285 */
+    for (size_t i = 0; i < n; i++) out[i] = (float)tanh((double)in[i]); /* matrix.hpp:285 */
 }
 JZO_API void jzo_dtanh(float* out, const float* in, size_t n) {
-    for (size_t i = 0; i < n; i++) out[i] = 1 - tanhf(in[i]) * tanhf(in[i]); /* matrix.hpp:309 */
+    for (size_t i = 0; i < n; i++) out[i] = (float)(1 - tanh((double)in[i]) * tanh((double)in[i])); /* matrix.hpp:309 */
 }
 JZO_API void jzo_square(float* out, const float* in, size_t n) {
     for (size_t i = 0; i < n; i++) out[i] = in[i] * in[i]; /* matrix.hpp:412 */
@@ -250,7 +250,7 @@ JZO_API void jzo_softmax_cols(float* out, const float* in, int rows, int cols, i
         float s = 0.0f;
         for (int i = 0; i < rows; i++) {
             /* M - ones*mx is add(B,1,-1): 1*x + (-1)*m (cpp/core.hpp:446) */
-            o[i] = expf(1.0f * v[i] + -1.0f * (1.0f * m));
+            o[i] = (float)exp((double)(1.0f * v[i] + -1.0f * (1.0f * m)));
             s += o[i] * 1.0f; /* gemv trans with ones: acc += Aj[i]*x[i] */
         }
         float inv = 1.0f / (1.0f * s + 1e-12f);
@@ -265,7 +265,7 @@ JZO_API void jzo_softmax_rows(float* out, const float* in, int rows, int cols, i
         for (int j = 0; j < cols; j++) m = m > in[(size_t)j * ld + i] ? m : in[(size_t)j * ld + i];
         float s = 0.0f;
         for (int j = 0; j < cols; j++) {
-            float e = expf(1.0f * in[(size_t)j * ld + i] + -1.0f * (1.0f * m));
+            float e = (float)exp((double)(1.0f * in[(size_t)j * ld + i] + -1.0f * (1.0f * m)));
             out[(size_t)j * ld + i] = e;
             s += e * 1.0f;
         }
@@ -331,14 +331,14 @@ JZO_API float jzo_softmax_xent(float* d, const float* logits, const int32_t* lab
         float m = -1e30f;
         for (int i = 0; i < K; i++) m = m > v[i] ? m : v[i];
         float s = 0.0f;
-        for (int i = 0; i < K; i++) s += expf(v[i] - m);
-        float lse = logf(s) + m;
+        for (int i = 0; i < K; i++) s += (float)exp((double)(v[i] - m));
+        float lse = (float)log((double)s) + m;
         total += v[labels[n]] - lse;
         if (d) {
             float invz = (float)(1.0 / (double)s); /* E / Z = hadmd(E, Z.eleminv(1.0)) */
             for (int i = 0; i < K; i++) {
                 float y = i == labels[n] ? 1.0f : 0.0f;
-                d[(size_t)n * ld + i] = -(y - expf(v[i] - m) * invz) * invnb;
+                d[(size_t)n * ld + i] = -(y - (float)exp((double)(v[i] - m)) * invz) * invnb;
             }
         }
     }
