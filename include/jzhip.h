@@ -258,6 +258,24 @@ int jzhip_attn_softmax_bwd(float* dS, const float* A, const float* dA, int S,
 int jzhip_softmax_xent(float* loss_out, float* dlogits, const float* logits,
                        const int32_t* labels, int K, int N, int ld);
 
+/* Multi-head self-attention core over the layouts TransformerLayer keeps
+ * (ml/layer.hpp:2843-2848): Q, K, V, H are (d_k, S*B) column-major with head hh
+ * in rows [hh*d_h, (hh+1)*d_h) and sequence b in columns [b*S, (b+1)*S); A is
+ * (S, S*B*heads) with block hh*B + b holding A[query, key].  Forward computes
+ * A = softmax_keys(Q_i^T K_i / sqrt(d_h), causal mask) and H_i = V_i A_i^T for
+ * every (head, sequence): the generic loop of ml/layer.hpp:2967-3006 (CUDA
+ * path :2880-2927) as batched launches with the mask applied on the device. */
+int jzhip_attention_fwd(float* H, float* A, const float* Q, const float* K,
+                        const float* V, int d_k, int heads, int S, int B,
+                        int causal);
+/* Backward of the above (ml/layer.hpp:3329-3363; CUDA path :3214-3283): from dH
+ * and the cached Q, K, V, A writes dQ, dK, dV; dA_scratch is caller-provided
+ * storage of the size of A. */
+int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch,
+                        const float* dH, const float* Q, const float* K,
+                        const float* V, const float* A, int d_k, int heads,
+                        int S, int B);
+
 /* ── LayerNorm ───────────────────────────────────────────────────────── */
 
 /* Per column of x (dim x N): mean, biased variance, inv = 1/sqrt(var+1e-5),

@@ -75,6 +75,130 @@ def build(force: bool = False, jobs: int = 6) -> Path:
     return LIB
 
 
+# ── host-side mirror: Matrix<ROCMfloat> + the reference's own programs ─────────
+#
+# juzhen_amd/cpp holds drop-in replacements for three files of the reference
+# tree (cpp/hipmatrix.cuh, cpp/hipmatrix.cpp, cpp/hipkernels.cpp).  They only
+# compile together with the reference's headers, so this step needs the
+# reference tree.  It never copies reference sources: it builds a directory of
+# symlinks ("overlay") in which those three names point at our files and every
+# other name points into the reference tree, compiles the reference's own
+# ROCm test programs in that overlay against libjzhip.so, and writes the
+# binaries (which contain compiled reference code) to oracle/_ref/bin/.
+REFERENCE_ROOT = Path(os.environ.get("JUZHEN_REFERENCE", "/root/reference"))
+OVERLAY = OBJ / "overlay"
+REF_BIN = ROOT / "oracle" / "_ref" / "bin"
+HOST_SRC = PKG / "cpp"
+OURS = {"hipmatrix.cuh", "hipmatrix.cpp", "hipkernels.cpp"}
+# a writable PROJECT_DIR that exists on any box (tests that dump files use it)
+PROJECT_DIR = "/tmp/jz_project"
+
+REFERENCE_PROGRAMS = [
+    "tests/testRocmDeviceProof.cu",
+    "tests/testRocmOpsSmoke.cu",
+    "tests/testRocmCpuParity.cu",
+    "tests/testbasic.cu",
+    "tests/testStackOps.cu",
+    "tests/testElementwiseReduceTorchDump.cu",
+    "tests/testConvBackendParity.cu",
+    "tests/testUNet.cu",
+    "tests/testTransformerRef.cu",
+    "tests/testTransformer.cu",
+]
+
+HOST_FLAGS = [
+    "-x", "hip", "--offload-arch=gfx950", "-std=c++20", "-O2", "-fPIC",
+    "-DROCM_HIP", "-DLOGGING_OFF", "-DJUZHEN_NO_BLAS", f'-DPROJECT_DIR="{PROJECT_DIR}"',
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-w",
+    f"-I{ROOT / 'include'}",
+]
+
+
+def _link_tree(src_dir: Path, dst_dir: Path, replace: dict[str, Path]):
+    dst_dir.mkdir(parents=True, exist_ok=True)
+    for f in src_dir.iterdir():
+        target = replace.get(f.name, f)
+        link = dst_dir / f.name
+        if link.is_symlink() or link.exists():
+            link.unlink()
+        link.symlink_to(target)
+
+
+def _relink(link: Path, target: Path):
+    if link.is_symlink() or link.exists():
+        link.unlink()
+    link.symlink_to(target)
+
+
+def make_overlay() -> Path:
+    """Symlink farm: the reference tree with our three cpp/ files swapped in,
+    and ml/util.cuh / ml/layer.hpp each followed by the one ROCm hook include a
+    maintainer appends to those files."""
+    _link_tree(REFERENCE_ROOT / "cpp", OVERLAY / "cpp", {n: HOST_SRC / n for n in OURS})
+    for extra in HOST_SRC.glob("hipfused*.hpp"):
+        _relink(OVERLAY / "cpp" / extra.name, extra)
+    _link_tree(REFERENCE_ROOT / "ml", OVERLAY / "ml", {})
+    hooks = {"util.cuh": "hipfused_util.hpp", "layer.hpp": "hipfused.hpp"}
+    for fname, hook in hooks.items():
+        if not (HOST_SRC / hook).exists():
+            continue
+        upstream = OVERLAY / "ml" / ("upstream_" + fname)
+        _relink(upstream, REFERENCE_ROOT / "ml" / fname)
+        wrapper = OVERLAY / "ml" / fname
+        wrapper.unlink()
+        wrapper.write_text(f'#include "./{upstream.name}"\n'
+                           f'#ifdef ROCM_HIP\n#include "../cpp/{hook}"\n#endif\n')
+    _link_tree(REFERENCE_ROOT / "tests", OVERLAY / "tests", {})
+    _link_tree(REFERENCE_ROOT / "examples", OVERLAY / "examples", {})
+    _relink(OVERLAY / "external", REFERENCE_ROOT / "external")
+    return OVERLAY
+
+
+def _hipcc(args: list[str], what: str):
+    r = subprocess.run([HIPCC, *args], capture_output=True, text=True)
+    if r.returncode != 0:
+        err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+        raise RuntimeError(f"{what} failed:\n{err[-6000:]}")
+
+
+def build_host(force: bool = False, jobs: int = 6):
+    """Compile the Matrix<ROCMfloat> mirror and the reference's ROCm programs.
+    Returns the list of binaries, or [] when the reference tree is absent."""
+    if not REFERENCE_ROOT.exists():
+        return sorted(REF_BIN.glob("*")) if REF_BIN.exists() else []
+    build()
+    ov = make_overlay()
+    REF_BIN.mkdir(parents=True, exist_ok=True)
+    hostobj = OBJ / "host"
+    hostobj.mkdir(parents=True, exist_ok=True)
+    ours = [HOST_SRC / n for n in sorted(OURS)] + list(HOST_SRC.glob("*.hpp"))
+
+    def compile_one(rel: str) -> Path:
+        src = ov / rel
+        obj = hostobj / (Path(rel).stem + ".o")
+        if force or _stale(obj, [src.resolve(), *ours, ROOT / "include" / "jzhip.h"]):
+            _hipcc([*HOST_FLAGS, "-c", str(src), "-o", str(obj)], f"compile {rel}")
+        return obj
+
+    lib_srcs = ["cpp/launcher.cu", "cpp/hipmatrix.cpp", "cpp/hipkernels.cpp"]
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        lib_objs = list(ex.map(compile_one, lib_srcs))
+        prog_objs = list(ex.map(compile_one, REFERENCE_PROGRAMS))
+    bins = []
+    for rel, obj in zip(REFERENCE_PROGRAMS, prog_objs):
+        out = REF_BIN / Path(rel).stem
+        if force or _stale(out, [obj, *lib_objs, LIB]):
+            _hipcc(["--offload-arch=gfx950", "-o", str(out), str(obj), *map(str, lib_objs),
+                    f"-L{LIB.parent}", "-ljzhip", "-Wl,-rpath,$ORIGIN/../../../juzhen_amd/lib"],
+                   f"link {out.name}")
+        bins.append(out)
+    return bins
+
+
 if __name__ == "__main__":
     path = build(force="--force" in sys.argv)
     print(path)
+    if "--host" in sys.argv:
+        for b in build_host(force="--force" in sys.argv):
+            print(b)

@@ -85,6 +85,8 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_attn_softmax": (I, [P, P, I, I, F, I, I]),
     "jzhip_attn_softmax_bwd": (I, [P, P, P, I, I, F, I]),
     "jzhip_softmax_xent": (I, [P, P, P, P, I, I, I]),
+    "jzhip_attention_fwd": (I, [P, P, P, P, P, I, I, I, I, I]),
+    "jzhip_attention_bwd": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I]),
     "jzhip_layernorm_fwd": (I, [P, P, P, P, P, P, I, I]),
     "jzhip_layernorm_bwd": (I, [P, P, P, P, P, I, I]),
     "jzhip_layernorm_param_grads": (I, [P, P, P, P, I, I]),

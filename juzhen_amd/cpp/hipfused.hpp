@@ -1,0 +1,165 @@
+// ROCm hook for ml/layer.hpp: include at the very end of that file,
+//
+//     #ifdef ROCM_HIP
+//     #include "../cpp/hipfused.hpp"
+//     #endif
+//
+// the counterpart of the `#ifdef CUDA` / `#ifdef APPLE_SILICON` blocks the
+// reference keeps inside LayerNorm and TransformerLayer (ml/layer.hpp:2595-2631,
+// 2646-2673, 2772-2798, 2880-2965, 3214-3283).  The members below are explicit
+// specialisations for ROCMfloat, so user code and the rest of ml/layer.hpp stay
+// untouched; without this include the generic formulation still compiles, but
+// TransformerLayer's causal mask is then written from the host into device
+// memory while the kernels that produce the scores are still in flight
+// (ml/layer.hpp:2979-2994), which races.
+//
+// What changes against the generic path:
+//   LayerNorm::forward / backward   one kernel each (+ one for dgamma/dbeta)
+//   TransformerLayer::add_bias      one broadcast kernel instead of a rank-1 GEMM
+//   TransformerLayer::eval/backward attention for all heads and sequences as
+//                                   batched GEMMs with the mask and softmax
+//                                   (and its backward) on the device
+#ifndef JZ_HIPFUSED_HPP
+#define JZ_HIPFUSED_HPP
+
+#include "jzhip.h"
+
+namespace Juzhen {
+
+namespace rocm_detail {
+inline float* p(const Matrix<ROCMfloat>& m) { return JzRocmFused::ptr(m); }
+inline void must(int rc, const char* what) {
+    if (rc != 0) {
+        std::cerr << "juzhen rocm: " << what << " failed with code " << rc << " (" << jzhip_error_string(rc)
+                  << ")" << std::endl;
+        ERROR_OUT;
+    }
+}
+// plain column-major copy of a possibly transposed operand
+inline Matrix<ROCMfloat> plain(const Matrix<ROCMfloat>& m) {
+    return m.get_transpose() ? JzRocmFused::materialise(m) : Matrix<ROCMfloat>(m);
+}
+}  // namespace rocm_detail
+
+// ── LayerNorm ────────────────────────────────────────────────────────────────
+
+template <>
+inline Matrix<ROCMfloat> LayerNorm<ROCMfloat>::forward(const Matrix<ROCMfloat>& x) {
+    using namespace rocm_detail;
+    if (x.get_transpose()) return forward(JzRocmFused::materialise(x));
+    const int N = (int)x.num_col();
+    if ((int)cached_xhat.num_col() != N || cached_xhat.get_transpose()) {
+        cached_xhat = Matrix<ROCMfloat>("ln_xhat", dim, N);
+        cached_inv = Matrix<ROCMfloat>("ln_inv", 1, N);
+    }
+    Matrix<ROCMfloat> y("ln_y", dim, N);
+    must(jzhip_layernorm_fwd(p(y), p(cached_xhat), p(cached_inv), p(x), p(gamma), p(beta), dim, N),
+         "layernorm_fwd");
+    return y;
+}
+
+template <>
+inline Matrix<ROCMfloat> LayerNorm<ROCMfloat>::backward(Matrix<ROCMfloat>&& dy, bool update) {
+    using namespace rocm_detail;
+    if (dy.get_transpose()) return backward(JzRocmFused::materialise(dy), update);
+    const int N = (int)dy.num_col();
+    Matrix<ROCMfloat> dx("ln_dx", dim, N);
+    must(jzhip_layernorm_bwd(p(dx), p(dy), p(gamma), p(cached_xhat), p(cached_inv), dim, N), "layernorm_bwd");
+    // dx reads gamma, so the parameter step comes second (ml/layer.hpp:2682-2686)
+    if (update) {
+        Matrix<ROCMfloat> dg("ln_dgamma", dim, 1), db("ln_dbeta", dim, 1);
+        must(jzhip_layernorm_param_grads(p(dg), p(db), p(dy), p(cached_xhat), dim, N), "layernorm_param_grads");
+        gamma -= adam_update(std::move(dg), adam_g);
+        beta -= adam_update(std::move(db), adam_b);
+    }
+    return dx;
+}
+
+// ── TransformerLayer ─────────────────────────────────────────────────────────
+
+template <>
+inline void TransformerLayer<ROCMfloat>::add_bias(Matrix<ROCMfloat>& y, const Matrix<ROCMfloat>& b) {
+    using namespace rocm_detail;
+    if (!y.get_transpose() && !b.get_transpose()) {
+        must(jzhip_add_bias(p(y), p(b), (int)y.num_row(), (int)y.num_col()), "add_bias");
+        return;
+    }
+    y += b * ones_1N;
+}
+
+template <>
+inline void TransformerLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+    using namespace rocm_detail;
+    using MD = Matrix<ROCMfloat>;
+    // pre-norm attention
+    cached_x1 = ln1.forward(input);
+    cached_Q = Wq * cached_x1;
+    cached_K = Wk * cached_x1;
+    cached_V = Wv * cached_x1;
+    must(jzhip_attention_fwd(p(cached_H), p(cached_A), p(cached_Q), p(cached_K), p(cached_V), d_k, num_heads,
+                             seq_len, batchN, causal ? 1 : 0),
+         "attention_fwd");
+    MD O = Wo * cached_H;
+    add_bias(O, bo);
+    cached_R = input + O;
+    // pre-norm feed-forward
+    cached_x2 = ln2.forward(cached_R);
+    cached_F1 = W1 * cached_x2;
+    add_bias(cached_F1, b1);
+    cached_F1_relu = relu(MD(cached_F1));
+    MD F = W2 * cached_F1_relu;
+    add_bias(F, b2);
+    this->val = cached_R + F;
+}
+
+template <>
+inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCMfloat>& input,
+                                                               Matrix<ROCMfloat>&& upstream_grad) {
+    using namespace rocm_detail;
+    using MD = Matrix<ROCMfloat>;
+    const int N = seq_len * batchN;
+    MD dout = plain(upstream_grad);  // read three times below; also the residual gradient
+
+    // feed-forward: F = W2 relu(W1 x2 + b1) + b2
+    MD dW2 = dout * cached_F1_relu.T();
+    MD db2 = sum(dout, 1);
+    MD dF1 = W2.T() * dout;
+    must(jzhip_drelu_mul(p(dF1), p(cached_F1), p(dF1), (size_t)d_ff * N), "drelu_mul");
+    MD dW1 = dF1 * cached_x2.T();
+    MD db1 = sum(dF1, 1);
+    MD dR = ln2.backward(W1.T() * dF1, this->need_update) + dout;
+
+    // output projection: O = Wo H + bo
+    MD dWo = dR * cached_H.T();
+    MD dbo = sum(dR, 1);
+    MD dH = Wo.T() * dR;
+
+    // attention core, all heads and sequences at once
+    MD dQ("dQ", d_k, N), dK("dK", d_k, N), dV("dV", d_k, N);
+    must(jzhip_attention_bwd(p(dQ), p(dK), p(dV), p(attn_dS_scratch), p(dH), p(cached_Q), p(cached_K),
+                             p(cached_V), p(cached_A), d_k, num_heads, seq_len, batchN),
+         "attention_bwd");
+
+    MD dWq = dQ * cached_x1.T();
+    MD dWk = dK * cached_x1.T();
+    MD dWv = dV * cached_x1.T();
+    MD dx1 = Wq.T() * dQ + Wk.T() * dK + Wv.T() * dV;
+    MD dx = ln1.backward(std::move(dx1), this->need_update) + dR;
+
+    if (this->need_update) {
+        Wq -= adam_update(std::move(dWq), adam_Wq);
+        Wk -= adam_update(std::move(dWk), adam_Wk);
+        Wv -= adam_update(std::move(dWv), adam_Wv);
+        Wo -= adam_update(std::move(dWo), adam_Wo);
+        bo -= adam_update(std::move(dbo), adam_bo);
+        W1 -= adam_update(std::move(dW1), adam_W1);
+        b1 -= adam_update(std::move(db1), adam_b1);
+        W2 -= adam_update(std::move(dW2), adam_W2);
+        b2 -= adam_update(std::move(db2), adam_b2);
+    }
+    return dx;
+}
+
+}  // namespace Juzhen
+
+#endif

@@ -1,0 +1,333 @@
+// Matrix<ROCMfloat> for MI355X (gfx950): drop-in for the reference's
+// cpp/hipmatrix.cuh.  The public surface (constructors, members, friends and the
+// free functions) is the one the reference declares (cpp/hipmatrix.cuh:40-162),
+// so cpp/operators.hpp, ml/layer.hpp and user programs compile unchanged.
+// Behind it every operation is one call into the C ABI of libjzhip.so
+// (include/jzhip.h); semantics are those of the CPU Matrix<float>
+// (cpp/core.hpp, cpp/matrix.hpp), including transpose flags on both operands.
+//
+// Additions over the reference header, all ROCm-only and found by ordinary
+// overload resolution (a non-template overload beats the generic template, the
+// mechanism the reference uses for its Metal backend, ml/layer.hpp:2333-2339):
+// fused col_softmax/row_softmax, adam_update, relu/d_relu and predict_one_hot.
+#ifndef HIPMATRIX_CUH
+#define HIPMATRIX_CUH
+
+#ifdef __HIPCC__
+#include <hip/hip_runtime.h>
+#endif
+
+#include <stdexcept>
+#include <vector>
+
+#include "core.hpp"
+#include "hipbackend.hpp"
+#include "matrix.hpp"
+#include "operators.hpp"
+
+// ── pool allocator hooks (cpp/memory.hpp:36-37) ─────────────────────────────
+template <>
+inline ROCMfloat* Memory<ROCMfloat>::_alloc(size_t size) {
+    float* p = nullptr;
+    if (Juzhen::RocmMalloc(&p, size ? size : 1) != 0 || p == nullptr) throw std::bad_alloc();
+    return reinterpret_cast<ROCMfloat*>(p);
+}
+
+template <>
+inline void Memory<ROCMfloat>::_free(ROCMfloat* ptr) {
+    Juzhen::RocmFree(reinterpret_cast<float*>(ptr));
+}
+
+template <class T>
+struct adam_state;
+
+// The stream every library call is enqueued on (include/jzhip.h); the
+// templates below launch on the same one so program order stays device order.
+extern "C" void* jzhip_get_stream(void);
+
+template <>
+class Matrix<ROCMfloat> {
+    // Field names are part of the contract: MatrixView<ROCMfloat> and the
+    // reduce/elemwise templates read them directly.
+    size_t numcol;
+    size_t numrow;
+    bool transpose;
+    std::string name;
+    std::shared_ptr<ROCMfloat[]> elements;
+
+    // view constructor: shares `elements`
+    Matrix<ROCMfloat>(const char* name, size_t numrow, size_t numcol, int trans,
+                      std::shared_ptr<ROCMfloat[]> elements);
+    // owning constructor: takes an uninitialised block from the pool
+    Matrix<ROCMfloat>(const char* name, size_t numrow, size_t numcol, int trans);
+
+    float* dev() const { return reinterpret_cast<float*>(elements.get()); }
+    size_t count() const { return numrow * numcol; }
+
+   public:
+    // ── construction / assignment ──
+    Matrix<ROCMfloat>() : Matrix<ROCMfloat>("un_init", 2, 2, 0) {}
+    Matrix<ROCMfloat>(const char* name, size_t numrow, size_t numcol)
+        : Matrix<ROCMfloat>(name, numrow, numcol, 0) {}
+    explicit Matrix<ROCMfloat>(const Matrix<float>& M);  // upload, keeps dims and flag
+    Matrix<ROCMfloat>(const Matrix<ROCMfloat>& M);       // deep copy
+    Matrix<ROCMfloat>(Matrix<ROCMfloat>&& M) noexcept;   // steals the buffer
+    Matrix<ROCMfloat>& operator=(const Matrix<ROCMfloat>& M);
+    Matrix<ROCMfloat>& operator=(Matrix<ROCMfloat>&& M) noexcept;
+
+    // ── shape / storage ──
+    inline size_t idx(size_t i, size_t j) const { return transpose ? i * numrow + j : j * numrow + i; }
+    inline size_t num_col() const { return transpose ? numrow : numcol; }
+    inline size_t num_row() const { return transpose ? numcol : numrow; }
+    inline size_t get_transpose() const { return transpose; }
+    std::string get_name() const { return name; }
+    const ROCMfloat* data() const { return elements.get(); }
+    // Device memory is not host-addressable; kept only so generic code that
+    // names elem() still compiles.  Use to_host() to read values.
+    inline ROCMfloat elem(size_t i, size_t j) const { return elements[idx(i, j)]; }
+    inline ROCMfloat& elem(size_t i, size_t j) { return elements[idx(i, j)]; }
+
+    // ── fill / factories ──
+    void ones();
+    void zeros();
+    static Matrix<ROCMfloat> randn(size_t m, size_t n);
+    static Matrix<ROCMfloat> rand(size_t m, size_t n);
+    static Matrix<ROCMfloat> ones(size_t m, size_t n);
+    static Matrix<ROCMfloat> zeros(size_t m, size_t n);
+
+    // ── the four operator concepts (cpp/operators.hpp:47-96) ──
+    Matrix<ROCMfloat> dot(const Matrix<ROCMfloat>& B) const;
+    Matrix<ROCMfloat> add(const Matrix<ROCMfloat>& B, float s1, float s2) const;
+    void add(const Matrix<ROCMfloat>& B, float s1, float s2);
+    Matrix<ROCMfloat> add(float a, float s1) const;
+    void add(float a, float s1);
+    Matrix<ROCMfloat> scale(float s1) const { return add(0, s1); }
+    void scale(float s1);
+    void eleminv(double l);
+    Matrix<ROCMfloat> eleminv(double l) const;
+
+    float norm() const;
+    const Matrix<ROCMfloat> T() const;
+    Matrix<float> to_host() const;
+
+    // ── rectangular views ──
+    Matrix<ROCMfloat> slice(size_t rstart, size_t rend, size_t cstart, size_t cend) const;
+    void slice(size_t rstart, size_t rend, size_t cstart, size_t cend, const Matrix<ROCMfloat>& M);
+    Matrix<ROCMfloat> rows(size_t rstart, size_t rend) const;
+    void rows(size_t rstart, size_t rend, const Matrix<ROCMfloat>& M);
+    Matrix<ROCMfloat> columns(size_t cstart, size_t cend) const;
+    void columns(size_t cstart, size_t cend, const Matrix<ROCMfloat>& M);
+
+    // ── friends (same set as the reference declares) ──
+    friend class MatrixView<ROCMfloat>;
+    friend Matrix<ROCMfloat> sum(const Matrix<ROCMfloat>& M, int dim);
+    friend Matrix<ROCMfloat> hadmd(const Matrix<ROCMfloat>& M1, const Matrix<ROCMfloat>& M2);
+    friend Matrix<ROCMfloat> hadmd(const Matrix<ROCMfloat>& M1, Matrix<ROCMfloat>&& M2);
+    friend Matrix<ROCMfloat> hadmd(Matrix<ROCMfloat>&& M1, const Matrix<ROCMfloat>& M2);
+    friend Matrix<ROCMfloat> hadmd(Matrix<ROCMfloat>&& M1, Matrix<ROCMfloat>&& M2);
+    friend Matrix<ROCMfloat> exp(const Matrix<ROCMfloat>& M);
+    friend Matrix<ROCMfloat> exp(Matrix<ROCMfloat>&& M);
+    friend Matrix<ROCMfloat> log(const Matrix<ROCMfloat>& M);
+    friend Matrix<ROCMfloat> tanh(const Matrix<ROCMfloat>& M);
+    friend Matrix<ROCMfloat> tanh(Matrix<ROCMfloat>&& M);
+    friend Matrix<ROCMfloat> d_tanh(const Matrix<ROCMfloat>& M);
+    friend Matrix<ROCMfloat> d_tanh(Matrix<ROCMfloat>&& M);
+    friend Matrix<ROCMfloat> square(const Matrix<ROCMfloat>& M);
+    friend Matrix<ROCMfloat> square(Matrix<ROCMfloat>&& M);
+    friend void copy(Matrix<ROCMfloat>& dest, const Matrix<ROCMfloat>& src);
+    friend Matrix<ROCMfloat>& fill(Matrix<ROCMfloat>& M, double a);
+    friend Matrix<ROCMfloat> hstack(std::vector<MatrixView<ROCMfloat>> matrices);
+    friend Matrix<ROCMfloat> vstack(std::vector<MatrixView<ROCMfloat>> matrices);
+    template <class Function>
+    friend Matrix<ROCMfloat> reduce(Function func, const Matrix<ROCMfloat>& M, int dim, int k);
+    template <class Function>
+    friend Matrix<ROCMfloat> elemwise(Function func, const Matrix<ROCMfloat>& M);
+    template <class Function>
+    friend Matrix<ROCMfloat> elemwise(Function func, Matrix<ROCMfloat>&& M);
+    friend std::ostream& operator<<(std::ostream& os, const Matrix<ROCMfloat>& M);
+    friend void write<ROCMfloat>(FILE* fp, const Matrix<ROCMfloat>& M);
+    friend void read<ROCMfloat>(FILE* fp, Matrix<ROCMfloat>& M);
+
+    // fused ROCm paths (defined in hipmatrix.cpp)
+    friend struct JzRocmFused;
+};
+
+Matrix<ROCMfloat> sum(const Matrix<ROCMfloat>& M, int dim);
+std::ostream& operator<<(std::ostream& os, const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> exp(const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> exp(Matrix<ROCMfloat>&& M);
+Matrix<ROCMfloat> log(const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> tanh(const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> tanh(Matrix<ROCMfloat>&& M);
+Matrix<ROCMfloat> d_tanh(const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> d_tanh(Matrix<ROCMfloat>&& M);
+Matrix<ROCMfloat> square(const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> square(Matrix<ROCMfloat>&& M);
+void copy(Matrix<ROCMfloat>& dest, const Matrix<ROCMfloat>& src);
+Matrix<ROCMfloat>& fill(Matrix<ROCMfloat>& M, double a);
+Matrix<ROCMfloat> hstack(std::vector<MatrixView<ROCMfloat>> matrices);
+Matrix<ROCMfloat> vstack(std::vector<MatrixView<ROCMfloat>> matrices);
+
+// ── fused overloads picked up by the unmodified layer templates ─────────────
+// relu / d_relu (ml/util.cuh:74-82): the generic templates go through a
+// device lambda; these call the fixed-function kernels and, unlike the
+// generic ones, really do reuse the rvalue's buffer.
+Matrix<ROCMfloat> relu(Matrix<ROCMfloat>&& M);
+Matrix<ROCMfloat> d_relu(Matrix<ROCMfloat>&& M);
+namespace Juzhen {
+// col_softmax / row_softmax (ml/layer.hpp:2344-2367): single-pass kernels.
+Matrix<ROCMfloat> col_softmax(const Matrix<ROCMfloat>& M);
+Matrix<ROCMfloat> row_softmax(const Matrix<ROCMfloat>& M);
+}  // namespace Juzhen
+
+// Internal access point for the fused paths.
+struct JzRocmFused {
+    static float* ptr(const Matrix<ROCMfloat>& M) { return M.dev(); }
+    static Matrix<ROCMfloat> like(const char* name, const Matrix<ROCMfloat>& M) {
+        return Matrix<ROCMfloat>(name, M.numrow, M.numcol, M.transpose);
+    }
+    static Matrix<ROCMfloat> make(const char* name, size_t r, size_t c, int trans) {
+        return Matrix<ROCMfloat>(name, r, c, trans);
+    }
+    static size_t phys_rows(const Matrix<ROCMfloat>& M) { return M.numrow; }
+    static size_t phys_cols(const Matrix<ROCMfloat>& M) { return M.numcol; }
+    // Materialise the logical transpose of M as a plain (flag 0) matrix.
+    static Matrix<ROCMfloat> materialise(const Matrix<ROCMfloat>& M);
+};
+
+// adam_update (ml/util.cuh:166-256) as one fused kernel with the arithmetic of
+// the CPU loop (ml/util.cuh:223-245).  adam_state is only forward-declared
+// here, so the body is a template that is instantiated at the end of the
+// including translation unit, where ml/util.cuh has completed the type.
+extern "C" int jzhip_adam_update(float* g, float* m, float* v, size_t count, float alpha, float beta1,
+                                 float beta2, float eps, int iteration);
+
+template <class State>
+Matrix<ROCMfloat> jz_rocm_adam_update(Matrix<ROCMfloat>&& g, State& st) {
+    if (!g.get_transpose() && !st.m.get_transpose() && !st.v.get_transpose()) {
+        const int rc = jzhip_adam_update(JzRocmFused::ptr(g), JzRocmFused::ptr(st.m), JzRocmFused::ptr(st.v),
+                                         g.num_row() * g.num_col(), st.alpha, st.beta1, st.beta2, st.eps,
+                                         st.iteration);
+        if (rc != 0) {
+            LOG_ERROR("jzhip_adam_update failed with code {}", rc);
+            ERROR_OUT;
+        }
+        st.iteration++;
+        return std::move(g);
+    }
+    // transposed operands: the generic formulation (ml/util.cuh:247-255)
+    st.m = st.beta1 * st.m + (1 - st.beta1) * g;
+    st.v = st.beta2 * st.v + (1 - st.beta2) * square(g);
+    auto m_hat = st.m / (1 - pow(st.beta1, st.iteration));
+    auto v_hat = st.v / (1 - pow(st.beta2, st.iteration));
+    g = st.alpha * m_hat / (sqrt(v_hat) + st.eps);
+    st.iteration++;
+    return std::move(g);
+}
+
+// Declared here so that it is visible before the layer templates are parsed;
+// defined in hipfused_util.hpp, which is included at the end of ml/util.cuh
+// (where adam_state is complete), the way ml/util.cuh:147-192 hooks CUDA.
+inline Matrix<ROCMfloat> adam_update(Matrix<ROCMfloat>&& g, adam_state<ROCMfloat>& state);
+
+#ifdef __HIPCC__
+
+// ── user-functor templates ──────────────────────────────────────────────────
+// elemwise<F> and reduce<F> take arbitrary device functors, so they have to be
+// header templates that launch from the user's translation unit.  elemwise is
+// a grid-stride kernel over float4 (the functor is applied per lane, so its
+// semantics are unchanged); reduce keeps the reference contract "one functor
+// call per reduced vector, on a contiguous vector the functor may overwrite".
+
+namespace jzrocm {
+constexpr int kThreads = 256;
+inline hipStream_t stream() { return static_cast<hipStream_t>(jzhip_get_stream()); }
+inline unsigned grid_for(size_t items) {
+    static int cus = 0;
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+                  ? prop.multiProcessorCount
+                  : 256;
+    }
+    size_t need = (items + kThreads - 1) / kThreads;
+    size_t cap = static_cast<size_t>(cus) * 8;
+    if (need < 1) need = 1;
+    return static_cast<unsigned>(need < cap ? need : cap);
+}
+
+template <class Function>
+__global__ __launch_bounds__(kThreads) void elemwise_kernel(Function func, float* dst,
+                                                            const float* src, size_t n, int vec) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (vec) {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride) {
+            const float4 x = reinterpret_cast<const float4*>(src)[i];
+            float4 y;
+            y.x = func(x.x);
+            y.y = func(x.y);
+            y.z = func(x.z);
+            y.w = func(x.w);
+            reinterpret_cast<float4*>(dst)[i] = y;
+        }
+        for (size_t j = n4 * 4 + tid; j < n; j += stride) dst[j] = func(src[j]);
+    } else {
+        for (size_t j = tid; j < n; j += stride) dst[j] = func(src[j]);
+    }
+}
+
+template <class Function>
+__global__ __launch_bounds__(kThreads) void reduce_kernel(Function func, float* vecdes, float* vec,
+                                                          size_t lenvec, size_t lenvecdes,
+                                                          size_t numvecs) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; i < numvecs; i += stride)
+        func(&vec[i * lenvec], &vecdes[i * lenvecdes], lenvec, lenvecdes);
+}
+}  // namespace jzrocm
+
+template <class Function>
+Matrix<ROCMfloat> elemwise(Function func, const Matrix<ROCMfloat>& M) {
+    Matrix<ROCMfloat> result("resM", M.numrow, M.numcol, M.transpose);
+    const size_t n = M.count();
+    const int vec = ((reinterpret_cast<uintptr_t>(M.dev()) | reinterpret_cast<uintptr_t>(result.dev())) & 15) == 0;
+    jzrocm::elemwise_kernel<<<jzrocm::grid_for(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+        func, result.dev(), M.dev(), n, vec);
+    return result;
+}
+
+template <class Function>
+Matrix<ROCMfloat> elemwise(Function func, Matrix<ROCMfloat>&& M) {
+    const size_t n = M.count();
+    const int vec = (reinterpret_cast<uintptr_t>(M.dev()) & 15) == 0;
+    jzrocm::elemwise_kernel<<<jzrocm::grid_for(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+        func, M.dev(), M.dev(), n, vec);
+    return std::move(M);
+}
+
+// Orientation table of the CPU oracle (cpp/matrix.hpp:202-250): the functor is
+// handed the physical columns directly when they are the vectors to reduce,
+// otherwise a private transposed copy.
+template <class Function>
+Matrix<ROCMfloat> reduce(Function func, const Matrix<ROCMfloat>& M, int dim, int k) {
+    const bool direct = (dim == 0) == !M.transpose;
+    if (direct) {
+        Matrix<ROCMfloat> result("resM", k, M.numcol);
+        jzrocm::reduce_kernel<<<jzrocm::grid_for(M.numcol), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+            func, result.dev(), M.dev(), M.numrow, k, M.numcol);
+        return M.transpose ? Matrix<ROCMfloat>(result.T()) : result;
+    }
+    // physical transpose of the buffer: its columns are the vectors to reduce
+    Matrix<ROCMfloat> t = JzRocmFused::materialise(M.transpose ? M : M.T());
+    Matrix<ROCMfloat> result("resM", k, t.numcol);
+    jzrocm::reduce_kernel<<<jzrocm::grid_for(t.numcol), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+        func, result.dev(), t.dev(), t.numrow, k, t.numcol);
+    return M.transpose ? result : Matrix<ROCMfloat>(result.T());
+}
+
+#endif  // __HIPCC__
+
+#endif

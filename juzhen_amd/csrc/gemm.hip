@@ -96,7 +96,8 @@ template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST>
 __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
-    long long strideB, long long strideC, int tiles_m, int tiles_n) {
+    long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
+    long long strideC2, int tiles_m, int tiles_n) {
     static_assert(WGM * WGN == kBlock / kWave, "four waves per workgroup");
     constexpr int BM = WGM * TM * 32;
     constexpr int BN = WGN * TN * 32;
@@ -131,10 +132,11 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
-    const int batch = blockIdx.z;
-    A += batch * strideA;
-    B += batch * strideB;
-    C += batch * strideC;
+    // two-level batch: z = inner + batch1*outer (e.g. sequence inside head)
+    const int b_in = blockIdx.z % batch1, b_out = blockIdx.z / batch1;
+    A += b_in * strideA + b_out * strideA2;
+    B += b_in * strideB + b_out * strideB2;
+    C += b_in * strideC + b_out * strideC2;
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -319,6 +321,8 @@ struct GemmArgs {
     float alpha, beta;
     long long sA, sB, sC;
     int batch;
+    long long sA2 = 0, sB2 = 0, sC2 = 0;  // outer batch level
+    int batch2 = 1;
 };
 
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB>
@@ -327,16 +331,16 @@ int launch_tile(const GemmArgs& g) {
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const bool fast = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && (g.lda % 4 == 0) &&
                       (g.ldb % 4 == 0) && aligned16(g.A) && aligned16(g.B) && (g.sA % 4 == 0) &&
-                      (g.sB % 4 == 0);
-    dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, 1, g.batch);
+                      (g.sB % 4 == 0) && (g.sA2 % 4 == 0) && (g.sB2 % 4 == 0);
+    dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, 1, g.batch * g.batch2);
     if (fast)
         gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true><<<grid, kBlock, 0, stream()>>>(
             g.A, g.B, g.C, g.M, g.N, g.K, g.lda, g.ldb, g.ldc, g.alpha, g.beta, g.sA, g.sB, g.sC,
-            tiles_m, tiles_n);
+            g.batch, g.sA2, g.sB2, g.sC2, tiles_m, tiles_n);
     else
         gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, false><<<grid, kBlock, 0, stream()>>>(
             g.A, g.B, g.C, g.M, g.N, g.K, g.lda, g.ldb, g.ldc, g.alpha, g.beta, g.sA, g.sB, g.sC,
-            tiles_m, tiles_n);
+            g.batch, g.sA2, g.sB2, g.sC2, tiles_m, tiles_n);
     return launch_rc();
 }
 
@@ -346,7 +350,7 @@ int launch_shape(const GemmArgs& g) {
     // keeping every CU busy.
     const long long cus = num_cus();
     auto tiles = [&](int bm, int bn) {
-        return static_cast<long long>((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
+        return static_cast<long long>((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch * g.batch2;
     };
     if (g.M <= 32) return launch_tile<1, 4, 1, 2, TA, TB>(g);   // 32 x 256
     if (g.N <= 32) return launch_tile<4, 1, 2, 1, TA, TB>(g);   // 256 x 32
@@ -386,6 +390,18 @@ int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans
 }
 
 }  // namespace
+
+// Two-level strided-batched GEMM for library-internal callers (attention):
+// problem (i, o) uses X + i*stride_x + o*stride_x2.
+int gemm_batched2(const float* A, const float* B, float* C, int m, int n, int k, bool ta, bool tb,
+                  int lda, int ldb, int ldc, long long sA, long long sB, long long sC, int batch,
+                  long long sA2, long long sB2, long long sC2, int batch2, float alpha, float beta) {
+    if (static_cast<long long>(batch) * batch2 > 65535) return -1;
+    GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
+               static_cast<size_t>(ldc), alpha, beta, sA, sB, sC, batch, sA2, sB2, sC2, batch2};
+    return gemm_dispatch(g, ta, tb);
+}
+
 }  // namespace jz
 
 using namespace jz;

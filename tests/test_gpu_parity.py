@@ -640,3 +640,44 @@ def test_rand(gpu):
     assert np.array_equal(to_host(d)[:1000], u[:1000])
     gpu.rand_uniform(dptr(d), 1000, 0)
     assert not np.array_equal(to_host(d)[:1000], u[:1000])
+
+
+# ── batched attention core ───────────────────────────────────────────────
+@pytest.mark.parametrize("d_k,heads,S,B,causal", [(8, 4, 3, 2, 1), (16, 2, 5, 3, 0), (64, 1, 17, 2, 1), (128, 2, 64, 3, 1),
+                                                  (512, 8, 32, 2, 1)])
+def test_attention_fwd_bwd(gpu, d_k, heads, S, B, causal):
+    """Against a float64 restatement of the per-(head, sequence) loop of
+    ml/layer.hpp:2967-3006 and 3329-3363 (the method of tests/testTransformerRef.cu:102-141)."""
+    r = rng(d_k + S + B)
+    N, dh = S * B, d_k // heads
+    Q, K, V, dH = (r.normal(0, 1, (N, d_k)).astype(np.float32) for _ in range(4))   # [col, row]
+    H = np.zeros((N, d_k)); A = np.zeros((heads * B, S, S))                           # A[blk][key][query]
+    dQ, dK, dV = np.zeros((N, d_k)), np.zeros((N, d_k)), np.zeros((N, d_k))
+    scale = 1.0 / np.sqrt(np.float32(dh))
+    for hh in range(heads):
+        for b in range(B):
+            rs, cs = slice(hh * dh, (hh + 1) * dh), slice(b * S, (b + 1) * S)
+            q, k, v, g = (X[cs, rs].astype(np.float64).T for X in (Q, K, V, dH))       # (dh, S)
+            s = (q.T @ k) * scale                                                      # [query, key]
+            if causal:
+                s[np.triu_indices(S, 1)] = -1e9
+            a = np.exp(s - s.max(1, keepdims=True))
+            a /= a.sum(1, keepdims=True)
+            H[cs, rs] = (v @ a.T).T
+            A[hh * B + b] = a.T
+            da = g.T @ v                                                               # [query, key]
+            ds = a * (da - (a * da).sum(1, keepdims=True)) * scale
+            dV[cs, rs] = (g @ a).T
+            dQ[cs, rs] = (k @ ds.T).T
+            dK[cs, rs] = (q @ ds).T
+    dHm, dAm = dev_empty(N * d_k), dev_empty(S * S * B * heads)
+    dq, dk, dv = to_dev(Q.reshape(-1)), to_dev(K.reshape(-1)), to_dev(V.reshape(-1))
+    gpu.attention_fwd(dptr(dHm), dptr(dAm), dptr(dq), dptr(dk), dptr(dv), d_k, heads, S, B, causal)
+    assert rel_err(to_host(dHm), H.reshape(-1)) <= TOL_GEMM
+    assert rel_err(to_host(dAm), A.reshape(-1)) <= TOL_RED
+    oq, ok_, ov, scratch = dev_empty(N * d_k), dev_empty(N * d_k), dev_empty(N * d_k), dev_empty(S * S * B * heads)
+    gpu.attention_bwd(dptr(oq), dptr(ok_), dptr(ov), dptr(scratch), dp(dH.reshape(-1)), dptr(dq), dptr(dk), dptr(dv),
+                      dptr(dAm), d_k, heads, S, B)
+    assert rel_err(to_host(ov), dV.reshape(-1)) <= TOL_GEMM
+    assert rel_err(to_host(oq), dQ.reshape(-1)) <= TOL_GEMM
+    assert rel_err(to_host(ok_), dK.reshape(-1)) <= TOL_GEMM
