@@ -196,9 +196,28 @@ def build_host(force: bool = False, jobs: int = 6):
     return bins
 
 
+# ── model harness (host C++ on the C ABI) ──────────────────────────────────────
+HARNESS_LIB = PKG / "lib" / "libjzlm.so"
+
+
+def build_harness(force: bool = False) -> Path:
+    """Compile the train-step harness library (plain host C++, links libjzhip)."""
+    build()
+    srcs = sorted((PKG / "harness").glob("*.cpp"))
+    if force or _stale(HARNESS_LIB, [*srcs, LIB, ROOT / "include" / "jzhip.h"]):
+        cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-fvisibility=hidden",
+               f"-I{ROOT / 'include'}", "-o", str(HARNESS_LIB), *map(str, srcs),
+               f"-L{LIB.parent}", "-ljzhip", "-Wl,-rpath,$ORIGIN"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"harness build failed:\n{r.stderr}")
+    return HARNESS_LIB
+
+
 if __name__ == "__main__":
     path = build(force="--force" in sys.argv)
     print(path)
+    print(build_harness(force="--force" in sys.argv))
     if "--host" in sys.argv:
         for b in build_host(force="--force" in sys.argv):
             print(b)

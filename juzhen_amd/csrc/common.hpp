@@ -28,7 +28,7 @@ inline int rc_of(hipError_t e) { return e == hipSuccess ? 0 : static_cast<int>(e
 // Device scratch for two-phase reductions; created once, never resized.
 // Returns nullptr on allocation failure. Capacity in floats.
 float* workspace();
-constexpr size_t kWorkspaceFloats = size_t(4) << 20;  // 16 MiB
+constexpr size_t kWorkspaceFloats = size_t(16) << 20;  // 64 MiB
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

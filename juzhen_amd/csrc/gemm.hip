@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
-    long long strideC2, int tiles_m, int tiles_n) {
+    long long strideC2, int tiles_m, int tiles_n, int k_chunk, long long split_stride) {
     static_assert(WGM * WGN == kBlock / kWave, "four waves per workgroup");
     constexpr int BM = WGM * TM * 32;
     constexpr int BN = WGN * TN * 32;
@@ -137,6 +137,10 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
     A += b_in * strideA + b_out * strideA2;
     B += b_in * strideB + b_out * strideB2;
     C += b_in * strideC + b_out * strideC2;
+    // split-K: blockIdx.y owns K range [k_lo, k_hi) and its own partial C
+    const int k_lo = blockIdx.y * k_chunk;
+    const int k_hi = (k_lo + k_chunk) < K ? (k_lo + k_chunk) : K;
+    C += blockIdx.y * split_stride;
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -154,9 +158,9 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
     TileLoader<BM, !TA> la;
     TileLoader<BN, TB> lb;
 
-    const int nk = (K + BK - 1) / BK;
-    la.template load<FAST>(A, lda, m0, 0, M, K);
-    lb.template load<FAST>(B, ldb, n0, 0, N, K);
+    const int nk = (k_hi - k_lo + BK - 1) / BK;
+    la.template load<FAST>(A, lda, m0, k_lo, M, k_hi);
+    lb.template load<FAST>(B, ldb, n0, k_lo, N, k_hi);
     la.store(As[0]);
     lb.store(Bs[0]);
     __syncthreads();
@@ -164,8 +168,8 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
     int cur = 0;
     for (int kt = 0; kt < nk; ++kt) {
         if (kt + 1 < nk) {
-            la.template load<FAST>(A, lda, m0, (kt + 1) * BK, M, K);
-            lb.template load<FAST>(B, ldb, n0, (kt + 1) * BK, N, K);
+            la.template load<FAST>(A, lda, m0, k_lo + (kt + 1) * BK, M, k_hi);
+            lb.template load<FAST>(B, ldb, n0, k_lo + (kt + 1) * BK, N, k_hi);
         }
         const float* as = As[cur] + wm * (TM * 32) + l32;
         const float* bs = Bs[cur] + wn * (TN * 32) + l32;
@@ -311,6 +315,22 @@ __global__ __launch_bounds__(kBlock) void add_bias_scalar_kernel(float* y, const
         y[i] += b[i % rows];
 }
 
+// C = alpha * sum_s part[s] + beta*C for split-K partials (each m x n, ld = m)
+__global__ __launch_bounds__(kBlock) void splitk_reduce_kernel(float* C, const float* part, int M, int N,
+                                                               size_t ldc, int splits, float alpha,
+                                                               float beta) {
+    const size_t total = static_cast<size_t>(M) * N;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s) acc += part[static_cast<size_t>(s) * total + i];
+        float* dst = C + (i / M) * ldc + (i % M);
+        float r = alpha * acc;
+        if (beta != 0.0f) r += beta * *dst;
+        *dst = r;
+    }
+}
+
 // ── dispatch ─────────────────────────────────────────────────────────────
 struct GemmArgs {
     const float* A;
@@ -329,18 +349,53 @@ template <int WGM, int WGN, int TM, int TN, bool TA, bool TB>
 int launch_tile(const GemmArgs& g) {
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    // Split K when the output alone cannot fill the chip (weight gradients:
+    // small m x n, very long k).  Partials go to the workspace and are summed
+    // in a fixed order, so results stay deterministic.
+    int splits = 1;
+    const long long tiles = static_cast<long long>(tiles_m) * tiles_n * g.batch * g.batch2;
+    const long long cus = num_cus();
+    if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 1024) {
+        splits = static_cast<int>((cus * 2 + tiles - 1) / tiles);
+        const int max_by_k = g.K / 256;
+        if (splits > max_by_k) splits = max_by_k;
+        const size_t per = static_cast<size_t>(g.M) * g.N;
+        while (splits > 1 && per * splits > kWorkspaceFloats) --splits;
+        if (splits < 2) splits = 1;
+    }
+    int k_chunk = g.K;
+    float* out = g.C;
+    size_t ldc = g.ldc;
+    float alpha = g.alpha, beta = g.beta;
+    long long split_stride = 0;
+    if (splits > 1) {
+        k_chunk = ((g.K + splits - 1) / splits + BK - 1) / BK * BK;
+        splits = (g.K + k_chunk - 1) / k_chunk;
+        out = workspace();
+        if (!out) return -2;
+        ldc = g.M;
+        alpha = 1.0f;
+        beta = 0.0f;
+        split_stride = static_cast<long long>(g.M) * g.N;
+    }
     const bool fast = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && (g.lda % 4 == 0) &&
                       (g.ldb % 4 == 0) && aligned16(g.A) && aligned16(g.B) && (g.sA % 4 == 0) &&
                       (g.sB % 4 == 0) && (g.sA2 % 4 == 0) && (g.sB2 % 4 == 0);
-    dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, 1, g.batch * g.batch2);
+    dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, splits, g.batch * g.batch2);
+    hipStream_t s = stream();
     if (fast)
-        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true><<<grid, kBlock, 0, stream()>>>(
-            g.A, g.B, g.C, g.M, g.N, g.K, g.lda, g.ldb, g.ldc, g.alpha, g.beta, g.sA, g.sB, g.sC,
-            g.batch, g.sA2, g.sB2, g.sC2, tiles_m, tiles_n);
+        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true><<<grid, kBlock, 0, s>>>(
+            g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2,
+            g.sB2, g.sC2, tiles_m, tiles_n, k_chunk, split_stride);
     else
-        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, false><<<grid, kBlock, 0, stream()>>>(
-            g.A, g.B, g.C, g.M, g.N, g.K, g.lda, g.ldb, g.ldc, g.alpha, g.beta, g.sA, g.sB, g.sC,
-            g.batch, g.sA2, g.sB2, g.sC2, tiles_m, tiles_n);
+        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, false><<<grid, kBlock, 0, s>>>(
+            g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2,
+            g.sB2, g.sC2, tiles_m, tiles_n, k_chunk, split_stride);
+    if (splits > 1) {
+        const size_t total = static_cast<size_t>(g.M) * g.N;
+        splitk_reduce_kernel<<<grid_for(total, kBlock, 4), kBlock, 0, s>>>(g.C, out, g.M, g.N, g.ldc, splits,
+                                                                           g.alpha, g.beta);
+    }
     return launch_rc();
 }
 

@@ -1,0 +1,357 @@
+// Character-level transformer language model trained on one MI355X through the
+// C ABI of libjzhip.so: the train-step harness of the benchmark configuration
+// (6 pre-LayerNorm decoder blocks, d_model 512, 8 heads, FFN 2048 with GELU,
+// tied embeddings, learned positional table, cross-entropy, AdamW).
+//
+// The block is the reference's TransformerLayer (ml/layer.hpp:2735-3447): same
+// tensors, same layouts (activations are (features, tokens) column-major with
+// token n = b*S + s), same forward/backward algebra, so with relu/adam/untied
+// options it reproduces a stack built from the reference's own classes
+// (examples/demo_transformer.cu:214-383: one-hot token+position input into a
+// LinearLayer, TransformerLayers, a LinearLayer head, LogisticLayer loss).
+// Embedding, positional table and head are expressed as GEMMs against one-hot
+// matrices, the reference's formulation (demo_transformer.cu:133-149), which
+// keeps them deterministic and checkable against the CPU path.
+//
+// Everything is preallocated at creation; a step issues only library calls
+// (no allocation, no host synchronisation).  The loss stays on the device until
+// jzlm_loss() is called.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "jzhip.h"
+
+#define JZLM_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+struct Config {
+    int vocab, d_model, heads, d_ff, layers, seq, batch;
+    int gelu;        // 1: exact-erf GELU FFN, 0: ReLU (the reference block)
+    int tied;        // 1: head = embedding^T, no biases on embedding/head; 0: separate head with biases
+    int adamw;       // 1: decoupled weight decay on matrices
+    float lr, weight_decay, beta1, beta2, eps;
+};
+
+struct Tensor {
+    std::string name;
+    int rows = 0, cols = 0;
+    float* w = nullptr;   // parameter
+    float* g = nullptr;   // gradient
+    float* m = nullptr;   // Adam first moment
+    float* v = nullptr;   // Adam second moment
+    bool decay = false;
+    size_t count() const { return static_cast<size_t>(rows) * cols; }
+};
+
+struct Block {
+    int Wq, Wk, Wv, Wo, bo, W1, b1, W2, b2, g1, be1, g2, be2;           // tensor indices
+    float *x1, *xhat1, *inv1, *Q, *K, *V, *A, *H, *R, *x2, *xhat2, *inv2, *F1, *F1a, *out;  // cached activations
+};
+
+struct Model {
+    Config c;
+    int N = 0;  // tokens per step
+    std::vector<Tensor> t;
+    std::vector<Block> blocks;
+    std::vector<float*> owned;
+    int E = -1, P = -1, be = -1, Wp = -1, bp = -1;
+    float *oh_tok = nullptr, *oh_pos = nullptr, *x0 = nullptr, *logits = nullptr, *dlogits = nullptr;
+    int32_t* targets = nullptr;
+    float* loss = nullptr;
+    // backward scratch shared by all blocks
+    float *dx = nullptr, *dR = nullptr, *dtmp = nullptr, *dQ = nullptr, *dK = nullptr, *dV = nullptr,
+          *dH = nullptr, *dA = nullptr, *dF1 = nullptr;
+    int iteration = 1;
+    int rc = 0;  // first failing return code, sticky
+
+    float* alloc(size_t n) {
+        float* p = nullptr;
+        int r = jzhip_malloc(&p, n);
+        if (r != 0 && rc == 0) rc = r;
+        owned.push_back(p);
+        return p;
+    }
+    int add(const std::string& name, int rows, int cols, bool decay) {
+        Tensor x;
+        x.name = name; x.rows = rows; x.cols = cols; x.decay = decay;
+        const size_t n = x.count();
+        x.w = alloc(n); x.g = alloc(n); x.m = alloc(n); x.v = alloc(n);
+        ck(jzhip_fill(x.w, n, 0.f)); ck(jzhip_fill(x.g, n, 0.f));
+        ck(jzhip_fill(x.m, n, 0.f)); ck(jzhip_fill(x.v, n, 0.f));
+        t.push_back(x);
+        return static_cast<int>(t.size()) - 1;
+    }
+    void ck(int r) { if (r != 0 && rc == 0) rc = r; }
+};
+
+// C(m x n) = alpha*op(A)op(B) + beta*C, dense operands
+inline void gemm(Model& M, const float* A, bool ta, const float* B, bool tb, float* C, int m, int n, int k,
+                 float beta = 0.f) {
+    M.ck(jzhip_gemm(A, B, C, m, n, k, ta, tb, ta ? k : m, tb ? n : k, m, 1.0f, beta));
+}
+
+void forward(Model& M) {
+    const Config& c = M.c;
+    const int d = c.d_model, N = M.N, ff = c.d_ff;
+    const size_t dN = static_cast<size_t>(d) * N;
+    // x0 = E * onehot(tokens) + P * onehot(positions) [+ embedding bias]
+    gemm(M, M.t[M.E].w, false, M.oh_tok, false, M.x0, d, N, c.vocab);
+    gemm(M, M.t[M.P].w, false, M.oh_pos, false, M.x0, d, N, c.seq, 1.0f);
+    if (M.be >= 0) M.ck(jzhip_add_bias(M.x0, M.t[M.be].w, d, N));
+    const float* x = M.x0;
+    for (Block& b : M.blocks) {
+        M.ck(jzhip_layernorm_fwd(b.x1, b.xhat1, b.inv1, x, M.t[b.g1].w, M.t[b.be1].w, d, N));
+        gemm(M, M.t[b.Wq].w, false, b.x1, false, b.Q, d, N, d);
+        gemm(M, M.t[b.Wk].w, false, b.x1, false, b.K, d, N, d);
+        gemm(M, M.t[b.Wv].w, false, b.x1, false, b.V, d, N, d);
+        M.ck(jzhip_attention_fwd(b.H, b.A, b.Q, b.K, b.V, d, c.heads, c.seq, c.batch, 1));
+        gemm(M, M.t[b.Wo].w, false, b.H, false, b.R, d, N, d);           // O
+        M.ck(jzhip_add_bias(b.R, M.t[b.bo].w, d, N));
+        M.ck(jzhip_axpby(b.R, x, b.R, dN, 1.0f, 1.0f));                  // R = x + O
+        M.ck(jzhip_layernorm_fwd(b.x2, b.xhat2, b.inv2, b.R, M.t[b.g2].w, M.t[b.be2].w, d, N));
+        gemm(M, M.t[b.W1].w, false, b.x2, false, b.F1, ff, N, d);
+        M.ck(jzhip_add_bias(b.F1, M.t[b.b1].w, ff, N));
+        const size_t fN = static_cast<size_t>(ff) * N;
+        M.ck(c.gelu ? jzhip_gelu(b.F1a, b.F1, fN) : jzhip_relu(b.F1a, b.F1, fN));
+        gemm(M, M.t[b.W2].w, false, b.F1a, false, b.out, d, N, ff);      // F
+        M.ck(jzhip_add_bias(b.out, M.t[b.b2].w, d, N));
+        M.ck(jzhip_axpby(b.out, b.R, b.out, dN, 1.0f, 1.0f));            // out = R + F
+        x = b.out;
+    }
+    if (c.tied) {
+        gemm(M, M.t[M.E].w, true, x, false, M.logits, c.vocab, N, d);    // E^T x
+    } else {
+        gemm(M, M.t[M.Wp].w, false, x, false, M.logits, c.vocab, N, d);
+        M.ck(jzhip_add_bias(M.logits, M.t[M.bp].w, c.vocab, N));
+    }
+}
+
+void step_tensor(Model& M, int idx) {
+    Tensor& x = M.t[idx];
+    const Config& c = M.c;
+    const float wd = (c.adamw && x.decay) ? c.weight_decay : 0.0f;
+    M.ck(jzhip_adamw_step(x.w, x.g, x.m, x.v, x.count(), c.lr, c.beta1, c.beta2, c.eps, wd, M.iteration));
+}
+
+void backward(Model& M, bool update) {
+    const Config& c = M.c;
+    const int d = c.d_model, N = M.N, ff = c.d_ff, V = c.vocab;
+    const size_t dN = static_cast<size_t>(d) * N;
+    const float* xL = M.blocks.empty() ? M.x0 : M.blocks.back().out;
+    M.ck(jzhip_softmax_xent(M.loss, M.dlogits, M.logits, M.targets, V, N, V));
+    float* dy = M.dx;  // gradient w.r.t. the current block's output
+    if (c.tied) {
+        gemm(M, M.t[M.E].w, false, M.dlogits, false, dy, d, N, V);       // E * dlogits
+        gemm(M, xL, false, M.dlogits, true, M.t[M.E].g, d, V, N);        // head part of dE
+    } else {
+        gemm(M, M.dlogits, false, xL, true, M.t[M.Wp].g, V, d, N);
+        M.ck(jzhip_sum_rows(M.t[M.bp].g, M.dlogits, V, N, V));
+        // The reference's dense layers step their weights before forming the
+        // gradient they hand down (Layer::backward, ml/layer.hpp:96-105: update(),
+        // then `return W().T() * t`); the untied head reproduces that order.
+        if (update) { step_tensor(M, M.Wp); step_tensor(M, M.bp); }
+        gemm(M, M.t[M.Wp].w, true, M.dlogits, false, dy, d, N, V);
+    }
+    for (int l = static_cast<int>(M.blocks.size()) - 1; l >= 0; --l) {
+        Block& b = M.blocks[l];
+        const float* xin = l == 0 ? M.x0 : M.blocks[l - 1].out;
+        const size_t fN = static_cast<size_t>(ff) * N;
+        // feed-forward
+        gemm(M, dy, false, b.F1a, true, M.t[b.W2].g, d, ff, N);
+        M.ck(jzhip_sum_rows(M.t[b.b2].g, dy, d, N, d));
+        gemm(M, M.t[b.W2].w, true, dy, false, M.dF1, ff, N, d);
+        M.ck(c.gelu ? jzhip_dgelu_mul(M.dF1, b.F1, M.dF1, fN) : jzhip_drelu_mul(M.dF1, b.F1, M.dF1, fN));
+        gemm(M, M.dF1, false, b.x2, true, M.t[b.W1].g, ff, d, N);
+        M.ck(jzhip_sum_rows(M.t[b.b1].g, M.dF1, ff, N, ff));
+        gemm(M, M.t[b.W1].w, true, M.dF1, false, M.dtmp, d, N, ff);      // dx2
+        M.ck(jzhip_layernorm_param_grads(M.t[b.g2].g, M.t[b.be2].g, M.dtmp, b.xhat2, d, N));
+        M.ck(jzhip_layernorm_bwd(M.dR, M.dtmp, M.t[b.g2].w, b.xhat2, b.inv2, d, N));
+        M.ck(jzhip_axpby(M.dR, M.dR, dy, dN, 1.0f, 1.0f));               // dR = LN2'(dx2) + dy
+        // output projection
+        gemm(M, M.dR, false, b.H, true, M.t[b.Wo].g, d, d, N);
+        M.ck(jzhip_sum_rows(M.t[b.bo].g, M.dR, d, N, d));
+        gemm(M, M.t[b.Wo].w, true, M.dR, false, M.dH, d, N, d);
+        // attention core
+        M.ck(jzhip_attention_bwd(M.dQ, M.dK, M.dV, M.dA, M.dH, b.Q, b.K, b.V, b.A, d, c.heads, c.seq, c.batch));
+        gemm(M, M.dQ, false, b.x1, true, M.t[b.Wq].g, d, d, N);
+        gemm(M, M.dK, false, b.x1, true, M.t[b.Wk].g, d, d, N);
+        gemm(M, M.dV, false, b.x1, true, M.t[b.Wv].g, d, d, N);
+        gemm(M, M.t[b.Wq].w, true, M.dQ, false, M.dtmp, d, N, d);
+        gemm(M, M.t[b.Wk].w, true, M.dK, false, M.dtmp, d, N, d, 1.0f);
+        gemm(M, M.t[b.Wv].w, true, M.dV, false, M.dtmp, d, N, d, 1.0f); // dx1
+        M.ck(jzhip_layernorm_param_grads(M.t[b.g1].g, M.t[b.be1].g, M.dtmp, b.xhat1, d, N));
+        M.ck(jzhip_layernorm_bwd(dy, M.dtmp, M.t[b.g1].w, b.xhat1, b.inv1, d, N));
+        M.ck(jzhip_axpby(dy, dy, M.dR, dN, 1.0f, 1.0f));                 // dx = LN1'(dx1) + dR
+        (void)xin;
+        if (update) {
+            for (int idx : {b.Wq, b.Wk, b.Wv, b.Wo, b.bo, b.W1, b.b1, b.W2, b.b2, b.g1, b.be1, b.g2, b.be2})
+                step_tensor(M, idx);
+        }
+    }
+    // embedding tables: dE (+)= dx0 * onehot_tok^T, dP = dx0 * onehot_pos^T
+    gemm(M, dy, false, M.oh_tok, true, M.t[M.E].g, d, V, N, c.tied ? 1.0f : 0.0f);
+    gemm(M, dy, false, M.oh_pos, true, M.t[M.P].g, d, c.seq, N);
+    if (M.be >= 0) M.ck(jzhip_sum_rows(M.t[M.be].g, dy, d, N, d));
+    if (update) {
+        step_tensor(M, M.E);
+        step_tensor(M, M.P);
+        if (M.be >= 0) step_tensor(M, M.be);
+        M.iteration++;
+    }
+}
+
+}  // namespace
+
+struct jzlm_config {
+    int vocab, d_model, heads, d_ff, layers, seq, batch, gelu, tied, adamw;
+    float lr, weight_decay, beta1, beta2, eps;
+};
+
+JZLM_API void* jzlm_create(const jzlm_config* cfg) {
+    if (!cfg || cfg->vocab <= 0 || cfg->d_model <= 0 || cfg->heads <= 0 || cfg->d_model % cfg->heads != 0 ||
+        cfg->d_ff <= 0 || cfg->layers < 0 || cfg->seq <= 0 || cfg->batch <= 0)
+        return nullptr;
+    Model* M = new Model;
+    Config& c = M->c;
+    c.vocab = cfg->vocab; c.d_model = cfg->d_model; c.heads = cfg->heads; c.d_ff = cfg->d_ff;
+    c.layers = cfg->layers; c.seq = cfg->seq; c.batch = cfg->batch; c.gelu = cfg->gelu; c.tied = cfg->tied;
+    c.adamw = cfg->adamw; c.lr = cfg->lr; c.weight_decay = cfg->weight_decay; c.beta1 = cfg->beta1;
+    c.beta2 = cfg->beta2; c.eps = cfg->eps;
+    const int d = c.d_model, ff = c.d_ff, V = c.vocab, S = c.seq;
+    const int N = M->N = c.seq * c.batch;
+    const size_t dN = static_cast<size_t>(d) * N, fN = static_cast<size_t>(ff) * N;
+    const size_t aN = static_cast<size_t>(S) * S * c.batch * c.heads;
+
+    M->E = M->add("embed", d, V, true);
+    M->P = M->add("pos", d, S, true);
+    if (!c.tied) {
+        M->be = M->add("embed_bias", d, 1, false);
+        M->Wp = M->add("head", V, d, true);
+        M->bp = M->add("head_bias", V, 1, false);
+    }
+    for (int l = 0; l < c.layers; ++l) {
+        Block b;
+        const std::string p = "block" + std::to_string(l) + ".";
+        b.Wq = M->add(p + "Wq", d, d, true);  b.Wk = M->add(p + "Wk", d, d, true);
+        b.Wv = M->add(p + "Wv", d, d, true);  b.Wo = M->add(p + "Wo", d, d, true);
+        b.bo = M->add(p + "bo", d, 1, false);
+        b.W1 = M->add(p + "W1", ff, d, true); b.b1 = M->add(p + "b1", ff, 1, false);
+        b.W2 = M->add(p + "W2", d, ff, true); b.b2 = M->add(p + "b2", d, 1, false);
+        b.g1 = M->add(p + "ln1_gamma", d, 1, false); b.be1 = M->add(p + "ln1_beta", d, 1, false);
+        b.g2 = M->add(p + "ln2_gamma", d, 1, false); b.be2 = M->add(p + "ln2_beta", d, 1, false);
+        M->ck(jzhip_fill(M->t[b.g1].w, d, 1.0f));
+        M->ck(jzhip_fill(M->t[b.g2].w, d, 1.0f));
+        b.x1 = M->alloc(dN); b.xhat1 = M->alloc(dN); b.inv1 = M->alloc(N);
+        b.Q = M->alloc(dN); b.K = M->alloc(dN); b.V = M->alloc(dN); b.A = M->alloc(aN); b.H = M->alloc(dN);
+        b.R = M->alloc(dN); b.x2 = M->alloc(dN); b.xhat2 = M->alloc(dN); b.inv2 = M->alloc(N);
+        b.F1 = M->alloc(fN); b.F1a = M->alloc(fN); b.out = M->alloc(dN);
+        M->blocks.push_back(b);
+    }
+    M->oh_tok = M->alloc(static_cast<size_t>(V) * N);
+    M->oh_pos = M->alloc(static_cast<size_t>(S) * N);
+    M->x0 = M->alloc(dN);
+    M->logits = M->alloc(static_cast<size_t>(V) * N);
+    M->dlogits = M->alloc(static_cast<size_t>(V) * N);
+    M->targets = reinterpret_cast<int32_t*>(M->alloc(N));
+    M->loss = M->alloc(1);
+    M->dx = M->alloc(dN); M->dR = M->alloc(dN); M->dtmp = M->alloc(dN);
+    M->dQ = M->alloc(dN); M->dK = M->alloc(dN); M->dV = M->alloc(dN); M->dH = M->alloc(dN);
+    M->dA = M->alloc(aN); M->dF1 = M->alloc(fN);
+    if (M->rc != 0) {
+        std::fprintf(stderr, "jzlm_create: device allocation failed (%s)\n", jzhip_error_string(M->rc));
+    }
+    return M;
+}
+
+JZLM_API void jzlm_destroy(void* h) {
+    Model* M = static_cast<Model*>(h);
+    if (!M) return;
+    jzhip_synchronize();
+    for (float* p : M->owned) jzhip_free(p);
+    delete M;
+}
+
+JZLM_API int jzlm_status(void* h) { return static_cast<Model*>(h)->rc; }
+JZLM_API int jzlm_num_tensors(void* h) { return static_cast<int>(static_cast<Model*>(h)->t.size()); }
+JZLM_API size_t jzlm_param_count(void* h) {
+    size_t n = 0;
+    for (const Tensor& x : static_cast<Model*>(h)->t) n += x.count();
+    return n;
+}
+JZLM_API const char* jzlm_tensor_name(void* h, int i) { return static_cast<Model*>(h)->t[i].name.c_str(); }
+JZLM_API int jzlm_tensor_rows(void* h, int i) { return static_cast<Model*>(h)->t[i].rows; }
+JZLM_API int jzlm_tensor_cols(void* h, int i) { return static_cast<Model*>(h)->t[i].cols; }
+
+// which: 0 parameter, 1 gradient, 2 Adam m, 3 Adam v.  Column-major host buffers.
+JZLM_API int jzlm_get(void* h, int i, int which, float* host) {
+    Tensor& x = static_cast<Model*>(h)->t[i];
+    float* src = which == 0 ? x.w : which == 1 ? x.g : which == 2 ? x.m : x.v;
+    return jzhip_memcpy_d2h(host, src, x.count());
+}
+JZLM_API int jzlm_set(void* h, int i, int which, const float* host) {
+    Tensor& x = static_cast<Model*>(h)->t[i];
+    float* dst = which == 0 ? x.w : which == 1 ? x.g : which == 2 ? x.m : x.v;
+    return jzhip_memcpy_h2d(dst, host, x.count());
+}
+
+// tokens: batch windows of seq+1 ids each (window b = tokens[b*(seq+1) ...]);
+// inputs are ids 0..seq-1 of a window, targets ids 1..seq.
+JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
+    Model* M = static_cast<Model*>(h);
+    const Config& c = M->c;
+    const int N = M->N;
+    std::vector<float> oh(static_cast<size_t>(c.vocab) * N, 0.0f), op(static_cast<size_t>(c.seq) * N, 0.0f);
+    std::vector<int32_t> tg(N);
+    for (int b = 0; b < c.batch; ++b)
+        for (int s = 0; s < c.seq; ++s) {
+            const int n = b * c.seq + s;
+            const int32_t tok = tokens[static_cast<size_t>(b) * (c.seq + 1) + s];
+            const int32_t nxt = tokens[static_cast<size_t>(b) * (c.seq + 1) + s + 1];
+            if (tok < 0 || tok >= c.vocab || nxt < 0 || nxt >= c.vocab) return -1;
+            oh[static_cast<size_t>(n) * c.vocab + tok] = 1.0f;
+            op[static_cast<size_t>(n) * c.seq + s] = 1.0f;
+            tg[n] = nxt;
+        }
+    int rc = jzhip_memcpy_h2d(M->oh_tok, oh.data(), oh.size());
+    if (rc == 0) rc = jzhip_memcpy_h2d(M->oh_pos, op.data(), op.size());
+    if (rc == 0) rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->targets), reinterpret_cast<const float*>(tg.data()), N);
+    return rc;
+}
+
+JZLM_API int jzlm_forward(void* h) {
+    Model* M = static_cast<Model*>(h);
+    forward(*M);
+    return M->rc;
+}
+// forward must have run; computes the loss and all gradients, applies the
+// optimiser when update != 0
+JZLM_API int jzlm_backward(void* h, int update) {
+    Model* M = static_cast<Model*>(h);
+    backward(*M, update != 0);
+    return M->rc;
+}
+// one training step: forward, loss, backward, optimiser
+JZLM_API int jzlm_step(void* h) {
+    Model* M = static_cast<Model*>(h);
+    forward(*M);
+    backward(*M, true);
+    return M->rc;
+}
+// loss of the last backward()/step(); synchronises
+JZLM_API float jzlm_loss(void* h) {
+    Model* M = static_cast<Model*>(h);
+    float v = NAN;
+    if (jzhip_memcpy_d2h(&v, M->loss, 1) != 0) return NAN;
+    return v;
+}
+JZLM_API int jzlm_logits(void* h, float* host) {
+    Model* M = static_cast<Model*>(h);
+    return jzhip_memcpy_d2h(host, M->logits, static_cast<size_t>(M->c.vocab) * M->N);
+}
+JZLM_API int jzlm_tokens_per_step(void* h) { return static_cast<Model*>(h)->N; }
+JZLM_API void jzlm_set_iteration(void* h, int it) { static_cast<Model*>(h)->iteration = it; }

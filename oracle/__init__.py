@@ -148,6 +148,11 @@ REF_SIGNATURES = {
     "jzref_block_eval": (None, [P, P, P]),
     "jzref_block_backward": (None, [P, P, P, P, I]),
     "jzref_mlp_step": (F, [I, P, P, PP, PP, PP, PP, PP, PP, P, P, I, F, I]),
+    "jzref_lm_create": (P, [I, I, I, I, I, I, I]),
+    "jzref_lm_destroy": (None, [P]),
+    "jzref_lm_param": (I, [P, I, I, I, P, I]),
+    "jzref_lm_set_lr": (None, [P, F]),
+    "jzref_lm_step": (F, [P, P, P]),
 }
 
 _ref = None

@@ -359,3 +359,70 @@ API float jzref_mlp_step(int nlayers, const int* kinds, const int* dims, float**
     }
     return value;
 }
+
+// ── character LM built from the reference's own classes ──────────────────
+// embed LinearLayer(d, V+S) on the stacked one-hot [token; position] input,
+// `layers` TransformerLayer<float> blocks, proj LinearLayer(V, d), LogisticLayer
+// loss, Adam — the wiring of examples/demo_transformer.cu:285-340.
+struct RefLM {
+    int V, d, heads, ff, layers, S, B, N;
+    std::unique_ptr<Juzhen::LinearLayer<float>> embed, proj;
+    std::vector<std::unique_ptr<Juzhen::TransformerLayer<float>>> blocks;
+    std::list<Layer<float>*> net;
+};
+
+API void* jzref_lm_create(int V, int d, int heads, int ff, int layers, int S, int B) {
+    using namespace Juzhen;
+    auto* m = new RefLM{V, d, heads, ff, layers, S, B, S * B};
+    m->embed = std::make_unique<LinearLayer<float>>(d, V + S, m->N);
+    m->proj = std::make_unique<LinearLayer<float>>(V, d, m->N);
+    for (int i = 0; i < layers; ++i)
+        m->blocks.push_back(std::make_unique<TransformerLayer<float>>(d, d, ff, S, B, heads));
+    m->net.push_back(m->proj.get());
+    for (int i = layers - 1; i >= 0; --i) m->net.push_back(m->blocks[i].get());
+    m->net.push_back(m->embed.get());
+    return m;
+}
+API void jzref_lm_destroy(void* h) { delete static_cast<RefLM*>(h); }
+
+// kind 0 embed.W (d x (V+S)), 1 embed.b, 2 proj.W (V x d), 3 proj.b, 4 block parameter `which` of block `layer`
+API int jzref_lm_param(void* h, int kind, int layer, int which, float* buf, int set) {
+    auto* m = static_cast<RefLM*>(h);
+    if (kind == 4) {
+        RefBlock tmp;  // reuse the block accessor through a non-owning view
+        tmp.layer.reset(m->blocks[layer].get());
+        tmp.d_model = m->d; tmp.d_k = m->d; tmp.d_ff = m->ff; tmp.S = m->S; tmp.B = m->B;
+        const int rc = jzref_block_param(&tmp, which, buf, set);
+        tmp.layer.release();
+        return rc;
+    }
+    Layer<float>* L = kind < 2 ? static_cast<Layer<float>*>(m->embed.get()) : m->proj.get();
+    MF& dst = (kind % 2 == 0) ? L->W() : L->b();
+    if (set) dst = mk(buf, (int)dst.num_row(), (int)dst.num_col(), 0);
+    else out_logical(buf, dst);
+    return 0;
+}
+
+API void jzref_lm_set_lr(void* h, float lr) {
+    auto* m = static_cast<RefLM*>(h);
+    for (auto* L : {static_cast<Layer<float>*>(m->embed.get()), static_cast<Layer<float>*>(m->proj.get())}) {
+        L->adamWstate().alpha = lr;
+        L->adambstate().alpha = lr;
+    }
+    for (auto& b : m->blocks) b->set_lr(lr);
+}
+
+// One training step (forward, loss, backprop with Adam).  X is the stacked
+// one-hot input ((V+S) x N), Y the one-hot targets (V x N).  Returns the loss
+// of the forward pass.
+API float jzref_lm_step(void* h, const float* X, const float* Y) {
+    using namespace Juzhen;
+    auto* m = static_cast<RefLM*>(h);
+    const MF x = mk(X, m->V + m->S, m->N, 0);
+    LogisticLayer<float> loss(m->N, mk(Y, m->V, m->N, 0));
+    m->net.push_front(&loss);
+    const float value = forward(m->net, x).elem(0, 0);
+    backprop(m->net, x);
+    m->net.pop_front();
+    return value;
+}

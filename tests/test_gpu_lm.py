@@ -1,0 +1,199 @@
+"""Train-step parity of the transformer LM harness.
+
+(a) In the reference's own configuration (ReLU FFN, Adam, untied head with
+    biases) the harness must track a model assembled from the reference's own
+    classes on the CPU (LinearLayer + TransformerLayer<float> + LogisticLayer,
+    examples/demo_transformer.cu:285-340, through oracle/_ref) for 100 steps:
+    relative loss error <= 1e-3.
+(b) The pieces the reference does not contain (GELU, tied embeddings, AdamW)
+    are not pinned by it; they are checked against an independent float64
+    PyTorch autograd model on the CPU (closed-form definitions only).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from util import hptr
+
+pytestmark = pytest.mark.gpu
+
+BLOCK_PARAMS = ["Wq", "Wk", "Wv", "Wo", "bo", "W1", "b1", "W2", "b2", "ln1_gamma", "ln1_beta", "ln2_gamma",
+                "ln2_beta"]
+
+
+def make_tokens(rng, vocab, batch, seq):
+    p = 1.0 / np.arange(1, vocab + 1) ** 1.1     # Zipf(s=1.1) over the vocabulary
+    p /= p.sum()
+    return rng.choice(vocab, size=(batch, seq + 1), p=p).astype(np.int32)
+
+
+def cm(a):
+    """(rows, cols) array -> dense column-major float32 vector"""
+    return np.ascontiguousarray(np.asarray(a, np.float32).T).reshape(-1)
+
+
+def test_reference_configuration_tracks_the_reference_cpu_model(gpu):
+    ref = oracle.load_ref()
+    if ref is None:
+        pytest.skip("oracle/_ref/libjzref.so not built")
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 13, 16, 4, 32, 2, 8, 3
+    N = S * B
+    lr = 2e-3
+    rng = np.random.default_rng(0)
+    m = CharLM(V, d, heads, ff, L, S, B, gelu=False, tied=False, adamw=False, lr=lr)
+    m.init_random(1)
+    m.set("embed_bias", rng.normal(0, 0.1, (d, 1)))
+    m.set("head_bias", rng.normal(0, 0.1, (V, 1)))
+    h = ref.jzref_lm_create(V, d, heads, ff, L, S, B)
+    keep = []
+
+    def give(kind, layer, which, arr):
+        buf = cm(arr)
+        keep.append(buf)
+        assert ref.jzref_lm_param(h, kind, layer, which, hptr(buf), 1) == 0
+
+    give(0, 0, 0, np.hstack([m.get("embed"), m.get("pos")]))
+    give(1, 0, 0, m.get("embed_bias"))
+    give(2, 0, 0, m.get("head"))
+    give(3, 0, 0, m.get("head_bias"))
+    for l in range(L):
+        for w, name in enumerate(BLOCK_PARAMS):
+            give(4, l, w, m.get(f"block{l}.{name}"))
+    ref.jzref_lm_set_lr(h, lr)
+
+    tokens = make_tokens(rng, V, B, S)
+    m.set_batch(tokens)
+    X = np.zeros((V + S, N), np.float32)
+    Y = np.zeros((V, N), np.float32)
+    for b in range(B):
+        for s in range(S):
+            n = b * S + s
+            X[tokens[b, s], n] = 1
+            X[V + s, n] = 1
+            Y[tokens[b, s + 1], n] = 1
+    Xc, Yc = cm(X), cm(Y)
+    worst = 0.0
+    first = last = None
+    for step in range(100):
+        want = ref.jzref_lm_step(h, hptr(Xc), hptr(Yc))
+        m.step()
+        got = m.loss()
+        worst = max(worst, abs(got - want) / abs(want))
+        first = want if first is None else first
+        last = want
+    print(f"reference-configuration LM: loss {first:.4f} -> {last:.4f}, worst rel err {worst:.2e}")
+    assert last < first                      # it trains
+    assert worst <= 1e-3
+    # parameters after 100 steps
+    buf = np.empty(d * d, np.float32)
+    ref.jzref_lm_param(h, 4, L - 1, 0, hptr(buf), 0)
+    got = cm(m.get(f"block{L - 1}.Wq"))
+    assert np.linalg.norm(got - buf) <= 1e-3 * np.linalg.norm(buf)
+    ref.jzref_lm_destroy(h)
+    m.close()
+
+
+def torch_twin(cfg, params, tokens, steps, lr, wd):
+    """float64 autograd restatement: pre-LN blocks, exact-erf GELU, tied head, AdamW."""
+    import torch
+    V, d, heads, ff, L, S, B = cfg
+    dh = d // heads
+    P = {k: torch.tensor(v, dtype=torch.float64, requires_grad=True) for k, v in params.items()}
+    opt_decay = [v for k, v in P.items() if v.shape[1] > 1]
+    opt_plain = [v for k, v in P.items() if v.shape[1] == 1]
+    opt = torch.optim.AdamW([{"params": opt_decay, "weight_decay": wd}, {"params": opt_plain, "weight_decay": 0.0}],
+                            lr=lr, betas=(0.9, 0.999), eps=1e-8)
+    tok = torch.tensor(tokens[:, :-1].reshape(-1), dtype=torch.long)
+    tgt = torch.tensor(tokens[:, 1:].reshape(-1), dtype=torch.long)
+    pos = torch.arange(S).repeat(B)
+    mask = torch.triu(torch.ones(S, S, dtype=torch.bool), 1)          # [query, key] key > query
+    losses = []
+    first_grads = {}
+
+    def ln(x, g, b):
+        mu = x.mean(0, keepdim=True)
+        var = ((x - mu) ** 2).mean(0, keepdim=True)
+        return (x - mu) / torch.sqrt(var + 1e-5) * g + b
+
+    for _ in range(steps):
+        x = P["embed"][:, tok] + P["pos"][:, pos]                       # (d, N)
+        for l in range(L):
+            p = lambda n: P[f"block{l}.{n}"]
+            x1 = ln(x, p("ln1_gamma"), p("ln1_beta"))
+            q, k, v = p("Wq") @ x1, p("Wk") @ x1, p("Wv") @ x1
+            H = torch.zeros_like(q)
+            for hh in range(heads):
+                for b in range(B):
+                    rs, cs = slice(hh * dh, (hh + 1) * dh), slice(b * S, (b + 1) * S)
+                    s = (q[rs, cs].T @ k[rs, cs]) / np.sqrt(dh)
+                    s = s.masked_fill(mask, -1e9)
+                    a = torch.softmax(s, dim=1)
+                    H[rs, cs] = v[rs, cs] @ a.T
+            R = x + p("Wo") @ H + p("bo")
+            x2 = ln(R, p("ln2_gamma"), p("ln2_beta"))
+            f1 = p("W1") @ x2 + p("b1")
+            x = R + p("W2") @ torch.nn.functional.gelu(f1) + p("b2")
+        logits = P["embed"].T @ x                                       # (V, N)
+        loss = torch.nn.functional.cross_entropy(logits.T, tgt)
+        losses.append(float(loss))
+        opt.zero_grad()
+        loss.backward()
+        if not first_grads:
+            first_grads.update({k: v.grad.detach().numpy().copy() for k, v in P.items()})
+        opt.step()
+    return losses, {k: v.detach().numpy() for k, v in P.items()}, first_grads
+
+
+def test_gelu_tied_adamw_against_float64_autograd(gpu):
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 17, 32, 4, 64, 2, 12, 4
+    lr, wd = 3e-3, 0.01
+    rng = np.random.default_rng(5)
+    m = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=True, adamw=True, lr=lr, weight_decay=wd)
+    m.init_random(2)
+    for n in m.names:                      # non-trivial biases / gains so every gradient path is live
+        r, c = m.shape(n)
+        if c == 1:
+            m.set(n, m.get(n) + rng.normal(0, 0.05, (r, 1)).astype(np.float32))
+    params = {n: m.get(n).astype(np.float64) for n in m.names}
+    tokens = make_tokens(rng, V, B, S)
+    m.set_batch(tokens)
+    steps = 100
+    want, final, _ = torch_twin((V, d, heads, ff, L, S, B), params, tokens, steps, lr, wd)
+    worst = 0.0
+    for i in range(steps):
+        m.step()
+        got = m.loss()
+        worst = max(worst, abs(got - want[i]) / abs(want[i]))
+    print(f"GELU/tied/AdamW LM: loss {want[0]:.4f} -> {want[-1]:.4f}, worst rel err {worst:.2e}")
+    assert want[-1] < want[0]
+    assert worst <= 1e-3                   # train-step losses after 100 steps
+    for n in ("embed", "pos", "block0.W1", "block1.Wq", "block1.ln2_gamma", "block0.b1"):
+        a, b = m.get(n), final[n]
+        assert np.linalg.norm(a - b) <= 2e-3 * np.linalg.norm(b), n
+    m.close()
+
+
+def test_gradients_against_float64_autograd(gpu):
+    """One backward pass: every parameter gradient against autograd (no optimiser)."""
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 11, 16, 2, 48, 1, 9, 3
+    rng = np.random.default_rng(7)
+    m = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=True, adamw=True, lr=0.0, weight_decay=0.0)
+    m.init_random(3)
+    for n in m.names:
+        r, c = m.shape(n)
+        if c == 1:
+            m.set(n, m.get(n) + rng.normal(0, 0.1, (r, 1)).astype(np.float32))
+    params = {n: m.get(n).astype(np.float64) for n in m.names}
+    tokens = make_tokens(rng, V, B, S)
+    m.set_batch(tokens)
+    m.forward()
+    m.backward(update=False)
+    losses, _, grads = torch_twin((V, d, heads, ff, L, S, B), params, tokens, 1, 0.0, 0.0)
+    assert abs(m.loss() - losses[0]) <= 1e-4 * abs(losses[0])
+    for name in m.names:
+        got, want = m.get(name, which=1), grads[name]
+        assert np.linalg.norm(got - want) <= 1e-3 * np.linalg.norm(want), name
+    m.close()
