@@ -1,0 +1,242 @@
+#!/usr/bin/env python3
+"""Headline benchmark: transformer train-step tokens/s on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Workload (BASELINE.json configs[3]): character-level LM, vocab 256 byte tokens
+drawn from Zipf(s=1.1), context 256, batch 64 (16 384 tokens per step), 6
+pre-LayerNorm decoder blocks, d_model 512, 8 heads, causal softmax attention,
+FFN 2048 with GELU, tied embeddings, learned positional table, cross-entropy,
+AdamW (lr 3e-4, wd 0.01), fp32 everywhere.  One step = forward + loss +
+backward + optimiser on a synthetic batch that is already resident in HBM.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the fp32 MFMA
+GEMM): algorithmic flops (2*m*n*k summed over its launches) divided by its
+launch time, measured with HIP events around every launch in separate
+instrumented steps after the timed region.  `cpu_baseline` times the
+reference's own CPU path (oracle/_ref, OpenBLAS build when available) on a
+bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+
+CFG = dict(vocab=256, d_model=512, heads=8, d_ff=2048, layers=6, seq=256, batch=64)
+
+
+def zipf_tokens(rng, vocab, batch, seq, s=1.1):
+    import numpy as np
+    p = 1.0 / np.arange(1, vocab + 1) ** s
+    p /= p.sum()
+    return rng.choice(vocab, size=(batch, seq + 1), p=p).astype(np.int32)
+
+
+class HipEvents:
+    """hipEvent timing on the stream the library launches on (plain HIP runtime)."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.hip.hipDeviceSynchronize.argtypes = []
+
+    def event(self):
+        e = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.hip.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return float(ms.value)
+
+    def sync(self):
+        assert self.hip.hipDeviceSynchronize() == 0
+
+
+def cpu_baseline(seconds_budget=40.0):
+    """Reference CPU path (nearest reference architecture: ReLU FFN, Adam, untied
+    head; examples/demo_transformer.cu wiring) at the benchmark's model size on a
+    bounded sample of sequences."""
+    import numpy as np
+    import oracle
+    ob = oracle.REF_DIR / "libjzref_openblas.so"
+    kind_note = "OpenBLAS"
+    lib = None
+    cores = 1
+    if ob.exists():
+        try:
+            lib = C.CDLL(str(ob))
+            for dep in sorted(Path("/usr/local/lib").glob("python3*/dist-packages/scipy.libs/libscipy_openblas*.so")):
+                blas = C.CDLL(str(dep))
+                want = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+                blas.scipy_openblas_set_num_threads(C.c_int(want))
+                blas.scipy_openblas_get_num_threads.restype = C.c_int
+                cores = int(blas.scipy_openblas_get_num_threads())
+                break
+        except OSError:
+            lib = None
+    if lib is None:
+        if not oracle.REF_LIB.exists():
+            return None
+        lib = C.CDLL(str(oracle.REF_LIB))
+        kind_note = "BLAS-free (cpp/cpulinalg.hpp)"
+        cores = 1
+    lib.jzref_init()
+    lib.jzref_lm_create.restype = C.c_void_p
+    lib.jzref_lm_create.argtypes = [C.c_int] * 7
+    lib.jzref_lm_step.restype = C.c_float
+    lib.jzref_lm_step.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.jzref_lm_destroy.argtypes = [C.c_void_p]
+    V, d, heads, ff, L, S = CFG["vocab"], CFG["d_model"], CFG["heads"], CFG["d_ff"], CFG["layers"], CFG["seq"]
+    B = 2 if kind_note == "OpenBLAS" else 1
+    N = S * B
+    rng = np.random.default_rng(0)
+    tok = zipf_tokens(rng, V, B, S)
+    X = np.zeros((N, V + S), np.float32)     # column-major ((V+S) x N)
+    Y = np.zeros((N, V), np.float32)
+    for b in range(B):
+        for s in range(S):
+            n = b * S + s
+            X[n, tok[b, s]] = 1
+            X[n, V + s] = 1
+            Y[n, tok[b, s + 1]] = 1
+    h = lib.jzref_lm_create(V, d, heads, ff, L, S, B)
+    t0 = time.perf_counter()
+    steps = 0
+    while True:
+        lib.jzref_lm_step(h, X.ctypes.data, Y.ctypes.data)
+        steps += 1
+        el = time.perf_counter() - t0
+        if el > seconds_budget * 0.5 or steps >= 3:
+            break
+    el = time.perf_counter() - t0
+    lib.jzref_lm_destroy(h)
+    return {
+        "value": round(N * steps / el, 2), "unit": "tokens/s", "cores": cores, "kind": "reference",
+        "sample": f"{steps} train step(s) of the reference's own CPU classes (LinearLayer + 6 TransformerLayer<float> "
+                  f"+ LogisticLayer, ReLU FFN, Adam; {kind_note} build) at d_model 512 / 8 heads / d_ff 2048 / "
+                  f"context 256 on {B} of the 64 sequences ({N} tokens per step); {cores} core(s) for BLAS, "
+                  f"1 core elsewhere; {el:.1f} s wall",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only; --gpus N with N > 1 is not supported "
+              "(the path has no collectives).", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch  # device presence check only; all compute goes through libjzhip.so
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from juzhen_amd import capi
+    from juzhen_amd.lm import CharLM
+
+    lib = capi.load()
+    ev = HipEvents()
+    stream = lib.jzhip_get_stream()
+
+    model = CharLM(**CFG, gelu=True, tied=True, adamw=True, lr=3e-4, weight_decay=0.01)
+    model.init_random(0)
+    rng = np.random.default_rng(1234)
+    model.set_batch(zipf_tokens(rng, CFG["vocab"], CFG["batch"], CFG["seq"]))
+    tokens_per_step = model.tokens_per_step
+
+    for _ in range(args.warmup):
+        model.step()
+    ev.sync()
+    first_loss = model.loss()
+
+    e0, e1 = ev.event(), ev.event()
+    ev.sync()
+    t0 = time.perf_counter()
+    ev.record(e0, stream)
+    for _ in range(args.steps):
+        model.step()
+    ev.record(e1, stream)
+    gpu_ms = ev.elapsed_ms(e0, e1)
+    ev.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    last_loss = model.loss()
+    ms_per_step = max(gpu_ms, wall_ms) / args.steps
+    value = tokens_per_step / (ms_per_step * 1e-3)
+
+    # instrumented steps: HIP events around every tiled-GEMM launch
+    lib.jzhip_profile_gemm(1)
+    prof_steps = 2
+    for _ in range(prof_steps):
+        model.step()
+    buf = C.create_string_buffer(1 << 16)
+    assert lib.jzhip_profile_gemm_report(buf, len(buf)) == 0
+    lib.jzhip_profile_gemm(0)
+    kernels = json.loads(buf.value.decode())
+    kernels.sort(key=lambda k: -k["total_ms"])
+    gemm_ms_per_step = sum(k["total_ms"] for k in kernels) / prof_steps
+    gemm_flops_per_step = sum(k["flops"] for k in kernels) / prof_steps
+    dom = kernels[0]
+    achieved = dom["flops"] / (dom["total_ms"] * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "kernel": dom["kernel"], "launches_per_step": dom["launches"] // prof_steps,
+        "avg_launch_us": round(dom["total_ms"] * 1e3 / dom["launches"], 2),
+        "flops_per_launch": round(dom["flops"] / dom["launches"], 1),
+        "all_gemm_kernels": {"tflops": round(gemm_flops_per_step / (gemm_ms_per_step * 1e-3) / 1e12, 2),
+                             "ms_per_step": round(gemm_ms_per_step, 3),
+                             "share_of_step": round(gemm_ms_per_step / ms_per_step, 3)},
+    }
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        try:
+            cpu = cpu_baseline()
+        except Exception as exc:  # the baseline must never take the GPU number down with it
+            cpu = {"value": None, "unit": "tokens/s", "cores": 0, "kind": "reference", "sample": f"failed: {exc}"}
+
+    out = {
+        "metric": "transformer train-step tokens/s", "value": round(value, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "char-LM train step: vocab 256 (Zipf 1.1), context 256, batch 64, 6 pre-LN blocks, "
+                               "d_model 512, 8 heads, FFN 2048 GELU, tied embeddings, learned positions, AdamW "
+                               "lr 3e-4 wd 0.01", "tokens_per_step": tokens_per_step,
+                   "parameters": int(model.param_count), "loss_first": round(first_loss, 4),
+                   "loss_last": round(last_loss, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 3)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    if cpu and cpu.get("value"):
+        out["speedup_vs_cpu_baseline"] = round(value / cpu["value"], 1)
+    model.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

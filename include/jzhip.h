@@ -218,6 +218,13 @@ int jzhip_gemm_strided_batched(const float* A, const float* B, float* C,
                                long long stride_a, long long stride_b,
                                long long stride_c, int batch,
                                float alpha, float beta);
+/* Measurement aid, no reference counterpart: while enabled, every launch of
+ * the tiled MFMA kernel is bracketed by HIP events on its stream.
+ * jzhip_profile_gemm_report synchronises and writes a JSON array with, per
+ * kernel instantiation, the launch count, the summed duration in ms and the
+ * summed algorithmic flops (2*m*n*k), then forgets the records. */
+int jzhip_profile_gemm(int enable);
+int jzhip_profile_gemm_report(char* json_out, size_t capacity);
 /* y(rows x cols, column-major, ld=rows) += b[i] broadcast over columns: the
  * rank-1 product `b * ones(1,N)` the layers use for every bias
  * (ml/layer.hpp:79,120,2797; CUDA add_bias_kernel ml/layer.hpp:2538-2542). */

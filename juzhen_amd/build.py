@@ -185,8 +185,30 @@ def build_host(force: bool = False, jobs: int = 6):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         lib_objs = list(ex.map(compile_one, lib_srcs))
         prog_objs = list(ex.map(compile_one, REFERENCE_PROGRAMS))
-    bins = []
-    for rel, obj in zip(REFERENCE_PROGRAMS, prog_objs):
+    # the benchmark-configuration harness, once per backend
+    cfg_src = PKG / "harness" / "configs.cu"
+    cfg_obj = hostobj / "configs_rocm.o"
+    if force or _stale(cfg_obj, [cfg_src, *ours, ROOT / "include" / "jzhip.h"]):
+        _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(cfg_src), "-o", str(cfg_obj)], "compile configs.cu (rocm)")
+    REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj)]
+    cpu_bin = REF_BIN / "configs_cpu"
+    if force or _stale(cpu_bin, [cfg_src]):
+        blas = sorted(Path("/usr/local/lib").glob("python3*/dist-packages/scipy.libs/libscipy_openblas*.so"))
+        cmd = ["g++", "-std=c++20", "-O2", "-x", "c++", "-DLOGGING_OFF", f'-DPROJECT_DIR="{PROJECT_DIR}"', "-w",
+               f"-I{REFERENCE_ROOT}", f"-I{REFERENCE_ROOT / 'tests'}"]
+        if blas:   # the reference's default CBLAS configuration (cpp/helper.hpp:190-250)
+            cmd += [f"-I{REFERENCE_ROOT / 'external' / 'OpenBLAS' / 'include'}"] + \
+                   [f"-Dcblas_{f}=scipy_cblas_{f}" for f in ("sgemm", "dgemm", "sgemv", "dgemv")]
+        else:      # BLAS-free configuration (cpp/cpulinalg.hpp)
+            cmd += ["-DJUZHEN_NO_BLAS", "-ffp-contract=off"]
+        cmd += [str(REFERENCE_ROOT / "cpp" / "launcher.cu"), str(cfg_src), "-o", str(cpu_bin)]
+        if blas:
+            cmd += ["-x", "none", str(blas[0]), f"-Wl,-rpath,{blas[0].parent}"]
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        if r.returncode != 0:
+            raise RuntimeError(f"configs.cu (cpu) failed:\n{r.stderr[-4000:]}")
+    bins = [cpu_bin]
+    for rel, obj in REFERENCE_PROGRAMS_ALL:
         out = REF_BIN / Path(rel).stem
         if force or _stale(out, [obj, *lib_objs, LIB]):
             _hipcc(["--offload-arch=gfx950", "-o", str(out), str(obj), *map(str, lib_objs),

@@ -79,6 +79,8 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_gemm_nn": (I, [P, P, P, I, I, I, F, F]),
     "jzhip_gemv": (I, [P, P, P, I, I, I, I, I, I, F, F]),
     "jzhip_gemm_strided_batched": (I, [P, P, P, I, I, I, I, I, I, I, I, LL, LL, LL, I, F, F]),
+    "jzhip_profile_gemm": (I, [I]),
+    "jzhip_profile_gemm_report": (I, [C.c_char_p, Z]),
     "jzhip_add_bias": (I, [P, P, I, I]),
     "jzhip_softmax_cols": (I, [P, P, I, I, I]),
     "jzhip_softmax_rows": (I, [P, P, I, I, I]),

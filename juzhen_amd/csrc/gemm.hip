@@ -13,8 +13,32 @@
 // writes 128-byte contiguous segments of the column-major C.
 #include "common.hpp"
 
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
 namespace jz {
 namespace {
+
+// Optional per-launch timing of the tiled kernel (jzhip_profile_gemm): HIP
+// events recorded on the launch stream around every launch, aggregated per
+// kernel instantiation when the report is read.
+struct GemmProfRecord {
+    hipEvent_t begin, end;
+    std::string kernel;
+    double flops;
+};
+struct GemmProf {
+    std::mutex mu;
+    bool on = false;
+    std::vector<GemmProfRecord> recs;
+};
+GemmProf& gemm_prof() {
+    static GemmProf p;
+    return p;
+}
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -383,6 +407,19 @@ int launch_tile(const GemmArgs& g) {
                       (g.sB % 4 == 0) && (g.sA2 % 4 == 0) && (g.sB2 % 4 == 0);
     dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, splits, g.batch * g.batch2);
     hipStream_t s = stream();
+    GemmProf& prof = gemm_prof();
+    GemmProfRecord rec;
+    const bool timing = prof.on;
+    if (timing) {
+        char name[96];
+        std::snprintf(name, sizeof name, "gemm_mfma_kernel<%d, %d, %d, %d, %s, %s, %s>", WGM, WGN, TM, TN,
+                      TA ? "true" : "false", TB ? "true" : "false", fast ? "true" : "false");
+        rec.kernel = name;
+        rec.flops = 2.0 * g.M * g.N * g.K * g.batch * g.batch2;
+        (void)hipEventCreate(&rec.begin);
+        (void)hipEventCreate(&rec.end);
+        (void)hipEventRecord(rec.begin, s);
+    }
     if (fast)
         gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true><<<grid, kBlock, 0, s>>>(
             g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2,
@@ -391,6 +428,11 @@ int launch_tile(const GemmArgs& g) {
         gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, false><<<grid, kBlock, 0, s>>>(
             g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2,
             g.sB2, g.sC2, tiles_m, tiles_n, k_chunk, split_stride);
+    if (timing) {
+        (void)hipEventRecord(rec.end, s);
+        std::lock_guard<std::mutex> lock(prof.mu);
+        prof.recs.push_back(rec);
+    }
     if (splits > 1) {
         const size_t total = static_cast<size_t>(g.M) * g.N;
         splitk_reduce_kernel<<<grid_for(total, kBlock, 4), kBlock, 0, s>>>(g.C, out, g.M, g.N, g.ldc, splits,
@@ -411,7 +453,12 @@ int launch_shape(const GemmArgs& g) {
     if (g.N <= 32) return launch_tile<4, 1, 2, 1, TA, TB>(g);   // 256 x 32
     if (g.M <= 64) return launch_tile<1, 4, 2, 1, TA, TB>(g);   // 64 x 128
     if (g.N <= 64) return launch_tile<4, 1, 1, 2, TA, TB>(g);   // 128 x 64
-    if (tiles(128, 128) < cus) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
+    // a long K is split across workgroups by launch_tile, so the big tile
+    // still fills the chip; otherwise fall back to 64 x 64 tiles
+    // (only when at least cus/8 big tiles exist: more than ~16 partial sums per
+    // output cost more in the reduction than the bigger tile saves)
+    const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && tiles(128, 128) * 8 >= cus;
+    if (tiles(128, 128) < cus && !splittable) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
     return launch_tile<2, 2, 2, 2, TA, TB>(g);                  // 128 x 128
 }
 
@@ -460,6 +507,48 @@ int gemm_batched2(const float* A, const float* B, float* C, int m, int n, int k,
 }  // namespace jz
 
 using namespace jz;
+
+JZ_API int jzhip_profile_gemm(int enable) {
+    GemmProf& p = gemm_prof();
+    std::lock_guard<std::mutex> lock(p.mu);
+    p.on = enable != 0;
+    return 0;
+}
+
+JZ_API int jzhip_profile_gemm_report(char* buf, size_t cap) {
+    if (!buf || cap == 0) return -1;
+    GemmProf& p = gemm_prof();
+    int rc = rc_of(hipStreamSynchronize(stream()));
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lock(p.mu);
+    struct Agg { long launches = 0; double ms = 0, flops = 0; };
+    std::map<std::string, Agg> agg;
+    for (GemmProfRecord& r : p.recs) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, r.begin, r.end) == hipSuccess) {
+            Agg& a = agg[r.kernel];
+            a.launches++;
+            a.ms += ms;
+            a.flops += r.flops;
+        }
+        (void)hipEventDestroy(r.begin);
+        (void)hipEventDestroy(r.end);
+    }
+    p.recs.clear();
+    std::string out = "[";
+    bool first = true;
+    for (const auto& kv : agg) {
+        char line[320];
+        std::snprintf(line, sizeof line, "%s{\"kernel\": \"%s\", \"launches\": %ld, \"total_ms\": %.6f, \"flops\": %.1f}",
+                      first ? "" : ", ", kv.first.c_str(), kv.second.launches, kv.second.ms, kv.second.flops);
+        out += line;
+        first = false;
+    }
+    out += "]";
+    if (out.size() + 1 > cap) return -1;
+    std::snprintf(buf, cap, "%s", out.c_str());
+    return 0;
+}
 
 JZ_API int jzhip_gemm_strided_batched(const float* A, const float* B, float* C, int m, int n, int k,
                                       int trans_a, int trans_b, int lda, int ldb, int ldc,

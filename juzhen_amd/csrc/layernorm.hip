@@ -216,18 +216,28 @@ __global__ __launch_bounds__(kBlock) void ln_param_partial_kernel(float* part, c
     }
 }
 
+// part is [chunk][2*dim]; a block owns 64 of the 2*dim outputs, its waves take
+// interleaved chunks and are combined through LDS.
 __global__ __launch_bounds__(kBlock) void ln_param_combine_kernel(float* dgamma, float* dbeta,
                                                                   const float* part, int dim,
                                                                   int chunks) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= dim) return;
-    float sg = 0.f, sb = 0.f;
-    for (int c = 0; c < chunks; ++c) {
-        sg += part[(static_cast<size_t>(c) * 2 + 0) * dim + i];
-        sb += part[(static_cast<size_t>(c) * 2 + 1) * dim + i];
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int i = blockIdx.x * kWave + lane;
+    const int n = 2 * dim;
+    float acc = 0.f;
+    if (i < n)
+        for (int c = wave; c < chunks; c += NW) acc += part[static_cast<size_t>(c) * n + i];
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && i < n) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += red[w][lane];
+        if (i < dim) dgamma[i] = s; else dbeta[i - dim] = s;
     }
-    dgamma[i] = sg;
-    dbeta[i] = sb;
 }
 
 }  // namespace
@@ -289,7 +299,6 @@ JZ_API int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float*
     hipStream_t s = stream();
     dim3 grid(row_blocks, chunks);
     ln_param_partial_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
-    ln_param_combine_kernel<<<(dim + kBlock - 1) / kBlock, kBlock, 0, s>>>(dgamma, dbeta, part, dim,
-                                                                          chunks);
+    ln_param_combine_kernel<<<(2 * dim + kWave - 1) / kWave, kBlock, 0, s>>>(dgamma, dbeta, part, dim, chunks);
     return launch_rc();
 }

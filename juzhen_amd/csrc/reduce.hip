@@ -53,14 +53,33 @@ __global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const floa
     }
 }
 
-// out[i] = sum_{c<chunks} part[c*n + i]
+// out[i] = sum_{c<chunks} part[c*n + i].  A block owns 64 outputs; its four
+// waves take interleaved chunks (lanes stay on consecutive i, so reads are
+// coalesced) and are combined through LDS.
 __global__ __launch_bounds__(kBlock) void combine_partials_kernel(float* out, const float* part,
                                                                   int n, int chunks) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
-    float acc = 0.f;
-    for (int c = 0; c < chunks; ++c) acc += part[static_cast<size_t>(c) * n + i];
-    out[i] = acc;
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int i = blockIdx.x * kWave + lane;
+    float acc0 = 0.f, acc1 = 0.f;
+    if (i < n) {
+        int c = wave;
+        for (; c + NW < chunks; c += 2 * NW) {
+            acc0 += part[static_cast<size_t>(c) * n + i];
+            acc1 += part[static_cast<size_t>(c + NW) * n + i];
+        }
+        if (c < chunks) acc0 += part[static_cast<size_t>(c) * n + i];
+    }
+    red[wave][lane] = acc0 + acc1;
+    __syncthreads();
+    if (wave == 0 && i < n) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += red[w][lane];
+        out[i] = s;
+    }
 }
 
 // ── row sums: out[i] = sum_j a[j*ld + i] ─────────────────────────────────
@@ -265,8 +284,7 @@ JZ_API int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, in
     else
         sum_cols_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
     if (chunks > 1) {
-        combine_partials_kernel<<<(numcol + kBlock - 1) / kBlock, kBlock, 0, s>>>(out, dst, numcol,
-                                                                                  chunks);
+        combine_partials_kernel<<<(numcol + kWave - 1) / kWave, kBlock, 0, s>>>(out, dst, numcol, chunks);
     }
     return launch_rc();
 }
@@ -296,8 +314,8 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
         sum_rows_short_kernel<<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(dst, a, numrow, total,
                                                                               active, span);
         if (blocks > 1) {
-            combine_partials_kernel<<<(numrow + kBlock - 1) / kBlock, kBlock, 0, s>>>(
-                out, dst, numrow, static_cast<int>(blocks));
+            combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kBlock, 0, s>>>(out, dst, numrow,
+                                                                                    static_cast<int>(blocks));
         }
         return launch_rc();
     }
@@ -320,8 +338,7 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
     else
         sum_rows_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
     if (chunks > 1) {
-        combine_partials_kernel<<<(numrow + kBlock - 1) / kBlock, kBlock, 0, s>>>(out, dst, numrow,
-                                                                                  chunks);
+        combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kBlock, 0, s>>>(out, dst, numrow, chunks);
     }
     return launch_rc();
 }
