@@ -36,6 +36,7 @@ __device__ __forceinline__ float adam_one(float gi, float& mi_io, float& vi_io, 
 template <bool FUSE_W, bool VEC>
 __global__ __launch_bounds__(kBlock) void adam_kernel(float* w, float* g, float* m, float* v,
                                                       size_t n, AdamConst c) {
+    // one float4 per thread, grid covers the data once (see elementwise.hip)
     const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
     const size_t tid = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
     if constexpr (VEC) {
@@ -115,7 +116,10 @@ template <bool FUSE_W>
 int launch_adam(float* w, float* g, float* m, float* v, size_t n, const AdamConst& c) {
     if (n == 0) return 0;
     const bool vec = aligned16(g) && aligned16(m) && aligned16(v) && (!FUSE_W || aligned16(w));
-    const unsigned grid = grid_for(vec ? (n + 3) / 4 : n, kBlock, 8);
+    const size_t items = vec ? (n + 3) / 4 : n;
+    const size_t blocks = (items + kBlock - 1) / kBlock;
+    if (blocks > 0x7fffffffull) return -1;
+    const unsigned grid = static_cast<unsigned>(blocks);
     if (vec)
         adam_kernel<FUSE_W, true><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
     else

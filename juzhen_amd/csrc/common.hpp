@@ -42,6 +42,17 @@ inline unsigned grid_for(size_t work, size_t per_block, int blocks_per_cu = 8) {
     return static_cast<unsigned>(need < cap ? need : cap);
 }
 
+// Grid that covers `work` items exactly once (`per_block` items per block).
+// Streaming kernels use this rather than a capped grid-stride loop: workgroups
+// are dispatched in id order, so the resident ones then stream one compact,
+// moving window of memory.
+inline unsigned grid_cover(size_t work, size_t per_block) {
+    size_t need = (work + per_block - 1) / per_block;
+    if (need < 1) need = 1;
+    if (need > 0x7fffffffull) need = 0x7fffffffull;  // kernels keep their stride loop for the excess
+    return static_cast<unsigned>(need);
+}
+
 // ── wave64 reductions: DPP inside a 16-lane row, bpermute across rows ────
 #ifdef __HIPCC__
 template <int CTRL>
@@ -85,6 +96,20 @@ __device__ __forceinline__ float block_allreduce(float v, Op op, float* smem, fl
 #pragma unroll
     for (int w = 0; w < NW; ++w) r = op(r, smem[w]);
     return r;
+}
+
+// Work split for "one wavefront per column" kernels: wave w of nw owns the
+// contiguous range [wave_begin, wave_end) of the n columns, so the waves that
+// are resident together stream one compact window of memory.
+__device__ __forceinline__ size_t wave_begin(size_t n, size_t w, size_t nw) {
+    const size_t per = (n + nw - 1) / nw;
+    const size_t b = w * per;
+    return b < n ? b : n;
+}
+__device__ __forceinline__ size_t wave_end(size_t n, size_t w, size_t nw) {
+    const size_t per = (n + nw - 1) / nw;
+    const size_t e = (w + 1) * per;
+    return e < n ? e : n;
 }
 
 // Unsigned division by a runtime-uniform divisor via multiply-high.

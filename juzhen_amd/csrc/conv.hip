@@ -184,9 +184,9 @@ int gather_patches(const float* img, float* col, const PatchGeom& g) {
     if (static_cast<size_t>(g.C) * g.H * g.W * g.N >= (size_t(1) << 31)) return -1;
     if (g.K % 4 == 0 && aligned16(col)) {
         const size_t tv = total / 4;
-        im2col_kernel<4><<<grid_for(tv, kBlock, 8), kBlock, 0, stream()>>>(img, col, g, make_fastdiv(g.K / 4), tv);
+        im2col_kernel<4><<<grid_cover(tv, kBlock), kBlock, 0, stream()>>>(img, col, g, make_fastdiv(g.K / 4), tv);
     } else {
-        im2col_kernel<1><<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(img, col, g, g.dK, total);
+        im2col_kernel<1><<<grid_cover(total, kBlock), kBlock, 0, stream()>>>(img, col, g, g.dK, total);
     }
     return launch_rc();
 }
@@ -195,7 +195,7 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
     const size_t total = static_cast<size_t>(g.C) * g.H * g.W * g.N;
     if (total >= (size_t(1) << 31)) return -1;
     if (static_cast<size_t>(g.K) * g.P * g.N >= (size_t(1) << 31)) return -1;
-    col2im_kernel<<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(col, img, bias, g, total);
+    col2im_kernel<<<grid_cover(total, kBlock), kBlock, 0, stream()>>>(col, img, bias, g, total);
     return launch_rc();
 }
 

@@ -471,7 +471,7 @@ int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans
               size_t incx, size_t incy, float alpha, float beta) {
     hipStream_t s = stream();
     if (trans) {
-        gemv_t_kernel<<<grid_for(n, kBlock / kWave, 8), kBlock, 0, s>>>(A, x, y, m, n, lda, incx, incy,
+        gemv_t_kernel<<<grid_cover(n, kBlock / kWave), kBlock, 0, s>>>(A, x, y, m, n, lda, incx, incy,
                                                                          alpha, beta);
         return launch_rc();
     }
@@ -612,7 +612,7 @@ JZ_API int jzhip_add_bias(float* y, const float* b, int rows, int cols) {
     if (rows <= 0 || cols <= 0 || !y || !b) return -1;
     const size_t total = static_cast<size_t>(rows) * cols;
     if (rows % 4 == 0 && aligned16(y) && aligned16(b)) {
-        add_bias_kernel<<<grid_for(total / 4, kBlock, 8), kBlock, 0, stream()>>>(y, b, rows, total / 4);
+        add_bias_kernel<<<grid_cover(total / 4, kBlock), kBlock, 0, stream()>>>(y, b, rows, total / 4);
     } else {
         add_bias_scalar_kernel<<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(y, b, rows, total);
     }

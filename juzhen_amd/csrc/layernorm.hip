@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_vec_kernel(float* y, float* xha
             b[v] = *reinterpret_cast<const float4*>(beta + r);
         }
     }
-    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
         const size_t base = col * dim;
         float4 xv[NV];
         float s = 0.f;
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic_kernel(float* y, float*
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
     const float invdim = 1.0f / static_cast<float>(dim);
-    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
         const size_t base = col * dim;
         float s = 0.f;
         for (int r = lane; r < dim; r += kWave) s += x[base + r];
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
         const int r = (lane + v * kWave) * 4;
         if (r < dim) g[v] = *reinterpret_cast<const float4*>(gamma + r);
     }
-    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
         const size_t base = col * dim;
         float4 d[NV], h[NV];
         float s1 = 0.f, s2 = 0.f;
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
     const float invdim = 1.0f / static_cast<float>(dim);
-    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
         const size_t base = col * dim;
         float s1 = 0.f, s2 = 0.f;
         for (int r = lane; r < dim; r += kWave) {
@@ -250,7 +250,7 @@ JZ_API int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const floa
     if (dim <= 0 || N <= 0 || !y || !xhat || !inv_std || !x || !gamma || !beta) return -1;
     const bool vec = (dim % 4 == 0) && dim <= 1024 && aligned16(x) && aligned16(y) &&
                      aligned16(xhat) && aligned16(gamma) && aligned16(beta);
-    const unsigned grid = grid_for(N, kBlock / kWave, 8);
+    const unsigned grid = grid_cover(N, kBlock / kWave);
     hipStream_t s = stream();
     if (vec && dim <= 256)
         ln_fwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
@@ -268,7 +268,7 @@ JZ_API int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma, c
     if (dim <= 0 || N <= 0 || !dx || !dy || !gamma || !xhat || !inv_std) return -1;
     const bool vec = (dim % 4 == 0) && dim <= 1024 && aligned16(dx) && aligned16(dy) &&
                      aligned16(xhat) && aligned16(gamma);
-    const unsigned grid = grid_for(N, kBlock / kWave, 8);
+    const unsigned grid = grid_cover(N, kBlock / kWave);
     hipStream_t s = stream();
     if (vec && dim <= 256)
         ln_bwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);

@@ -277,7 +277,7 @@ JZ_API int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, in
         if (!dst) return -2;
     }
     const size_t items = static_cast<size_t>(numcol) * chunks;
-    const unsigned grid = grid_for(items, kBlock / kWave, 8);
+    const unsigned grid = grid_cover(items, kBlock / kWave);
     hipStream_t s = stream();
     if (vec)
         sum_cols_kernel<4><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
@@ -358,14 +358,14 @@ JZ_API int jzhip_nrm2(float* out_device, const float* x, size_t count) {
 
 JZ_API int jzhip_max_cols(float* out, const float* a, int numrow, int numcol, int ld) {
     if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
-    const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+    const unsigned grid = grid_cover(numcol, kBlock / kWave);
     max_cols_kernel<false><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
     return launch_rc();
 }
 
 JZ_API int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numcol, int ld) {
     if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
-    const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+    const unsigned grid = grid_cover(numcol, kBlock / kWave);
     max_cols_kernel<true><<<grid, kBlock, 0, stream()>>>(nullptr, out, a, numrow, numcol, ld);
     return launch_rc();
 }

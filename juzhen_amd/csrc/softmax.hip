@@ -32,7 +32,7 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_kernel(float* out, const 
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
-    for (size_t col = wave0; col < numcol; col += nwaves) {
+    for (size_t col = wave_begin(numcol, wave0, nwaves), col_end = wave_end(numcol, wave0, nwaves); col < col_end; ++col) {
         const float* p = in + col * ld;
         float* q = out + col * ld;
         const int qidx = xf.S ? static_cast<int>(col % xf.S) : 0;  // query index of this column
@@ -156,6 +156,141 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(float* out, const 
     }
 }
 
+// Row softmax with the whole row held in registers: 64 row lanes x 4 column
+// phases, NV columns per thread (numcol <= 4*NV), one read and one write per
+// element.  Used for attention score blocks (S <= 256) and other short rows.
+template <int NV>
+__global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(float* out, const float* in,
+                                                                  int numrow, int numcol, size_t ld,
+                                                                  size_t batch_stride, ScoreXform xf) {
+    constexpr int RPB = kWave, CP = kBlock / kWave;
+    __shared__ float red[CP][RPB];
+    const int rl = threadIdx.x % RPB;
+    const int cp = threadIdx.x / RPB;
+    const int row = blockIdx.x * RPB + rl;
+    const float* p = in + static_cast<size_t>(blockIdx.y) * batch_stride;
+    float* q = out + static_cast<size_t>(blockIdx.y) * batch_stride;
+    const bool live = row < numrow;
+    const bool causal = xf.S && xf.causal;
+    float x[NV];
+    float m = -1e30f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = cp + v * CP;
+        float t = -INFINITY;
+        if (live && c < numcol) {
+            if (causal && c > row) {
+                t = -1e9f;  // masked key (ml/layer.hpp:2979-2994); never loaded
+            } else {
+                t = p[static_cast<size_t>(c) * ld + row];
+                if (xf.S) t = t * xf.scale;
+            }
+            m = m > t ? m : t;
+        }
+        x[v] = t;
+    }
+    red[cp][rl] = m;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < CP; ++k) m = m > red[k][rl] ? m : red[k][rl];
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = cp + v * CP;
+        x[v] = (live && c < numcol) ? expf(x[v] - m) : 0.f;
+        s += x[v];
+    }
+    red[cp][rl] = s;
+    __syncthreads();
+    s = 0.f;
+#pragma unroll
+    for (int k = 0; k < CP; ++k) s += red[k][rl];
+    const float inv = 1.0f / (s + 1e-12f);
+    if (live) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int c = cp + v * CP;
+            if (c < numcol) q[static_cast<size_t>(c) * ld + row] = x[v] * inv;
+        }
+    }
+}
+
+// Long rows: columns are split into chunks over grid.y.  Pass A leaves one
+// (max, sum) pair per (row, chunk) in the workspace (online softmax inside the
+// chunk); pass B folds the pairs of a row and writes its chunk.  12 bytes per
+// element instead of the 16 of a three-sweep kernel, and rows x chunks
+// workgroups instead of rows/64.
+__global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* part, const float* in,
+                                                                      int numrow, int numcol,
+                                                                      size_t ld, int chunk_len) {
+    constexpr int RPB = kWave, CP = kBlock / kWave;
+    __shared__ float redm[CP][RPB], reds[CP][RPB];
+    const int rl = threadIdx.x % RPB, cp = threadIdx.x / RPB;
+    const int row = blockIdx.x * RPB + rl;
+    const int c0 = blockIdx.y * chunk_len;
+    const int c1 = (c0 + chunk_len) < numcol ? (c0 + chunk_len) : numcol;
+    float m = -1e30f, s = 0.f;
+    if (row < numrow) {
+        for (int c = c0 + cp; c < c1; c += CP) {
+            const float t = in[static_cast<size_t>(c) * ld + row];
+            if (t > m) {
+                s = s * expf(m - t) + 1.0f;
+                m = t;
+            } else {
+                s += expf(t - m);
+            }
+        }
+    }
+    redm[cp][rl] = m;
+    reds[cp][rl] = s;
+    __syncthreads();
+    if (cp == 0 && row < numrow) {
+        float M = -1e30f;
+#pragma unroll
+        for (int k = 0; k < CP; ++k) M = M > redm[k][rl] ? M : redm[k][rl];
+        float S = 0.f;
+#pragma unroll
+        for (int k = 0; k < CP; ++k) S += reds[k][rl] * expf(redm[k][rl] - M);
+        const size_t o = (static_cast<size_t>(blockIdx.y) * numrow + row) * 2;
+        part[o] = M;
+        part[o + 1] = S;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, const float* in,
+                                                                    const float* part, int numrow,
+                                                                    int numcol, size_t ld,
+                                                                    int chunk_len, int chunks) {
+    constexpr int RPB = kWave, CP = kBlock / kWave;
+    __shared__ float row_m[RPB], row_inv[RPB];
+    const int rl = threadIdx.x % RPB, cp = threadIdx.x / RPB;
+    const int row = blockIdx.x * RPB + rl;
+    if (cp == 0 && row < numrow) {
+        float M = -1e30f;
+        for (int k = 0; k < chunks; ++k) {
+            const float mk = part[(static_cast<size_t>(k) * numrow + row) * 2];
+            M = M > mk ? M : mk;
+        }
+        float S = 0.f;
+        for (int k = 0; k < chunks; ++k) {
+            const size_t o = (static_cast<size_t>(k) * numrow + row) * 2;
+            S += part[o + 1] * expf(part[o] - M);
+        }
+        row_m[rl] = M;
+        row_inv[rl] = 1.0f / (S + 1e-12f);
+    }
+    __syncthreads();
+    if (row >= numrow) return;
+    const float M = row_m[rl], inv = row_inv[rl];
+    const int c0 = blockIdx.y * chunk_len;
+    const int c1 = (c0 + chunk_len) < numcol ? (c0 + chunk_len) : numcol;
+    for (int c = c0 + cp; c < c1; c += CP) {
+        const size_t i = static_cast<size_t>(c) * ld + row;
+        out[i] = expf(in[i] - M) * inv;
+    }
+}
+
 // ── softmax backward: dS = A*(dA - sum_keys(A*dA))*scale ─────────────────
 template <int NV>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_cols_kernel(float* dS, const float* A,
@@ -164,7 +299,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_cols_kernel(float* dS, con
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
-    for (size_t col = wave0; col < numcol; col += nwaves) {
+    for (size_t col = wave_begin(numcol, wave0, nwaves), col_end = wave_end(numcol, wave0, nwaves); col < col_end; ++col) {
         const size_t base = col * numrow;
         float a[NV], g[NV];
         float dot = 0.f;
@@ -225,7 +360,7 @@ __global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, fl
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
-    for (size_t col = wave0; col < static_cast<size_t>(N); col += nwaves) {
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
         const float* p = logits + col * ld;
         const int label = labels[col];
         float x[NV];
@@ -286,7 +421,7 @@ int dispatch_nv(int numrow, Args... args) {
 template <int NV>
 struct SoftmaxColsL {
     static int run(float* out, const float* in, int numrow, size_t numcol, size_t ld, ScoreXform xf) {
-        const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+        const unsigned grid = grid_cover(numcol, kBlock / kWave);
         softmax_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld, xf);
         return launch_rc();
     }
@@ -294,7 +429,7 @@ struct SoftmaxColsL {
 template <int NV>
 struct SoftmaxBwdColsL {
     static int run(float* dS, const float* A, const float* dA, int numrow, size_t numcol, float scale) {
-        const unsigned grid = grid_for(numcol, kBlock / kWave, 8);
+        const unsigned grid = grid_cover(numcol, kBlock / kWave);
         softmax_bwd_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(dS, A, dA, numrow, numcol, scale);
         return launch_rc();
     }
@@ -303,7 +438,7 @@ template <int NV>
 struct XentL {
     static int run(float* per_sample, float* dlogits, const float* logits, const int32_t* labels,
                    int K, int N, size_t ld) {
-        const unsigned grid = grid_for(N, kBlock / kWave, 8);
+        const unsigned grid = grid_cover(N, kBlock / kWave);
         xent_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, labels, K, N,
                                                             ld, static_cast<float>(1.0 / N));
         return launch_rc();
@@ -322,15 +457,42 @@ int softmax_cols_impl(float* out, const float* in, int numrow, size_t numcol, si
 int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_t ld, int batch,
                       size_t batch_stride, ScoreXform xf) {
     if (batch > 65535) return -1;
-    // small problems: 16-row strips give 4x more blocks than 64-row strips
-    const bool small = static_cast<size_t>((numrow + 63) / 64) * batch < static_cast<size_t>(num_cus()) * 2;
-    if (small) {
-        dim3 grid((numrow + 15) / 16, batch);
-        softmax_rows_kernel<16><<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld, batch_stride, xf);
-    } else {
-        dim3 grid((numrow + 63) / 64, batch);
-        softmax_rows_kernel<64><<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+    hipStream_t s = stream();
+    const int row_blocks = (numrow + kWave - 1) / kWave;
+    if (numcol <= 256) {
+        // whole row in registers
+        dim3 grid(row_blocks, batch);
+        if (numcol <= 16)
+            softmax_rows_reg_kernel<4><<<grid, kBlock, 0, s>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+        else if (numcol <= 64)
+            softmax_rows_reg_kernel<16><<<grid, kBlock, 0, s>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+        else if (numcol <= 128)
+            softmax_rows_reg_kernel<32><<<grid, kBlock, 0, s>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+        else
+            softmax_rows_reg_kernel<64><<<grid, kBlock, 0, s>>>(out, in, numrow, numcol, ld, batch_stride, xf);
+        return launch_rc();
     }
+    if (batch == 1 && !xf.S) {
+        // long rows: split the columns so that row_blocks x chunks fills the chip
+        int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
+        if (chunks > numcol / 32) chunks = numcol / 32;
+        if (chunks < 1) chunks = 1;
+        if (chunks > 4096) chunks = 4096;
+        while (chunks > 1 && static_cast<size_t>(chunks) * numrow * 2 > kWorkspaceFloats) --chunks;
+        const int chunk_len = (numcol + chunks - 1) / chunks;
+        chunks = (numcol + chunk_len - 1) / chunk_len;
+        if (static_cast<size_t>(chunks) * numrow * 2 <= kWorkspaceFloats) {
+            float* part = workspace();
+            if (!part) return -2;
+            dim3 grid(row_blocks, chunks);
+            softmax_rows_partial_kernel<<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
+            softmax_rows_apply_kernel<<<grid, kBlock, 0, s>>>(out, in, part, numrow, numcol, ld, chunk_len, chunks);
+            return launch_rc();
+        }
+    }
+    // general fallback: three sweeps per 64-row strip
+    dim3 grid(row_blocks, batch);
+    softmax_rows_kernel<64><<<grid, kBlock, 0, s>>>(out, in, numrow, numcol, ld, batch_stride, xf);
     return launch_rc();
 }
 
