@@ -41,9 +41,18 @@ GemmProf& gemm_prof() {
 }
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+// native vector type for staging registers (HIP's float4 is a struct around a
+// union, which kept the staging array in scratch memory)
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int BK = 16;
-constexpr int kPad = 4;  // keeps 16-byte alignment of LDS rows, skews banks
+#ifndef JZ_GEMM_BK
+#define JZ_GEMM_BK 16
+#endif
+#ifndef JZ_GEMM_PAD
+#define JZ_GEMM_PAD 4
+#endif
+constexpr int BK = JZ_GEMM_BK;     // K extent of one LDS stage
+constexpr int kPad = JZ_GEMM_PAD;  // keeps 16-byte alignment of LDS rows, skews banks
 
 // Global -> register staging for one operand tile of EXT (BM or BN) x BK.
 // MNC = true : the operand is contiguous along its m/n index (A not
@@ -54,62 +63,73 @@ template <int EXT, bool MNC>
 struct TileLoader {
     static constexpr int kVecs = EXT * BK / 4;             // float4 per tile
     static constexpr int kPasses = (kVecs + kBlock - 1) / kBlock;
-    float4 reg[kPasses];
 
     // FAST: tile fully inside the matrix, ld % 4 == 0, base 16-byte aligned.
     template <bool FAST>
-    __device__ __forceinline__ void load(const float* __restrict__ p, size_t ld, int x0, int k0,
-                                         int X, int K) {
+    static __device__ __forceinline__ void load(floatx4 (&reg)[kPasses], const float* __restrict__ p,
+                                                size_t ld, int x0, int k0, int X, int K) {
 #pragma unroll
         for (int ps = 0; ps < kPasses; ++ps) {
             const int v = threadIdx.x + ps * kBlock;
-            if (kVecs % kBlock != 0 && v >= kVecs) break;
-            int x, k;
-            if constexpr (MNC) {
-                x = (v % (EXT / 4)) * 4;
-                k = v / (EXT / 4);
-            } else {
-                k = (v % (BK / 4)) * 4;
-                x = v / (BK / 4);
-            }
-            const int gx = x0 + x, gk = k0 + k;
-            if constexpr (FAST) {
-                const float* src = MNC ? p + static_cast<size_t>(gk) * ld + gx
-                                       : p + static_cast<size_t>(gx) * ld + gk;
-                reg[ps] = *reinterpret_cast<const float4*>(src);
-            } else {
-                float t[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int ex = MNC ? gx + e : gx;
-                    const int ek = MNC ? gk : gk + e;
-                    t[e] = (ex < X && ek < K)
-                               ? (MNC ? p[static_cast<size_t>(ek) * ld + ex] : p[static_cast<size_t>(ex) * ld + ek])
-                               : 0.0f;
+            // (no early exit: the loop must unroll fully so reg[] stays in registers)
+            if (kVecs % kBlock == 0 || v < kVecs) {
+                int x, k;
+                if constexpr (MNC) {
+                    x = (v % (EXT / 4)) * 4;
+                    k = v / (EXT / 4);
+                } else {
+                    k = (v % (BK / 4)) * 4;
+                    x = v / (BK / 4);
                 }
-                reg[ps] = make_float4(t[0], t[1], t[2], t[3]);
+                const int gx = x0 + x, gk = k0 + k;
+                if constexpr (FAST) {
+                    const float* src = MNC ? p + static_cast<size_t>(gk) * ld + gx
+                                           : p + static_cast<size_t>(gx) * ld + gk;
+                    reg[ps] = *reinterpret_cast<const floatx4*>(src);
+                } else {
+                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (MNC) {
+                        if (gk < K) {
+                            const float* src = p + static_cast<size_t>(gk) * ld + gx;
+                            if (gx + 0 < X) t.x = src[0];
+                            if (gx + 1 < X) t.y = src[1];
+                            if (gx + 2 < X) t.z = src[2];
+                            if (gx + 3 < X) t.w = src[3];
+                        }
+                    } else {
+                        if (gx < X) {
+                            const float* src = p + static_cast<size_t>(gx) * ld + gk;
+                            if (gk + 0 < K) t.x = src[0];
+                            if (gk + 1 < K) t.y = src[1];
+                            if (gk + 2 < K) t.z = src[2];
+                            if (gk + 3 < K) t.w = src[3];
+                        }
+                    }
+                    reg[ps] = t;
+                }
             }
         }
     }
 
     // registers -> LDS tile laid out [BK][EXT + kPad]
-    __device__ __forceinline__ void store(float* __restrict__ s) const {
+    static __device__ __forceinline__ void store(const floatx4 (&reg)[kPasses], float* __restrict__ s) {
         constexpr int LD = EXT + kPad;
 #pragma unroll
         for (int ps = 0; ps < kPasses; ++ps) {
             const int v = threadIdx.x + ps * kBlock;
-            if (kVecs % kBlock != 0 && v >= kVecs) break;
-            if constexpr (MNC) {
-                const int x = (v % (EXT / 4)) * 4;
-                const int k = v / (EXT / 4);
-                *reinterpret_cast<float4*>(s + k * LD + x) = reg[ps];
-            } else {
-                const int k = (v % (BK / 4)) * 4;
-                const int x = v / (BK / 4);
-                s[(k + 0) * LD + x] = reg[ps].x;
-                s[(k + 1) * LD + x] = reg[ps].y;
-                s[(k + 2) * LD + x] = reg[ps].z;
-                s[(k + 3) * LD + x] = reg[ps].w;
+            if (kVecs % kBlock == 0 || v < kVecs) {
+                if constexpr (MNC) {
+                    const int x = (v % (EXT / 4)) * 4;
+                    const int k = v / (EXT / 4);
+                    *reinterpret_cast<floatx4*>(s + k * LD + x) = reg[ps];
+                } else {
+                    const int k = (v % (BK / 4)) * 4;
+                    const int x = v / (BK / 4);
+                    s[(k + 0) * LD + x] = reg[ps].x;
+                    s[(k + 1) * LD + x] = reg[ps].y;
+                    s[(k + 2) * LD + x] = reg[ps].z;
+                    s[(k + 3) * LD + x] = reg[ps].w;
+                }
             }
         }
     }
@@ -117,7 +137,7 @@ struct TileLoader {
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST>
-__global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
+__global__ __launch_bounds__(kBlock, 2) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
@@ -179,21 +199,22 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    TileLoader<BM, !TA> la;
-    TileLoader<BN, TB> lb;
+    using LA = TileLoader<BM, !TA>;
+    using LB = TileLoader<BN, TB>;
+    floatx4 ra[LA::kPasses], rb[LB::kPasses];  // next stage in flight, global -> registers
 
     const int nk = (k_hi - k_lo + BK - 1) / BK;
-    la.template load<FAST>(A, lda, m0, k_lo, M, k_hi);
-    lb.template load<FAST>(B, ldb, n0, k_lo, N, k_hi);
-    la.store(As[0]);
-    lb.store(Bs[0]);
+    LA::template load<FAST>(ra, A, lda, m0, k_lo, M, k_hi);
+    LB::template load<FAST>(rb, B, ldb, n0, k_lo, N, k_hi);
+    LA::store(ra, As[0]);
+    LB::store(rb, Bs[0]);
     __syncthreads();
 
     int cur = 0;
     for (int kt = 0; kt < nk; ++kt) {
         if (kt + 1 < nk) {
-            la.template load<FAST>(A, lda, m0, k_lo + (kt + 1) * BK, M, k_hi);
-            lb.template load<FAST>(B, ldb, n0, k_lo + (kt + 1) * BK, N, k_hi);
+            LA::template load<FAST>(ra, A, lda, m0, k_lo + (kt + 1) * BK, M, k_hi);
+            LB::template load<FAST>(rb, B, ldb, n0, k_lo + (kt + 1) * BK, N, k_hi);
         }
         const float* as = As[cur] + wm * (TM * 32) + l32;
         const float* bs = Bs[cur] + wn * (TN * 32) + l32;
@@ -211,8 +232,8 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma_kernel(
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j], af[i], acc[i][j], 0, 0, 0);
         }
         if (kt + 1 < nk) {
-            la.store(As[cur ^ 1]);
-            lb.store(Bs[cur ^ 1]);
+            LA::store(ra, As[cur ^ 1]);
+            LB::store(rb, Bs[cur ^ 1]);
         }
         __syncthreads();
         cur ^= 1;
