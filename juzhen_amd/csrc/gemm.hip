@@ -45,6 +45,9 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // union, which kept the staging array in scratch memory)
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+#ifndef JZ_GEMM_OCC
+#define JZ_GEMM_OCC 2
+#endif
 #ifndef JZ_GEMM_BK
 #define JZ_GEMM_BK 16
 #endif
@@ -137,7 +140,7 @@ struct TileLoader {
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST>
-__global__ __launch_bounds__(kBlock, 2) void gemm_mfma_kernel(
+__global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
@@ -210,33 +213,56 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_mfma_kernel(
     LB::store(rb, Bs[0]);
     __syncthreads();
 
+    // Software pipeline: the operand fragments of MFMA step kk+1 are read from
+    // LDS before the MFMAs of step kk are issued, and the first fragments of
+    // the next K stage are read right after the barrier, ahead of the last
+    // MFMAs of the current stage, so every LDS read has four MFMAs (256
+    // cycles) to land in.
+    constexpr int KS = BK / 2;  // MFMA steps per stage
+    static_assert(KS % 2 == 0, "fragment double buffer assumes an even step count");
+    float af[2][TM], bf[2][TN];
+    const int a_off = wm * (TM * 32) + l32 + h * LDA_S;
+    const int b_off = wn * (TN * 32) + l32 + h * LDB_S;
+    auto read_frags = [&](int slot, const float* as, const float* bs, int kk) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[slot][i] = as[2 * kk * LDA_S + i * 32];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bf[slot][j] = bs[2 * kk * LDB_S + j * 32];
+    };
+    auto mfma_step = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
+    };
+
     int cur = 0;
+    read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
     for (int kt = 0; kt < nk; ++kt) {
-        if (kt + 1 < nk) {
+        const bool more = kt + 1 < nk;
+        if (more) {
             LA::template load<FAST>(ra, A, lda, m0, k_lo + (kt + 1) * BK, M, k_hi);
             LB::template load<FAST>(rb, B, ldb, n0, k_lo + (kt + 1) * BK, N, k_hi);
         }
-        const float* as = As[cur] + wm * (TM * 32) + l32;
-        const float* bs = Bs[cur] + wn * (TN * 32) + l32;
+        const float* as = As[cur] + a_off;
+        const float* bs = Bs[cur] + b_off;
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = as[(kk + h) * LDA_S + i * 32];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) bf[j] = bs[(kk + h) * LDB_S + j * 32];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j], af[i], acc[i][j], 0, 0, 0);
+        for (int kk = 0; kk < KS - 1; ++kk) {
+            read_frags((kk + 1) & 1, as, bs, kk + 1);
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs they do not feed
+            mfma_step(kk & 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (kt + 1 < nk) {
+        if (more) {
             LA::store(ra, As[cur ^ 1]);
             LB::store(rb, Bs[cur ^ 1]);
         }
         __syncthreads();
         cur ^= 1;
+        if (more) read_frags(0, As[cur] + a_off, Bs[cur] + b_off, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step((KS - 1) & 1);
     }
 
     // Epilogue.  Register v of lane (h, l32) holds C(row, col) with

@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Per-kernel roofline report for the MI355X backend.
+
+    python -m juzhen_amd.opbench [--groups gemm,ew,reduce,fused,conv] [--out FILE]
+
+Every line is one C-ABI entry point at one shape: median and p95 launch time
+over 20 samples after 3 warm-ups (the reference's convention,
+tests/benchmarkCoreOps.cu:35-54 and tests/benchmarkTrainingStep.cu:73-74),
+the algorithmic bytes or flops of the call, and the fraction of the bound that
+applies (HBM 8 TB/s for streaming kernels, 157.3 TFLOP/s fp32 MFMA for GEMM).
+A sample is a HIP-event pair around enough back-to-back launches to last
+about 100 us, so short kernels are not priced at event resolution.
+
+The report is a Markdown table on stdout (or --out).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import sys
+from pathlib import Path
+
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+sys.path.insert(0, str(ROOT))
+
+from juzhen_amd import capi  # noqa: E402
+
+HBM_GBS = 8000.0
+MFMA_TFLOPS = 157.3
+
+
+class _Events:
+    def __init__(self):
+        h = self.hip = C.CDLL("libamdhip64.so")
+        h.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        h.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        h.hipEventSynchronize.argtypes = [C.c_void_p]
+        h.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.a, self.b = C.c_void_p(), C.c_void_p()
+        assert h.hipEventCreate(C.byref(self.a)) == 0 and h.hipEventCreate(C.byref(self.b)) == 0
+
+    def time_ms(self, fn, reps, stream):
+        h = self.hip
+        assert h.hipEventRecord(self.a, stream) == 0
+        for _ in range(reps):
+            fn()
+        assert h.hipEventRecord(self.b, stream) == 0
+        assert h.hipEventSynchronize(self.b) == 0
+        ms = C.c_float()
+        assert h.hipEventElapsedTime(C.byref(ms), self.a, self.b) == 0
+        return ms.value / reps
+
+
+class Report:
+    def __init__(self):
+        self.lib = capi.load()
+        self.jz = capi.jz
+        self.ev = _Events()
+        self.stream = C.c_void_p(self.lib.jzhip_get_stream())
+        self.rows = []
+
+    def run(self, group, name, shape, fn, *, bytes_=None, flops=None, samples=20, warm=3):
+        for _ in range(warm):
+            fn()
+        first = self.ev.time_ms(fn, 1, self.stream)
+        reps = max(1, min(64, int(0.1 / max(first, 1e-4))))
+        ts = sorted(self.ev.time_ms(fn, reps, self.stream) for _ in range(samples))
+        med = ts[len(ts) // 2]
+        p95 = ts[min(len(ts) - 1, int(round(0.95 * (len(ts) - 1))))]
+        if flops is not None:
+            ach = flops / (med * 1e-3) / 1e12
+            self.rows.append((group, name, shape, med, p95, f"{flops / 1e9:.2f} GF", f"{ach:.1f} TFLOP/s", ach / MFMA_TFLOPS, "mfma"))
+        else:
+            ach = bytes_ / (med * 1e-3) / 1e9
+            self.rows.append((group, name, shape, med, p95, f"{bytes_ / 1e6:.2f} MB", f"{ach:.0f} GB/s", ach / HBM_GBS, "hbm"))
+        print(f"{group} {name} {shape}: {med * 1e3:.1f} us  {self.rows[-1][6]}", file=sys.stderr, flush=True)
+
+    def markdown(self):
+        out = ["| group | entry point | shape | median us | p95 us | algorithmic | achieved | bound | frac |",
+               "|---|---|---|---:|---:|---:|---:|---|---:|"]
+        for g, n, s, med, p95, alg, ach, frac, bound in self.rows:
+            out.append(f"| {g} | {n} | {s} | {med * 1e3:.1f} | {p95 * 1e3:.1f} | {alg} | {ach} | {bound} | {frac:.2f} |")
+        return "\n".join(out) + "\n"
+
+
+def P(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def dev(n, fill=None):
+    if fill is None:
+        return torch.randn(n, device="cuda")
+    return torch.full((n,), float(fill), device="cuda")
+
+
+def bench_gemm(r):
+    jz = r.jz
+    shapes = [
+        # (label, m, n, k, ta, tb)
+        ("C1 chain NN", 1024, 1024, 1024, 0, 0),
+        ("C2 fwd NN", 256, 4096, 256, 0, 0), ("C2 dW NT", 256, 256, 4096, 0, 1), ("C2 dx TN", 256, 4096, 256, 1, 0),
+        ("C3 conv2 fwd TN", 64, 25088, 288, 1, 0), ("C3 conv2 dW NT", 288, 64, 25088, 0, 1),
+        ("C3 conv2 dcol NN", 288, 25088, 64, 0, 0),
+        ("C4 proj NN", 512, 16384, 512, 0, 0), ("C4 ffn1 NN", 2048, 16384, 512, 0, 0),
+        ("C4 ffn2 NN", 512, 16384, 2048, 0, 0), ("C4 dx TN", 512, 16384, 2048, 1, 0),
+        ("C4 dx TN", 2048, 16384, 512, 1, 0), ("C4 dW NT", 512, 512, 16384, 0, 1),
+        ("C4 dW NT", 2048, 512, 16384, 0, 1), ("C4 dW NT", 512, 2048, 16384, 0, 1),
+        ("C4 logits TN", 256, 16384, 512, 1, 0),
+        ("square NN", 4096, 4096, 4096, 0, 0), ("square NT", 4096, 4096, 4096, 0, 1),
+        ("square TN", 4096, 4096, 4096, 1, 0), ("square TT", 4096, 4096, 4096, 1, 1),
+        ("square NN", 8192, 8192, 8192, 0, 0), ("square TN", 8192, 8192, 8192, 1, 0),
+    ]
+    for label, m, n, k, ta, tb in shapes:
+        A, B, Cm = dev(m * k), dev(k * n), dev(m * n, 0)
+        lda, ldb = (k if ta else m), (n if tb else k)
+        r.run("gemm", f"jzhip_gemm {label}", f"{m}x{n}x{k}",
+              lambda: jz.gemm(P(A), P(B), P(Cm), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0), flops=2.0 * m * n * k)
+    # attention-shaped strided batches (C4: 512 blocks of 256x256x64)
+    S, dk, nb = 256, 64, 512
+    Q, K, A_ = dev(S * dk * nb), dev(S * dk * nb), dev(S * S * nb, 0)
+    r.run("gemm", "jzhip_gemm_strided_batched QK^T", f"{S}x{S}x{dk} x{nb}",
+          lambda: jz.gemm_strided_batched(P(Q), P(K), P(A_), S, S, dk, 1, 0, dk, dk, S, dk * S, dk * S, S * S, nb, 1.0, 0.0),
+          flops=2.0 * S * S * dk * nb)
+    r.run("gemm", "jzhip_gemm_strided_batched AV", f"{dk}x{S}x{S} x{nb}",
+          lambda: jz.gemm_strided_batched(P(Q), P(A_), P(K), dk, S, S, 0, 0, dk, S, dk, dk * S, S * S, dk * S, nb, 1.0, 0.0),
+          flops=2.0 * S * S * dk * nb)
+
+
+def bench_ew(r):
+    jz = r.jz
+    for lg in (20, 22, 24, 26, 28):
+        n = 1 << lg
+        a, b, o = dev(n), dev(n), dev(n, 0)
+        a.abs_().add_(0.5)
+        tag = f"2^{lg}"
+        for name, fn, bpe in [
+            ("jzhip_copy", lambda: jz.copy(P(o), P(a), n), 8), ("jzhip_fill", lambda: jz.fill(P(o), n, 1.0), 4),
+            ("jzhip_exp", lambda: jz.exp(P(o), P(a), n), 8), ("jzhip_log", lambda: jz.log(P(o), P(a), n), 8),
+            ("jzhip_tanh", lambda: jz.tanh(P(o), P(a), n), 8), ("jzhip_affine", lambda: jz.affine(P(o), P(a), n, 0.2, 1.0), 8),
+            ("jzhip_eleminv", lambda: jz.eleminv(P(o), P(a), n, 1.0), 8),
+            ("jzhip_axpby", lambda: jz.axpby(P(o), P(a), P(b), n, 1.0, 2.0), 12),
+            ("jzhip_hadamard", lambda: jz.hadamard(P(o), P(a), P(b), n), 12),
+            ("jzhip_gelu", lambda: jz.gelu(P(o), P(a), n), 8),
+        ]:
+            r.run("elementwise", name, tag, fn, bytes_=bpe * n)
+    # logical-transpose forms (one operand stored transposed): C1 size and a large one
+    for rows, cols in ((1024, 1024), (8192, 8192)):
+        n = rows * cols
+        a, b, o = dev(n), dev(n), dev(n, 0)
+        r.run("elementwise", "jzhip_axpby2d (B transposed)", f"{rows}x{cols}",
+              lambda: jz.axpby2d(P(o), rows, 0, P(a), rows, 0, P(b), cols, 1, rows, cols, 1.0, 1.0), bytes_=12 * n)
+        r.run("elementwise", "jzhip_copy2d (transpose)", f"{rows}x{cols}",
+              lambda: jz.copy2d(P(o), rows, 0, 0, 0, P(a), cols, 1, 0, 0, rows, cols), bytes_=8 * n)
+
+
+def bench_reduce(r):
+    jz = r.jz
+    for rows, cols in ((1024, 1024), (256, 4096), (512, 16384), (2048, 16384), (64, 25088), (16384, 16384)):
+        a, o = dev(rows * cols), dev(max(rows, cols) * 2, 0)
+        s = f"{rows}x{cols}"
+        r.run("reduce", "jzhip_sum_cols", s, lambda: jz.sum_cols(P(o), P(a), rows, cols, rows), bytes_=4 * (rows * cols + cols))
+        r.run("reduce", "jzhip_sum_rows", s, lambda: jz.sum_rows(P(o), P(a), rows, cols, rows), bytes_=4 * (rows * cols + rows))
+        r.run("reduce", "jzhip_max_cols", s, lambda: jz.max_cols(P(o), P(a), rows, cols, rows), bytes_=4 * (rows * cols + cols))
+        r.run("reduce", "jzhip_nrm2", s, lambda: jz.nrm2(P(o), P(a), rows * cols), bytes_=4 * rows * cols)
+        r.run("reduce", "jzhip_softmax_cols", s, lambda: jz.softmax_cols(P(a), P(a), rows, cols, rows), bytes_=8 * rows * cols)
+        r.run("reduce", "jzhip_softmax_rows", s, lambda: jz.softmax_rows(P(a), P(a), rows, cols, rows), bytes_=8 * rows * cols)
+    # loss of C3 and C4: softmax cross-entropy over columns
+    for k, nb in ((10, 128), (256, 16384)):
+        z, g, loss = dev(k * nb), dev(k * nb, 0), dev(1, 0)
+        lab = torch.randint(0, k, (nb,), device="cuda", dtype=torch.int32)
+        r.run("reduce", "jzhip_softmax_xent", f"{k}x{nb}", lambda: jz.softmax_xent(P(loss), P(g), P(z), P(lab), k, nb, k),
+              bytes_=8 * k * nb + 4 * nb)
+
+
+def bench_fused(r):
+    jz = r.jz
+    for dim, N in ((512, 16384), (512, 262144)):
+        x, y, xh = dev(dim * N), dev(dim * N, 0), dev(dim * N, 0)
+        inv, g, b, dg, db = dev(N, 1), dev(dim, 1), dev(dim, 0), dev(dim, 0), dev(dim, 0)
+        s = f"{dim}x{N}"
+        r.run("fused", "jzhip_layernorm_fwd", s, lambda: jz.layernorm_fwd(P(y), P(xh), P(inv), P(x), P(g), P(b), dim, N),
+              bytes_=4 * (3 * dim * N + N + 2 * dim))
+        r.run("fused", "jzhip_layernorm_bwd", s, lambda: jz.layernorm_bwd(P(y), P(x), P(g), P(xh), P(inv), dim, N),
+              bytes_=4 * (3 * dim * N + N + dim))
+        r.run("fused", "jzhip_layernorm_param_grads", s, lambda: jz.layernorm_param_grads(P(dg), P(db), P(x), P(xh), dim, N),
+              bytes_=4 * (2 * dim * N + 2 * dim))
+    for n in (1 << 20, 19_000_000, 1 << 27):
+        w, g, m, v = dev(n), dev(n), dev(n, 0), dev(n, 0)
+        r.run("fused", "jzhip_adam_update", f"{n}", lambda: jz.adam_update(P(g), P(m), P(v), n, 1e-3, 0.9, 0.999, 1e-8, 3), bytes_=24 * n)
+        r.run("fused", "jzhip_adamw_step", f"{n}", lambda: jz.adamw_step(P(w), P(g), P(m), P(v), n, 1e-3, 0.9, 0.999, 1e-8, 0.01, 3),
+              bytes_=28 * n)
+    S, nblk = 256, 512
+    a, o, da = dev(S * S * nblk), dev(S * S * nblk, 0), dev(S * S * nblk)
+    for kar in (0, 1):
+        s = f"{S}x{S} x{nblk} keys_along_rows={kar}"
+        r.run("fused", "jzhip_attn_softmax (causal)", s, lambda: jz.attn_softmax(P(o), P(a), S, nblk, 0.125, 1, kar), bytes_=8 * a.numel())
+        r.run("fused", "jzhip_attn_softmax_bwd", s, lambda: jz.attn_softmax_bwd(P(da), P(o), P(da), S, nblk, 0.125, kar), bytes_=12 * a.numel())
+    # attention core of C4 (QK^T, mask+softmax, AV and their backward)
+    dk, heads, B = 64, 8, 64
+    N = S * B
+    Q, K, V, H = (dev(dk * heads * N) for _ in range(4))
+    A = dev(S * S * heads * B, 0)
+    dQ, dK, dV, dA = dev(dk * heads * N, 0), dev(dk * heads * N, 0), dev(dk * heads * N, 0), dev(S * S * heads * B, 0)
+    fl = 4.0 * S * S * dk * heads * B
+    r.run("fused", "jzhip_attention_fwd", f"S{S} d_k{dk} h{heads} B{B}",
+          lambda: jz.attention_fwd(P(H), P(A), P(Q), P(K), P(V), dk, heads, S, B, 1), flops=fl)
+    r.run("fused", "jzhip_attention_bwd", f"S{S} d_k{dk} h{heads} B{B}",
+          lambda: jz.attention_bwd(P(dQ), P(dK), P(dV), P(dA), P(H), P(Q), P(K), P(V), P(A), dk, heads, S, B), flops=2 * fl)
+
+
+def bench_conv(r):
+    jz = r.jz
+    for label, N, Cc, H, W, k, pad, s in (("C3 conv1", 128, 1, 28, 28, 3, 1, 1), ("C3 conv2", 128, 32, 28, 28, 3, 1, 2),
+                                          ("C5 enc", 128, 64, 32, 32, 3, 1, 2), ("C5 dec1", 128, 128, 32, 32, 3, 1, 1)):
+        Ho = (H + 2 * pad - k) // s + 1
+        K, Pp = Cc * k * k, Ho * Ho
+        x, col = dev(Cc * H * W * N), dev(K * Pp * N, 0)
+        args = (Cc, H, W, k, k, pad, pad, s, s, Ho, Ho, N)
+        byt = 4 * (x.numel() + col.numel())
+        shape = f"{label} N{N} C{Cc} {H}x{W} k{k} s{s}"
+        r.run("conv", "jzhip_im2col", shape, lambda: jz.im2col(P(x), P(col), *args), bytes_=byt)
+        r.run("conv", "jzhip_col2im", shape, lambda: jz.col2im(P(col), P(x), *args), bytes_=byt)
+        Co = 64
+        y2d, out, bias = dev(Co * Pp * N), dev(Co * Pp * N, 0), dev(Co, 0)
+        r.run("conv", "jzhip_conv_forward_reshape_bias", f"{label} C_out{Co} P{Pp} N{N}",
+              lambda: jz.conv_forward_reshape_bias(P(y2d), P(out), P(bias), Co, Pp, N), bytes_=8 * y2d.numel())
+        r.run("conv", "jzhip_conv_backward_reshape", f"{label} C_out{Co} P{Pp} N{N}",
+              lambda: jz.conv_backward_reshape(P(out), P(y2d), Co, Pp, N), bytes_=8 * y2d.numel())
+
+
+GROUPS = {"gemm": bench_gemm, "ew": bench_ew, "reduce": bench_reduce, "fused": bench_fused, "conv": bench_conv}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--groups", default=",".join(GROUPS))
+    ap.add_argument("--out", default=None)
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        sys.exit("opbench needs a GPU")
+    r = Report()
+    for g in args.groups.split(","):
+        GROUPS[g](r)
+        torch.cuda.empty_cache()
+    text = r.markdown()
+    if args.out:
+        Path(args.out).write_text(text)
+    else:
+        print(text)
+
+
+if __name__ == "__main__":
+    main()

@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 
 import oracle
+from oracle.lm_check import track_reference_lm
 from util import hptr
 
 pytestmark = pytest.mark.gpu
@@ -45,43 +46,10 @@ def test_reference_configuration_tracks_the_reference_cpu_model(gpu):
     m.init_random(1)
     m.set("embed_bias", rng.normal(0, 0.1, (d, 1)))
     m.set("head_bias", rng.normal(0, 0.1, (V, 1)))
-    h = ref.jzref_lm_create(V, d, heads, ff, L, S, B)
-    keep = []
-
-    def give(kind, layer, which, arr):
-        buf = cm(arr)
-        keep.append(buf)
-        assert ref.jzref_lm_param(h, kind, layer, which, hptr(buf), 1) == 0
-
-    give(0, 0, 0, np.hstack([m.get("embed"), m.get("pos")]))
-    give(1, 0, 0, m.get("embed_bias"))
-    give(2, 0, 0, m.get("head"))
-    give(3, 0, 0, m.get("head_bias"))
-    for l in range(L):
-        for w, name in enumerate(BLOCK_PARAMS):
-            give(4, l, w, m.get(f"block{l}.{name}"))
-    ref.jzref_lm_set_lr(h, lr)
-
     tokens = make_tokens(rng, V, B, S)
-    m.set_batch(tokens)
-    X = np.zeros((V + S, N), np.float32)
-    Y = np.zeros((V, N), np.float32)
-    for b in range(B):
-        for s in range(S):
-            n = b * S + s
-            X[tokens[b, s], n] = 1
-            X[V + s, n] = 1
-            Y[tokens[b, s + 1], n] = 1
-    Xc, Yc = cm(X), cm(Y)
-    worst = 0.0
-    first = last = None
-    for step in range(100):
-        want = ref.jzref_lm_step(h, hptr(Xc), hptr(Yc))
-        m.step()
-        got = m.loss()
-        worst = max(worst, abs(got - want) / abs(want))
-        first = want if first is None else first
-        last = want
+    want, got, h = track_reference_lm(ref, m, (V, d, heads, ff, L, S, B), tokens, 100, lr)
+    worst = float(np.max(np.abs(got - want) / np.abs(want)))
+    first, last = want[0], want[-1]
     print(f"reference-configuration LM: loss {first:.4f} -> {last:.4f}, worst rel err {worst:.2e}")
     assert last < first                      # it trains
     assert worst <= 1e-3
