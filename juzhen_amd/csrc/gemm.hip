@@ -62,80 +62,131 @@ constexpr int kPad = JZ_GEMM_PAD;  // keeps 16-byte alignment of LDS rows, skews
 //              transposed, or B transposed): element (x, k) at p[k*ld + x].
 // MNC = false: contiguous along k (A transposed, or B not transposed):
 //              element (x, k) at p[x*ld + k].
-template <int EXT, bool MNC>
+// T is the number of 32-wide MFMA tiles a wave owns along this operand.  The
+// LDS tile is [BK][EXT + kPad] with the T tiles of a wave interleaved inside
+// each row (x = w*32T + i*32 + l is kept at w*32T + l*T + i), so that a lane
+// fetches its T fragment values of one k with a single 4T-byte read at an
+// immediate offset.
+template <int EXT, bool MNC, int T>
 struct TileLoader {
     static constexpr int kVecs = EXT * BK / 4;             // float4 per tile
     static constexpr int kPasses = (kVecs + kBlock - 1) / kBlock;
+    static constexpr int LD = EXT + kPad;
 
-    // FAST: tile fully inside the matrix, ld % 4 == 0, base 16-byte aligned.
-    template <bool FAST>
-    static __device__ __forceinline__ void load(floatx4 (&reg)[kPasses], const float* __restrict__ p,
-                                                size_t ld, int x0, int k0, int X, int K) {
+    static __device__ __forceinline__ int pos(int x) {
+        return (x / (32 * T)) * (32 * T) + (x % 32) * T + (x / 32) % T;
+    }
+    static __device__ __forceinline__ void coords(int ps, int& x, int& k) {
+        const int v = threadIdx.x + ps * kBlock;
+        if constexpr (MNC) {
+            x = (v % (EXT / 4)) * 4;
+            k = v / (EXT / 4);
+        } else {
+            k = (v % (BK / 4)) * 4;
+            x = v / (BK / 4);
+        }
+    }
+    static __device__ __forceinline__ bool active(int ps) {
+        return kVecs % kBlock == 0 || threadIdx.x + ps * kBlock < kVecs;
+    }
+
+    // Fast path (tile inside the matrix, ld % 4 == 0, 16-byte aligned base,
+    // 256*ld*4 < 2^32): per-thread 32-bit element offsets from the tile origin
+    // are computed once; each K stage adds them to a wave-uniform pointer.
+    static __device__ __forceinline__ void offsets(unsigned (&off)[kPasses], unsigned ld) {
 #pragma unroll
         for (int ps = 0; ps < kPasses; ++ps) {
-            const int v = threadIdx.x + ps * kBlock;
+            int x, k;
+            coords(ps, x, k);
+            off[ps] = MNC ? static_cast<unsigned>(k) * ld + x : static_cast<unsigned>(x) * ld + k;
+        }
+    }
+    // origin: p advanced to (x0, k0) of the stage
+    static __device__ __forceinline__ const float* origin(const float* p, size_t ld, int x0, int k0) {
+        return MNC ? p + static_cast<size_t>(k0) * ld + x0 : p + static_cast<size_t>(x0) * ld + k0;
+    }
+    static __device__ __forceinline__ void load_fast(floatx4 (&reg)[kPasses], const float* __restrict__ org,
+                                                     const unsigned (&off)[kPasses]) {
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps)
+            if (active(ps)) reg[ps] = *reinterpret_cast<const floatx4*>(org + off[ps]);
+    }
+
+    // Bounds-checked path for edge tiles and unaligned operands.
+    static __device__ __forceinline__ void load_checked(floatx4 (&reg)[kPasses], const float* __restrict__ p,
+                                                        size_t ld, int x0, int k0, int X, int K) {
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
             // (no early exit: the loop must unroll fully so reg[] stays in registers)
-            if (kVecs % kBlock == 0 || v < kVecs) {
+            if (active(ps)) {
                 int x, k;
-                if constexpr (MNC) {
-                    x = (v % (EXT / 4)) * 4;
-                    k = v / (EXT / 4);
-                } else {
-                    k = (v % (BK / 4)) * 4;
-                    x = v / (BK / 4);
-                }
+                coords(ps, x, k);
                 const int gx = x0 + x, gk = k0 + k;
-                if constexpr (FAST) {
-                    const float* src = MNC ? p + static_cast<size_t>(gk) * ld + gx
-                                           : p + static_cast<size_t>(gx) * ld + gk;
-                    reg[ps] = *reinterpret_cast<const floatx4*>(src);
-                } else {
-                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
-                    if constexpr (MNC) {
-                        if (gk < K) {
-                            const float* src = p + static_cast<size_t>(gk) * ld + gx;
-                            if (gx + 0 < X) t.x = src[0];
-                            if (gx + 1 < X) t.y = src[1];
-                            if (gx + 2 < X) t.z = src[2];
-                            if (gx + 3 < X) t.w = src[3];
-                        }
-                    } else {
-                        if (gx < X) {
-                            const float* src = p + static_cast<size_t>(gx) * ld + gk;
-                            if (gk + 0 < K) t.x = src[0];
-                            if (gk + 1 < K) t.y = src[1];
-                            if (gk + 2 < K) t.z = src[2];
-                            if (gk + 3 < K) t.w = src[3];
-                        }
+                floatx4 t = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (MNC) {
+                    if (gk < K) {
+                        const float* src = p + static_cast<size_t>(gk) * ld + gx;
+                        if (gx + 0 < X) t.x = src[0];
+                        if (gx + 1 < X) t.y = src[1];
+                        if (gx + 2 < X) t.z = src[2];
+                        if (gx + 3 < X) t.w = src[3];
                     }
-                    reg[ps] = t;
+                } else {
+                    if (gx < X) {
+                        const float* src = p + static_cast<size_t>(gx) * ld + gk;
+                        if (gk + 0 < K) t.x = src[0];
+                        if (gk + 1 < K) t.y = src[1];
+                        if (gk + 2 < K) t.z = src[2];
+                        if (gk + 3 < K) t.w = src[3];
+                    }
                 }
+                reg[ps] = t;
             }
         }
     }
 
-    // registers -> LDS tile laid out [BK][EXT + kPad]
+    // registers -> LDS
     static __device__ __forceinline__ void store(const floatx4 (&reg)[kPasses], float* __restrict__ s) {
-        constexpr int LD = EXT + kPad;
 #pragma unroll
         for (int ps = 0; ps < kPasses; ++ps) {
-            const int v = threadIdx.x + ps * kBlock;
-            if (kVecs % kBlock == 0 || v < kVecs) {
+            if (active(ps)) {
+                int x, k;
+                coords(ps, x, k);
                 if constexpr (MNC) {
-                    const int x = (v % (EXT / 4)) * 4;
-                    const int k = v / (EXT / 4);
-                    *reinterpret_cast<floatx4*>(s + k * LD + x) = reg[ps];
+                    float* d = s + k * LD + pos(x);  // x % 4 == 0: the four values share a tile
+                    if constexpr (T == 1) {
+                        *reinterpret_cast<floatx4*>(d) = reg[ps];
+                    } else {
+                        d[0 * T] = reg[ps].x;
+                        d[1 * T] = reg[ps].y;
+                        d[2 * T] = reg[ps].z;
+                        d[3 * T] = reg[ps].w;
+                    }
                 } else {
-                    const int k = (v % (BK / 4)) * 4;
-                    const int x = v / (BK / 4);
-                    s[(k + 0) * LD + x] = reg[ps].x;
-                    s[(k + 1) * LD + x] = reg[ps].y;
-                    s[(k + 2) * LD + x] = reg[ps].z;
-                    s[(k + 3) * LD + x] = reg[ps].w;
+                    float* d = s + k * LD + pos(x);
+                    d[0 * LD] = reg[ps].x;
+                    d[1 * LD] = reg[ps].y;
+                    d[2 * LD] = reg[ps].z;
+                    d[3 * LD] = reg[ps].w;
                 }
             }
         }
     }
+};
+
+// T fragment values of one lane, read from LDS with one 4T-byte access
+template <int T>
+struct Frag {
+    typedef float vec __attribute__((ext_vector_type(T)));
+    vec v;
+    __device__ __forceinline__ void read(const float* p) { v = *reinterpret_cast<const vec*>(p); }
+    __device__ __forceinline__ float operator[](int i) const { return v[i]; }
+};
+template <>
+struct Frag<1> {
+    float v;
+    __device__ __forceinline__ void read(const float* p) { v = *p; }
+    __device__ __forceinline__ float operator[](int) const { return v; }
 };
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
@@ -202,13 +253,26 @@ __global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    using LA = TileLoader<BM, !TA>;
-    using LB = TileLoader<BN, TB>;
+    using LA = TileLoader<BM, !TA, TM>;
+    using LB = TileLoader<BN, TB, TN>;
     floatx4 ra[LA::kPasses], rb[LB::kPasses];  // next stage in flight, global -> registers
+    unsigned offa[LA::kPasses], offb[LB::kPasses];
+    if constexpr (FAST) {
+        LA::offsets(offa, static_cast<unsigned>(lda));
+        LB::offsets(offb, static_cast<unsigned>(ldb));
+    }
+    auto load_stage = [&](int k0) {
+        if constexpr (FAST) {
+            LA::load_fast(ra, LA::origin(A, lda, m0, k0), offa);
+            LB::load_fast(rb, LB::origin(B, ldb, n0, k0), offb);
+        } else {
+            LA::load_checked(ra, A, lda, m0, k0, M, k_hi);
+            LB::load_checked(rb, B, ldb, n0, k0, N, k_hi);
+        }
+    };
 
     const int nk = (k_hi - k_lo + BK - 1) / BK;
-    LA::template load<FAST>(ra, A, lda, m0, k_lo, M, k_hi);
-    LB::template load<FAST>(rb, B, ldb, n0, k_lo, N, k_hi);
+    load_stage(k_lo);
     LA::store(ra, As[0]);
     LB::store(rb, Bs[0]);
     __syncthreads();
@@ -220,31 +284,28 @@ __global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
     // cycles) to land in.
     constexpr int KS = BK / 2;  // MFMA steps per stage
     static_assert(KS % 2 == 0, "fragment double buffer assumes an even step count");
-    float af[2][TM], bf[2][TN];
-    const int a_off = wm * (TM * 32) + l32 + h * LDA_S;
-    const int b_off = wn * (TN * 32) + l32 + h * LDB_S;
+    Frag<TM> af[2];
+    Frag<TN> bf[2];
+    const int a_off = wm * (TM * 32) + l32 * TM + h * LDA_S;
+    const int b_off = wn * (TN * 32) + l32 * TN + h * LDB_S;
     auto read_frags = [&](int slot, const float* as, const float* bs, int kk) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) af[slot][i] = as[2 * kk * LDA_S + i * 32];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) bf[slot][j] = bs[2 * kk * LDB_S + j * 32];
+        af[slot].read(as + 2 * kk * LDA_S);
+        bf[slot].read(bs + 2 * kk * LDB_S);
     };
     auto mfma_step = [&](int slot) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[slot][j], af[slot][i],
+                                                                 acc[i][j], 0, 0, 0);
     };
 
     int cur = 0;
     read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
     for (int kt = 0; kt < nk; ++kt) {
         const bool more = kt + 1 < nk;
-        if (more) {
-            LA::template load<FAST>(ra, A, lda, m0, k_lo + (kt + 1) * BK, M, k_hi);
-            LB::template load<FAST>(rb, B, ldb, n0, k_lo + (kt + 1) * BK, N, k_hi);
-        }
+        if (more) load_stage(k_lo + (kt + 1) * BK);
         const float* as = As[cur] + a_off;
         const float* bs = Bs[cur] + b_off;
 #pragma unroll
@@ -451,7 +512,8 @@ int launch_tile(const GemmArgs& g) {
     }
     const bool fast = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && (g.lda % 4 == 0) &&
                       (g.ldb % 4 == 0) && aligned16(g.A) && aligned16(g.B) && (g.sA % 4 == 0) &&
-                      (g.sB % 4 == 0) && (g.sA2 % 4 == 0) && (g.sB2 % 4 == 0);
+                      (g.sB % 4 == 0) && (g.sA2 % 4 == 0) && (g.sB2 % 4 == 0) && g.lda < (1u << 22) &&
+                      g.ldb < (1u << 22);
     dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, splits, g.batch * g.batch2);
     hipStream_t s = stream();
     GemmProf& prof = gemm_prof();
