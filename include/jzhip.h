@@ -202,6 +202,23 @@ int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numcol, int 
 int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, int k,
                int trans_a, int trans_b, int lda, int ldb, int ldc,
                float alpha, float beta);
+/* GEMM with the layer's elementwise tail fused into the store of C, for the
+ * chains dense layers issue after a product (ml/layer.hpp:83-105 `W*x + b*ones`,
+ * :335-345 activation, :3005-3024 residual adds of TransformerLayer): with
+ * v = alpha*op(A)op(B) + beta*C element by element, in this order
+ *   bias != NULL      : v += bias[row]                    (RocmGemm k=1 broadcast + RocmAxpby)
+ *   act 1 relu, 2 gelu: aux(row,col) = v when aux != NULL (the pre-activation
+ *                       the backward pass needs), then v = act(v)
+ *   act 3, 4          : v *= relu'(aux(row,col)) / gelu'(aux(row,col))   (hadmd(d_act(pre), up))
+ *   residual != NULL  : v += residual(row,col)
+ * Each step rounds like the separate kernel it replaces, so the result is
+ * bit-identical to jzhip_gemm followed by jzhip_add_bias / jzhip_gelu /
+ * jzhip_dgelu_mul / jzhip_axpby(1,1).  aux has leading dimension ld_aux,
+ * residual ldr; residual may alias C. */
+int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int n,
+                     int k, int trans_a, int trans_b, int lda, int ldb, int ldc,
+                     float alpha, float beta, const float* bias, int act,
+                     float* aux, int ld_aux, const float* residual, int ldr);
 /* Juzhen::RocmGemmNN (cpp/hipbackend.hpp:94-95). */
 int jzhip_gemm_nn(const float* A, const float* B, float* C, int m, int n, int k,
                   float alpha, float beta);
@@ -282,6 +299,17 @@ int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch,
                         const float* dH, const float* Q, const float* K,
                         const float* V, const float* A, int d_k, int heads,
                         int S, int B);
+/* The same two calls for operands that live inside wider matrices (Q, K, V as
+ * row blocks of one stacked (3*d_k, S*B) projection and likewise dQ, dK, dV):
+ * ld_qkv / ld_dqkv / ld_h / ld_dh are the leading dimensions of those buffers. */
+int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q,
+                           const float* K, const float* V, int ld_qkv, int d_k,
+                           int heads, int S, int B, int causal);
+int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv,
+                           float* dA_scratch, const float* dH, int ld_dh,
+                           const float* Q, const float* K, const float* V,
+                           int ld_qkv, const float* A, int d_k, int heads, int S,
+                           int B);
 
 /* ── LayerNorm ───────────────────────────────────────────────────────── */
 
@@ -295,6 +323,13 @@ int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const float* x,
  * (ml/layer.hpp:2674-2681; CUDA kernel :2512-2534). */
 int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma,
                         const float* xhat, const float* inv_std, int dim, int N);
+/* dx = layernorm_bwd(dy) + res in one pass (res may be NULL or alias dx): the
+ * residual branch of a pre-LN block adds the skip gradient right after the
+ * LayerNorm backward (ml/layer.hpp:3287-3299, 3372-3376); rounds like the
+ * separate add. */
+int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float* gamma,
+                                 const float* xhat, const float* inv_std,
+                                 const float* res, int dim, int N);
 /* dgamma[i] = sum_c dy*xhat, dbeta[i] = sum_c dy in one pass over dy/xhat:
  * the two sum(...,1) calls of ml/layer.hpp:2683-2686. */
 int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,

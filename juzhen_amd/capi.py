@@ -78,6 +78,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_gemm": (I, [P, P, P, I, I, I, I, I, I, I, I, F, F]),
     "jzhip_gemm_nn": (I, [P, P, P, I, I, I, F, F]),
     "jzhip_gemv": (I, [P, P, P, I, I, I, I, I, I, F, F]),
+    "jzhip_gemm_fused": (I, [P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P, I, P, I]),
     "jzhip_gemm_strided_batched": (I, [P, P, P, I, I, I, I, I, I, I, I, LL, LL, LL, I, F, F]),
     "jzhip_profile_gemm": (I, [I]),
     "jzhip_profile_gemm_report": (I, [C.c_char_p, Z]),
@@ -87,10 +88,13 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_attn_softmax": (I, [P, P, I, I, F, I, I]),
     "jzhip_attn_softmax_bwd": (I, [P, P, P, I, I, F, I]),
     "jzhip_softmax_xent": (I, [P, P, P, P, I, I, I]),
+    "jzhip_attention_fwd_ld": (I, [P, I, P, P, P, P, I, I, I, I, I, I]),
+    "jzhip_attention_bwd_ld": (I, [P, P, P, I, P, P, I, P, P, P, I, P, I, I, I, I]),
     "jzhip_attention_fwd": (I, [P, P, P, P, P, I, I, I, I, I]),
     "jzhip_attention_bwd": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I]),
     "jzhip_layernorm_fwd": (I, [P, P, P, P, P, P, I, I]),
     "jzhip_layernorm_bwd": (I, [P, P, P, P, P, I, I]),
+    "jzhip_layernorm_bwd_residual": (I, [P, P, P, P, P, P, I, I]),
     "jzhip_layernorm_param_grads": (I, [P, P, P, P, I, I]),
     "jzhip_adam_update": (I, [P, P, P, Z, F, F, F, F, I]),
     "jzhip_adamw_step": (I, [P, P, P, P, Z, F, F, F, F, F, I]),

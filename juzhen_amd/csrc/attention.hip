@@ -17,51 +17,68 @@ int gemm_batched2(const float* A, const float* B, float* C, int m, int n, int k,
                   long long sA2, long long sB2, long long sC2, int batch2, float alpha, float beta);
 }
 
-JZ_API int jzhip_attention_fwd(float* H, float* A, const float* Q, const float* K, const float* V,
-                               int d_k, int heads, int S, int B, int causal) {
+JZ_API int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q, const float* K,
+                                  const float* V, int ld_qkv, int d_k, int heads, int S, int B,
+                                  int causal) {
     if (d_k <= 0 || heads <= 0 || S <= 0 || B <= 0 || d_k % heads != 0) return -1;
-    if (!H || !A || !Q || !K || !V) return -1;
+    if (!H || !A || !Q || !K || !V || ld_h < d_k || ld_qkv < d_k) return -1;
     const int d_h = d_k / heads;
-    const long long seq = static_cast<long long>(S) * d_k;   // next sequence in Q/K/V/H
-    const long long blk = static_cast<long long>(S) * S;     // next score block
+    const long long seq = static_cast<long long>(S) * ld_qkv;  // next sequence in Q/K/V
+    const long long seq_h = static_cast<long long>(S) * ld_h;  // next sequence in H
+    const long long blk = static_cast<long long>(S) * S;       // next score block
     const float scale = 1.0f / sqrtf(static_cast<float>(d_h));
     // scores[q, k] = <Q_i[:, q], K_i[:, k]>
-    int rc = jz::gemm_batched2(Q, K, A, S, S, d_h, true, false, d_k, d_k, S, seq, seq, blk, B, d_h, d_h,
+    int rc = jz::gemm_batched2(Q, K, A, S, S, d_h, true, false, ld_qkv, ld_qkv, S, seq, seq, blk, B, d_h, d_h,
                                blk * B, heads, 1.0f, 0.0f);
     if (rc) return rc;
     // A = softmax over keys of (scores*scale, masked)
     rc = jzhip_attn_softmax(A, A, S, B * heads, scale, causal, 0);
     if (rc) return rc;
     // H_i = V_i * A_i^T
-    return jz::gemm_batched2(V, A, H, d_h, S, S, false, true, d_k, S, d_k, seq, blk, seq, B, d_h, blk * B,
-                             d_h, heads, 1.0f, 0.0f);
+    return jz::gemm_batched2(V, A, H, d_h, S, S, false, true, ld_qkv, S, ld_h, seq, blk, seq_h, B, d_h,
+                             blk * B, d_h, heads, 1.0f, 0.0f);
 }
 
-JZ_API int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch, const float* dH,
-                               const float* Q, const float* K, const float* V, const float* A,
-                               int d_k, int heads, int S, int B) {
+JZ_API int jzhip_attention_fwd(float* H, float* A, const float* Q, const float* K, const float* V,
+                               int d_k, int heads, int S, int B, int causal) {
+    return jzhip_attention_fwd_ld(H, d_k, A, Q, K, V, d_k, d_k, heads, S, B, causal);
+}
+
+JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, float* dA_scratch,
+                                  const float* dH, int ld_dh, const float* Q, const float* K,
+                                  const float* V, int ld_qkv, const float* A, int d_k, int heads,
+                                  int S, int B) {
     if (d_k <= 0 || heads <= 0 || S <= 0 || B <= 0 || d_k % heads != 0) return -1;
     if (!dQ || !dK || !dV || !dA_scratch || !dH || !Q || !K || !V || !A) return -1;
+    if (ld_dqkv < d_k || ld_dh < d_k || ld_qkv < d_k) return -1;
     const int d_h = d_k / heads;
-    const long long seq = static_cast<long long>(S) * d_k;
+    const long long seq = static_cast<long long>(S) * ld_qkv;
+    const long long seq_d = static_cast<long long>(S) * ld_dqkv;
+    const long long seq_h = static_cast<long long>(S) * ld_dh;
     const long long blk = static_cast<long long>(S) * S;
     const float scale = 1.0f / sqrtf(static_cast<float>(d_h));
     // dV_i = dH_i * A_i
-    int rc = jz::gemm_batched2(dH, A, dV, d_h, S, S, false, false, d_k, S, d_k, seq, blk, seq, B, d_h,
+    int rc = jz::gemm_batched2(dH, A, dV, d_h, S, S, false, false, ld_dh, S, ld_dqkv, seq_h, blk, seq_d, B, d_h,
                                blk * B, d_h, heads, 1.0f, 0.0f);
     if (rc) return rc;
     // dA_i[q, k] = <dH_i[:, q], V_i[:, k]>
-    rc = jz::gemm_batched2(dH, V, dA_scratch, S, S, d_h, true, false, d_k, d_k, S, seq, seq, blk, B, d_h, d_h,
-                           blk * B, heads, 1.0f, 0.0f);
+    rc = jz::gemm_batched2(dH, V, dA_scratch, S, S, d_h, true, false, ld_dh, ld_qkv, S, seq_h, seq, blk, B, d_h,
+                           d_h, blk * B, heads, 1.0f, 0.0f);
     if (rc) return rc;
     // dS = A .* (dA - rowsum(A .* dA)) * scale, in place
     rc = jzhip_attn_softmax_bwd(dA_scratch, A, dA_scratch, S, B * heads, scale, 0);
     if (rc) return rc;
     // dQ_i = K_i * dS_i^T
-    rc = jz::gemm_batched2(K, dA_scratch, dQ, d_h, S, S, false, true, d_k, S, d_k, seq, blk, seq, B, d_h,
+    rc = jz::gemm_batched2(K, dA_scratch, dQ, d_h, S, S, false, true, ld_qkv, S, ld_dqkv, seq, blk, seq_d, B, d_h,
                            blk * B, d_h, heads, 1.0f, 0.0f);
     if (rc) return rc;
     // dK_i = Q_i * dS_i
-    return jz::gemm_batched2(Q, dA_scratch, dK, d_h, S, S, false, false, d_k, S, d_k, seq, blk, seq, B, d_h,
-                             blk * B, d_h, heads, 1.0f, 0.0f);
+    return jz::gemm_batched2(Q, dA_scratch, dK, d_h, S, S, false, false, ld_qkv, S, ld_dqkv, seq, blk, seq_d, B,
+                             d_h, blk * B, d_h, heads, 1.0f, 0.0f);
+}
+
+JZ_API int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch, const float* dH,
+                               const float* Q, const float* K, const float* V, const float* A,
+                               int d_k, int heads, int S, int B) {
+    return jzhip_attention_bwd_ld(dQ, dK, dV, d_k, dA_scratch, dH, d_k, Q, K, V, d_k, A, d_k, heads, S, B);
 }

@@ -11,6 +11,7 @@
 // and gfx950's fp32 mul/add/div/sqrt are IEEE correctly rounded, so the
 // multiply-add chains here are bit-identical to the oracle.
 #include "common.hpp"
+#include "activations.hpp"
 
 #include <cmath>
 
@@ -55,10 +56,10 @@ struct EleminvF {  // cpp/core.hpp:472-482: double division, then narrowing
     __device__ float operator()(float x) const { return static_cast<float>(l / static_cast<double>(x)); }
 };
 struct ReluF {  // ml/util.cuh:74-77
-    __device__ float operator()(float x) const { return x > 0.0f ? x : 0.0f; }
+    __device__ float operator()(float x) const { return relu_f(x); }
 };
 struct DReluF {  // ml/util.cuh:79-82
-    __device__ float operator()(float x) const { return x > 0.0f ? 1.0f : 0.0f; }
+    __device__ float operator()(float x) const { return drelu_f(x); }
 };
 struct SqrtF {  // cpp/juzhen.hpp:71-79
     __device__ float operator()(float x) const { return sqrtf(x); }
@@ -68,9 +69,7 @@ struct ClampF {  // ml/util.cuh:84-89
     __device__ float operator()(float x) const { return x < lo ? lo : (x > hi ? hi : x); }
 };
 struct GeluF {  // 0.5*x*(1+erf(x/sqrt(2)))
-    __device__ float operator()(float x) const {
-        return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
-    }
+    __device__ float operator()(float x) const { return gelu_f(x); }
 };
 struct AxpbyF {  // cpp/core.hpp:414-449: s1*a + s2*b
     float s1, s2;
@@ -80,14 +79,10 @@ struct HadamardF {  // cpp/matrix.hpp:428-474
     __device__ float operator()(float a, float b) const { return a * b; }
 };
 struct DReluMulF {  // hadmd(d_relu(pre), up): up * mask
-    __device__ float operator()(float pre, float up) const { return up * (pre > 0.0f ? 1.0f : 0.0f); }
+    __device__ float operator()(float pre, float up) const { return up * drelu_f(pre); }
 };
 struct DGeluMulF {  // up * d/dx gelu(pre)
-    __device__ float operator()(float x, float up) const {
-        const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752440f));
-        const float pdf = 0.39894228040143267794f * expf(-0.5f * x * x);
-        return up * (cdf + x * pdf);
-    }
+    __device__ float operator()(float x, float up) const { return up * dgelu_f(x); }
 };
 
 // ── kernels ──────────────────────────────────────────────────────────────

@@ -12,6 +12,7 @@
 // register then maps to 32 consecutive rows of one column of C, so the epilogue
 // writes 128-byte contiguous segments of the column-major C.
 #include "common.hpp"
+#include "activations.hpp"
 
 #include <cstdio>
 #include <map>
@@ -71,10 +72,18 @@ template <int EXT, bool MNC, int T>
 struct TileLoader {
     static constexpr int kVecs = EXT * BK / 4;             // float4 per tile
     static constexpr int kPasses = (kVecs + kBlock - 1) / kBlock;
-    static constexpr int LD = EXT + kPad;
+    // Interleaving two tiles turns the float4 of a contiguous operand into four
+    // stride-2 stores; skewing each wave's 64-float group by two banks keeps the
+    // 32 lanes of such a store on distinct banks.  The row pitch is rounded up to
+    // 4 (mod 16) floats so that the four k-rows written by a k-contiguous
+    // operand (lanes = 8 x-values times 4 k-quads) also land on distinct banks.
+    static constexpr int kSkew = (T == 2) ? 2 : 0;
+    static constexpr int kGroup = 32 * T + kSkew;          // floats per wave group in a row
+    static constexpr int kRow = (EXT / (32 * T)) * kGroup;
+    static constexpr int LD = kRow + ((4 - kRow % 16) + 16) % 16;
 
     static __device__ __forceinline__ int pos(int x) {
-        return (x / (32 * T)) * (32 * T) + (x % 32) * T + (x / 32) % T;
+        return (x / (32 * T)) * kGroup + (x % 32) * T + (x / 32) % T;
     }
     static __device__ __forceinline__ void coords(int ps, int& x, int& k) {
         const int v = threadIdx.x + ps * kBlock;
@@ -148,7 +157,11 @@ struct TileLoader {
     // registers -> LDS
     static __device__ __forceinline__ void store(const floatx4 (&reg)[kPasses], float* __restrict__ s) {
 #pragma unroll
-        for (int ps = 0; ps < kPasses; ++ps) {
+        for (int ps = 0; ps < kPasses; ++ps) store_pass(reg, s, ps);
+    }
+    static __device__ __forceinline__ void store_pass(const floatx4 (&reg)[kPasses], float* __restrict__ s,
+                                                      int ps) {
+        {
             if (active(ps)) {
                 int x, k;
                 coords(ps, x, k);
@@ -174,6 +187,24 @@ struct TileLoader {
     }
 };
 
+// Optional work fused into the store of C (jzhip_gemm_fused).  With v the
+// value alpha*acc + beta*C of element (row, col), in this order:
+//   v += bias[row]
+//   act 1/2 (relu/gelu): aux_out(row, col) = v when aux_out is set, v = act(v)
+//   act 3/4            : v *= drelu/dgelu(aux_in(row, col))
+//   v += res(row, col)
+// Every step rounds as the separate kernel it replaces.
+struct Epilogue {
+    const float* bias = nullptr;
+    const float* res = nullptr;
+    size_t ldr = 0;
+    const float* aux_in = nullptr;
+    float* aux_out = nullptr;
+    size_t ld_aux = 0;
+    int act = 0;
+    int any = 0;
+};
+
 // T fragment values of one lane, read from LDS with one 4T-byte access
 template <int T>
 struct Frag {
@@ -190,17 +221,19 @@ struct Frag<1> {
 };
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
-template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST>
-__global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
+template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST, bool EPI>
+__global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
-    long long strideC2, int tiles_m, int tiles_n, int k_chunk, long long split_stride) {
+    long long strideC2, int tiles_m, int tiles_n, int k_chunk, long long split_stride, Epilogue ep) {
     static_assert(WGM * WGN == kBlock / kWave, "four waves per workgroup");
     constexpr int BM = WGM * TM * 32;
     constexpr int BN = WGN * TN * 32;
-    constexpr int LDA_S = BM + kPad;
-    constexpr int LDB_S = BN + kPad;
+    using LA = TileLoader<BM, !TA, TM>;
+    using LB = TileLoader<BN, TB, TN>;
+    constexpr int LDA_S = LA::LD;
+    constexpr int LDB_S = LB::LD;
     __shared__ __attribute__((aligned(16))) float As[2][BK * LDA_S];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB_S];
 
@@ -253,8 +286,6 @@ __global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    using LA = TileLoader<BM, !TA, TM>;
-    using LB = TileLoader<BN, TB, TN>;
     floatx4 ra[LA::kPasses], rb[LB::kPasses];  // next stage in flight, global -> registers
     unsigned offa[LA::kPasses], offb[LB::kPasses];
     if constexpr (FAST) {
@@ -276,18 +307,26 @@ __global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
     LA::store(ra, As[0]);
     LB::store(rb, Bs[0]);
     __syncthreads();
+    if (nk > 1) load_stage(k_lo + BK);   // stage 1 waits in registers
 
-    // Software pipeline: the operand fragments of MFMA step kk+1 are read from
-    // LDS before the MFMAs of step kk are issued, and the first fragments of
-    // the next K stage are read right after the barrier, ahead of the last
-    // MFMAs of the current stage, so every LDS read has four MFMAs (256
-    // cycles) to land in.
+    // Software pipeline of one K stage (KS MFMA steps of k = 2):
+    //  * the operand fragments of step kk+1 are read from LDS before the MFMAs of
+    //    step kk are issued, and the first fragments of the next stage right
+    //    after the barrier, ahead of the last MFMAs of this stage: every LDS
+    //    read has four MFMAs (256 cycles) to land in;
+    //  * the staging registers (stage t+1, loaded during the previous stage) go
+    //    to the other LDS buffer one float4-pass per MFMA step instead of in a
+    //    burst before the barrier, so fragment reads of the other workgroups on
+    //    the CU never queue behind a block of stores;
+    //  * the global loads of stage t+2 are issued once those registers are free.
     constexpr int KS = BK / 2;  // MFMA steps per stage
     static_assert(KS % 2 == 0, "fragment double buffer assumes an even step count");
+    constexpr int kStorePasses = LA::kPasses + LB::kPasses;
+    static_assert(kStorePasses <= KS - 2, "staging stores must fit the MFMA steps of a stage");
     Frag<TM> af[2];
     Frag<TN> bf[2];
-    const int a_off = wm * (TM * 32) + l32 * TM + h * LDA_S;
-    const int b_off = wn * (TN * 32) + l32 * TN + h * LDB_S;
+    const int a_off = wm * LA::kGroup + l32 * TM + h * LDA_S;
+    const int b_off = wn * LB::kGroup + l32 * TN + h * LDB_S;
     auto read_frags = [&](int slot, const float* as, const float* bs, int kk) {
         af[slot].read(as + 2 * kk * LDA_S);
         bf[slot].read(bs + 2 * kk * LDB_S);
@@ -305,19 +344,19 @@ __global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
     read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
     for (int kt = 0; kt < nk; ++kt) {
         const bool more = kt + 1 < nk;
-        if (more) load_stage(k_lo + (kt + 1) * BK);
         const float* as = As[cur] + a_off;
         const float* bs = Bs[cur] + b_off;
 #pragma unroll
         for (int kk = 0; kk < KS - 1; ++kk) {
             read_frags((kk + 1) & 1, as, bs, kk + 1);
+            if (more) {
+                if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
+                else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
+            }
+            if (kk == kStorePasses && kt + 2 < nk) load_stage(k_lo + (kt + 2) * BK);
             __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs they do not feed
             mfma_step(kk & 1);
             __builtin_amdgcn_sched_barrier(0);
-        }
-        if (more) {
-            LA::store(ra, As[cur ^ 1]);
-            LB::store(rb, Bs[cur ^ 1]);
         }
         __syncthreads();
         cur ^= 1;
@@ -328,21 +367,65 @@ __global__ __launch_bounds__(kBlock, JZ_GEMM_OCC) void gemm_mfma_kernel(
 
     // Epilogue.  Register v of lane (h, l32) holds C(row, col) with
     // row = l32 and col = 8*(v/4) + 4*h + v%4 inside the 32x32 tile.
+    if constexpr (!EPI) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int row = m0 + (wm * TM + i) * 32 + l32;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int cbase = n0 + (wn * TN + j) * 32 + 4 * h;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int col = cbase + 8 * (v / 4) + (v % 4);
+                    if (FAST || (row < M && col < N)) {
+                        float* dst = C + static_cast<size_t>(col) * ldc + row;
+                        float r = alpha * acc[i][j][v];
+                        if (beta != 0.0f) r += beta * *dst;
+                        *dst = r;
+                    }
+                }
+            }
+        }
+        return;
+    }
+    // Fused tail.  Addresses are a wave-uniform pointer (tile origin and column,
+    // scalar registers) plus one 32-bit lane offset per array, so the tail costs
+    // three address registers instead of one pointer per element.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int wm_u = wave_u % WGM, wn_u = wave_u / WGM;
+    const unsigned lane_c = static_cast<unsigned>(4 * h) * static_cast<unsigned>(ldc) + l32;
+    const unsigned lane_r = static_cast<unsigned>(4 * h) * static_cast<unsigned>(ep.ldr) + l32;
+    const unsigned lane_a = static_cast<unsigned>(4 * h) * static_cast<unsigned>(ep.ld_aux) + l32;
+    const float* aux_in = ep.aux_in;
+    float* aux_out = ep.aux_out;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int row = m0 + (wm * TM + i) * 32 + l32;
+        const int row0 = m0 + (wm_u * TM + i) * 32;
+        const int row = row0 + l32;
+        const float bias = (ep.bias && (FAST || row < M)) ? ep.bias[row] : 0.0f;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            const int cbase = n0 + (wn * TN + j) * 32 + 4 * h;
+            const int col0 = n0 + (wn_u * TN + j) * 32;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int col = cbase + 8 * (v / 4) + (v % 4);
+                const int cu = col0 + 8 * (v / 4) + (v % 4);   // uniform part of the column
+                const int col = cu + 4 * h;
                 if (FAST || (row < M && col < N)) {
-                    float* dst = C + static_cast<size_t>(col) * ldc + row;
+                    float* dst = C + (static_cast<size_t>(cu) * ldc + row0) + lane_c;
                     float r = alpha * acc[i][j][v];
                     if (beta != 0.0f) r += beta * *dst;
+                    if (ep.bias) r += bias;
+                    if (ep.act == 1 || ep.act == 2) {
+                        if (aux_out) (aux_out + (static_cast<size_t>(cu) * ep.ld_aux + row0))[lane_a] = r;
+                        r = ep.act == 1 ? relu_f(r) : gelu_f(r);
+                    } else if (ep.act == 3 || ep.act == 4) {
+                        const float pre = (aux_in + (static_cast<size_t>(cu) * ep.ld_aux + row0))[lane_a];
+                        r = r * (ep.act == 3 ? drelu_f(pre) : dgelu_f(pre));
+                    }
+                    if (ep.res) r += (ep.res + (static_cast<size_t>(cu) * ep.ldr + row0))[lane_r];
                     *dst = r;
                 }
+                if (v % 4 == 3) __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
@@ -475,6 +558,7 @@ struct GemmArgs {
     int batch;
     long long sA2 = 0, sB2 = 0, sC2 = 0;  // outer batch level
     int batch2 = 1;
+    Epilogue ep;
 };
 
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB>
@@ -487,7 +571,7 @@ int launch_tile(const GemmArgs& g) {
     int splits = 1;
     const long long tiles = static_cast<long long>(tiles_m) * tiles_n * g.batch * g.batch2;
     const long long cus = num_cus();
-    if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 1024) {
+    if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 1024 && !g.ep.any) {
         splits = static_cast<int>((cus * 2 + tiles - 1) / tiles);
         const int max_by_k = g.K / 256;
         if (splits > max_by_k) splits = max_by_k;
@@ -521,22 +605,25 @@ int launch_tile(const GemmArgs& g) {
     const bool timing = prof.on;
     if (timing) {
         char name[96];
-        std::snprintf(name, sizeof name, "gemm_mfma_kernel<%d, %d, %d, %d, %s, %s, %s>", WGM, WGN, TM, TN,
-                      TA ? "true" : "false", TB ? "true" : "false", fast ? "true" : "false");
+        std::snprintf(name, sizeof name, "gemm_mfma_kernel<%d, %d, %d, %d, %s, %s, %s, %s>", WGM, WGN, TM, TN,
+                      TA ? "true" : "false", TB ? "true" : "false", fast ? "true" : "false",
+                      g.ep.any ? "true" : "false");
         rec.kernel = name;
         rec.flops = 2.0 * g.M * g.N * g.K * g.batch * g.batch2;
         (void)hipEventCreate(&rec.begin);
         (void)hipEventCreate(&rec.end);
         (void)hipEventRecord(rec.begin, s);
     }
-    if (fast)
-        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true><<<grid, kBlock, 0, s>>>(
-            g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2,
-            g.sB2, g.sC2, tiles_m, tiles_n, k_chunk, split_stride);
-    else
-        gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, false><<<grid, kBlock, 0, s>>>(
-            g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2,
-            g.sB2, g.sC2, tiles_m, tiles_n, k_chunk, split_stride);
+#define JZ_LAUNCH_GEMM(FASTV, EPIV)                                                                         \
+    gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, FASTV, EPIV><<<grid, kBlock, 0, s>>>(                        \
+        g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2, g.sB2, \
+        g.sC2, tiles_m, tiles_n, k_chunk, split_stride, g.ep)
+    if (g.ep.any) {
+        if (fast) JZ_LAUNCH_GEMM(true, true); else JZ_LAUNCH_GEMM(false, true);
+    } else {
+        if (fast) JZ_LAUNCH_GEMM(true, false); else JZ_LAUNCH_GEMM(false, false);
+    }
+#undef JZ_LAUNCH_GEMM
     if (timing) {
         (void)hipEventRecord(rec.end, s);
         std::lock_guard<std::mutex> lock(prof.mu);
@@ -566,7 +653,7 @@ int launch_shape(const GemmArgs& g) {
     // still fills the chip; otherwise fall back to 64 x 64 tiles
     // (only when at least cus/8 big tiles exist: more than ~16 partial sums per
     // output cost more in the reduction than the bigger tile saves)
-    const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && tiles(128, 128) * 8 >= cus;
+    const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && tiles(128, 128) * 8 >= cus && !g.ep.any;
     if (tiles(128, 128) < cus && !splittable) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
     return launch_tile<2, 2, 2, 2, TA, TB>(g);                  // 128 x 128
 }
@@ -701,6 +788,30 @@ JZ_API int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, in
     }
     GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
                static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
+    return gemm_dispatch(g, trans_a != 0, trans_b != 0);
+}
+
+JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int n, int k, int trans_a,
+                            int trans_b, int lda, int ldb, int ldc, float alpha, float beta,
+                            const float* bias, int act, float* aux, int ld_aux, const float* residual,
+                            int ldr) {
+    if (m <= 0 || n <= 0 || k <= 0) return -1;
+    if (!A || !B || !C) return -1;
+    if (lda < (trans_a ? k : m) || ldb < (trans_b ? n : k) || ldc < m) return -1;
+    if (act < 0 || act > 4) return -1;
+    if ((act == 3 || act == 4) && !aux) return -1;
+    if (aux && ld_aux < m) return -1;
+    if (residual && ldr < m) return -1;
+    GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
+               static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
+    g.ep.bias = bias;
+    g.ep.act = act;
+    if (act == 1 || act == 2) g.ep.aux_out = aux;
+    if (act == 3 || act == 4) g.ep.aux_in = aux;
+    g.ep.ld_aux = static_cast<size_t>(ld_aux);
+    g.ep.res = residual;
+    g.ep.ldr = static_cast<size_t>(ldr);
+    g.ep.any = (bias || act || residual) ? 1 : 0;
     return gemm_dispatch(g, trans_a != 0, trans_b != 0);
 }
 

@@ -107,7 +107,8 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic_kernel(float* y, float*
 template <int NV>
 __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const float* dy,
                                                             const float* gamma, const float* xhat,
-                                                            const float* inv_std, int dim, int N) {
+                                                            const float* inv_std, const float* res,
+                                                            int dim, int N) {
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
@@ -145,6 +146,10 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
                 o.y = inv * (d[v].y - m1 - h[v].y * m2);
                 o.z = inv * (d[v].z - m1 - h[v].z * m2);
                 o.w = inv * (d[v].w - m1 - h[v].w * m2);
+                if (res) {  // dx = LN'(dy) + res, rounded like a separate add
+                    const float4 rr = *reinterpret_cast<const float4*>(res + base + r);
+                    o.x += rr.x; o.y += rr.y; o.z += rr.z; o.w += rr.w;
+                }
                 *reinterpret_cast<float4*>(dx + base + r) = o;
             }
         }
@@ -154,8 +159,8 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
 __global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const float* dy,
                                                                 const float* gamma,
                                                                 const float* xhat,
-                                                                const float* inv_std, int dim,
-                                                                int N) {
+                                                                const float* inv_std,
+                                                                const float* res, int dim, int N) {
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
@@ -173,7 +178,9 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const
         const float inv = inv_std[col];
         for (int r = lane; r < dim; r += kWave) {
             const float d = dy[base + r] * gamma[r];
-            dx[base + r] = inv * (d - m1 - xhat[base + r] * m2);
+            float o = inv * (d - m1 - xhat[base + r] * m2);
+            if (res) o += res[base + r];
+            dx[base + r] = o;
         }
     }
 }
@@ -263,22 +270,28 @@ JZ_API int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const floa
     return launch_rc();
 }
 
-JZ_API int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma, const float* xhat,
-                               const float* inv_std, int dim, int N) {
+JZ_API int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float* gamma,
+                                        const float* xhat, const float* inv_std, const float* res,
+                                        int dim, int N) {
     if (dim <= 0 || N <= 0 || !dx || !dy || !gamma || !xhat || !inv_std) return -1;
     const bool vec = (dim % 4 == 0) && dim <= 1024 && aligned16(dx) && aligned16(dy) &&
-                     aligned16(xhat) && aligned16(gamma);
+                     aligned16(xhat) && aligned16(gamma) && (!res || aligned16(res));
     const unsigned grid = grid_cover(N, kBlock / kWave);
     hipStream_t s = stream();
     if (vec && dim <= 256)
-        ln_bwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+        ln_bwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     else if (vec && dim <= 512)
-        ln_bwd_vec_kernel<2><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+        ln_bwd_vec_kernel<2><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     else if (vec)
-        ln_bwd_vec_kernel<4><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+        ln_bwd_vec_kernel<4><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     else
-        ln_bwd_generic_kernel<<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, dim, N);
+        ln_bwd_generic_kernel<<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     return launch_rc();
+}
+
+JZ_API int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma, const float* xhat,
+                               const float* inv_std, int dim, int N) {
+    return jzhip_layernorm_bwd_residual(dx, dy, gamma, xhat, inv_std, nullptr, dim, N);
 }
 
 JZ_API int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,

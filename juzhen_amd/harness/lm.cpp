@@ -37,20 +37,33 @@ struct Config {
     float lr, weight_decay, beta1, beta2, eps;
 };
 
+// Parameters live in a few arenas (one per optimiser group) that hold weights,
+// gradients and both Adam moments at equal offsets, so the optimiser is one
+// fused AdamW launch per group instead of one per tensor.  A tensor is a
+// (rows x cols) view with leading dimension ld: Wq, Wk, Wv are the three row
+// blocks of one stacked (3d x d) projection matrix (ld = 3d).
+enum Group { kDecay = 0, kPlain = 1, kHeadDecay = 2, kHeadPlain = 3, kGroups = 4 };
+
 struct Tensor {
     std::string name;
-    int rows = 0, cols = 0;
+    int rows = 0, cols = 0, ld = 0;
+    int group = kPlain;
+    size_t offset = 0;    // floats from the arena start
     float* w = nullptr;   // parameter
     float* g = nullptr;   // gradient
     float* m = nullptr;   // Adam first moment
     float* v = nullptr;   // Adam second moment
-    bool decay = false;
     size_t count() const { return static_cast<size_t>(rows) * cols; }
+};
+
+struct Arena {
+    size_t used = 0;
+    float *w = nullptr, *g = nullptr, *m = nullptr, *v = nullptr;
 };
 
 struct Block {
     int Wq, Wk, Wv, Wo, bo, W1, b1, W2, b2, g1, be1, g2, be2;           // tensor indices
-    float *x1, *xhat1, *inv1, *Q, *K, *V, *A, *H, *R, *x2, *xhat2, *inv2, *F1, *F1a, *out;  // cached activations
+    float *x1, *xhat1, *inv1, *QKV, *A, *H, *R, *x2, *xhat2, *inv2, *F1, *F1a, *out;  // cached activations
 };
 
 struct Model {
@@ -59,13 +72,16 @@ struct Model {
     std::vector<Tensor> t;
     std::vector<Block> blocks;
     std::vector<float*> owned;
+    Arena arena[kGroups];
     int E = -1, P = -1, be = -1, Wp = -1, bp = -1;
     float *oh_tok = nullptr, *oh_pos = nullptr, *x0 = nullptr, *logits = nullptr, *dlogits = nullptr;
     int32_t* targets = nullptr;
     float* loss = nullptr;
     // backward scratch shared by all blocks
-    float *dx = nullptr, *dR = nullptr, *dtmp = nullptr, *dQ = nullptr, *dK = nullptr, *dV = nullptr,
-          *dH = nullptr, *dA = nullptr, *dF1 = nullptr;
+    float *dx = nullptr, *dR = nullptr, *dtmp = nullptr, *dQKV = nullptr, *dH = nullptr, *dA = nullptr,
+          *dF1 = nullptr;
+    float* io = nullptr;  // dense staging for get/set of strided views
+    size_t io_floats = 0;
     int iteration = 1;
     int rc = 0;  // first failing return code, sticky
 
@@ -76,72 +92,103 @@ struct Model {
         owned.push_back(p);
         return p;
     }
-    int add(const std::string& name, int rows, int cols, bool decay) {
+    // Reserve rows x cols (contiguous) in a group's arena; pointers are bound by finish().
+    int add(const std::string& name, int rows, int cols, int group) {
         Tensor x;
-        x.name = name; x.rows = rows; x.cols = cols; x.decay = decay;
-        const size_t n = x.count();
-        x.w = alloc(n); x.g = alloc(n); x.m = alloc(n); x.v = alloc(n);
-        ck(jzhip_fill(x.w, n, 0.f)); ck(jzhip_fill(x.g, n, 0.f));
-        ck(jzhip_fill(x.m, n, 0.f)); ck(jzhip_fill(x.v, n, 0.f));
+        x.name = name; x.rows = rows; x.cols = cols; x.ld = rows; x.group = group;
+        x.offset = arena[group].used;
+        arena[group].used += (x.count() + 3) / 4 * 4;   // keep every tensor 16-byte aligned
         t.push_back(x);
         return static_cast<int>(t.size()) - 1;
+    }
+    // Three row blocks of one stacked (3*rows x cols) matrix.
+    void add_stacked3(const std::string& n0, const std::string& n1, const std::string& n2, int rows, int cols,
+                      int group, int& i0, int& i1, int& i2) {
+        const size_t base = arena[group].used;
+        arena[group].used += (static_cast<size_t>(3) * rows * cols + 3) / 4 * 4;
+        const std::string* names[3] = {&n0, &n1, &n2};
+        int* idx[3] = {&i0, &i1, &i2};
+        for (int k = 0; k < 3; ++k) {
+            Tensor x;
+            x.name = *names[k]; x.rows = rows; x.cols = cols; x.ld = 3 * rows; x.group = group;
+            x.offset = base + static_cast<size_t>(k) * rows;
+            t.push_back(x);
+            *idx[k] = static_cast<int>(t.size()) - 1;
+        }
+    }
+    void finish() {
+        for (Arena& a : arena) {
+            if (a.used == 0) continue;
+            a.w = alloc(a.used); a.g = alloc(a.used); a.m = alloc(a.used); a.v = alloc(a.used);
+            if (rc != 0) return;
+            ck(jzhip_fill(a.w, a.used, 0.f)); ck(jzhip_fill(a.g, a.used, 0.f));
+            ck(jzhip_fill(a.m, a.used, 0.f)); ck(jzhip_fill(a.v, a.used, 0.f));
+        }
+        for (Tensor& x : t) {
+            Arena& a = arena[x.group];
+            x.w = a.w + x.offset; x.g = a.g + x.offset; x.m = a.m + x.offset; x.v = a.v + x.offset;
+            if (x.count() > io_floats) io_floats = x.count();
+        }
+        io = alloc(io_floats);
     }
     void ck(int r) { if (r != 0 && rc == 0) rc = r; }
 };
 
-// C(m x n) = alpha*op(A)op(B) + beta*C, dense operands
+// C(m x n) = alpha*op(A)op(B) + beta*C, dense operands unless ld is given
 inline void gemm(Model& M, const float* A, bool ta, const float* B, bool tb, float* C, int m, int n, int k,
-                 float beta = 0.f) {
-    M.ck(jzhip_gemm(A, B, C, m, n, k, ta, tb, ta ? k : m, tb ? n : k, m, 1.0f, beta));
+                 float beta = 0.f, int lda = 0, int ldb = 0, int ldc = 0) {
+    M.ck(jzhip_gemm(A, B, C, m, n, k, ta, tb, lda ? lda : (ta ? k : m), ldb ? ldb : (tb ? n : k),
+                    ldc ? ldc : m, 1.0f, beta));
+}
+// C = act(A*B + bias) + residual with the elementwise tail fused into the store
+// (act codes of jzhip_gemm_fused); operands dense, A possibly transposed
+inline void gemm_tail(Model& M, const float* A, bool ta, const float* B, float* C, int m, int n, int k,
+                      const float* bias, int act, float* aux, const float* residual, float beta = 0.f) {
+    M.ck(jzhip_gemm_fused(A, B, C, m, n, k, ta, 0, ta ? k : m, k, m, 1.0f, beta, bias, act, aux, m, residual, m));
 }
 
 void forward(Model& M) {
     const Config& c = M.c;
     const int d = c.d_model, N = M.N, ff = c.d_ff;
-    const size_t dN = static_cast<size_t>(d) * N;
     // x0 = E * onehot(tokens) + P * onehot(positions) [+ embedding bias]
     gemm(M, M.t[M.E].w, false, M.oh_tok, false, M.x0, d, N, c.vocab);
-    gemm(M, M.t[M.P].w, false, M.oh_pos, false, M.x0, d, N, c.seq, 1.0f);
-    if (M.be >= 0) M.ck(jzhip_add_bias(M.x0, M.t[M.be].w, d, N));
+    gemm_tail(M, M.t[M.P].w, false, M.oh_pos, M.x0, d, N, c.seq, M.be >= 0 ? M.t[M.be].w : nullptr, 0, nullptr,
+              nullptr, 1.0f);
     const float* x = M.x0;
     for (Block& b : M.blocks) {
         M.ck(jzhip_layernorm_fwd(b.x1, b.xhat1, b.inv1, x, M.t[b.g1].w, M.t[b.be1].w, d, N));
-        gemm(M, M.t[b.Wq].w, false, b.x1, false, b.Q, d, N, d);
-        gemm(M, M.t[b.Wk].w, false, b.x1, false, b.K, d, N, d);
-        gemm(M, M.t[b.Wv].w, false, b.x1, false, b.V, d, N, d);
-        M.ck(jzhip_attention_fwd(b.H, b.A, b.Q, b.K, b.V, d, c.heads, c.seq, c.batch, 1));
-        gemm(M, M.t[b.Wo].w, false, b.H, false, b.R, d, N, d);           // O
-        M.ck(jzhip_add_bias(b.R, M.t[b.bo].w, d, N));
-        M.ck(jzhip_axpby(b.R, x, b.R, dN, 1.0f, 1.0f));                  // R = x + O
+        // Q, K, V in one product against the stacked projection
+        gemm(M, M.t[b.Wq].w, false, b.x1, false, b.QKV, 3 * d, N, d);
+        M.ck(jzhip_attention_fwd_ld(b.H, d, b.A, b.QKV, b.QKV + d, b.QKV + 2 * d, 3 * d, d, c.heads, c.seq,
+                                    c.batch, 1));
+        // R = x + (Wo*H + bo)
+        gemm_tail(M, M.t[b.Wo].w, false, b.H, b.R, d, N, d, M.t[b.bo].w, 0, nullptr, x);
         M.ck(jzhip_layernorm_fwd(b.x2, b.xhat2, b.inv2, b.R, M.t[b.g2].w, M.t[b.be2].w, d, N));
-        gemm(M, M.t[b.W1].w, false, b.x2, false, b.F1, ff, N, d);
-        M.ck(jzhip_add_bias(b.F1, M.t[b.b1].w, ff, N));
-        const size_t fN = static_cast<size_t>(ff) * N;
-        M.ck(c.gelu ? jzhip_gelu(b.F1a, b.F1, fN) : jzhip_relu(b.F1a, b.F1, fN));
-        gemm(M, M.t[b.W2].w, false, b.F1a, false, b.out, d, N, ff);      // F
-        M.ck(jzhip_add_bias(b.out, M.t[b.b2].w, d, N));
-        M.ck(jzhip_axpby(b.out, b.R, b.out, dN, 1.0f, 1.0f));            // out = R + F
+        // F1 = W1*x2 + b1 (kept for the backward pass), F1a = act(F1)
+        gemm_tail(M, M.t[b.W1].w, false, b.x2, b.F1a, ff, N, d, M.t[b.b1].w, c.gelu ? 2 : 1, b.F1, nullptr);
+        // out = R + (W2*F1a + b2)
+        gemm_tail(M, M.t[b.W2].w, false, b.F1a, b.out, d, N, ff, M.t[b.b2].w, 0, nullptr, b.R);
         x = b.out;
     }
     if (c.tied) {
         gemm(M, M.t[M.E].w, true, x, false, M.logits, c.vocab, N, d);    // E^T x
     } else {
-        gemm(M, M.t[M.Wp].w, false, x, false, M.logits, c.vocab, N, d);
-        M.ck(jzhip_add_bias(M.logits, M.t[M.bp].w, c.vocab, N));
+        gemm_tail(M, M.t[M.Wp].w, false, x, M.logits, c.vocab, N, d, M.t[M.bp].w, 0, nullptr, nullptr);
     }
 }
 
-void step_tensor(Model& M, int idx) {
-    Tensor& x = M.t[idx];
+void step_group(Model& M, int group) {
     const Config& c = M.c;
-    const float wd = (c.adamw && x.decay) ? c.weight_decay : 0.0f;
-    M.ck(jzhip_adamw_step(x.w, x.g, x.m, x.v, x.count(), c.lr, c.beta1, c.beta2, c.eps, wd, M.iteration));
+    Arena& a = M.arena[group];
+    if (a.used == 0) return;
+    const bool decay = group == kDecay || group == kHeadDecay;
+    const float wd = (c.adamw && decay) ? c.weight_decay : 0.0f;
+    M.ck(jzhip_adamw_step(a.w, a.g, a.m, a.v, a.used, c.lr, c.beta1, c.beta2, c.eps, wd, M.iteration));
 }
 
 void backward(Model& M, bool update) {
     const Config& c = M.c;
     const int d = c.d_model, N = M.N, ff = c.d_ff, V = c.vocab;
-    const size_t dN = static_cast<size_t>(d) * N;
     const float* xL = M.blocks.empty() ? M.x0 : M.blocks.back().out;
     M.ck(jzhip_softmax_xent(M.loss, M.dlogits, M.logits, M.targets, V, N, V));
     float* dy = M.dx;  // gradient w.r.t. the current block's output
@@ -154,53 +201,42 @@ void backward(Model& M, bool update) {
         // The reference's dense layers step their weights before forming the
         // gradient they hand down (Layer::backward, ml/layer.hpp:96-105: update(),
         // then `return W().T() * t`); the untied head reproduces that order.
-        if (update) { step_tensor(M, M.Wp); step_tensor(M, M.bp); }
+        if (update) { step_group(M, kHeadDecay); step_group(M, kHeadPlain); }
         gemm(M, M.t[M.Wp].w, true, M.dlogits, false, dy, d, N, V);
     }
     for (int l = static_cast<int>(M.blocks.size()) - 1; l >= 0; --l) {
         Block& b = M.blocks[l];
-        const float* xin = l == 0 ? M.x0 : M.blocks[l - 1].out;
-        const size_t fN = static_cast<size_t>(ff) * N;
         // feed-forward
         gemm(M, dy, false, b.F1a, true, M.t[b.W2].g, d, ff, N);
         M.ck(jzhip_sum_rows(M.t[b.b2].g, dy, d, N, d));
-        gemm(M, M.t[b.W2].w, true, dy, false, M.dF1, ff, N, d);
-        M.ck(c.gelu ? jzhip_dgelu_mul(M.dF1, b.F1, M.dF1, fN) : jzhip_drelu_mul(M.dF1, b.F1, M.dF1, fN));
+        // dF1 = (W2^T dy) .* act'(F1)
+        gemm_tail(M, M.t[b.W2].w, true, dy, M.dF1, ff, N, d, nullptr, c.gelu ? 4 : 3, b.F1, nullptr);
         gemm(M, M.dF1, false, b.x2, true, M.t[b.W1].g, ff, d, N);
         M.ck(jzhip_sum_rows(M.t[b.b1].g, M.dF1, ff, N, ff));
         gemm(M, M.t[b.W1].w, true, M.dF1, false, M.dtmp, d, N, ff);      // dx2
         M.ck(jzhip_layernorm_param_grads(M.t[b.g2].g, M.t[b.be2].g, M.dtmp, b.xhat2, d, N));
-        M.ck(jzhip_layernorm_bwd(M.dR, M.dtmp, M.t[b.g2].w, b.xhat2, b.inv2, d, N));
-        M.ck(jzhip_axpby(M.dR, M.dR, dy, dN, 1.0f, 1.0f));               // dR = LN2'(dx2) + dy
+        // dR = LN2'(dx2) + dy
+        M.ck(jzhip_layernorm_bwd_residual(M.dR, M.dtmp, M.t[b.g2].w, b.xhat2, b.inv2, dy, d, N));
         // output projection
         gemm(M, M.dR, false, b.H, true, M.t[b.Wo].g, d, d, N);
         M.ck(jzhip_sum_rows(M.t[b.bo].g, M.dR, d, N, d));
         gemm(M, M.t[b.Wo].w, true, M.dR, false, M.dH, d, N, d);
-        // attention core
-        M.ck(jzhip_attention_bwd(M.dQ, M.dK, M.dV, M.dA, M.dH, b.Q, b.K, b.V, b.A, d, c.heads, c.seq, c.batch));
-        gemm(M, M.dQ, false, b.x1, true, M.t[b.Wq].g, d, d, N);
-        gemm(M, M.dK, false, b.x1, true, M.t[b.Wk].g, d, d, N);
-        gemm(M, M.dV, false, b.x1, true, M.t[b.Wv].g, d, d, N);
-        gemm(M, M.t[b.Wq].w, true, M.dQ, false, M.dtmp, d, N, d);
-        gemm(M, M.t[b.Wk].w, true, M.dK, false, M.dtmp, d, N, d, 1.0f);
-        gemm(M, M.t[b.Wv].w, true, M.dV, false, M.dtmp, d, N, d, 1.0f); // dx1
+        // attention core, gradients into the stacked (3d x N) buffer
+        M.ck(jzhip_attention_bwd_ld(M.dQKV, M.dQKV + d, M.dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
+                                    b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch));
+        gemm(M, M.dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
+        gemm(M, M.t[b.Wq].w, true, M.dQKV, false, M.dtmp, d, N, 3 * d);        // dx1
         M.ck(jzhip_layernorm_param_grads(M.t[b.g1].g, M.t[b.be1].g, M.dtmp, b.xhat1, d, N));
-        M.ck(jzhip_layernorm_bwd(dy, M.dtmp, M.t[b.g1].w, b.xhat1, b.inv1, d, N));
-        M.ck(jzhip_axpby(dy, dy, M.dR, dN, 1.0f, 1.0f));                 // dx = LN1'(dx1) + dR
-        (void)xin;
-        if (update) {
-            for (int idx : {b.Wq, b.Wk, b.Wv, b.Wo, b.bo, b.W1, b.b1, b.W2, b.b2, b.g1, b.be1, b.g2, b.be2})
-                step_tensor(M, idx);
-        }
+        // dx = LN1'(dx1) + dR
+        M.ck(jzhip_layernorm_bwd_residual(dy, M.dtmp, M.t[b.g1].w, b.xhat1, b.inv1, M.dR, d, N));
     }
     // embedding tables: dE (+)= dx0 * onehot_tok^T, dP = dx0 * onehot_pos^T
     gemm(M, dy, false, M.oh_tok, true, M.t[M.E].g, d, V, N, c.tied ? 1.0f : 0.0f);
     gemm(M, dy, false, M.oh_pos, true, M.t[M.P].g, d, c.seq, N);
     if (M.be >= 0) M.ck(jzhip_sum_rows(M.t[M.be].g, dy, d, N, d));
     if (update) {
-        step_tensor(M, M.E);
-        step_tensor(M, M.P);
-        if (M.be >= 0) step_tensor(M, M.be);
+        step_group(M, kDecay);
+        step_group(M, kPlain);
         M.iteration++;
     }
 }
@@ -227,30 +263,34 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
     const size_t dN = static_cast<size_t>(d) * N, fN = static_cast<size_t>(ff) * N;
     const size_t aN = static_cast<size_t>(S) * S * c.batch * c.heads;
 
-    M->E = M->add("embed", d, V, true);
-    M->P = M->add("pos", d, S, true);
+    M->E = M->add("embed", d, V, kDecay);
+    M->P = M->add("pos", d, S, kDecay);
     if (!c.tied) {
-        M->be = M->add("embed_bias", d, 1, false);
-        M->Wp = M->add("head", V, d, true);
-        M->bp = M->add("head_bias", V, 1, false);
+        M->be = M->add("embed_bias", d, 1, kPlain);
+        M->Wp = M->add("head", V, d, kHeadDecay);
+        M->bp = M->add("head_bias", V, 1, kHeadPlain);
     }
+    M->blocks.resize(c.layers);
     for (int l = 0; l < c.layers; ++l) {
-        Block b;
+        Block& b = M->blocks[l];
         const std::string p = "block" + std::to_string(l) + ".";
-        b.Wq = M->add(p + "Wq", d, d, true);  b.Wk = M->add(p + "Wk", d, d, true);
-        b.Wv = M->add(p + "Wv", d, d, true);  b.Wo = M->add(p + "Wo", d, d, true);
-        b.bo = M->add(p + "bo", d, 1, false);
-        b.W1 = M->add(p + "W1", ff, d, true); b.b1 = M->add(p + "b1", ff, 1, false);
-        b.W2 = M->add(p + "W2", d, ff, true); b.b2 = M->add(p + "b2", d, 1, false);
-        b.g1 = M->add(p + "ln1_gamma", d, 1, false); b.be1 = M->add(p + "ln1_beta", d, 1, false);
-        b.g2 = M->add(p + "ln2_gamma", d, 1, false); b.be2 = M->add(p + "ln2_beta", d, 1, false);
+        M->add_stacked3(p + "Wq", p + "Wk", p + "Wv", d, d, kDecay, b.Wq, b.Wk, b.Wv);
+        b.Wo = M->add(p + "Wo", d, d, kDecay);
+        b.bo = M->add(p + "bo", d, 1, kPlain);
+        b.W1 = M->add(p + "W1", ff, d, kDecay); b.b1 = M->add(p + "b1", ff, 1, kPlain);
+        b.W2 = M->add(p + "W2", d, ff, kDecay); b.b2 = M->add(p + "b2", d, 1, kPlain);
+        b.g1 = M->add(p + "ln1_gamma", d, 1, kPlain); b.be1 = M->add(p + "ln1_beta", d, 1, kPlain);
+        b.g2 = M->add(p + "ln2_gamma", d, 1, kPlain); b.be2 = M->add(p + "ln2_beta", d, 1, kPlain);
+    }
+    M->finish();
+    for (int l = 0; l < c.layers && M->rc == 0; ++l) {
+        Block& b = M->blocks[l];
         M->ck(jzhip_fill(M->t[b.g1].w, d, 1.0f));
         M->ck(jzhip_fill(M->t[b.g2].w, d, 1.0f));
         b.x1 = M->alloc(dN); b.xhat1 = M->alloc(dN); b.inv1 = M->alloc(N);
-        b.Q = M->alloc(dN); b.K = M->alloc(dN); b.V = M->alloc(dN); b.A = M->alloc(aN); b.H = M->alloc(dN);
+        b.QKV = M->alloc(3 * dN); b.A = M->alloc(aN); b.H = M->alloc(dN);
         b.R = M->alloc(dN); b.x2 = M->alloc(dN); b.xhat2 = M->alloc(dN); b.inv2 = M->alloc(N);
         b.F1 = M->alloc(fN); b.F1a = M->alloc(fN); b.out = M->alloc(dN);
-        M->blocks.push_back(b);
     }
     M->oh_tok = M->alloc(static_cast<size_t>(V) * N);
     M->oh_pos = M->alloc(static_cast<size_t>(S) * N);
@@ -260,7 +300,7 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
     M->targets = reinterpret_cast<int32_t*>(M->alloc(N));
     M->loss = M->alloc(1);
     M->dx = M->alloc(dN); M->dR = M->alloc(dN); M->dtmp = M->alloc(dN);
-    M->dQ = M->alloc(dN); M->dK = M->alloc(dN); M->dV = M->alloc(dN); M->dH = M->alloc(dN);
+    M->dQKV = M->alloc(3 * dN); M->dH = M->alloc(dN);
     M->dA = M->alloc(aN); M->dF1 = M->alloc(fN);
     if (M->rc != 0) {
         std::fprintf(stderr, "jzlm_create: device allocation failed (%s)\n", jzhip_error_string(M->rc));
@@ -289,14 +329,20 @@ JZLM_API int jzlm_tensor_cols(void* h, int i) { return static_cast<Model*>(h)->t
 
 // which: 0 parameter, 1 gradient, 2 Adam m, 3 Adam v.  Column-major host buffers.
 JZLM_API int jzlm_get(void* h, int i, int which, float* host) {
-    Tensor& x = static_cast<Model*>(h)->t[i];
+    Model* M = static_cast<Model*>(h);
+    Tensor& x = M->t[i];
     float* src = which == 0 ? x.w : which == 1 ? x.g : which == 2 ? x.m : x.v;
-    return jzhip_memcpy_d2h(host, src, x.count());
+    if (x.ld == x.rows) return jzhip_memcpy_d2h(host, src, x.count());
+    int rc = jzhip_copy2d(M->io, x.rows, 0, 0, 0, src, x.ld, 0, 0, 0, x.rows, x.cols);
+    return rc ? rc : jzhip_memcpy_d2h(host, M->io, x.count());
 }
 JZLM_API int jzlm_set(void* h, int i, int which, const float* host) {
-    Tensor& x = static_cast<Model*>(h)->t[i];
+    Model* M = static_cast<Model*>(h);
+    Tensor& x = M->t[i];
     float* dst = which == 0 ? x.w : which == 1 ? x.g : which == 2 ? x.m : x.v;
-    return jzhip_memcpy_h2d(dst, host, x.count());
+    if (x.ld == x.rows) return jzhip_memcpy_h2d(dst, host, x.count());
+    int rc = jzhip_memcpy_h2d(M->io, host, x.count());
+    return rc ? rc : jzhip_copy2d(dst, x.ld, 0, 0, 0, M->io, x.rows, 0, 0, 0, x.rows, x.cols);
 }
 
 // tokens: batch windows of seq+1 ids each (window b = tokens[b*(seq+1) ...]);

@@ -303,6 +303,76 @@ def test_gemm_variants(gpu, oracle_lib, m, n, k, ta, tb):
             assert np.array_equal(g2[:, m:], C0.reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 5, 7), (64, 64, 64), (129, 127, 17), (256, 512, 128), (128, 1024, 96)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1)])
+@pytest.mark.parametrize("act", [0, 1, 2, 3, 4])
+def test_gemm_fused_epilogue(gpu, m, n, k, ta, tb, act):
+    """bias / activation / residual fused into the store of C: bit-identical to
+    jzhip_gemm followed by the separate kernels, and within the GEMM tolerance
+    of the float64 closed form (erf-GELU from math.erf)."""
+    import math
+    r = rng(m * 31 + n * 7 + k + act)
+    lda, ldb = (k if ta else m), (n if tb else k)
+    A = (r.normal(0, 1, lda * (m if ta else k)) / np.sqrt(k)).astype(np.float32)
+    B = r.normal(0, 1, ldb * (k if tb else n)).astype(np.float32)
+    bias = r.normal(0, 1, m).astype(np.float32)
+    res = r.normal(0, 1, m * n).astype(np.float32)
+    pre = r.normal(0, 1, m * n).astype(np.float32)      # saved pre-activation for act 3/4
+    dA, dB, dbias, dres = to_dev(A), to_dev(B), to_dev(bias), to_dev(res)
+    # separate kernels
+    dC = dev_empty(m * n)
+    daux = to_dev(pre) if act in (3, 4) else dev_empty(m * n)
+    gpu.gemm(dptr(dA), dptr(dB), dptr(dC), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0)
+    gpu.add_bias(dptr(dC), dptr(dbias), m, n)
+    want_aux = to_host(dC).copy()
+    if act == 1:
+        gpu.relu(dptr(dC), dptr(dC), m * n)
+    elif act == 2:
+        gpu.gelu(dptr(dC), dptr(dC), m * n)
+    elif act == 3:
+        gpu.drelu_mul(dptr(dC), dptr(daux), dptr(dC), m * n)
+    elif act == 4:
+        gpu.dgelu_mul(dptr(dC), dptr(daux), dptr(dC), m * n)
+    gpu.axpby(dptr(dC), dptr(dC), dptr(dres), m * n, 1.0, 1.0)
+    want = to_host(dC)
+    # fused
+    dF = dev_empty(m * n)
+    daux2 = to_dev(pre) if act in (3, 4) else dev_empty(m * n)
+    gpu.gemm_fused(dptr(dA), dptr(dB), dptr(dF), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0, dptr(dbias), act,
+                   dptr(daux2) if act else None, m, dptr(dres), m)
+    got = to_host(dF)
+    assert np.array_equal(got, want)
+    if act in (1, 2):
+        assert np.array_equal(to_host(daux2), want_aux)
+    # closed form in float64
+    Am = A.astype(np.float64).reshape(-1, lda).T
+    Bm = B.astype(np.float64).reshape(-1, ldb).T
+    opA = Am.T if ta else Am
+    opB = Bm.T if tb else Bm
+    v = opA @ opB + bias.astype(np.float64)[:, None]
+    erf = np.vectorize(math.erf)
+    P = pre.astype(np.float64).reshape(n, m).T
+    if act == 1:
+        v = np.maximum(v, 0)
+    elif act == 2:
+        v = 0.5 * v * (1 + erf(v / math.sqrt(2)))
+    elif act == 3:
+        v = v * (P > 0)
+    elif act == 4:
+        v = v * (0.5 * (1 + erf(P / math.sqrt(2))) + P * np.exp(-0.5 * P * P) / math.sqrt(2 * math.pi))
+    v = v + res.astype(np.float64).reshape(n, m).T
+    assert rel_err(got, v.T.reshape(-1)) <= TOL_GEMM
+
+
+def test_gemm_fused_rejects_bad_arguments(gpu):
+    from juzhen_amd import capi
+    lib = capi.load()
+    d = dev_empty(16)
+    assert lib.jzhip_gemm_fused(dptr(d), dptr(d), dptr(d), 2, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0, None, 7, None, 2, None, 2) == -1
+    assert lib.jzhip_gemm_fused(dptr(d), dptr(d), dptr(d), 2, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0, None, 3, None, 2, None, 2) == -1
+    assert lib.jzhip_gemm_fused(dptr(d), dptr(d), dptr(d), 2, 2, 2, 0, 0, 2, 2, 2, 1.0, 0.0, None, 0, None, 2, dptr(d), 1) == -1
+
+
 def test_gemm_known_answer(gpu):
     """tests/testRocmDeviceProof.cu:36-41: [[1,2],[3,4]]*[[5,6],[7,8]] = [[19,22],[43,50]]."""
     A = np.array([1, 3, 2, 4], np.float32)  # column-major
@@ -467,6 +537,14 @@ def test_layernorm(gpu, oracle_lib, dim, N):
     ddx = dev_empty(dim * N)
     gpu.layernorm_bwd(dptr(ddx), dp(g), dptr(dg), dp(xh), dp(inv), dim, N)
     assert rel_err(to_host(ddx), dx) <= TOL_RED
+    # the fused skip-gradient add equals the separate add bit for bit
+    res = r.normal(0, 1, dim * N).astype(np.float32)
+    dres = to_dev(res)
+    dfused = dev_empty(dim * N)
+    gpu.layernorm_bwd_residual(dptr(dfused), dp(g), dptr(dg), dp(xh), dp(inv), dptr(dres), dim, N)
+    gpu.axpby(dptr(ddx), dptr(ddx), dptr(dres), dim * N, 1.0, 1.0)
+    assert np.array_equal(to_host(dfused), to_host(ddx))
+    assert rel_err(to_host(dfused), dx.astype(np.float64) + res) <= TOL_RED
 
     rg, rb = np.empty(dim, np.float32), np.empty(dim, np.float32)
     oracle_lib.jzo_layernorm_param_grads(hptr(rg), hptr(rb), hptr(g), hptr(xh), dim, N)
@@ -681,3 +759,20 @@ def test_attention_fwd_bwd(gpu, d_k, heads, S, B, causal):
     assert rel_err(to_host(ov), dV.reshape(-1)) <= TOL_GEMM
     assert rel_err(to_host(oq), dQ.reshape(-1)) <= TOL_GEMM
     assert rel_err(to_host(ok_), dK.reshape(-1)) <= TOL_GEMM
+    # the same operands as row blocks of stacked (3*d_k, N) buffers give the same bits
+    import torch
+    ld = 3 * d_k
+    qkv = torch.stack([dq.view(N, d_k), dk.view(N, d_k), dv.view(N, d_k)], dim=1).contiguous().view(-1)
+    base = qkv.data_ptr()
+    Hs, As = dev_empty(N * d_k), dev_empty(S * S * B * heads)
+    pq, pk, pv = (C.c_void_p(base + 4 * i * d_k) for i in range(3))
+    gpu.attention_fwd_ld(dptr(Hs), d_k, dptr(As), pq, pk, pv, ld, d_k, heads, S, B, causal)
+    assert np.array_equal(to_host(Hs), to_host(dHm)) and np.array_equal(to_host(As), to_host(dAm))
+    dqkv = dev_empty(3 * N * d_k)
+    ob = dqkv.data_ptr()
+    gpu.attention_bwd_ld(C.c_void_p(ob), C.c_void_p(ob + 4 * d_k), C.c_void_p(ob + 8 * d_k), ld, dptr(scratch),
+                         dp(dH.reshape(-1)), d_k, pq, pk, pv, ld, dptr(As), d_k, heads, S, B)
+    got = to_host(dqkv).reshape(N, 3, d_k)
+    assert np.array_equal(got[:, 0].reshape(-1), to_host(oq))
+    assert np.array_equal(got[:, 1].reshape(-1), to_host(ok_))
+    assert np.array_equal(got[:, 2].reshape(-1), to_host(ov))
