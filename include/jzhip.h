@@ -301,7 +301,12 @@ int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch,
                         int S, int B);
 /* The same two calls for operands that live inside wider matrices (Q, K, V as
  * row blocks of one stacked (3*d_k, S*B) projection and likewise dQ, dK, dV):
- * ld_qkv / ld_dqkv / ld_h / ld_dh are the leading dimensions of those buffers. */
+ * ld_qkv / ld_dqkv / ld_h / ld_dh are the leading dimensions of those buffers.
+ * causal != 0 in the backward call states that A came from a causal forward
+ * call (exact zeros above the diagonal), which lets it skip those key tiles.
+ * For head widths 32 and 64 with S a multiple of 32 up to 256 both calls run
+ * as one fused kernel per pass (scores, softmax and the second product in
+ * registers); other shapes take batched GEMMs and the softmax kernels. */
 int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q,
                            const float* K, const float* V, int ld_qkv, int d_k,
                            int heads, int S, int B, int causal);
@@ -309,7 +314,7 @@ int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv,
                            float* dA_scratch, const float* dH, int ld_dh,
                            const float* Q, const float* K, const float* V,
                            int ld_qkv, const float* A, int d_k, int heads, int S,
-                           int B);
+                           int B, int causal);
 
 /* ── LayerNorm ───────────────────────────────────────────────────────── */
 

@@ -17,6 +17,338 @@ int gemm_batched2(const float* A, const float* B, float* C, int m, int n, int k,
                   long long sA2, long long sB2, long long sC2, int batch2, float alpha, float beta);
 }
 
+
+namespace jz {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// One workgroup per (head, sequence) block, everything for that block in one
+// launch.  Forward (BWD = false):
+//     P = softmax_keys(scale * K^T Q, causal mask)   -> A (kept for the backward pass)
+//     H = V P
+// Backward core (BWD = true), with P read back from A:
+//     dA = V^T dH,  dS = P .* (dA - sum_keys(P .* dA)) * scale   -> dS
+//     dQ = K dS
+// (dV = dH P^T and dK = Q dS^T reduce over queries and stay batched GEMMs.)
+//
+// Both passes are "scores-like product, per-query row operation, second
+// product": X1 (Q or dH) x M1 (K or V) gives a (keys x queries) matrix whose
+// 32x32 MFMA tiles keep the query along the lanes and the keys along the
+// accumulator registers, so the softmax (or its backward) is an in-register
+// reduction plus one exchange between the two half-waves, and the second
+// product takes its B operand (P or dS) straight from those registers: the
+// S x S matrix never goes through LDS and is written to HBM once.
+//
+// A wave owns 32 queries at a time (all their keys: up to 8 tiles = 128
+// accumulator registers), two such groups per wave, paired (g, G-1-g) so the
+// causal triangle gives every wave the same work.  M1 is staged in LDS as
+// [d][key] (pitch S+1), M2 as [key][d] (pitch DH+4); X1 fragments are read
+// straight from global memory (each lane 32 consecutive floats of its query's
+// column: half-wave h contracts d in [h*DH/2, (h+1)*DH/2)).
+constexpr int kMaxKeyTiles = 8;   // S <= 256
+constexpr int kAttnThreads = 512;  // eight waves: one query group each, two per SIMD
+constexpr int kLD1 = 32 * kMaxKeyTiles + 1;   // pitch of the [d][key] staging, whatever S is
+
+// One group of 32 queries against its first 2*NP key tiles (NP compile-time so
+// that the accumulator tiles stay in registers without predication).
+template <int DH, bool BWD, int NP>
+__device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, float* __restrict__ Ablk,
+                                           float* __restrict__ dSblk, const float* __restrict__ x1, int ld_x1,
+                                           const float* t1, const float* t2, int S, int G, int g,
+                                           int l32, int h, float scale, int causal) {
+    constexpr int HD = DH / 2;        // contraction steps of the first product
+    constexpr int NDT = DH / 32;      // 32-row tiles of the second product's output
+    constexpr int LD2 = DH + 4;
+    constexpr int NT = 2 * NP;
+    constexpr int LD1 = kLD1;
+    const int q = g * 32 + l32;       // query index inside the block
+    // S x S block addressing: wave-uniform key row plus one lane offset
+    const unsigned lane_off = static_cast<unsigned>(4 * h) * static_cast<unsigned>(S) + q;
+
+    // this lane's X1 fragments: d = HD*h + kk for kk = 0..HD-1
+    float xf[HD];
+    {
+        const float* src = x1 + static_cast<size_t>(q) * ld_x1 + HD * h;
+#pragma unroll
+        for (int i = 0; i < HD / 4; ++i) {
+            const floatx4 t = *reinterpret_cast<const floatx4*>(src + 4 * i);
+            xf[4 * i] = t.x; xf[4 * i + 1] = t.y; xf[4 * i + 2] = t.z; xf[4 * i + 3] = t.w;
+        }
+    }
+
+    // first product, two key tiles at a time
+    floatx16 sc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[t][v] = 0.0f;
+#pragma unroll
+    for (int tp = 0; tp < NP; ++tp) {
+        const float* base = t1 + 64 * tp;
+        float a0 = base[0], a1 = base[32];
+#pragma unroll
+        for (int kk = 0; kk < HD; ++kk) {
+            float n0 = 0.f, n1 = 0.f;
+            if (kk + 1 < HD) {
+                n0 = base[(kk + 1) * LD1];
+                n1 = base[(kk + 1) * LD1 + 32];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            sc[2 * tp] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, xf[kk], sc[2 * tp], 0, 0, 0);
+            sc[2 * tp + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, xf[kk], sc[2 * tp + 1], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            a0 = n0; a1 = n1;
+        }
+    }
+
+    // per-query row operation; register v of tile t is key 32t + 8(v/4) + 4h + v%4
+    if constexpr (!BWD) {
+        float m = -1e30f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
+                float x = sc[t][v] * scale;
+                if ((causal && key > q) || key >= S) x = -1e9f;   // ml/layer.hpp:2979-2994; tile past S
+                sc[t][v] = x;
+                m = m > x ? m : x;
+            }
+        }
+        {
+            const float o = __shfl_xor(m, 32);
+            m = m > o ? m : o;
+        }
+        float sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float e = expf(sc[t][v] - m);
+                sc[t][v] = e;
+                sum += e;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        sum += __shfl_xor(sum, 32);
+        const float inv = 1.0f / (sum + 1e-12f);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
+                const float pv = sc[t][v] * inv;
+                sc[t][v] = pv;
+                const int ku = 32 * t + 8 * (v / 4) + (v % 4);
+                if (32 * t < S) (Ablk + static_cast<size_t>(ku) * S)[lane_off] = pv;
+            }
+        }
+    } else {
+        // P is read twice (dot product, then dS) instead of being held in 16*NT more
+        // registers; the second wave of the SIMD covers the latency.  S is a
+        // multiple of 32, so a tile lies entirely inside or outside the block.
+        float dot = 0.f;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (32 * t < S) {
+                float pv[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int ku = 32 * t + 8 * (v / 4) + (v % 4);
+                    pv[v] = (Ablk + static_cast<size_t>(ku) * S)[lane_off];
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) dot += pv[v] * sc[t][v];
+            }
+        }
+        dot += __shfl_xor(dot, 32);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (32 * t < S) {
+                float pv[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int ku = 32 * t + 8 * (v / 4) + (v % 4);
+                    pv[v] = (Ablk + static_cast<size_t>(ku) * S)[lane_off];
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int ku = 32 * t + 8 * (v / 4) + (v % 4);
+                    const float ds = (pv[v] * (sc[t][v] - dot)) * scale;
+                    sc[t][v] = ds;
+                    (dSblk + static_cast<size_t>(ku) * S)[lane_off] = ds;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sc[t][v] = 0.0f;
+            }
+        }
+    }
+    // key tiles past the causal range hold exact zeros
+    for (int t = NT; t < G; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int ku = 32 * t + 8 * (v / 4) + (v % 4);
+            ((BWD ? dSblk : Ablk) + static_cast<size_t>(ku) * S)[lane_off] = 0.0f;
+        }
+
+    // second product: Out[d][query] = sum_key M2[d][key] * sc[key][query]
+    floatx16 oacc[NDT];
+#pragma unroll
+    for (int u = 0; u < NDT; ++u)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[u][v] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        if (32 * t < S) {   // (an odd tile count leaves one all-zero tile in the last pair)
+            float an[NDT];
+#pragma unroll
+            for (int u = 0; u < NDT; ++u) an[u] = t2[(32 * t) * LD2 + 32 * u];
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                float ac[NDT];
+#pragma unroll
+                for (int u = 0; u < NDT; ++u) ac[u] = an[u];
+                if (s + 1 < 16) {
+                    const int keyn = 32 * t + 8 * ((s + 1) / 4) + ((s + 1) % 4);   // + 4h is in t2
+#pragma unroll
+                    for (int u = 0; u < NDT; ++u) an[u] = t2[keyn * LD2 + 32 * u];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < NDT; ++u)
+                    oacc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(ac[u], sc[t][s], oacc[u], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    // Out(d, query): register v of tile u is d = 32u + 8(v/4) + 4h + v%4
+    float* dst = out + static_cast<size_t>(q) * ld_out + 4 * h;
+#pragma unroll
+    for (int u = 0; u < NDT; ++u)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+            floatx4 o = {oacc[u][4 * v4], oacc[u][4 * v4 + 1], oacc[u][4 * v4 + 2], oacc[u][4 * v4 + 3]};
+            *reinterpret_cast<floatx4*>(dst + 32 * u + 8 * v4) = o;
+        }
+}
+
+template <int DH, bool BWD>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
+    float* __restrict__ Out, int ld_out, float* __restrict__ Aio, float* __restrict__ dS_out,
+    const float* __restrict__ X1, int ld_x1, const float* __restrict__ M1, const float* __restrict__ M2,
+    int ld_m, int heads, int S, int B, float scale, int causal) {
+    constexpr int HD = DH / 2;
+    constexpr int LD2 = DH + 4;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int LD1 = kLD1;
+    // LDS rows past S (the second tile of an odd last pair) are read but only
+    // multiply masked or zero entries; the buffers are sized for an even tile count.
+    const int S2 = (S + 63) / 64 * 64;
+    float* T1 = lds;                                    // [DH][LD1], LD1 >= S2 + 1 ...
+    (void)S2;
+    float* T2 = lds + ((DH * LD1 + 64 + 3) / 4) * 4;    // [S2][LD2]
+
+    const int blk = blockIdx.x;            // hh*B + b
+    const int hh = blk / B, b = blk % B;
+    const size_t col0 = static_cast<size_t>(b) * S;
+    const float* m1 = M1 + col0 * ld_m + hh * DH;
+    const float* m2 = M2 + col0 * ld_m + hh * DH;
+    const float* x1 = X1 + col0 * ld_x1 + hh * DH;
+    float* out = Out + col0 * ld_out + hh * DH;
+    const size_t blk_off = static_cast<size_t>(blk) * S * S;
+    float* Ablk = Aio + blk_off;
+    float* dSblk = BWD ? dS_out + blk_off : nullptr;
+
+    // stage M1 transposed and M2 as it lies: all global loads of a thread first
+    // (they are independent), then the LDS stores
+    {
+        constexpr int kIters = (DH / 4) * 32 * kMaxKeyTiles / kAttnThreads;
+        const int total = (DH / 4) * S;
+        floatx4 ra[kIters], rc[kIters];
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+            const int v = threadIdx.x + i * kAttnThreads;
+            if (v < total) {
+                const int dq = v % (DH / 4), tok = v / (DH / 4);
+                ra[i] = *reinterpret_cast<const floatx4*>(m1 + static_cast<size_t>(tok) * ld_m + 4 * dq);
+                rc[i] = *reinterpret_cast<const floatx4*>(m2 + static_cast<size_t>(tok) * ld_m + 4 * dq);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+            const int v = threadIdx.x + i * kAttnThreads;
+            if (v < total) {
+                const int dq = v % (DH / 4), tok = v / (DH / 4);
+                float* d1 = T1 + (4 * dq) * LD1 + tok;
+                d1[0] = ra[i].x; d1[LD1] = ra[i].y; d1[2 * LD1] = ra[i].z; d1[3 * LD1] = ra[i].w;
+                *reinterpret_cast<floatx4*>(T2 + tok * LD2 + 4 * dq) = rc[i];
+            }
+        }
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int l32 = lane & 31, h = lane >> 5;
+    const int G = S / 32;
+    const float* t1 = T1 + (HD * h) * LD1 + l32;
+    const float* t2 = T2 + (4 * h) * LD2 + l32;
+
+    // wave w < 4 takes group w, wave w >= 4 takes group G-1-(w-4): the two waves
+    // of a SIMD (w, w+4) share the causal triangle evenly
+    {
+        const int g = wave < 4 ? wave : G - 1 - (wave - 4);
+        const bool mine = wave < 4 ? (wave < (G + 1) / 2) : (wave - 4 < G / 2);
+        if (mine) {
+            const int nkt = causal ? g + 1 : G;          // key tiles that are not entirely masked
+            switch ((nkt + 1) / 2) {
+            case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
+            case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
+            case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
+            default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
+            }
+        }
+    }
+}
+
+size_t attn_core_lds_bytes(int d_h, int S) {
+    const size_t S2 = static_cast<size_t>(S + 63) / 64 * 64;
+    return (static_cast<size_t>((d_h * kLD1 + 64 + 3) / 4 * 4) + S2 * (d_h + 4)) * sizeof(float);
+}
+
+// The fused kernel covers head widths 32 and 64 with S a multiple of 32 up to
+// 256 and 16-byte aligned operands; other shapes take the batched-GEMM path.
+bool attn_core_ok(int d_h, int S, int heads, int B, const void* p0, const void* p1, const void* p2, const void* p3,
+                  int ld_a, int ld_b, int ld_c) {
+    if (!(d_h == 32 || d_h == 64)) return false;
+    if (S % 32 != 0 || S > 32 * kMaxKeyTiles) return false;
+    if (static_cast<long long>(heads) * B > 0x7fffffffLL) return false;
+    if (ld_a % 4 || ld_b % 4 || ld_c % 4) return false;
+    return aligned16(p0) && aligned16(p1) && aligned16(p2) && aligned16(p3);
+}
+
+template <int DH, bool BWD>
+int launch_attn_core(float* Out, int ld_out, float* Aio, float* dS, const float* X1, int ld_x1, const float* M1,
+                     const float* M2, int ld_m, int heads, int S, int B, float scale, int causal) {
+    const size_t lds = attn_core_lds_bytes(DH, S);
+    static bool configured = false;   // per instantiation
+    if (!configured) {
+        int rc = rc_of(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_core_kernel<DH, BWD>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        if (rc) return rc;
+        configured = true;
+    }
+    attn_core_kernel<DH, BWD><<<heads * B, kAttnThreads, lds, stream()>>>(Out, ld_out, Aio, dS, X1, ld_x1, M1, M2, ld_m,
+                                                                   heads, S, B, scale, causal);
+    return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
 JZ_API int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q, const float* K,
                                   const float* V, int ld_qkv, int d_k, int heads, int S, int B,
                                   int causal) {
@@ -27,6 +359,13 @@ JZ_API int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q, 
     const long long seq_h = static_cast<long long>(S) * ld_h;  // next sequence in H
     const long long blk = static_cast<long long>(S) * S;       // next score block
     const float scale = 1.0f / sqrtf(static_cast<float>(d_h));
+    if (jz::attn_core_ok(d_h, S, heads, B, H, Q, K, V, ld_h, ld_qkv, ld_qkv)) {
+        if (d_h == 64)
+            return jz::launch_attn_core<64, false>(H, ld_h, A, nullptr, Q, ld_qkv, K, V, ld_qkv, heads, S, B, scale,
+                                                   causal);
+        return jz::launch_attn_core<32, false>(H, ld_h, A, nullptr, Q, ld_qkv, K, V, ld_qkv, heads, S, B, scale,
+                                               causal);
+    }
     // scores[q, k] = <Q_i[:, q], K_i[:, k]>
     int rc = jz::gemm_batched2(Q, K, A, S, S, d_h, true, false, ld_qkv, ld_qkv, S, seq, seq, blk, B, d_h, d_h,
                                blk * B, heads, 1.0f, 0.0f);
@@ -47,7 +386,7 @@ JZ_API int jzhip_attention_fwd(float* H, float* A, const float* Q, const float* 
 JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, float* dA_scratch,
                                   const float* dH, int ld_dh, const float* Q, const float* K,
                                   const float* V, int ld_qkv, const float* A, int d_k, int heads,
-                                  int S, int B) {
+                                  int S, int B, int causal) {
     if (d_k <= 0 || heads <= 0 || S <= 0 || B <= 0 || d_k % heads != 0) return -1;
     if (!dQ || !dK || !dV || !dA_scratch || !dH || !Q || !K || !V || !A) return -1;
     if (ld_dqkv < d_k || ld_dh < d_k || ld_qkv < d_k) return -1;
@@ -61,6 +400,18 @@ JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, 
     int rc = jz::gemm_batched2(dH, A, dV, d_h, S, S, false, false, ld_dh, S, ld_dqkv, seq_h, blk, seq_d, B, d_h,
                                blk * B, d_h, heads, 1.0f, 0.0f);
     if (rc) return rc;
+    if (jz::attn_core_ok(d_h, S, heads, B, dQ, dH, K, V, ld_dqkv, ld_dh, ld_qkv)) {
+        // dA, dS and dQ in one launch; with causal set the key tiles above the
+        // diagonal (exact zeros in A) are skipped
+        rc = d_h == 64 ? jz::launch_attn_core<64, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, dH, ld_dh, V,
+                                                        K, ld_qkv, heads, S, B, scale, causal)
+                       : jz::launch_attn_core<32, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, dH, ld_dh, V,
+                                                        K, ld_qkv, heads, S, B, scale, causal);
+        if (rc) return rc;
+        // dK_i = Q_i * dS_i
+        return jz::gemm_batched2(Q, dA_scratch, dK, d_h, S, S, false, false, ld_qkv, S, ld_dqkv, seq, blk, seq_d, B,
+                                 d_h, blk * B, d_h, heads, 1.0f, 0.0f);
+    }
     // dA_i[q, k] = <dH_i[:, q], V_i[:, k]>
     rc = jz::gemm_batched2(dH, V, dA_scratch, S, S, d_h, true, false, ld_dh, ld_qkv, S, seq_h, seq, blk, B, d_h,
                            d_h, blk * B, heads, 1.0f, 0.0f);
@@ -80,5 +431,5 @@ JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, 
 JZ_API int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch, const float* dH,
                                const float* Q, const float* K, const float* V, const float* A,
                                int d_k, int heads, int S, int B) {
-    return jzhip_attention_bwd_ld(dQ, dK, dV, d_k, dA_scratch, dH, d_k, Q, K, V, d_k, A, d_k, heads, S, B);
+    return jzhip_attention_bwd_ld(dQ, dK, dV, d_k, dA_scratch, dH, d_k, Q, K, V, d_k, A, d_k, heads, S, B, 0);
 }

@@ -223,7 +223,7 @@ void backward(Model& M, bool update) {
         gemm(M, M.t[b.Wo].w, true, M.dR, false, M.dH, d, N, d);
         // attention core, gradients into the stacked (3d x N) buffer
         M.ck(jzhip_attention_bwd_ld(M.dQKV, M.dQKV + d, M.dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
-                                    b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch));
+                                    b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch, 1));
         gemm(M, M.dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
         gemm(M, M.t[b.Wq].w, true, M.dQKV, false, M.dtmp, d, N, 3 * d);        // dx1
         M.ck(jzhip_layernorm_param_grads(M.t[b.g1].g, M.t[b.be1].g, M.dtmp, b.xhat1, d, N));

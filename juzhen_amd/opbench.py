@@ -198,12 +198,12 @@ def bench_fused(r):
         r.run("fused", "jzhip_attn_softmax (causal)", s, lambda: jz.attn_softmax(P(o), P(a), S, nblk, 0.125, 1, kar), bytes_=8 * a.numel())
         r.run("fused", "jzhip_attn_softmax_bwd", s, lambda: jz.attn_softmax_bwd(P(da), P(o), P(da), S, nblk, 0.125, kar), bytes_=12 * a.numel())
     # attention core of C4 (QK^T, mask+softmax, AV and their backward)
-    dk, heads, B = 64, 8, 64
+    dk, heads, B = 512, 8, 64
     N = S * B
     Q, K, V, H = (dev(dk * heads * N) for _ in range(4))
     A = dev(S * S * heads * B, 0)
     dQ, dK, dV, dA = dev(dk * heads * N, 0), dev(dk * heads * N, 0), dev(dk * heads * N, 0), dev(S * S * heads * B, 0)
-    fl = 4.0 * S * S * dk * heads * B
+    fl = 4.0 * S * S * dk * B
     r.run("fused", "jzhip_attention_fwd", f"S{S} d_k{dk} h{heads} B{B}",
           lambda: jz.attention_fwd(P(H), P(A), P(Q), P(K), P(V), dk, heads, S, B, 1), flops=fl)
     r.run("fused", "jzhip_attention_bwd", f"S{S} d_k{dk} h{heads} B{B}",

@@ -722,7 +722,8 @@ def test_rand(gpu):
 
 # ── batched attention core ───────────────────────────────────────────────
 @pytest.mark.parametrize("d_k,heads,S,B,causal", [(8, 4, 3, 2, 1), (16, 2, 5, 3, 0), (64, 1, 17, 2, 1), (128, 2, 64, 3, 1),
-                                                  (512, 8, 32, 2, 1)])
+                                                  (512, 8, 32, 2, 1), (512, 8, 256, 2, 1), (256, 4, 128, 1, 0),
+                                                  (64, 2, 96, 2, 1), (128, 2, 160, 1, 1), (128, 4, 224, 1, 0)])
 def test_attention_fwd_bwd(gpu, d_k, heads, S, B, causal):
     """Against a float64 restatement of the per-(head, sequence) loop of
     ml/layer.hpp:2967-3006 and 3329-3363 (the method of tests/testTransformerRef.cu:102-141)."""
@@ -771,7 +772,7 @@ def test_attention_fwd_bwd(gpu, d_k, heads, S, B, causal):
     dqkv = dev_empty(3 * N * d_k)
     ob = dqkv.data_ptr()
     gpu.attention_bwd_ld(C.c_void_p(ob), C.c_void_p(ob + 4 * d_k), C.c_void_p(ob + 8 * d_k), ld, dptr(scratch),
-                         dp(dH.reshape(-1)), d_k, pq, pk, pv, ld, dptr(As), d_k, heads, S, B)
+                         dp(dH.reshape(-1)), d_k, pq, pk, pv, ld, dptr(As), d_k, heads, S, B, causal)
     got = to_host(dqkv).reshape(N, 3, d_k)
     assert np.array_equal(got[:, 0].reshape(-1), to_host(oq))
     assert np.array_equal(got[:, 1].reshape(-1), to_host(ok_))
