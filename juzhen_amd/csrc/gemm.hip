@@ -18,6 +18,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 namespace jz {
@@ -390,44 +391,97 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kerne
     }
     // Fused tail.  Addresses are a wave-uniform pointer (tile origin and column,
     // scalar registers) plus one 32-bit lane offset per array, so the tail costs
-    // three address registers instead of one pointer per element.
+    // three address registers instead of one pointer per element.  Per 32x32
+    // tile the residual and saved pre-activation values are requested in one
+    // batch before any arithmetic, and the activation is chosen once per tile.
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int wm_u = wave_u % WGM, wn_u = wave_u / WGM;
     const unsigned lane_c = static_cast<unsigned>(4 * h) * static_cast<unsigned>(ldc) + l32;
     const unsigned lane_r = static_cast<unsigned>(4 * h) * static_cast<unsigned>(ep.ldr) + l32;
     const unsigned lane_a = static_cast<unsigned>(4 * h) * static_cast<unsigned>(ep.ld_aux) + l32;
-    const float* aux_in = ep.aux_in;
-    float* aux_out = ep.aux_out;
+    auto live = [&](int row0, int col0, int v) {
+        return FAST || (row0 + l32 < M && col0 + 8 * (v / 4) + (v % 4) + 4 * h < N);
+    };
+    // residual (r) and saved pre-activation (x) values of one tile, one batch of loads
+    auto tail_fetch = [&](auto& r, auto& x, int row0, int col0, auto act_c, auto res_c) {
+        constexpr int ACT = decltype(act_c)::value;
+        constexpr bool RES = decltype(res_c)::value;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int row0 = m0 + (wm_u * TM + i) * 32;
-        const int row = row0 + l32;
-        const float bias = (ep.bias && (FAST || row < M)) ? ep.bias[row] : 0.0f;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col0 = n0 + (wn_u * TN + j) * 32;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int cu = col0 + 8 * (v / 4) + (v % 4);   // uniform part of the column
-                const int col = cu + 4 * h;
-                if (FAST || (row < M && col < N)) {
-                    float* dst = C + (static_cast<size_t>(cu) * ldc + row0) + lane_c;
-                    float r = alpha * acc[i][j][v];
-                    if (beta != 0.0f) r += beta * *dst;
-                    if (ep.bias) r += bias;
-                    if (ep.act == 1 || ep.act == 2) {
-                        if (aux_out) (aux_out + (static_cast<size_t>(cu) * ep.ld_aux + row0))[lane_a] = r;
-                        r = ep.act == 1 ? relu_f(r) : gelu_f(r);
-                    } else if (ep.act == 3 || ep.act == 4) {
-                        const float pre = (aux_in + (static_cast<size_t>(cu) * ep.ld_aux + row0))[lane_a];
-                        r = r * (ep.act == 3 ? drelu_f(pre) : dgelu_f(pre));
-                    }
-                    if (ep.res) r += (ep.res + (static_cast<size_t>(cu) * ep.ldr + row0))[lane_r];
-                    *dst = r;
-                }
-                if (v % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        for (int v = 0; v < 16; ++v) {
+            const int cu = col0 + 8 * (v / 4) + (v % 4);   // wave-uniform part of the column
+            if constexpr (RES) r[v] = 0.0f;
+            if constexpr (ACT == 3 || ACT == 4) x[v] = 0.0f;
+            if (live(row0, col0, v)) {
+                if constexpr (RES) r[v] = (ep.res + (static_cast<size_t>(cu) * ep.ldr + row0))[lane_r];
+                if constexpr (ACT == 3 || ACT == 4)
+                    x[v] = (ep.aux_in + (static_cast<size_t>(cu) * ep.ld_aux + row0))[lane_a];
             }
         }
+    };
+    auto tail_tile = [&](const floatx16& a, const auto& r, const auto& x, int row0, int col0, float bias,
+                         auto act_c, auto res_c) {
+        constexpr int ACT = decltype(act_c)::value;
+        constexpr bool RES = decltype(res_c)::value;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int cu = col0 + 8 * (v / 4) + (v % 4);
+            if (live(row0, col0, v)) {
+                float* dst = C + (static_cast<size_t>(cu) * ldc + row0) + lane_c;
+                float t = alpha * a[v];
+                if (beta != 0.0f) t += beta * *dst;
+                if (ep.bias) t += bias;
+                if constexpr (ACT == 1 || ACT == 2) {
+                    if (ep.aux_out) (ep.aux_out + (static_cast<size_t>(cu) * ep.ld_aux + row0))[lane_a] = t;
+                    t = ACT == 1 ? relu_f(t) : gelu_f(t);
+                } else if constexpr (ACT == 3) {
+                    t = t * drelu_f(x[v]);
+                } else if constexpr (ACT == 4) {
+                    t = t * dgelu_f(x[v]);
+                }
+                if constexpr (RES) t += r[v];
+                *dst = t;
+            }
+            if (v % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // tiles in order; the loads of tile n+1 are in flight while tile n is finished
+    auto tail_all = [&](auto act_c, auto res_c) {
+        constexpr int ACT = decltype(act_c)::value;
+        constexpr bool RES = decltype(res_c)::value;
+        // (both arrays at once would not fit beside the accumulators: that rare form is not pipelined)
+        constexpr int NBUF = ((ACT == 3 || ACT == 4) && RES) ? 1 : 2;
+        float r[NBUF][RES ? 16 : 1], x[NBUF][(ACT == 3 || ACT == 4) ? 16 : 1];
+        auto rows = [&](int n) { return m0 + (wm_u * TM + n / TN) * 32; };
+        auto cols = [&](int n) { return n0 + (wn_u * TN + n % TN) * 32; };
+        tail_fetch(r[0], x[0], rows(0), cols(0), act_c, res_c);
+#pragma unroll
+        for (int n = 0; n < TM * TN; ++n) {
+            if constexpr (NBUF == 2) {
+                if (n + 1 < TM * TN)
+                    tail_fetch(r[(n + 1) & 1], x[(n + 1) & 1], rows(n + 1), cols(n + 1), act_c, res_c);
+            } else if (n > 0) {
+                tail_fetch(r[0], x[0], rows(n), cols(n), act_c, res_c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const int row = rows(n) + l32;
+            const float bias = (ep.bias && (FAST || row < M)) ? ep.bias[row] : 0.0f;
+            tail_tile(acc[n / TN][n % TN], r[n % NBUF], x[n % NBUF], rows(n), cols(n), bias, act_c, res_c);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    using std::integral_constant;
+    using std::bool_constant;
+    switch (ep.act * 2 + (ep.res ? 1 : 0)) {
+    case 1: tail_all(integral_constant<int, 0>{}, bool_constant<true>{}); break;
+    case 2: tail_all(integral_constant<int, 1>{}, bool_constant<false>{}); break;
+    case 3: tail_all(integral_constant<int, 1>{}, bool_constant<true>{}); break;
+    case 4: tail_all(integral_constant<int, 2>{}, bool_constant<false>{}); break;
+    case 5: tail_all(integral_constant<int, 2>{}, bool_constant<true>{}); break;
+    case 6: tail_all(integral_constant<int, 3>{}, bool_constant<false>{}); break;
+    case 7: tail_all(integral_constant<int, 3>{}, bool_constant<true>{}); break;
+    case 8: tail_all(integral_constant<int, 4>{}, bool_constant<false>{}); break;
+    case 9: tail_all(integral_constant<int, 4>{}, bool_constant<true>{}); break;
+    default: tail_all(integral_constant<int, 0>{}, bool_constant<false>{}); break;
     }
 }
 

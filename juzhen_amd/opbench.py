@@ -117,6 +117,18 @@ def bench_gemm(r):
         lda, ldb = (k if ta else m), (n if tb else k)
         r.run("gemm", f"jzhip_gemm {label}", f"{m}x{n}x{k}",
               lambda: jz.gemm(P(A), P(B), P(Cm), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0), flops=2.0 * m * n * k)
+    # products with the layer's elementwise tail fused into the store (C4 shapes)
+    for label, m, n, k, ta, act, use_res in (("C4 Wo: bias+residual NN", 512, 16384, 512, 0, 0, 1),
+                                             ("C4 W2: bias+residual NN", 512, 16384, 2048, 0, 0, 1),
+                                             ("C4 W1: bias+gelu(+pre) NN", 2048, 16384, 512, 0, 2, 0),
+                                             ("C4 dF1: .*gelu'(pre) TN", 2048, 16384, 512, 1, 4, 0)):
+        A, B, Cm = dev(m * k), dev(k * n), dev(m * n, 0)
+        bias, aux, res = dev(m), dev(m * n), dev(m * n)
+        lda = k if ta else m
+        r.run("gemm", f"jzhip_gemm_fused {label}", f"{m}x{n}x{k}",
+              lambda: jz.gemm_fused(P(A), P(B), P(Cm), m, n, k, ta, 0, lda, k, m, 1.0, 0.0,
+                                    P(bias) if act != 4 else None, act, P(aux) if act else None, m,
+                                    P(res) if use_res else None, m), flops=2.0 * m * n * k)
     # attention-shaped strided batches (C4: 512 blocks of 256x256x64)
     S, dk, nb = 256, 64, 512
     Q, K, A_ = dev(S * dk * nb), dev(S * dk * nb), dev(S * S * nb, 0)
