@@ -10,6 +10,7 @@
 #include "common.hpp"
 
 #include <cmath>
+#include <type_traits>
 
 namespace jz {
 int gemm_batched2(const float* A, const float* B, float* C, int m, int n, int k, bool ta, bool tb,
@@ -47,6 +48,18 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // [d][key] (pitch S+1), M2 as [key][d] (pitch DH+4); X1 fragments are read
 // straight from global memory (each lane 32 consecutive floats of its query's
 // column: half-wave h contracts d in [h*DH/2, (h+1)*DH/2)).
+// e^x for x <= 0 through the hardware exp2: x*log2(e) is formed with its
+// rounding error (fma) and the error is folded back in, which keeps the result
+// within about 2 ulp; libm's expf costs an order of magnitude more
+// instructions and made the softmax the longest phase of the kernel.
+__device__ __forceinline__ float exp_neg(float x) {
+    const float l2e = 1.44269504088896341f;
+    x = x > -100.0f ? x : -100.0f;   // masked scores (-1e9) end as an exact +0
+    const float t = x * l2e;
+    const float err = fmaf(x, l2e, -t) + x * 1.92596299112661746e-8f;   // low bits of the product and of log2(e)
+    return __builtin_amdgcn_exp2f(t) * (1.0f + 0.693147180559945309f * err);
+}
+
 constexpr int kMaxKeyTiles = 8;   // S <= 256
 constexpr int kAttnThreads = 512;  // eight waves: one query group each, two per SIMD
 constexpr int kLD1 = 32 * kMaxKeyTiles + 1;   // pitch of the [d][key] staging, whatever S is
@@ -55,7 +68,7 @@ constexpr int kLD1 = 32 * kMaxKeyTiles + 1;   // pitch of the [d][key] staging, 
 // that the accumulator tiles stay in registers without predication).
 template <int DH, bool BWD, int NP>
 __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, float* __restrict__ Ablk,
-                                           float* __restrict__ dSblk, const float* __restrict__ x1, int ld_x1,
+                                           float* __restrict__ dSblk, const float (&xf)[DH / 2],
                                            const float* t1, const float* t2, int S, int G, int g,
                                            int l32, int h, float scale, int causal) {
     constexpr int HD = DH / 2;        // contraction steps of the first product
@@ -67,41 +80,40 @@ __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, 
     // S x S block addressing: wave-uniform key row plus one lane offset
     const unsigned lane_off = static_cast<unsigned>(4 * h) * static_cast<unsigned>(S) + q;
 
-    // this lane's X1 fragments: d = HD*h + kk for kk = 0..HD-1
-    float xf[HD];
-    {
-        const float* src = x1 + static_cast<size_t>(q) * ld_x1 + HD * h;
-#pragma unroll
-        for (int i = 0; i < HD / 4; ++i) {
-            const floatx4 t = *reinterpret_cast<const floatx4*>(src + 4 * i);
-            xf[4 * i] = t.x; xf[4 * i + 1] = t.y; xf[4 * i + 2] = t.z; xf[4 * i + 3] = t.w;
-        }
-    }
-
     // first product, two key tiles at a time
     floatx16 sc[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int v = 0; v < 16; ++v) sc[t][v] = 0.0f;
+    // four key tiles per contraction step where there are that many (four
+    // independent MFMAs cover the latency of the next step's LDS reads), then a
+    // remaining pair
+    auto first_product = [&](auto nt_c, int t0) {
+        constexpr int W = decltype(nt_c)::value;   // tiles handled together
+        const float* base = t1 + 32 * t0;
+        float a[W], n[W];
 #pragma unroll
-    for (int tp = 0; tp < NP; ++tp) {
-        const float* base = t1 + 64 * tp;
-        float a0 = base[0], a1 = base[32];
+        for (int w = 0; w < W; ++w) a[w] = base[32 * w];
 #pragma unroll
         for (int kk = 0; kk < HD; ++kk) {
-            float n0 = 0.f, n1 = 0.f;
             if (kk + 1 < HD) {
-                n0 = base[(kk + 1) * LD1];
-                n1 = base[(kk + 1) * LD1 + 32];
+#pragma unroll
+                for (int w = 0; w < W; ++w) n[w] = base[(kk + 1) * LD1 + 32 * w];
             }
             __builtin_amdgcn_sched_barrier(0);
-            sc[2 * tp] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, xf[kk], sc[2 * tp], 0, 0, 0);
-            sc[2 * tp + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, xf[kk], sc[2 * tp + 1], 0, 0, 0);
+#pragma unroll
+            for (int w = 0; w < W; ++w)
+                sc[t0 + w] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[w], xf[kk], sc[t0 + w], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            a0 = n0; a1 = n1;
+#pragma unroll
+            for (int w = 0; w < W; ++w) a[w] = n[w];
         }
-    }
+    };
+    if constexpr (NT >= 4) first_product(std::integral_constant<int, 4>{}, 0);
+    if constexpr (NT == 8) first_product(std::integral_constant<int, 4>{}, 4);
+    if constexpr (NT == 2) first_product(std::integral_constant<int, 2>{}, 0);
+    if constexpr (NT == 6) first_product(std::integral_constant<int, 2>{}, 4);
 
     // per-query row operation; register v of tile t is key 32t + 8(v/4) + 4h + v%4
     if constexpr (!BWD) {
@@ -126,7 +138,7 @@ __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, 
         for (int t = 0; t < NT; ++t) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float e = expf(sc[t][v] - m);
+                const float e = exp_neg(sc[t][v] - m);
                 sc[t][v] = e;
                 sum += e;
             }
@@ -262,6 +274,26 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
     float* Ablk = Aio + blk_off;
     float* dSblk = BWD ? dS_out + blk_off : nullptr;
 
+    // wave w < 4 takes query group w, wave w >= 4 takes group G-1-(w-4): the two
+    // waves of a SIMD (w, w+4) share the causal triangle evenly
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int l32 = lane & 31, h = lane >> 5;
+    const int G = S / 32;
+    const int g = wave < 4 ? wave : G - 1 - (wave - 4);
+    const bool mine = wave < 4 ? (wave < (G + 1) / 2) : (wave - 4 < G / 2);
+    // this lane's X1 fragments (d = HD*h + kk for kk = 0..HD-1), requested before
+    // the staging so that they arrive behind it
+    float xf[HD];
+    if (mine) {
+        const float* src = x1 + static_cast<size_t>(g * 32 + l32) * ld_x1 + HD * h;
+#pragma unroll
+        for (int i = 0; i < HD / 4; ++i) {
+            const floatx4 t = *reinterpret_cast<const floatx4*>(src + 4 * i);
+            xf[4 * i] = t.x; xf[4 * i + 1] = t.y; xf[4 * i + 2] = t.z; xf[4 * i + 3] = t.w;
+        }
+    }
+
     // stage M1 transposed and M2 as it lies: all global loads of a thread first
     // (they are independent), then the LDS stores
     {
@@ -290,25 +322,17 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
     }
     __syncthreads();
 
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int l32 = lane & 31, h = lane >> 5;
-    const int G = S / 32;
     const float* t1 = T1 + (HD * h) * LD1 + l32;
     const float* t2 = T2 + (4 * h) * LD2 + l32;
 
-    // wave w < 4 takes group w, wave w >= 4 takes group G-1-(w-4): the two waves
-    // of a SIMD (w, w+4) share the causal triangle evenly
     {
-        const int g = wave < 4 ? wave : G - 1 - (wave - 4);
-        const bool mine = wave < 4 ? (wave < (G + 1) / 2) : (wave - 4 < G / 2);
         if (mine) {
             const int nkt = causal ? g + 1 : G;          // key tiles that are not entirely masked
             switch ((nkt + 1) / 2) {
-            case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
-            case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
-            case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
-            default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, x1, ld_x1, t1, t2, S, G, g, l32, h, scale, causal); break;
+            case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
+            case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
+            case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
+            default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
             }
         }
     }

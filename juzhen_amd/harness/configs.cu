@@ -8,7 +8,7 @@
 // and dumped as raw float32 files for element-wise comparison.
 //
 // Selected through the environment (the library owns main(), cpp/launcher.cu):
-//   JZ_CONFIG = c1 | c2 | c3      JZ_STEPS = training steps      JZ_OUT = dump dir
+//   JZ_CONFIG = c1 | c2 | c3 | c5  JZ_STEPS = training steps     JZ_OUT = dump dir
 //   JZ_SCALE  = full | small      (small shrinks batch/width for quick runs)
 #include <chrono>
 #include <cstdio>
@@ -195,6 +195,148 @@ int run_c3(const std::string& out, bool small, int steps) {
     return 0;
 }
 
+// ── C5: rectified-flow conv UNet, CIFAR-10 shape (wiring of
+//    examples/demo_cnn_rectified.cu:210-315 and its step :476-535, with two
+//    conv+ReLU blocks per level and an additive sinusoidal time embedding) ──
+struct UNet {
+    int nb, H, c1, c2, c3;
+    ConvLayer e1a, e1b, e2a, e2b, e3a, e3b, d2a, d2b, d1a, d1b, head;
+    ConvTransLayer up2, up1;
+    Matrix<D> T1, T2, T3, Td2, Td1;                       // time embeddings, one per level
+    Matrix<D> a1, s1, a2, s2, a3, m, cat2, ad2, dd2, cat1, ad1, dd1;
+
+    UNet(int nb_, int H_, int c1_, int c2_, int c3_)
+        : nb(nb_), H(H_), c1(c1_), c2(c2_), c3(c3_),
+          e1a(nb, 3, H, H, c1, 3, 3, 1, 1, true), e1b(nb, c1, H, H, c1, 3, 3, 1, 1, true),
+          e2a(nb, c1, H, H, c2, 3, 3, 1, 2, true), e2b(nb, c2, H / 2, H / 2, c2, 3, 3, 1, 1, true),
+          e3a(nb, c2, H / 2, H / 2, c3, 3, 3, 1, 2, true), e3b(nb, c3, H / 4, H / 4, c3, 3, 3, 1, 1, true),
+          d2a(nb, 2 * c2, H / 2, H / 2, c2, 3, 3, 1, 1, true), d2b(nb, c2, H / 2, H / 2, c2, 3, 3, 1, 1, true),
+          d1a(nb, 2 * c1, H, H, c1, 3, 3, 1, 1, true), d1b(nb, c1, H, H, c1, 3, 3, 1, 1, true),
+          head(nb, c1, H, H, 3, 3, 3, 1, 1, false),
+          up2(nb, c3, H / 4, H / 4, c2, 4, 4, 1, 2, true), up1(nb, c2, H / 2, H / 2, c1, 4, 4, 1, 2, true) {}
+
+    std::vector<Layer<D>*> layers() {
+        return {&e1a, &e1b, &e2a, &e2b, &e3a, &e3b, &up2, &d2a, &d2b, &up1, &d1a, &d1b, &head};
+    }
+
+    // emb(c*P + p, n) = sin(2^(c/2) * pi * t_n) for even c, cos(...) for odd c
+    static Matrix<float> time_embedding(int C, int P, const std::vector<float>& t) {
+        Matrix<float> e("temb", C * P, (int)t.size());
+        for (size_t n = 0; n < t.size(); ++n)
+            for (int c = 0; c < C; ++c) {
+                const float f = std::ldexp(3.14159265358979323846f, (c / 2) % 6);
+                const float v = 0.1f * ((c & 1) ? std::cos(f * t[n]) : std::sin(f * t[n]));
+                for (int p = 0; p < P; ++p) e.elem((size_t)c * P + p, n) = v;
+            }
+        return e;
+    }
+    void set_time(const std::vector<float>& t) {
+        const int P = H * H;
+        T1 = Matrix<D>(time_embedding(c1, P, t));
+        T2 = Matrix<D>(time_embedding(c2, P / 4, t));
+        T3 = Matrix<D>(time_embedding(c3, P / 16, t));
+        Td2 = Matrix<D>(time_embedding(c2, P / 4, t));
+        Td1 = Matrix<D>(time_embedding(c1, P, t));
+    }
+
+    const Matrix<D>& fwd(const Matrix<D>& x) {
+        e1a.eval(x);    a1 = e1a.value() + T1;
+        e1b.eval(a1);   s1 = e1b.value();
+        e2a.eval(s1);   a2 = e2a.value() + T2;
+        e2b.eval(a2);   s2 = e2b.value();
+        e3a.eval(s2);   a3 = e3a.value() + T3;
+        e3b.eval(a3);   m = e3b.value();
+        up2.eval(m);    cat2 = vstack(std::vector<MatrixView<D>>{MatrixView<D>(up2.value()), MatrixView<D>(s2)});
+        d2a.eval(cat2); ad2 = d2a.value() + Td2;
+        d2b.eval(ad2);  dd2 = d2b.value();
+        up1.eval(dd2);  cat1 = vstack(std::vector<MatrixView<D>>{MatrixView<D>(up1.value()), MatrixView<D>(s1)});
+        d1a.eval(cat1); ad1 = d1a.value() + Td1;
+        d1b.eval(ad1);  dd1 = d1b.value();
+        head.eval(dd1);
+        return head.value();
+    }
+    void bwd(const Matrix<D>& x, Matrix<D>&& g) {
+        auto g0 = head.backward(dd1, std::move(g));
+        auto g1 = d1b.backward(ad1, std::move(g0));
+        auto gc1 = d1a.backward(cat1, std::move(g1));
+        const size_t k1 = (size_t)c1 * H * H;
+        auto gu1 = gc1.rows(0, k1);
+        auto gs1 = gc1.rows(k1, gc1.num_row());
+        auto g2 = up1.backward(dd2, std::move(gu1));
+        auto g3 = d2b.backward(ad2, std::move(g2));
+        auto gc2 = d2a.backward(cat2, std::move(g3));
+        const size_t k2 = (size_t)c2 * (H / 2) * (H / 2);
+        auto gu2 = gc2.rows(0, k2);
+        auto gs2 = gc2.rows(k2, gc2.num_row());
+        auto g4 = up2.backward(m, std::move(gu2));
+        auto g5 = e3b.backward(a3, std::move(g4));
+        auto g6 = e3a.backward(s2, std::move(g5));
+        g6 = g6 + gs2;
+        auto g7 = e2b.backward(a2, std::move(g6));
+        auto g8 = e2a.backward(s1, std::move(g7));
+        g8 = g8 + gs1;
+        auto g9 = e1b.backward(a1, std::move(g8));
+        e1a.backward(x, std::move(g9));
+    }
+};
+
+int run_c5(const std::string& out, bool small, int steps) {
+    const int nb = small ? 4 : 128, H = small ? 16 : 32;
+    const int c1 = small ? 8 : 64, c2 = small ? 16 : 128, c3 = small ? 32 : 256;
+    const int d = 3 * H * H;
+    std::mt19937 g(23);
+    UNet net(nb, H, c1, c2, c3);
+    for (Layer<D>* l : net.layers()) {
+        // He-normal over the patch fan-in, zero biases, Adam alpha 2e-4
+        const size_t nw = l->W().num_row() * l->W().num_col();
+        const size_t cout = l->b().num_row();
+        const float sd = std::sqrt(2.0f / (float)(nw / cout));
+        l->W() = Matrix<D>(host_normal((int)l->W().num_row(), (int)l->W().num_col(), g, sd));
+        l->b() = Matrix<D>(Matrix<float>::zeros(cout, 1));
+        l->adamWstate().alpha = 2e-4f;
+        l->adambstate().alpha = 2e-4f;
+    }
+    // one fixed batch: x1 = clip(N(0,1), -1, 1), x0 = N(0,1), t = U[0,1]
+    Matrix<float> x1h = host_normal(d, nb, g, 1.0f);
+    for (size_t i = 0; i < (size_t)d * nb; ++i) {
+        float& v = const_cast<float*>(x1h.data())[i];
+        v = v < -1.f ? -1.f : (v > 1.f ? 1.f : v);
+    }
+    const Matrix<float> x0h = host_normal(d, nb, g, 1.0f);
+    std::vector<float> t(nb);
+    {
+        std::uniform_real_distribution<float> u(0.f, 1.f);
+        for (float& v : t) v = u(g);
+    }
+    // x_t = (1-t) x0 + t x1 and the target velocity x1 - x0, formed on the host
+    Matrix<float> xth("xt", d, nb), vth("vt", d, nb);
+    for (int n = 0; n < nb; ++n)
+        for (int p = 0; p < d; ++p) {
+            xth.elem(p, n) = (1.f - t[n]) * x0h.elem(p, n) + t[n] * x1h.elem(p, n);
+            vth.elem(p, n) = x1h.elem(p, n) - x0h.elem(p, n);
+        }
+    const Matrix<D> xt(xth), vt(vth);
+    net.set_time(t);
+    Matrix<float> losses("losses", 1, steps);
+    double t0 = 0;
+    for (int it = 0; it < steps; ++it) {
+        if (it == 1) t0 = now_ms();
+        const Matrix<D>& pred = net.fwd(xt);
+        if (it == 0) dump(out, "c5_pred0", host(pred));
+        Matrix<D> diff = pred - vt;
+        losses.elem(0, it) = item(sum(sum(square(Matrix<D>(diff)), 0), 1)) / (float)nb;   // demo_cnn_rectified.cu:531-534
+        Matrix<D> grad = 2.0f * diff / (float)nb;
+        net.bwd(xt, std::move(grad));
+    }
+    if (steps > 1) std::printf("RESULT c5_ms_per_step %.4f\n", (now_ms() - t0) / (steps - 1));
+    std::printf("RESULT c5_loss_first %.8g\nRESULT c5_loss_last %.8g\n", losses.elem(0, 0), losses.elem(0, steps - 1));
+    dump(out, "c5_losses", losses);
+    dump(out, "c5_head_W", host(net.head.W()));
+    dump(out, "c5_e1a_W", host(net.e1a.W()));
+    dump(out, "c5_up2_W", host(net.up2.W()));
+    return 0;
+}
+
 }  // namespace
 
 int compute() {
@@ -206,6 +348,7 @@ int compute() {
     if (cfg == "c1") return run_c1(out, small);
     if (cfg == "c2") return run_c2(out, small, steps);
     if (cfg == "c3") return run_c3(out, small, steps);
+    if (cfg == "c5") return run_c5(out, small, steps);
     std::printf("unknown JZ_CONFIG %s\n", cfg.c_str());
     return 1;
 }

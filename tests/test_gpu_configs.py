@@ -1,4 +1,4 @@
-"""Benchmark configurations 1-3 through the drop-in boundary: the same Juzhen
+"""Benchmark configurations 1-3 and 5 through the drop-in boundary: the same Juzhen
 program (juzhen_amd/harness/configs.cu) built against the reference's CPU
 Matrix<float> and against this backend's Matrix<ROCMfloat>, run on identical
 host-generated inputs, compared element-wise.
@@ -91,4 +91,25 @@ def test_c3_cnn_training(gpu, tmp_path, scale, steps):
     assert lc[-1] < lc[0]
     assert worst <= 1e-3
     for name in ("c3_conv1_W", "c3_fc_b"):
+        assert rel(load(tmp_path, name, "rocm"), load(tmp_path, name, "cpu")) <= 2e-3
+
+
+@pytest.mark.parametrize("scale,steps", [("small", 30), ("full", 5)])
+def test_c5_rectified_flow_unet_training(gpu, tmp_path, scale, steps):
+    """Conv / transposed-conv UNet (channels 64/128/256, two conv+ReLU per level,
+    skip connections through vstack/rows, additive sinusoidal time embedding),
+    MSE on the velocity x1 - x0, Adam 2e-4: first prediction and every loss of
+    the run against the reference CPU classes on the same host-generated batch."""
+    res = run_both(tmp_path, "c5", scale, steps)
+    lc, lg = load(tmp_path, "c5_losses", "cpu"), load(tmp_path, "c5_losses", "rocm")
+    assert lc.size == steps and lg.size == steps
+    worst = float(np.max(np.abs(lg - lc) / np.abs(lc)))
+    e0 = rel(load(tmp_path, "c5_pred0", "rocm"), load(tmp_path, "c5_pred0", "cpu"))
+    print(f"c5 {scale}: first prediction rel err {e0:.2e}; loss {lc[0]:.4f} -> {lc[-1]:.4f}, worst rel err over "
+          f"{steps} steps {worst:.2e}; ms/step cpu {res['cpu'].get('c5_ms_per_step')} "
+          f"rocm {res['rocm'].get('c5_ms_per_step')}")
+    assert e0 <= 1e-3
+    assert lc[-1] < lc[0]
+    assert worst <= 1e-3
+    for name in ("c5_head_W", "c5_e1a_W", "c5_up2_W"):
         assert rel(load(tmp_path, name, "rocm"), load(tmp_path, name, "cpu")) <= 2e-3
