@@ -172,6 +172,182 @@ int transpose_batched(float* dst, const float* src, const float* bias, int R, in
     return launch_rc();
 }
 
+// ── row-tiled forms for the layer-sized problems ─────────────────────────
+// The two kernels above are gather-bound: a thread's reads jump by a column
+// (K floats) or a channel plane between neighbours.  The row forms move a
+// strip of the image (or of the patch matrix) through LDS so that both the
+// HBM reads and the HBM writes are contiguous runs.
+constexpr int kPatchChunk = 256;   // k values per workgroup of im2col_rows: one float4 per lane
+
+// One workgroup = one row ph of the patch grid, one sample n, one chunk of 256
+// consecutive k.  The image rows that chunk touches (its channels x kH rows,
+// zero-filled where the window hangs over the border) are staged in LDS; then
+// every wave writes whole 1 KB pieces of patch columns: lane l owns k = k0+4l..k0+4l+3
+// for all pw, so its four LDS offsets are computed once.
+__global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __restrict__ img,
+                                                             float* __restrict__ col, PatchGeom g,
+                                                             int WT, FastDiv dWT, FastDiv dkH) {
+    extern __shared__ float tile[];   // [channels of the chunk][kH][WT]
+    const int KK = g.kH * g.kW;
+    const int k0 = blockIdx.x * kPatchChunk;
+    const int k1 = (k0 + kPatchChunk) < g.K ? (k0 + kPatchChunk) : g.K;
+    const int ph = blockIdx.y, n = blockIdx.z;
+    const int c_lo = fdiv(static_cast<uint32_t>(k0), g.dKK);
+    const int c_hi = fdiv(static_cast<uint32_t>(k1 - 1), g.dKK);
+    const int rows = (c_hi - c_lo + 1) * g.kH;
+    const int h0 = ph * g.stride_h - g.pad_h;
+    const float* src = img + static_cast<size_t>(n) * (g.C * g.H * g.W) + static_cast<size_t>(c_lo) * g.H * g.W;
+    // (eight independent loads in flight per thread, then their LDS stores)
+    constexpr int kBatch = 8;
+    for (int idx0 = threadIdx.x; idx0 < rows * WT; idx0 += kBlock * kBatch) {
+        float v[kBatch];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int idx = idx0 + b * kBlock;
+            v[b] = 0.0f;
+            if (idx < rows * WT) {
+                const uint32_t r = fdiv(static_cast<uint32_t>(idx), dWT);
+                const int w = idx - static_cast<int>(r) * WT;
+                const uint32_t chl = fdiv(r, dkH);
+                const int kh = static_cast<int>(r - chl * g.kH);
+                const int ih = h0 + kh, iw = w - g.pad_w;
+                if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+                    v[b] = src[(static_cast<size_t>(chl) * g.H + ih) * g.W + iw];
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int idx = idx0 + b * kBlock;
+            if (idx < rows * WT) tile[idx] = v[b];
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int kq = k0 + 4 * lane;
+    if (kq >= k1) return;
+    int off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t k = static_cast<uint32_t>(kq + j);
+        const uint32_t ch = fdiv(k, g.dKK);
+        const uint32_t rem = k - ch * KK;
+        const uint32_t kh = fdiv(rem, g.dkW);
+        const uint32_t kw = rem - kh * g.kW;
+        off[j] = static_cast<int>(((ch - c_lo) * g.kH + kh) * WT + kw);
+    }
+    float* dst = col + (static_cast<size_t>(n) * g.P + static_cast<size_t>(ph) * g.Wp) * g.K + kq;
+    for (int pw = wave; pw < g.Wp; pw += kBlock / kWave) {
+        const int w = pw * g.stride_w;
+        const float4 v = make_float4(tile[off[0] + w], tile[off[1] + w], tile[off[2] + w], tile[off[3] + w]);
+        *reinterpret_cast<float4*>(dst + static_cast<size_t>(pw) * g.K) = v;
+    }
+}
+
+// One workgroup = R image rows of CC channels of one sample.  The patch-matrix
+// entries those rows collect (the k range of the CC channels, for every pw of
+// the ph rows involved) are staged in LDS with contiguous reads; the sums are
+// then formed in the CPU's order (kh, kw descending) out of LDS and written as
+// whole image rows.  The pitch is odd so that lanes walking along pw hit
+// distinct banks.
+__global__ __launch_bounds__(kBlock) void col2im_rows_kernel(const float* __restrict__ col,
+                                                             float* __restrict__ img,
+                                                             const float* __restrict__ bias, PatchGeom g,
+                                                             int CC, int R, int pitch, int vec4, FastDiv dL,
+                                                             FastDiv dR, FastDiv dsh, FastDiv dsw) {
+    extern __shared__ float tile[];   // [ph rows][Wp][pitch]
+    const int KK = g.kH * g.kW;
+    // (the launcher picks CC dividing C and R dividing H, so every workgroup is full)
+    const int c0 = blockIdx.x * CC;
+    const int cc = CC;
+    const int ih0 = blockIdx.y * R;
+    const int rcnt = R;
+    const int n = blockIdx.z;
+    // patch rows with ph*stride - pad + kh inside [ih0, ih0 + rcnt)
+    int lo = ih0 + g.pad_h - (g.kH - 1);
+    lo = lo <= 0 ? 0 : (lo + g.stride_h - 1) / g.stride_h;
+    int hi = (ih0 + rcnt - 1 + g.pad_h) / g.stride_h;
+    if (hi > g.Hp - 1) hi = g.Hp - 1;
+    const int NR = hi - lo + 1;   // may be <= 0: nothing to collect
+    const int L = cc * KK;        // contiguous floats per patch column
+    if (NR > 0) {
+        const size_t col0 = static_cast<size_t>(n) * g.P + static_cast<size_t>(lo) * g.Wp;
+        const int ncols = NR * g.Wp;
+        const float* base = col + col0 * g.K + static_cast<size_t>(c0) * KK;
+        // eight independent loads in flight per thread, then their LDS stores;
+        // float4 loads when the runs are 16-byte aligned (L and K multiples of 4)
+        constexpr int kBatch = 8;
+        if (vec4) {
+            const int L4 = L / 4;
+            const int count = ncols * L4;
+            for (int idx0 = threadIdx.x; idx0 < count; idx0 += kBlock * kBatch) {
+                float4 v[kBatch];
+                int dst[kBatch];
+#pragma unroll
+                for (int b = 0; b < kBatch; ++b) {
+                    const int idx = idx0 + b * kBlock;
+                    dst[b] = -1;
+                    if (idx < count) {
+                        const int cidx = static_cast<int>(fdiv(static_cast<uint32_t>(idx), dL));   // dL divides by L/4 here
+                        const int kk = (idx - cidx * L4) * 4;
+                        dst[b] = cidx * pitch + kk;
+                        v[b] = *reinterpret_cast<const float4*>(base + static_cast<size_t>(cidx) * g.K + kk);
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < kBatch; ++b)
+                    if (dst[b] >= 0) {
+                        float* d = tile + dst[b];
+                        d[0] = v[b].x; d[1] = v[b].y; d[2] = v[b].z; d[3] = v[b].w;
+                    }
+            }
+        } else {
+            const int count = ncols * L;
+            for (int idx0 = threadIdx.x; idx0 < count; idx0 += kBlock * kBatch) {
+                float v[kBatch];
+                int dst[kBatch];
+#pragma unroll
+                for (int b = 0; b < kBatch; ++b) {
+                    const int idx = idx0 + b * kBlock;
+                    dst[b] = -1;
+                    if (idx < count) {
+                        const int cidx = static_cast<int>(fdiv(static_cast<uint32_t>(idx), dL));
+                        const int kk = idx - cidx * L;
+                        dst[b] = cidx * pitch + kk;
+                        v[b] = base[static_cast<size_t>(cidx) * g.K + kk];
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < kBatch; ++b)
+                    if (dst[b] >= 0) tile[dst[b]] = v[b];
+            }
+        }
+    }
+    __syncthreads();
+    const int total = cc * rcnt * g.W;
+    for (int idx = threadIdx.x; idx < total; idx += kBlock) {
+        const uint32_t t = fdiv(static_cast<uint32_t>(idx), g.dW);
+        const int iw = idx - static_cast<int>(t) * g.W;
+        const int cl = static_cast<int>(fdiv(t, dR));
+        const int ih = ih0 + (static_cast<int>(t) - cl * rcnt);
+        float val = bias ? bias[c0 + cl] : 0.0f;
+        for (int kh = g.kH - 1; kh >= 0; --kh) {
+            const int hn = ih + g.pad_h - kh;
+            if (hn < 0) continue;
+            const int ph = static_cast<int>(fdiv(static_cast<uint32_t>(hn), dsh));
+            if (ph * g.stride_h != hn || ph >= g.Hp) continue;
+            const float* row = tile + static_cast<size_t>(ph - lo) * g.Wp * pitch + cl * KK + kh * g.kW;
+            for (int kw = g.kW - 1; kw >= 0; --kw) {
+                const int wn = iw + g.pad_w - kw;
+                if (wn < 0) continue;
+                const int pw = static_cast<int>(fdiv(static_cast<uint32_t>(wn), dsw));
+                if (pw * g.stride_w != wn || pw >= g.Wp) continue;
+                val += row[pw * pitch + kw];
+            }
+        }
+        img[static_cast<size_t>(n) * (g.C * g.H * g.W) + (static_cast<size_t>(c0 + cl) * g.H + ih) * g.W + iw] = val;
+    }
+}
+
 bool geom_ok(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int stride_h, int stride_w,
              int Hp, int Wp, int N) {
     return C > 0 && H > 0 && W > 0 && kH > 0 && kW > 0 && pad_h >= 0 && pad_w >= 0 && stride_h > 0 &&
@@ -182,6 +358,16 @@ int gather_patches(const float* img, float* col, const PatchGeom& g) {
     const size_t total = static_cast<size_t>(g.K) * g.P * g.N;
     if (total >= (size_t(1) << 31)) return -1;
     if (static_cast<size_t>(g.C) * g.H * g.W * g.N >= (size_t(1) << 31)) return -1;
+    if (g.K % 4 == 0 && g.K >= 64 && aligned16(col) && g.N <= 65535 && g.Hp <= 65535) {
+        const int WT = (g.Wp - 1) * g.stride_w + g.kW;
+        const int nch_max = kPatchChunk / (g.kH * g.kW) + 2;
+        const size_t lds = static_cast<size_t>(nch_max) * g.kH * WT * sizeof(float);
+        if (lds <= 48 * 1024) {
+            dim3 grid((g.K + kPatchChunk - 1) / kPatchChunk, g.Hp, g.N);
+            im2col_rows_kernel<<<grid, kBlock, lds, stream()>>>(img, col, g, WT, make_fastdiv(WT), make_fastdiv(g.kH));
+            return launch_rc();
+        }
+    }
     if (g.K % 4 == 0 && aligned16(col)) {
         const size_t tv = total / 4;
         im2col_kernel<4><<<grid_cover(tv, kBlock), kBlock, 0, stream()>>>(img, col, g, make_fastdiv(g.K / 4), tv);
@@ -195,6 +381,29 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
     const size_t total = static_cast<size_t>(g.C) * g.H * g.W * g.N;
     if (total >= (size_t(1) << 31)) return -1;
     if (static_cast<size_t>(g.K) * g.P * g.N >= (size_t(1) << 31)) return -1;
+    if (g.N <= 65535 && g.W <= 1024) {
+        // channels and image rows per workgroup: as many as keep the staged strip
+        // under 40 KB (four workgroups per CU), preferring a channel-chunk count
+        // that is a multiple of 8 so that the workgroups sharing patch rows
+        // (same chunk, neighbouring rows) meet in one XCD's L2
+        const int KK = g.kH * g.kW;
+        int R = 4, CC = 8;
+        auto bytes = [&](int cc, int r) {
+            const int nr = (r - 1 + g.kH - 1) / g.stride_h + 1;
+            return static_cast<size_t>(nr) * g.Wp * ((cc * KK) | 1) * sizeof(float);
+        };
+        while (R > 1 && g.H % R != 0) R /= 2;
+        while (CC > 1 && (g.C % CC != 0 || bytes(CC, R) > 40 * 1024)) CC /= 2;
+        while (R > 1 && bytes(CC, R) > 40 * 1024) R /= 2;
+        if (bytes(CC, R) <= 40 * 1024 && g.H / R <= 65535) {
+            dim3 grid(g.C / CC, g.H / R, g.N);
+            const int vec4 = ((CC * KK) % 4 == 0 && g.K % 4 == 0 && aligned16(col)) ? 1 : 0;
+            col2im_rows_kernel<<<grid, kBlock, bytes(CC, R), stream()>>>(
+                col, img, bias, g, CC, R, (CC * KK) | 1, vec4, make_fastdiv(vec4 ? CC * KK / 4 : CC * KK), make_fastdiv(R),
+                make_fastdiv(g.stride_h), make_fastdiv(g.stride_w));
+            return launch_rc();
+        }
+    }
     col2im_kernel<<<grid_cover(total, kBlock), kBlock, 0, stream()>>>(col, img, bias, g, total);
     return launch_rc();
 }

@@ -613,6 +613,13 @@ CONV_CASES = [
     (2, 32, 28, 28, 3, 3, 1, 2),
     (2, 3, 10, 10, 4, 4, 1, 2),
     (2, 5, 7, 9, 3, 2, 1, 3),
+    # layer-sized: the row-tiled kernels (K % 4 == 0, K >= 64), chunk edges inside a channel
+    (2, 64, 32, 32, 3, 3, 1, 1),
+    (3, 128, 16, 16, 3, 3, 1, 2),
+    (2, 36, 13, 11, 3, 3, 1, 1),
+    (2, 20, 9, 10, 5, 5, 2, 2),
+    (1, 16, 8, 8, 2, 2, 0, 1),
+    (2, 256, 8, 8, 3, 3, 1, 1),
 ]
 
 
@@ -675,6 +682,9 @@ CT_CASES = [
     (2, 4, 8, 8, 4, 4, 1, 2),
     (3, 1, 3, 5, 2, 2, 0, 2),
     (2, 2, 4, 4, 3, 3, 1, 3),
+    (2, 64, 16, 16, 4, 4, 1, 2),
+    (2, 128, 8, 8, 4, 4, 1, 2),
+    (3, 12, 7, 5, 3, 3, 1, 2),
 ]
 
 
