@@ -91,6 +91,54 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_long_kernel(float* out, c
     }
 }
 
+// Medium-long columns (1024 < numrow <= 16384): one block per column with the
+// column held in registers (NV4 float4 per thread), so it is still one read
+// and one write per element.
+template <int NV4>
+__global__ __launch_bounds__(kBlock) void softmax_cols_block_kernel(float* out, const float* in,
+                                                                    int numrow, size_t numcol,
+                                                                    size_t ld) {
+    __shared__ float red[kBlock / kWave];
+    for (size_t col = blockIdx.x; col < numcol; col += gridDim.x) {
+        const float* p = in + col * ld;
+        float* q = out + col * ld;
+        float4 x[NV4];
+        float m = -1e30f;
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) {
+            const int r = (threadIdx.x + v * kBlock) * 4;
+            if (r < numrow) {   // numrow % 4 == 0 on this path
+                x[v] = *reinterpret_cast<const float4*>(p + r);
+                const float a = x[v].x > x[v].y ? x[v].x : x[v].y;
+                const float b = x[v].z > x[v].w ? x[v].z : x[v].w;
+                const float c = a > b ? a : b;
+                m = m > c ? m : c;
+            }
+        }
+        m = block_allreduce<kBlock / kWave>(m, MaxOp{}, red, -1e30f);
+        float s = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) {
+            const int r = (threadIdx.x + v * kBlock) * 4;
+            if (r < numrow) {
+                x[v].x = expf(x[v].x - m); x[v].y = expf(x[v].y - m);
+                x[v].z = expf(x[v].z - m); x[v].w = expf(x[v].w - m);
+                s += (x[v].x + x[v].y) + (x[v].z + x[v].w);
+            }
+        }
+        s = block_allreduce<kBlock / kWave>(s, SumOp{}, red, 0.f);
+        const float inv = 1.0f / (s + 1e-12f);
+#pragma unroll
+        for (int v = 0; v < NV4; ++v) {
+            const int r = (threadIdx.x + v * kBlock) * 4;
+            if (r < numrow) {
+                x[v].x *= inv; x[v].y *= inv; x[v].z *= inv; x[v].w *= inv;
+                *reinterpret_cast<float4*>(q + r) = x[v];
+            }
+        }
+    }
+}
+
 // ── distributions along rows (stride ld) ─────────────────────────────────
 // A block owns RPB consecutive rows of one matrix (blockIdx.y selects the
 // matrix of a batch); its 256 threads are RPB row lanes x (256/RPB) column
@@ -217,10 +265,14 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(float* out, co
 }
 
 // Long rows: columns are split into chunks over grid.y.  Pass A leaves one
-// (max, sum) pair per (row, chunk) in the workspace (online softmax inside the
-// chunk); pass B folds the pairs of a row and writes its chunk.  12 bytes per
-// element instead of the 16 of a three-sweep kernel, and rows x chunks
-// workgroups instead of rows/64.
+// (max, sum) pair per (chunk, row) in the workspace (online softmax inside the
+// chunk), a small fold kernel turns them into (max, 1/sum) per row, pass B
+// writes the result: 12 bytes per element instead of the 16 of a three-sweep
+// kernel, and rows x chunks workgroups instead of rows/64.  The column loops
+// are unrolled eight deep so that eight loads are in flight per thread.
+// part layout: [chunk][2][numrow]; rowstat layout: [2][numrow].
+constexpr int kRowUnroll = 8;
+
 __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* part, const float* in,
                                                                       int numrow, int numcol,
                                                                       size_t ld, int chunk_len) {
@@ -232,14 +284,24 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* par
     const int c1 = (c0 + chunk_len) < numcol ? (c0 + chunk_len) : numcol;
     float m = -1e30f, s = 0.f;
     if (row < numrow) {
-        for (int c = c0 + cp; c < c1; c += CP) {
-            const float t = in[static_cast<size_t>(c) * ld + row];
-            if (t > m) {
-                s = s * expf(m - t) + 1.0f;
-                m = t;
-            } else {
-                s += expf(t - m);
+        for (int c = c0 + cp; c < c1; c += CP * kRowUnroll) {
+            float t[kRowUnroll];
+            float tm = -1e30f;
+#pragma unroll
+            for (int u = 0; u < kRowUnroll; ++u) {
+                const int cc = c + u * CP;
+                t[u] = cc < c1 ? in[static_cast<size_t>(cc) * ld + row] : -1e30f;
+                tm = tm > t[u] ? tm : t[u];
             }
+            const float mn = m > tm ? m : tm;
+            float acc = s * expf(m - mn);
+#pragma unroll
+            for (int u = 0; u < kRowUnroll; ++u) {
+                const int cc = c + u * CP;
+                if (cc < c1) acc += expf(t[u] - mn);
+            }
+            s = acc;
+            m = mn;
         }
     }
     redm[cp][rl] = m;
@@ -252,42 +314,126 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* par
         float S = 0.f;
 #pragma unroll
         for (int k = 0; k < CP; ++k) S += reds[k][rl] * expf(redm[k][rl] - M);
-        const size_t o = (static_cast<size_t>(blockIdx.y) * numrow + row) * 2;
+        const size_t o = static_cast<size_t>(blockIdx.y) * 2 * numrow + row;
         part[o] = M;
-        part[o + 1] = S;
+        part[o + numrow] = S;
+    }
+}
+
+// (max, sum) pairs of a row over all chunks -> (max, 1/(sum + 1e-12)).
+// 64 row lanes x 16 chunk phases per block, four pairs in flight per thread.
+constexpr int kFoldThreads = 1024;
+__global__ __launch_bounds__(kFoldThreads) void softmax_rows_fold_kernel(float* rowstat, const float* part,
+                                                                         int numrow, int chunks) {
+    constexpr int RPB = kWave, CP = kFoldThreads / kWave;
+    __shared__ float redm[CP][RPB], reds[CP][RPB];
+    const int rl = threadIdx.x % RPB, cp = threadIdx.x / RPB;
+    const int row = blockIdx.x * RPB + rl;
+    float m = -1e30f, s = 0.f;
+    if (row < numrow) {
+        for (int k = cp; k < chunks; k += CP * 4) {
+            float mk[4], sk[4];
+            float tm = -1e30f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int kk = k + u * CP;
+                const size_t o = static_cast<size_t>(kk) * 2 * numrow + row;
+                mk[u] = kk < chunks ? part[o] : -1e30f;
+                sk[u] = kk < chunks ? part[o + numrow] : 0.f;
+                tm = tm > mk[u] ? tm : mk[u];
+            }
+            const float mn = m > tm ? m : tm;
+            float acc = s * expf(m - mn);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc += sk[u] * expf(mk[u] - mn);
+            s = acc;
+            m = mn;
+        }
+    }
+    redm[cp][rl] = m;
+    reds[cp][rl] = s;
+    __syncthreads();
+    if (cp == 0 && row < numrow) {
+        float M = -1e30f;
+#pragma unroll
+        for (int k = 0; k < CP; ++k) M = M > redm[k][rl] ? M : redm[k][rl];
+        float S = 0.f;
+#pragma unroll
+        for (int k = 0; k < CP; ++k) S += reds[k][rl] * expf(redm[k][rl] - M);
+        rowstat[row] = M;
+        rowstat[numrow + row] = 1.0f / (S + 1e-12f);
     }
 }
 
 __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, const float* in,
-                                                                    const float* part, int numrow,
+                                                                    const float* rowstat, int numrow,
                                                                     int numcol, size_t ld,
-                                                                    int chunk_len, int chunks) {
+                                                                    int chunk_len) {
     constexpr int RPB = kWave, CP = kBlock / kWave;
-    __shared__ float row_m[RPB], row_inv[RPB];
     const int rl = threadIdx.x % RPB, cp = threadIdx.x / RPB;
     const int row = blockIdx.x * RPB + rl;
-    if (cp == 0 && row < numrow) {
-        float M = -1e30f;
-        for (int k = 0; k < chunks; ++k) {
-            const float mk = part[(static_cast<size_t>(k) * numrow + row) * 2];
-            M = M > mk ? M : mk;
-        }
-        float S = 0.f;
-        for (int k = 0; k < chunks; ++k) {
-            const size_t o = (static_cast<size_t>(k) * numrow + row) * 2;
-            S += part[o + 1] * expf(part[o] - M);
-        }
-        row_m[rl] = M;
-        row_inv[rl] = 1.0f / (S + 1e-12f);
-    }
-    __syncthreads();
     if (row >= numrow) return;
-    const float M = row_m[rl], inv = row_inv[rl];
+    const float M = rowstat[row], inv = rowstat[numrow + row];
     const int c0 = blockIdx.y * chunk_len;
     const int c1 = (c0 + chunk_len) < numcol ? (c0 + chunk_len) : numcol;
-    for (int c = c0 + cp; c < c1; c += CP) {
-        const size_t i = static_cast<size_t>(c) * ld + row;
-        out[i] = expf(in[i] - M) * inv;
+    for (int c = c0 + cp; c < c1; c += CP * kRowUnroll) {
+        float t[kRowUnroll];
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int cc = c + u * CP;
+            t[u] = cc < c1 ? in[static_cast<size_t>(cc) * ld + row] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int cc = c + u * CP;
+            if (cc < c1) out[static_cast<size_t>(cc) * ld + row] = expf(t[u] - M) * inv;
+        }
+    }
+}
+
+// Rows of up to 2048 columns held in registers by a 1024-thread block: 16 row
+// lanes x 64 column phases, NV columns per thread.  One read and one write per
+// element with numrow/16 workgroups (the 64-row form above leaves most of the
+// chip idle on a 1024 x 1024 matrix).
+constexpr int kWideThreads = 1024, kWideRows = 16, kWidePhases = kWideThreads / kWideRows;
+template <int NV>
+__global__ __launch_bounds__(kWideThreads) void softmax_rows_wide_kernel(float* out, const float* in,
+                                                                         int numrow, int numcol,
+                                                                         size_t ld) {
+    __shared__ float red[kWidePhases][kWideRows + 1];
+    const int rl = threadIdx.x % kWideRows, cp = threadIdx.x / kWideRows;
+    const int row = blockIdx.x * kWideRows + rl;
+    const bool live = row < numrow;
+    float x[NV];
+    float m = -1e30f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = cp + v * kWidePhases;
+        x[v] = (live && c < numcol) ? in[static_cast<size_t>(c) * ld + row] : -1e30f;
+        m = m > x[v] ? m : x[v];
+    }
+    red[cp][rl] = m;
+    __syncthreads();
+    for (int k = 0; k < kWidePhases; ++k) m = m > red[k][rl] ? m : red[k][rl];
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = cp + v * kWidePhases;
+        x[v] = (live && c < numcol) ? expf(x[v] - m) : 0.f;
+        s += x[v];
+    }
+    red[cp][rl] = s;
+    __syncthreads();
+    s = 0.f;
+    for (int k = 0; k < kWidePhases; ++k) s += red[k][rl];
+    const float inv = 1.0f / (s + 1e-12f);
+    if (live) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int c = cp + v * kWidePhases;
+            if (c < numcol) out[static_cast<size_t>(c) * ld + row] = x[v] * inv;
+        }
     }
 }
 
@@ -449,6 +595,20 @@ int softmax_cols_impl(float* out, const float* in, int numrow, size_t numcol, si
                       ScoreXform xf) {
     if (numrow <= 1024) return dispatch_nv<SoftmaxColsL>(numrow, out, in, numrow, numcol, ld, xf);
     if (xf.S) return -1;
+    if (numrow % 4 == 0 && ld % 4 == 0 && numrow <= 16 * 1024 && aligned16(in) && aligned16(out) &&
+        numcol <= 0x7fffffffull) {
+        const unsigned grid = static_cast<unsigned>(numcol);
+        hipStream_t st = stream();
+        if (numrow <= 2048)
+            softmax_cols_block_kernel<2><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+        else if (numrow <= 4096)
+            softmax_cols_block_kernel<4><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+        else if (numrow <= 8192)
+            softmax_cols_block_kernel<8><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+        else
+            softmax_cols_block_kernel<16><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+        return launch_rc();
+    }
     const unsigned grid = grid_for(numcol, 1, 8);
     softmax_cols_long_kernel<<<grid, kBlock, 0, stream()>>>(out, in, numrow, numcol, ld);
     return launch_rc();
@@ -473,20 +633,34 @@ int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_
         return launch_rc();
     }
     if (batch == 1 && !xf.S) {
+        if (numcol <= 2048 && numrow >= 512) {
+            // medium rows: registers of a 1024-thread block, numrow/16 workgroups
+            const unsigned grid = (numrow + kWideRows - 1) / kWideRows;
+            if (numcol <= 512)
+                softmax_rows_wide_kernel<8><<<grid, kWideThreads, 0, s>>>(out, in, numrow, numcol, ld);
+            else if (numcol <= 1024)
+                softmax_rows_wide_kernel<16><<<grid, kWideThreads, 0, s>>>(out, in, numrow, numcol, ld);
+            else
+                softmax_rows_wide_kernel<32><<<grid, kWideThreads, 0, s>>>(out, in, numrow, numcol, ld);
+            return launch_rc();
+        }
         // long rows: split the columns so that row_blocks x chunks fills the chip
-        int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
+        int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 8 + row_blocks - 1) / row_blocks);
         if (chunks > numcol / 32) chunks = numcol / 32;
         if (chunks < 1) chunks = 1;
-        if (chunks > 4096) chunks = 4096;
-        while (chunks > 1 && static_cast<size_t>(chunks) * numrow * 2 > kWorkspaceFloats) --chunks;
+        if (chunks > 512) chunks = 512;   // the fold walks them once per row
+        auto need = [&](int ch) { return (static_cast<size_t>(ch) + 1) * numrow * 2; };
+        while (chunks > 1 && need(chunks) > kWorkspaceFloats) --chunks;
         const int chunk_len = (numcol + chunks - 1) / chunks;
         chunks = (numcol + chunk_len - 1) / chunk_len;
-        if (static_cast<size_t>(chunks) * numrow * 2 <= kWorkspaceFloats) {
+        if (need(chunks) <= kWorkspaceFloats) {
             float* part = workspace();
             if (!part) return -2;
+            float* rowstat = part + static_cast<size_t>(chunks) * numrow * 2;
             dim3 grid(row_blocks, chunks);
             softmax_rows_partial_kernel<<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
-            softmax_rows_apply_kernel<<<grid, kBlock, 0, s>>>(out, in, part, numrow, numcol, ld, chunk_len, chunks);
+            softmax_rows_fold_kernel<<<row_blocks, kFoldThreads, 0, s>>>(rowstat, part, numrow, chunks);
+            softmax_rows_apply_kernel<<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
             return launch_rc();
         }
     }
