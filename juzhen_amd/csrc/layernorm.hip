@@ -223,20 +223,84 @@ __global__ __launch_bounds__(kBlock) void ln_param_partial_kernel(float* part, c
     }
 }
 
+// float4 form (dim % 4 == 0, aligned operands): a lane owns four rows, a wave
+// 256 rows; each wave walks its columns four at a time, so eight 16-byte loads
+// are in flight per lane.
+__global__ __launch_bounds__(kBlock) void ln_param_partial_vec_kernel(float* part, const float* dy,
+                                                                      const float* xhat, int dim, int N,
+                                                                      int chunk_len) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ float4 red[2][NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = (blockIdx.x * kWave + lane) * 4;
+    const int chunk = blockIdx.y;
+    const int c_begin = chunk * chunk_len;
+    int c_end = c_begin + chunk_len;
+    if (c_end > N) c_end = N;
+    float4 ag = make_float4(0.f, 0.f, 0.f, 0.f), ab = ag;
+    if (row < dim) {
+        for (int c = c_begin + wave; c < c_end; c += NW * 4) {
+            float4 d[4], h[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int cc = c + u * NW;
+                if (cc < c_end) {
+                    const size_t i = static_cast<size_t>(cc) * dim + row;
+                    d[u] = *reinterpret_cast<const float4*>(dy + i);
+                    h[u] = *reinterpret_cast<const float4*>(xhat + i);
+                } else {
+                    d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    h[u] = d[u];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                ag.x += d[u].x * h[u].x; ag.y += d[u].y * h[u].y; ag.z += d[u].z * h[u].z; ag.w += d[u].w * h[u].w;
+                ab.x += d[u].x; ab.y += d[u].y; ab.z += d[u].z; ab.w += d[u].w;
+            }
+        }
+    }
+    red[0][wave][lane] = ag;
+    red[1][wave][lane] = ab;
+    __syncthreads();
+    if (wave == 0 && row < dim) {
+        float4 sg = make_float4(0.f, 0.f, 0.f, 0.f), sb = sg;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float4 a = red[0][w][lane], b = red[1][w][lane];
+            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
+            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+        }
+        *reinterpret_cast<float4*>(part + (static_cast<size_t>(chunk) * 2 + 0) * dim + row) = sg;
+        *reinterpret_cast<float4*>(part + (static_cast<size_t>(chunk) * 2 + 1) * dim + row) = sb;
+    }
+}
+
 // part is [chunk][2*dim]; a block owns 64 of the 2*dim outputs, its waves take
 // interleaved chunks and are combined through LDS.
-__global__ __launch_bounds__(kBlock) void ln_param_combine_kernel(float* dgamma, float* dbeta,
-                                                                  const float* part, int dim,
-                                                                  int chunks) {
-    constexpr int NW = kBlock / kWave;
+constexpr int kCombineThreads = 1024;
+__global__ __launch_bounds__(kCombineThreads) void ln_param_combine_kernel(float* dgamma, float* dbeta,
+                                                                           const float* part, int dim,
+                                                                           int chunks) {
+    constexpr int NW = kCombineThreads / kWave;
     __shared__ float red[NW][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int i = blockIdx.x * kWave + lane;
     const int n = 2 * dim;
     float acc = 0.f;
-    if (i < n)
-        for (int c = wave; c < chunks; c += NW) acc += part[static_cast<size_t>(c) * n + i];
+    if (i < n) {
+        int c = wave;
+        for (; c + 3 * NW < chunks; c += 4 * NW) {   // four loads in flight
+            const float a0 = part[static_cast<size_t>(c) * n + i];
+            const float a1 = part[static_cast<size_t>(c + NW) * n + i];
+            const float a2 = part[static_cast<size_t>(c + 2 * NW) * n + i];
+            const float a3 = part[static_cast<size_t>(c + 3 * NW) * n + i];
+            acc += (a0 + a1) + (a2 + a3);
+        }
+        for (; c < chunks; c += NW) acc += part[static_cast<size_t>(c) * n + i];
+    }
     red[wave][lane] = acc;
     __syncthreads();
     if (wave == 0 && i < n) {
@@ -297,10 +361,11 @@ JZ_API int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma, c
 JZ_API int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,
                                        const float* xhat, int dim, int N) {
     if (dim <= 0 || N <= 0 || !dgamma || !dbeta || !dy || !xhat) return -1;
-    const int row_blocks = (dim + kWave - 1) / kWave;
+    const bool vec = dim % 4 == 0 && aligned16(dy) && aligned16(xhat);
+    const int row_blocks = vec ? (dim / 4 + kWave - 1) / kWave : (dim + kWave - 1) / kWave;
     size_t want = static_cast<size_t>(num_cus()) * 4;
     int chunks = static_cast<int>((want + row_blocks - 1) / row_blocks);
-    if (chunks > N / 16) chunks = N / 16;
+    if (chunks > N / 32) chunks = N / 32;
     if (chunks < 1) chunks = 1;
     if (chunks > 65535) chunks = 65535;
     while (chunks > 1 && static_cast<size_t>(chunks) * 2 * dim > kWorkspaceFloats) --chunks;
@@ -311,7 +376,11 @@ JZ_API int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float*
     if (!part) return -2;
     hipStream_t s = stream();
     dim3 grid(row_blocks, chunks);
-    ln_param_partial_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
-    ln_param_combine_kernel<<<(2 * dim + kWave - 1) / kWave, kBlock, 0, s>>>(dgamma, dbeta, part, dim, chunks);
+    if (vec) {
+        ln_param_partial_vec_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
+    } else {
+        ln_param_partial_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
+    }
+    ln_param_combine_kernel<<<(2 * dim + kWave - 1) / kWave, kCombineThreads, 0, s>>>(dgamma, dbeta, part, dim, chunks);
     return launch_rc();
 }

@@ -219,7 +219,21 @@ __global__ __launch_bounds__(kBlock) void max_cols_kernel(float* out_val, int32_
             best = p[lane];
             bidx = lane;
         }
-        for (int r = lane + kWave; r < numrow; r += kWave) {
+        int r = lane + kWave;
+        // eight loads in flight per lane, visited in row order
+        for (; r + 7 * kWave < numrow; r += 8 * kWave) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = p[r + u * kWave];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (best < v[u]) {
+                    best = v[u];
+                    bidx = r + u * kWave;
+                }
+            }
+        }
+        for (; r < numrow; r += kWave) {
             const float v = p[r];
             if (best < v) {
                 best = v;
