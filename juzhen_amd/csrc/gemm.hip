@@ -241,10 +241,19 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kerne
     // Tile rasterisation.  Workgroups are dealt round-robin to the 8 XCDs, so
     // ids congruent mod 8 share an L2; give each XCD a contiguous run of the
     // tile order, and walk that order in column panels of 8 tile-rows so a
-    // panel's A rows and B columns stay L2-resident.
+    // panel's A rows and B columns stay L2-resident.  With split-K the K chunk
+    // is the fastest-varying part of the workgroup id instead: an XCD then
+    // works on one chunk of K for all tiles, so each operand panel of that
+    // chunk is fetched into one L2 only.
     const int ntiles = tiles_m * tiles_n;
+    const int splits = gridDim.y;          // (y carries only the count; see below)
     int pid = blockIdx.x;
-    {
+    int chunk = 0;
+    if (splits > 1) {
+        const int lin = blockIdx.x + blockIdx.y * gridDim.x;   // dispatch order
+        chunk = lin % splits;
+        pid = lin / splits;
+    } else {
         constexpr int kXcd = 8;
         const int per = ntiles / kXcd;
         const int rem = ntiles % kXcd;
@@ -269,10 +278,10 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kerne
     A += b_in * strideA + b_out * strideA2;
     B += b_in * strideB + b_out * strideB2;
     C += b_in * strideC + b_out * strideC2;
-    // split-K: blockIdx.y owns K range [k_lo, k_hi) and its own partial C
-    const int k_lo = blockIdx.y * k_chunk;
+    // split-K: a chunk owns K range [k_lo, k_hi) and its own partial C
+    const int k_lo = chunk * k_chunk;
     const int k_hi = (k_lo + k_chunk) < K ? (k_lo + k_chunk) : K;
-    C += blockIdx.y * split_stride;
+    C += chunk * split_stride;
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
