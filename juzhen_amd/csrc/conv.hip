@@ -158,8 +158,55 @@ __global__ __launch_bounds__(kT * 8) void transpose_batched_kernel(float* dst, c
     }
 }
 
+// float4 form (R, C multiples of 4, aligned buffers): 64x64 tiles, 256 threads
+constexpr int kTV = 64;
+__global__ __launch_bounds__(kBlock) void transpose_batched_vec_kernel(float* dst, const float* src,
+                                                                       const float* bias, int R, int C,
+                                                                       unsigned tiles_r) {
+    __shared__ float tile[kTV][kTV + 1];
+    const size_t boff = static_cast<size_t>(blockIdx.y) * R * C;
+    const int r0 = static_cast<int>(blockIdx.x % tiles_r) * kTV;
+    const int c0 = static_cast<int>(blockIdx.x / tiles_r) * kTV;
+    const int q = threadIdx.x % 16, l = threadIdx.x / 16;
+#pragma unroll
+    for (int k = 0; k < kTV; k += 16) {
+        const int r = r0 + 4 * q, c = c0 + l + k;
+        if (r < R && c < C) {
+            const float4 v = *reinterpret_cast<const float4*>(src + boff + static_cast<size_t>(c) * R + r);
+            float* d = &tile[l + k][4 * q];   // tile[c][r]
+            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kTV; k += 16) {
+        const int c = c0 + 4 * q, r = r0 + l + k;
+        if (r < R && c < C) {
+            float4 v = make_float4(tile[4 * q][l + k], tile[4 * q + 1][l + k], tile[4 * q + 2][l + k],
+                                   tile[4 * q + 3][l + k]);
+            if (bias) {
+                const float bb = bias[r];
+                v.x = v.x + bb; v.y = v.y + bb; v.z = v.z + bb; v.w = v.w + bb;
+            }
+            *reinterpret_cast<float4*>(dst + boff + static_cast<size_t>(r) * C + c) = v;
+        }
+    }
+}
+
 int transpose_batched(float* dst, const float* src, const float* bias, int R, int C, int batch) {
     if (R <= 0 || C <= 0 || batch <= 0 || !dst || !src) return -1;
+    const bool vec = R % 4 == 0 && C % 4 == 0 && aligned16(dst) && aligned16(src);
+    if (vec) {
+        const unsigned tr = (R + kTV - 1) / kTV, tc = (C + kTV - 1) / kTV;
+        int done = 0;
+        while (done < batch) {
+            const int nb = (batch - done) < 65535 ? (batch - done) : 65535;
+            const size_t off = static_cast<size_t>(done) * R * C;
+            transpose_batched_vec_kernel<<<dim3(tr * tc, nb), kBlock, 0, stream()>>>(dst + off, src + off, bias, R, C, tr);
+            done += nb;
+        }
+        return launch_rc();
+    }
     const unsigned tiles_r = (R + kT - 1) / kT, tiles_c = (C + kT - 1) / kT;
     int done = 0;
     while (done < batch) {

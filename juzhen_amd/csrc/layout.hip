@@ -64,10 +64,75 @@ __global__ __launch_bounds__(kTile* kRowsPerPass) void ew2d_kernel(
     }
 }
 
+// float4 form of the kernel above for 16-byte aligned operands whose extents and
+// leading dimensions are multiples of 4: 64x64 tiles, every global access a
+// float4, relatively transposed operands turned in LDS (pitch 65).
+constexpr int kTileV = 64;
+template <int OP>
+__global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
+    float* out, size_t ldo, const float* a, size_t lda, int rel_a, const float* b, size_t ldb,
+    int rel_b, size_t R, size_t C, unsigned tiles_r, float s1, float s2) {
+    __shared__ float ta[kTileV][kTileV + 1];
+    __shared__ float tb[OP == kOpCopy ? 1 : kTileV][kTileV + 1];
+    const unsigned tile = blockIdx.x;
+    const size_t r0 = static_cast<size_t>(tile % tiles_r) * kTileV;
+    const size_t c0 = static_cast<size_t>(tile / tiles_r) * kTileV;
+    const int q = threadIdx.x % 16;    // float4 slot along the contiguous index
+    const int l = threadIdx.x / 16;    // line inside a pass of 16
+    auto stage = [&](float (*t)[kTileV + 1], const float* x, size_t ldx) {
+#pragma unroll
+        for (int k = 0; k < kTileV; k += 16) {
+            const size_t r = r0 + l + k, c = c0 + 4 * q;
+            if (r < R && c < C) {
+                const float4 v = *reinterpret_cast<const float4*>(x + r * ldx + c);
+                float* d = &t[l + k][4 * q];
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            }
+        }
+    };
+    if (rel_a) stage(ta, a, lda);
+    if constexpr (OP != kOpCopy) {
+        if (rel_b) stage(tb, b, ldb);
+    }
+    if (rel_a || (OP != kOpCopy && rel_b)) __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kTileV; k += 16) {
+        const int cl = l + k;
+        const size_t r = r0 + 4 * q, c = c0 + cl;
+        if (r < R && c < C) {
+            float4 va;
+            if (rel_a) va = make_float4(ta[4 * q][cl], ta[4 * q + 1][cl], ta[4 * q + 2][cl], ta[4 * q + 3][cl]);
+            else va = *reinterpret_cast<const float4*>(a + c * lda + r);
+            float4 res = va;
+            if constexpr (OP != kOpCopy) {
+                float4 vb;
+                if (rel_b) vb = make_float4(tb[4 * q][cl], tb[4 * q + 1][cl], tb[4 * q + 2][cl], tb[4 * q + 3][cl]);
+                else vb = *reinterpret_cast<const float4*>(b + c * ldb + r);
+                if constexpr (OP == kOpAxpby) {
+                    res.x = s1 * va.x + s2 * vb.x; res.y = s1 * va.y + s2 * vb.y;
+                    res.z = s1 * va.z + s2 * vb.z; res.w = s1 * va.w + s2 * vb.w;
+                } else {
+                    res.x = va.x * vb.x; res.y = va.y * vb.y; res.z = va.z * vb.z; res.w = va.w * vb.w;
+                }
+            }
+            *reinterpret_cast<float4*>(out + c * ldo + r) = res;
+        }
+    }
+}
+
 template <int OP>
 int launch2d(float* out, size_t ldo, const float* a, size_t lda, int rel_a, const float* b,
              size_t ldb, int rel_b, size_t R, size_t C, float s1, float s2) {
     if (R == 0 || C == 0) return 0;
+    const bool vec = R % 4 == 0 && C % 4 == 0 && ldo % 4 == 0 && lda % 4 == 0 && aligned16(out) && aligned16(a) &&
+                     (OP == kOpCopy || (ldb % 4 == 0 && aligned16(b)));
+    if (vec) {
+        const size_t tr = (R + kTileV - 1) / kTileV, tc = (C + kTileV - 1) / kTileV;
+        if (tr * tc > 0x7fffffffull) return -1;
+        ew2d_vec_kernel<OP><<<static_cast<unsigned>(tr * tc), kBlock, 0, stream()>>>(
+            out, ldo, a, lda, rel_a, b, ldb, rel_b, R, C, static_cast<unsigned>(tr), s1, s2);
+        return launch_rc();
+    }
     const size_t tiles_r = (R + kTile - 1) / kTile;
     const size_t tiles_c = (C + kTile - 1) / kTile;
     if (tiles_r * tiles_c > 0x7fffffffull) return -1;
