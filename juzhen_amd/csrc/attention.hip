@@ -36,18 +36,18 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 //
 // Both passes are "scores-like product, per-query row operation, second
 // product": X1 (Q or dH) x M1 (K or V) gives a (keys x queries) matrix whose
-// 32x32 MFMA tiles keep the query along the lanes and the keys along the
+// 16x16 MFMA tiles keep the query along the lanes and the keys along the
 // accumulator registers, so the softmax (or its backward) is an in-register
-// reduction plus one exchange between the two half-waves, and the second
+// reduction plus two exchanges between the four lane groups, and the second
 // product takes its B operand (P or dS) straight from those registers: the
 // S x S matrix never goes through LDS and is written to HBM once.
 //
-// A wave owns 32 queries at a time (all their keys: up to 8 tiles = 128
-// accumulator registers), two such groups per wave, paired (g, G-1-g) so the
-// causal triangle gives every wave the same work.  M1 is staged in LDS as
-// [d][key] (pitch S+1), M2 as [key][d] (pitch DH+4); X1 fragments are read
-// straight from global memory (each lane 32 consecutive floats of its query's
-// column: half-wave h contracts d in [h*DH/2, (h+1)*DH/2)).
+// A wave owns 16 queries (all their keys: up to 16 tiles = 64 accumulator
+// registers); sixteen waves cover S = 256, four per SIMD, assigned so that the
+// causal triangle gives every SIMD the same work.  M1 is staged in LDS as
+// [d][key], M2 as [key][d] (pitch DH+4); X1 fragments are read straight from
+// global memory (each lane DH/4 consecutive floats of its query's column: lane
+// group kq contracts d in [kq*DH/4, (kq+1)*DH/4)).
 // e^x for x <= 0 through the hardware exp2: x*log2(e) is formed with its
 // rounding error (fma) and the error is folded back in, which keeps the result
 // within about 2 ulp; libm's expf costs an order of magnitude more
@@ -60,208 +60,213 @@ __device__ __forceinline__ float exp_neg(float x) {
     return __builtin_amdgcn_exp2f(t) * (1.0f + 0.693147180559945309f * err);
 }
 
-constexpr int kMaxKeyTiles = 8;   // S <= 256
-constexpr int kAttnThreads = 512;  // eight waves: one query group each, two per SIMD
-constexpr int kLD1 = 32 * kMaxKeyTiles + 1;   // pitch of the [d][key] staging, whatever S is
+constexpr int kMaxKeys = 256;      // S <= 256
+constexpr int kAttnThreads = 1024;  // sixteen waves, one group of 16 queries each, four per SIMD
+// pitch of the [d][key] staging, whatever S is: the four lane groups of a
+// fragment read rows DH/4 apart, which this pitch puts 16 banks apart, and the
+// transposing staging stores stay conflict-free
+template <int DH> constexpr int kLD1 = DH == 64 ? kMaxKeys + 1 : kMaxKeys + 2;
 
-// One group of 32 queries against its first 2*NP key tiles (NP compile-time so
-// that the accumulator tiles stay in registers without predication).
-template <int DH, bool BWD, int NP>
+// One group of 16 queries against its first 4*NQ tiles of 16 keys (NQ
+// compile-time so that the accumulator tiles stay in registers without
+// predication); nkt <= 4*NQ tiles take part, the others are entirely masked.
+// Lane (l16, kq): query 16g + l16; register v of score tile t is key
+// 16t + 4kq + v (v_mfma_f32_16x16x4_f32 accumulator layout), so the softmax is
+// an in-lane reduction plus two exchanges between the four lane groups, and
+// step s of the second product contracts exactly the keys held in register s.
+template <int DH, bool BWD, int NQ>
 __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, float* __restrict__ Ablk,
-                                           float* __restrict__ dSblk, const float (&xf)[DH / 2],
-                                           const float* t1, const float* t2, int S, int G, int g,
-                                           int l32, int h, float scale, int causal) {
-    constexpr int HD = DH / 2;        // contraction steps of the first product
-    constexpr int NDT = DH / 32;      // 32-row tiles of the second product's output
+                                           float* __restrict__ dSblk, const float (&xf)[DH / 4],
+                                           const float* t1, const float* t2, int S, int nkt, int g,
+                                           int l16, int kq, float scale, int causal) {
+    constexpr int HD4 = DH / 4;       // contraction steps of the first product
+    constexpr int NDT = DH / 16;      // 16-row tiles of the second product's output
     constexpr int LD2 = DH + 4;
-    constexpr int NT = 2 * NP;
-    constexpr int LD1 = kLD1;
-    const int q = g * 32 + l32;       // query index inside the block
+    constexpr int NT = 4 * NQ;
+    constexpr int LD1 = kLD1<DH>;
+    const int q = g * 16 + l16;       // query index inside the block
     // S x S block addressing: wave-uniform key row plus one lane offset
-    const unsigned lane_off = static_cast<unsigned>(4 * h) * static_cast<unsigned>(S) + q;
+    const unsigned lane_off = static_cast<unsigned>(4 * kq) * static_cast<unsigned>(S) + q;
 
-    // first product, two key tiles at a time
-    floatx16 sc[NT];
+    // first product, four key tiles per contraction step (four independent MFMAs
+    // cover the latency of the next step's LDS reads)
+    floatx4 sc[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) sc[t][v] = 0.0f;
-    // four key tiles per contraction step where there are that many (four
-    // independent MFMAs cover the latency of the next step's LDS reads), then a
-    // remaining pair
-    auto first_product = [&](auto nt_c, int t0) {
-        constexpr int W = decltype(nt_c)::value;   // tiles handled together
-        const float* base = t1 + 32 * t0;
-        float a[W], n[W];
+        for (int v = 0; v < 4; ++v) sc[t][v] = 0.0f;
 #pragma unroll
-        for (int w = 0; w < W; ++w) a[w] = base[32 * w];
+    for (int tq = 0; tq < NQ; ++tq) {
+        const float* base = t1 + 64 * tq;
+        float a[4], n[4];
 #pragma unroll
-        for (int kk = 0; kk < HD; ++kk) {
-            if (kk + 1 < HD) {
+        for (int w = 0; w < 4; ++w) a[w] = base[16 * w];
 #pragma unroll
-                for (int w = 0; w < W; ++w) n[w] = base[(kk + 1) * LD1 + 32 * w];
+        for (int kk = 0; kk < HD4; ++kk) {
+            if (kk + 1 < HD4) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) n[w] = base[(kk + 1) * LD1 + 16 * w];
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int w = 0; w < W; ++w)
-                sc[t0 + w] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[w], xf[kk], sc[t0 + w], 0, 0, 0);
+            for (int w = 0; w < 4; ++w)
+                sc[4 * tq + w] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[w], xf[kk], sc[4 * tq + w], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int w = 0; w < W; ++w) a[w] = n[w];
+            for (int w = 0; w < 4; ++w) a[w] = n[w];
         }
-    };
-    if constexpr (NT >= 4) first_product(std::integral_constant<int, 4>{}, 0);
-    if constexpr (NT == 8) first_product(std::integral_constant<int, 4>{}, 4);
-    if constexpr (NT == 2) first_product(std::integral_constant<int, 2>{}, 0);
-    if constexpr (NT == 6) first_product(std::integral_constant<int, 2>{}, 4);
+    }
 
-    // per-query row operation; register v of tile t is key 32t + 8(v/4) + 4h + v%4
+    // per-query row operation over the nkt tiles that are not entirely masked
     if constexpr (!BWD) {
         float m = -1e30f;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
+            if (t < nkt) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int key = 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
-                float x = sc[t][v] * scale;
-                if ((causal && key > q) || key >= S) x = -1e9f;   // ml/layer.hpp:2979-2994; tile past S
-                sc[t][v] = x;
-                m = m > x ? m : x;
+                for (int v = 0; v < 4; ++v) {
+                    const int key = 16 * t + 4 * kq + v;
+                    float x = sc[t][v] * scale;
+                    if (causal && key > q) x = -1e9f;   // ml/layer.hpp:2979-2994
+                    sc[t][v] = x;
+                    m = m > x ? m : x;
+                }
             }
         }
         {
-            const float o = __shfl_xor(m, 32);
+            float o = __shfl_xor(m, 16);
+            m = m > o ? m : o;
+            o = __shfl_xor(m, 32);
             m = m > o ? m : o;
         }
         float sum = 0.f;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
+            if (t < nkt) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float e = exp_neg(sc[t][v] - m);
-                sc[t][v] = e;
-                sum += e;
+                for (int v = 0; v < 4; ++v) {
+                    const float e = exp_neg(sc[t][v] - m);
+                    sc[t][v] = e;
+                    sum += e;
+                }
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
+        sum += __shfl_xor(sum, 16);
         sum += __shfl_xor(sum, 32);
         const float inv = 1.0f / (sum + 1e-12f);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
+            if (t < nkt) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int key = 32 * t + 8 * (v / 4) + 4 * h + (v % 4);
-                const float pv = sc[t][v] * inv;
-                sc[t][v] = pv;
-                const int ku = 32 * t + 8 * (v / 4) + (v % 4);
-                if (32 * t < S) (Ablk + static_cast<size_t>(ku) * S)[lane_off] = pv;
+                for (int v = 0; v < 4; ++v) {
+                    const float pv = sc[t][v] * inv;
+                    sc[t][v] = pv;
+                    (Ablk + static_cast<size_t>(16 * t + v) * S)[lane_off] = pv;
+                }
             }
         }
     } else {
-        // P is read twice (dot product, then dS) instead of being held in 16*NT more
-        // registers; the second wave of the SIMD covers the latency.  S is a
-        // multiple of 32, so a tile lies entirely inside or outside the block.
+        // P is read twice (dot product, then dS) instead of being held in 4*NT more
+        // registers; the other waves of the SIMD cover the latency.
         float dot = 0.f;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if (32 * t < S) {
-                float pv[16];
+        for (int tq = 0; tq < NQ; ++tq) {
+            float pv[16];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int ku = 32 * t + 8 * (v / 4) + (v % 4);
-                    pv[v] = (Ablk + static_cast<size_t>(ku) * S)[lane_off];
+            for (int w = 0; w < 4; ++w)
+                if (4 * tq + w < nkt) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        pv[4 * w + v] = (Ablk + static_cast<size_t>(16 * (4 * tq + w) + v) * S)[lane_off];
                 }
 #pragma unroll
-                for (int v = 0; v < 16; ++v) dot += pv[v] * sc[t][v];
-            }
+            for (int w = 0; w < 4; ++w)
+                if (4 * tq + w < nkt) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) dot += pv[4 * w + v] * sc[4 * tq + w][v];
+                }
         }
+        dot += __shfl_xor(dot, 16);
         dot += __shfl_xor(dot, 32);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if (32 * t < S) {
-                float pv[16];
+        for (int tq = 0; tq < NQ; ++tq) {
+            float pv[16];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int ku = 32 * t + 8 * (v / 4) + (v % 4);
-                    pv[v] = (Ablk + static_cast<size_t>(ku) * S)[lane_off];
+            for (int w = 0; w < 4; ++w)
+                if (4 * tq + w < nkt) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        pv[4 * w + v] = (Ablk + static_cast<size_t>(16 * (4 * tq + w) + v) * S)[lane_off];
                 }
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int ku = 32 * t + 8 * (v / 4) + (v % 4);
-                    const float ds = (pv[v] * (sc[t][v] - dot)) * scale;
-                    sc[t][v] = ds;
-                    (dSblk + static_cast<size_t>(ku) * S)[lane_off] = ds;
-                }
-            } else {
+            for (int w = 0; w < 4; ++w) {
+                const int t = 4 * tq + w;
+                if (t < nkt) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) sc[t][v] = 0.0f;
+                    for (int v = 0; v < 4; ++v) {
+                        const float ds = (pv[4 * w + v] * (sc[t][v] - dot)) * scale;
+                        sc[t][v] = ds;
+                        (dSblk + static_cast<size_t>(16 * t + v) * S)[lane_off] = ds;
+                    }
+                }
             }
         }
     }
     // key tiles past the causal range hold exact zeros
-    for (int t = NT; t < G; ++t)
+    for (int t = nkt; t < S / 16; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int ku = 32 * t + 8 * (v / 4) + (v % 4);
-            ((BWD ? dSblk : Ablk) + static_cast<size_t>(ku) * S)[lane_off] = 0.0f;
-        }
+        for (int v = 0; v < 4; ++v) ((BWD ? dSblk : Ablk) + static_cast<size_t>(16 * t + v) * S)[lane_off] = 0.0f;
 
-    // second product: Out[d][query] = sum_key M2[d][key] * sc[key][query]
-    floatx16 oacc[NDT];
+    // second product: Out[d][query] = sum_key M2[d][key] * sc[key][query]; the
+    // skipped tiles are a suffix, so the fragment prefetch can run ahead freely
+    floatx4 oacc[NDT];
 #pragma unroll
     for (int u = 0; u < NDT; ++u)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[u][v] = 0.0f;
+        for (int v = 0; v < 4; ++v) oacc[u][v] = 0.0f;
+    float an[NDT];
+#pragma unroll
+    for (int u = 0; u < NDT; ++u) an[u] = t2[16 * u];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        if (32 * t < S) {   // (an odd tile count leaves one all-zero tile in the last pair)
-            float an[NDT];
+        if (t < nkt) {
 #pragma unroll
-            for (int u = 0; u < NDT; ++u) an[u] = t2[(32 * t) * LD2 + 32 * u];
-#pragma unroll
-            for (int s = 0; s < 16; ++s) {
+            for (int s = 0; s < 4; ++s) {
                 float ac[NDT];
 #pragma unroll
                 for (int u = 0; u < NDT; ++u) ac[u] = an[u];
-                if (s + 1 < 16) {
-                    const int keyn = 32 * t + 8 * ((s + 1) / 4) + ((s + 1) % 4);   // + 4h is in t2
+                if (4 * t + s + 1 < 4 * NT) {
+                    const int keyn = s + 1 < 4 ? 16 * t + s + 1 : 16 * (t + 1);   // + 4kq is in t2
 #pragma unroll
-                    for (int u = 0; u < NDT; ++u) an[u] = t2[keyn * LD2 + 32 * u];
+                    for (int u = 0; u < NDT; ++u) an[u] = t2[keyn * LD2 + 16 * u];
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int u = 0; u < NDT; ++u)
-                    oacc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(ac[u], sc[t][s], oacc[u], 0, 0, 0);
+                    oacc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(ac[u], sc[t][s], oacc[u], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
-    // Out(d, query): register v of tile u is d = 32u + 8(v/4) + 4h + v%4
-    float* dst = out + static_cast<size_t>(q) * ld_out + 4 * h;
+    // Out(d, query): register v of tile u is d = 16u + 4kq + v
+    float* dst = out + static_cast<size_t>(q) * ld_out + 4 * kq;
 #pragma unroll
-    for (int u = 0; u < NDT; ++u)
-#pragma unroll
-        for (int v4 = 0; v4 < 4; ++v4) {
-            floatx4 o = {oacc[u][4 * v4], oacc[u][4 * v4 + 1], oacc[u][4 * v4 + 2], oacc[u][4 * v4 + 3]};
-            *reinterpret_cast<floatx4*>(dst + 32 * u + 8 * v4) = o;
-        }
+    for (int u = 0; u < NDT; ++u) *reinterpret_cast<floatx4*>(dst + 16 * u) = oacc[u];
 }
 
 template <int DH, bool BWD>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
+__global__ __launch_bounds__(kAttnThreads) void attn_core_kernel(
     float* __restrict__ Out, int ld_out, float* __restrict__ Aio, float* __restrict__ dS_out,
     const float* __restrict__ X1, int ld_x1, const float* __restrict__ M1, const float* __restrict__ M2,
     int ld_m, int heads, int S, int B, float scale, int causal) {
-    constexpr int HD = DH / 2;
+    constexpr int HD4 = DH / 4;
     constexpr int LD2 = DH + 4;
+    constexpr int LD1 = kLD1<DH>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    constexpr int LD1 = kLD1;
-    // LDS rows past S (the second tile of an odd last pair) are read but only
-    // multiply masked or zero entries; the buffers are sized for an even tile count.
-    const int S2 = (S + 63) / 64 * 64;
-    float* T1 = lds;                                    // [DH][LD1], LD1 >= S2 + 1 ...
-    (void)S2;
-    float* T2 = lds + ((DH * LD1 + 64 + 3) / 4) * 4;    // [S2][LD2]
+    // LDS columns / rows past S (up to the next multiple of 64) are read by the
+    // tiles that complete a group of four but never enter a result.
+    float* T1 = lds;                                    // [DH][LD1]
+    float* T2 = lds + ((DH * LD1 + 3) / 4) * 4;         // [S rounded up to 64][LD2]
 
     const int blk = blockIdx.x;            // hh*B + b
     const int hh = blk / B, b = blk % B;
@@ -274,21 +279,22 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
     float* Ablk = Aio + blk_off;
     float* dSblk = BWD ? dS_out + blk_off : nullptr;
 
-    // wave w < 4 takes query group w, wave w >= 4 takes group G-1-(w-4): the two
-    // waves of a SIMD (w, w+4) share the causal triangle evenly
+    // the four waves of a SIMD (w, w+4, w+8, w+12) take query groups s, 7-s,
+    // 8+s, 15-s: with the causal triangle every SIMD gets the same work
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int l32 = lane & 31, h = lane >> 5;
-    const int G = S / 32;
-    const int g = wave < 4 ? wave : G - 1 - (wave - 4);
-    const bool mine = wave < 4 ? (wave < (G + 1) / 2) : (wave - 4 < G / 2);
-    // this lane's X1 fragments (d = HD*h + kk for kk = 0..HD-1), requested before
-    // the staging so that they arrive behind it
-    float xf[HD];
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int GQ = S / 16;
+    const int ws = wave & 3, wj = wave >> 2;
+    const int g = wj == 0 ? ws : wj == 1 ? 7 - ws : wj == 2 ? 8 + ws : 15 - ws;
+    const bool mine = g < GQ;
+    // this lane's X1 fragments (d = HD4*kq + kk for kk = 0..HD4-1), requested
+    // before the staging so that they arrive behind it
+    float xf[HD4];
     if (mine) {
-        const float* src = x1 + static_cast<size_t>(g * 32 + l32) * ld_x1 + HD * h;
+        const float* src = x1 + static_cast<size_t>(g * 16 + l16) * ld_x1 + HD4 * kq;
 #pragma unroll
-        for (int i = 0; i < HD / 4; ++i) {
+        for (int i = 0; i < HD4 / 4; ++i) {
             const floatx4 t = *reinterpret_cast<const floatx4*>(src + 4 * i);
             xf[4 * i] = t.x; xf[4 * i + 1] = t.y; xf[4 * i + 2] = t.z; xf[4 * i + 3] = t.w;
         }
@@ -297,7 +303,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
     // stage M1 transposed and M2 as it lies: all global loads of a thread first
     // (they are independent), then the LDS stores
     {
-        constexpr int kIters = (DH / 4) * 32 * kMaxKeyTiles / kAttnThreads;
+        constexpr int kIters = (DH / 4) * kMaxKeys / kAttnThreads;
         const int total = (DH / 4) * S;
         floatx4 ra[kIters], rc[kIters];
 #pragma unroll
@@ -322,25 +328,24 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_core_kernel(
     }
     __syncthreads();
 
-    const float* t1 = T1 + (HD * h) * LD1 + l32;
-    const float* t2 = T2 + (4 * h) * LD2 + l32;
+    const float* t1 = T1 + (HD4 * kq) * LD1 + l16;
+    const float* t2 = T2 + (4 * kq) * LD2 + l16;
 
-    {
-        if (mine) {
-            const int nkt = causal ? g + 1 : G;          // key tiles that are not entirely masked
-            switch ((nkt + 1) / 2) {
-            case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
-            case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
-            case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
-            default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, G, g, l32, h, scale, causal); break;
-            }
+    if (mine) {
+        const int nkt = causal ? g + 1 : GQ;          // key tiles that are not entirely masked
+        switch ((nkt + 3) / 4) {
+        case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
         }
     }
 }
 
 size_t attn_core_lds_bytes(int d_h, int S) {
     const size_t S2 = static_cast<size_t>(S + 63) / 64 * 64;
-    return (static_cast<size_t>((d_h * kLD1 + 64 + 3) / 4 * 4) + S2 * (d_h + 4)) * sizeof(float);
+    const size_t ld1 = d_h == 64 ? kLD1<64> : kLD1<32>;
+    return ((d_h * ld1 + 3) / 4 * 4 + S2 * (d_h + 4)) * sizeof(float);
 }
 
 // The fused kernel covers head widths 32 and 64 with S a multiple of 32 up to
@@ -348,7 +353,7 @@ size_t attn_core_lds_bytes(int d_h, int S) {
 bool attn_core_ok(int d_h, int S, int heads, int B, const void* p0, const void* p1, const void* p2, const void* p3,
                   int ld_a, int ld_b, int ld_c) {
     if (!(d_h == 32 || d_h == 64)) return false;
-    if (S % 32 != 0 || S > 32 * kMaxKeyTiles) return false;
+    if (S % 32 != 0 || S > kMaxKeys) return false;
     if (static_cast<long long>(heads) * B > 0x7fffffffLL) return false;
     if (ld_a % 4 || ld_b % 4 || ld_c % 4) return false;
     return aligned16(p0) && aligned16(p1) && aligned16(p2) && aligned16(p3);

@@ -53,26 +53,32 @@ __global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const floa
     }
 }
 
-// out[i] = sum_{c<chunks} part[c*n + i].  A block owns 64 outputs; its four
+// out[i] = sum_{c<chunks} part[c*n + i].  A block owns 64 outputs; its sixteen
 // waves take interleaved chunks (lanes stay on consecutive i, so reads are
-// coalesced) and are combined through LDS.
-__global__ __launch_bounds__(kBlock) void combine_partials_kernel(float* out, const float* part,
-                                                                  int n, int chunks) {
-    constexpr int NW = kBlock / kWave;
+// coalesced), eight loads in flight each, and are combined through LDS.
+constexpr int kCombineBlock = 1024;
+__global__ __launch_bounds__(kCombineBlock) void combine_partials_kernel(float* out, const float* part,
+                                                                         int n, int chunks) {
+    constexpr int NW = kCombineBlock / kWave;
+    constexpr int U = 8;
     __shared__ float red[NW][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int i = blockIdx.x * kWave + lane;
-    float acc0 = 0.f, acc1 = 0.f;
+    float acc = 0.f;
     if (i < n) {
+        const float* p = part + i;
         int c = wave;
-        for (; c + NW < chunks; c += 2 * NW) {
-            acc0 += part[static_cast<size_t>(c) * n + i];
-            acc1 += part[static_cast<size_t>(c + NW) * n + i];
+        for (; c + (U - 1) * NW < chunks; c += U * NW) {
+            float x[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) x[u] = p[static_cast<size_t>(c + u * NW) * n];
+#pragma unroll
+            for (int u = 0; u < U; ++u) acc += x[u];
         }
-        if (c < chunks) acc0 += part[static_cast<size_t>(c) * n + i];
+        for (; c < chunks; c += NW) acc += p[static_cast<size_t>(c) * n];
     }
-    red[wave][lane] = acc0 + acc1;
+    red[wave][lane] = acc;
     __syncthreads();
     if (wave == 0 && i < n) {
         float s = 0.f;
@@ -298,7 +304,7 @@ JZ_API int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, in
     else
         sum_cols_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
     if (chunks > 1) {
-        combine_partials_kernel<<<(numcol + kWave - 1) / kWave, kBlock, 0, s>>>(out, dst, numcol, chunks);
+        combine_partials_kernel<<<(numcol + kWave - 1) / kWave, kCombineBlock, 0, s>>>(out, dst, numcol, chunks);
     }
     return launch_rc();
 }
@@ -328,8 +334,8 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
         sum_rows_short_kernel<<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(dst, a, numrow, total,
                                                                               active, span);
         if (blocks > 1) {
-            combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kBlock, 0, s>>>(out, dst, numrow,
-                                                                                    static_cast<int>(blocks));
+            combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kCombineBlock, 0, s>>>(
+                out, dst, numrow, static_cast<int>(blocks));
         }
         return launch_rc();
     }
@@ -352,7 +358,7 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
     else
         sum_rows_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
     if (chunks > 1) {
-        combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kBlock, 0, s>>>(out, dst, numrow, chunks);
+        combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kCombineBlock, 0, s>>>(out, dst, numrow, chunks);
     }
     return launch_rc();
 }
