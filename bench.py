@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: transformer train-step tokens/s on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--serial] [--no-cpu-baseline]
 
 Workload (BASELINE.json configs[3]): character-level LM, vocab 256 byte tokens
 drawn from Zipf(s=1.1), context 256, batch 64 (16 384 tokens per step), 6
@@ -10,10 +10,17 @@ FFN 2048 with GELU, tied embeddings, learned positional table, cross-entropy,
 AdamW (lr 3e-4, wd 0.01), fp32 everywhere.  One step = forward + loss +
 backward + optimiser on a synthetic batch that is already resident in HBM.
 
+The timed steps issue the backward pass on two streams: weight, bias and
+LayerNorm-parameter gradients (leaves of the backward graph) on a second
+stream beside the gradient chain.  `--serial` keeps everything on one stream in
+program order, which is what a per-kernel trace needs: concurrent kernels share
+the CUs, so their individual durations stop measuring the kernel.
+
 Prints ONE JSON line.  `roofline` describes the dominant kernel (the fp32 MFMA
 GEMM): algorithmic flops (2*m*n*k summed over its launches) divided by its
 launch time, measured with HIP events around every launch in separate
-instrumented steps after the timed region.  `cpu_baseline` times the
+instrumented steps after the timed region; those steps always run on one
+stream.  `cpu_baseline` times the
 reference's own CPU path (oracle/_ref, OpenBLAS build when available) on a
 bounded sample of the same workload.
 """
@@ -158,6 +165,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--serial", action="store_true",
+                    help="one stream, program order, also in the timed steps (for per-kernel traces and counters)")
     ap.add_argument("--cpu-baseline-only", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy of 2^26 floats three times, so that a counter run of this "
@@ -186,7 +195,7 @@ def main():
     ev = HipEvents()
     stream = lib.jzhip_get_stream()
 
-    model = CharLM(**CFG, gelu=True, tied=True, adamw=True, lr=3e-4, weight_decay=0.01)
+    model = CharLM(**CFG, gelu=True, tied=True, adamw=True, lr=3e-4, weight_decay=0.01, overlap=not args.serial)
     model.init_random(0)
     rng = np.random.default_rng(1234)
     model.set_batch(zipf_tokens(rng, CFG["vocab"], CFG["batch"], CFG["seq"]))
@@ -219,7 +228,8 @@ def main():
     ms_per_step = max(gpu_ms, wall_ms) / args.steps
     value = tokens_per_step / (ms_per_step * 1e-3)
 
-    # instrumented steps: HIP events around every tiled-GEMM launch
+    # instrumented steps: HIP events around every tiled-GEMM launch, one stream
+    model.set_overlap(False)
     lib.jzhip_profile_gemm(1)
     prof_steps = 2
     for _ in range(prof_steps):
@@ -240,6 +250,7 @@ def main():
         "kernel": dom["kernel"], "launches_per_step": dom["launches"] // prof_steps,
         "avg_launch_us": round(dom["total_ms"] * 1e3 / dom["launches"], 2),
         "flops_per_launch": round(dom["flops"] / dom["launches"], 1),
+        "measured_in": "instrumented steps on one stream (as with --serial)",
         "all_gemm_kernels": {"tflops": round(gemm_flops_per_step / (gemm_ms_per_step * 1e-3) / 1e12, 2),
                              "ms_per_step": round(gemm_ms_per_step, 3),
                              "share_of_step": round(gemm_ms_per_step / ms_per_step, 3)},
@@ -263,6 +274,7 @@ def main():
         "config": {"workload": "char-LM train step: vocab 256 (Zipf 1.1), context 256, batch 64, 6 pre-LN blocks, "
                                "d_model 512, 8 heads, FFN 2048 GELU, tied embeddings, learned positions, AdamW "
                                "lr 3e-4 wd 0.01", "tokens_per_step": tokens_per_step,
+                   "backward_streams": 1 if args.serial else 2,
                    "parameters": int(model.param_count), "loss_first": round(first_loss, 4),
                    "loss_last": round(last_loss, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 3)},
         "roofline": roofline,

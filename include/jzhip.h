@@ -18,8 +18,8 @@
  *     reference's null-stream launches (cpp/hipkernels.cpp:610-622).  Only
  *     the memcpy calls and `jzhip_synchronize` block the host.
  *   - no entry point allocates device memory behind the caller's back except
- *     `jzhip_malloc` and the one-time lazily created reduction workspace
- *     (see `jzhip_workspace_bytes`).
+ *     `jzhip_malloc` and the lazily created reduction workspace, one per
+ *     stream that needs it (see `jzhip_workspace_bytes`).
  *
  * Citations `file:line` refer to the reference tree (anewgithubname/Juzhen).
  */
@@ -63,8 +63,23 @@ int jzhip_set_stream(void* hip_stream);
 void* jzhip_get_stream(void);
 /* Block until the current stream is idle. */
 int jzhip_synchronize(void);
-/* Bytes of the lazily created reduction workspace (0 before first use). */
+/* Bytes of the lazily created reduction workspaces (0 before first use): one
+ * per stream that has run a call needing partial results, so that calls
+ * issued on different streams never share scratch storage. */
 size_t jzhip_workspace_bytes(void);
+/* No reference counterpart (cpp/hipkernels.cpp:458-461 runs everything on the
+ * null stream): a second stream and the events that order work between
+ * streams, for callers that overlap independent products (weight gradients
+ * against the gradient chain).  `jzhip_stream_create` makes a non-blocking
+ * stream of default priority; `jzhip_event_record` marks the current stream's
+ * position and `jzhip_stream_wait_event` makes everything issued afterwards
+ * on the current stream wait for that mark.  Neither blocks the host. */
+int jzhip_stream_create(void** out_stream);
+int jzhip_stream_destroy(void* hip_stream);
+int jzhip_event_create(void** out_event);
+int jzhip_event_destroy(void* event);
+int jzhip_event_record(void* event);
+int jzhip_stream_wait_event(void* event);
 
 /* ── random numbers ──────────────────────────────────────────────────── */
 

@@ -35,6 +35,12 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_get_stream": (P, []),
     "jzhip_synchronize": (I, []),
     "jzhip_workspace_bytes": (Z, []),
+    "jzhip_stream_create": (I, [P]),
+    "jzhip_stream_destroy": (I, [P]),
+    "jzhip_event_create": (I, [P]),
+    "jzhip_event_destroy": (I, [P]),
+    "jzhip_event_record": (I, [P]),
+    "jzhip_stream_wait_event": (I, [P]),
     "jzhip_rand_uniform": (I, [P, Z, U64]),
     "jzhip_rand_normal": (I, [P, Z, F, F, U64]),
     "jzhip_fill": (I, [P, Z, F]),

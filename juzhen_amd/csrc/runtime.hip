@@ -11,7 +11,15 @@ namespace jz {
 namespace {
 std::atomic<hipStream_t> g_stream{nullptr};
 std::atomic<int> g_cus{0};
-std::atomic<float*> g_workspace{nullptr};
+// One workspace per stream that has asked for one: launches on different
+// streams may run concurrently and must not share partial-result storage.
+constexpr int kMaxWorkspaces = 16;
+struct WorkspaceSlot {
+    std::atomic<float*> ptr{nullptr};
+    hipStream_t owner = nullptr;
+};
+WorkspaceSlot g_ws[kMaxWorkspaces];
+std::atomic<int> g_ws_count{0};
 std::mutex g_ws_mutex;
 }  // namespace
 
@@ -32,17 +40,23 @@ int num_cus() {
 }
 
 float* workspace() {
-    float* w = g_workspace.load(std::memory_order_acquire);
-    if (w) return w;
+    const hipStream_t s = stream();
+    const int n = g_ws_count.load(std::memory_order_acquire);
+    for (int i = 0; i < n; ++i)
+        if (g_ws[i].owner == s) return g_ws[i].ptr.load(std::memory_order_relaxed);
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    w = g_workspace.load(std::memory_order_acquire);
-    if (w) return w;
+    const int m = g_ws_count.load(std::memory_order_acquire);
+    for (int i = n; i < m; ++i)
+        if (g_ws[i].owner == s) return g_ws[i].ptr.load(std::memory_order_relaxed);
+    if (m == kMaxWorkspaces) return nullptr;
     void* p = nullptr;
     if (hipMalloc(&p, kWorkspaceFloats * sizeof(float)) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
-    g_workspace.store(static_cast<float*>(p), std::memory_order_release);
+    g_ws[m].owner = s;
+    g_ws[m].ptr.store(static_cast<float*>(p), std::memory_order_relaxed);
+    g_ws_count.store(m + 1, std::memory_order_release);
     return static_cast<float*>(p);
 }
 
@@ -122,5 +136,38 @@ JZ_API void* jzhip_get_stream(void) { return jz::stream(); }
 JZ_API int jzhip_synchronize(void) { return jz::rc_of(hipStreamSynchronize(jz::stream())); }
 
 JZ_API size_t jzhip_workspace_bytes(void) {
-    return jz::g_workspace.load(std::memory_order_acquire) ? jz::kWorkspaceFloats * sizeof(float) : 0;
+    return static_cast<size_t>(jz::g_ws_count.load(std::memory_order_acquire)) * jz::kWorkspaceFloats * sizeof(float);
+}
+
+JZ_API int jzhip_stream_create(void** out_stream) {
+    if (!out_stream) return -1;
+    hipStream_t s = nullptr;
+    // default priority; non-blocking so that it does not serialise against the null stream
+    const int rc = jz::rc_of(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out_stream = rc ? nullptr : s;
+    return rc;
+}
+JZ_API int jzhip_stream_destroy(void* hip_stream) {
+    if (!hip_stream) return 0;
+    if (jz::stream() == static_cast<hipStream_t>(hip_stream)) jzhip_set_stream(nullptr);
+    return jz::rc_of(hipStreamDestroy(static_cast<hipStream_t>(hip_stream)));
+}
+JZ_API int jzhip_event_create(void** out_event) {
+    if (!out_event) return -1;
+    hipEvent_t e = nullptr;
+    const int rc = jz::rc_of(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    *out_event = rc ? nullptr : e;
+    return rc;
+}
+JZ_API int jzhip_event_destroy(void* event) {
+    if (!event) return 0;
+    return jz::rc_of(hipEventDestroy(static_cast<hipEvent_t>(event)));
+}
+JZ_API int jzhip_event_record(void* event) {
+    if (!event) return -1;
+    return jz::rc_of(hipEventRecord(static_cast<hipEvent_t>(event), jz::stream()));
+}
+JZ_API int jzhip_stream_wait_event(void* event) {
+    if (!event) return -1;
+    return jz::rc_of(hipStreamWaitEvent(jz::stream(), static_cast<hipEvent_t>(event), 0));
 }

@@ -19,6 +19,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -78,8 +79,19 @@ struct Model {
     int32_t* targets = nullptr;
     float* loss = nullptr;
     // backward scratch shared by all blocks
-    float *dx = nullptr, *dR = nullptr, *dtmp = nullptr, *dQKV = nullptr, *dH = nullptr, *dA = nullptr,
-          *dF1 = nullptr;
+    // (the ones the weight-gradient products read exist twice, alternating by
+    // block, and the block-output gradient three times: see backward())
+    float *dx[3] = {}, *dR[2] = {}, *dtmp[2] = {}, *dtmp1[2] = {}, *dQKV[2] = {}, *dF1[2] = {};
+    float *dH = nullptr, *dA = nullptr;
+    // Weight, bias and LayerNorm-parameter gradients are leaves of the backward
+    // graph: with `overlap` they go to a second stream and fill the gaps the
+    // gradient chain leaves (tile prologues and tails, bandwidth-bound kernels).
+    bool overlap = true;
+    void* side = nullptr;
+    static constexpr int kEvents = 8, kDone = 4;
+    void* ev[kEvents] = {};
+    void* done[kDone] = {};   // side stream finished a block's weight gradients
+    int ev_next = 0;
     float* io = nullptr;  // dense staging for get/set of strided views
     size_t io_floats = 0;
     int iteration = 1;
@@ -186,15 +198,59 @@ void step_group(Model& M, int group) {
     M.ck(jzhip_adamw_step(a.w, a.g, a.m, a.v, a.used, c.lr, c.beta1, c.beta2, c.eps, wd, M.iteration));
 }
 
+// The backward pass on two streams.  `fork()` makes the side stream wait for
+// everything issued so far on the main stream and routes the next calls to it;
+// `back()` returns to the main stream without waiting; `mark(i)` records the
+// side stream's position in done[i % kDone] and `await(i)` makes the main
+// stream wait for that mark; `join()` makes the main stream wait for
+// everything issued so far on the side stream.
+struct Lanes {
+    Model& M;
+    void* main_stream;
+    bool on;
+    explicit Lanes(Model& m) : M(m), main_stream(jzhip_get_stream()), on(m.overlap && m.side != nullptr) {}
+    void* next_event() { void* e = M.ev[M.ev_next]; M.ev_next = (M.ev_next + 1) % Model::kEvents; return e; }
+    void fork() {
+        if (!on) return;
+        void* e = next_event();
+        M.ck(jzhip_event_record(e));
+        M.ck(jzhip_set_stream(M.side));
+        M.ck(jzhip_stream_wait_event(e));
+    }
+    void back() {
+        if (on) M.ck(jzhip_set_stream(main_stream));
+    }
+    void mark(int i) {
+        if (!on) return;
+        M.ck(jzhip_set_stream(M.side));
+        M.ck(jzhip_event_record(M.done[i % Model::kDone]));
+        M.ck(jzhip_set_stream(main_stream));
+    }
+    void await(int i) {
+        if (on) M.ck(jzhip_stream_wait_event(M.done[i % Model::kDone]));
+    }
+    void join() {
+        if (!on) return;
+        void* e = next_event();
+        M.ck(jzhip_set_stream(M.side));
+        M.ck(jzhip_event_record(e));
+        M.ck(jzhip_set_stream(main_stream));
+        M.ck(jzhip_stream_wait_event(e));
+    }
+};
+
 void backward(Model& M, bool update) {
     const Config& c = M.c;
     const int d = c.d_model, N = M.N, ff = c.d_ff, V = c.vocab;
     const float* xL = M.blocks.empty() ? M.x0 : M.blocks.back().out;
+    Lanes lanes(M);
     M.ck(jzhip_softmax_xent(M.loss, M.dlogits, M.logits, M.targets, V, N, V));
-    float* dy = M.dx;  // gradient w.r.t. the current block's output
+    float* dy = M.dx[0];  // gradient w.r.t. the current block's output
     if (c.tied) {
         gemm(M, M.t[M.E].w, false, M.dlogits, false, dy, d, N, V);       // E * dlogits
+        lanes.fork();
         gemm(M, xL, false, M.dlogits, true, M.t[M.E].g, d, V, N);        // head part of dE
+        lanes.back();
     } else {
         gemm(M, M.dlogits, false, xL, true, M.t[M.Wp].g, V, d, N);
         M.ck(jzhip_sum_rows(M.t[M.bp].g, M.dlogits, V, N, V));
@@ -204,32 +260,60 @@ void backward(Model& M, bool update) {
         if (update) { step_group(M, kHeadDecay); step_group(M, kHeadPlain); }
         gemm(M, M.t[M.Wp].w, true, M.dlogits, false, dy, d, N, V);
     }
-    for (int l = static_cast<int>(M.blocks.size()) - 1; l >= 0; --l) {
-        Block& b = M.blocks[l];
+    const int L = static_cast<int>(M.blocks.size());
+    for (int i = 0; i < L; ++i) {   // i-th block from the top
+        Block& b = M.blocks[L - 1 - i];
+        // Scratch gradients alternate between two sets by block (three for the
+        // block-output gradient, which is written one block before it is read by
+        // the side stream): set i % 2 is rewritten here, so the side stream must
+        // have finished the weight gradients of block i - 2, and may still be
+        // working on those of block i - 1.
+        if (i >= 2) lanes.await(i - 2);
+        float* dF1 = M.dF1[i % 2];
+        float* dx2 = M.dtmp[i % 2];
+        float* dx1 = M.dtmp1[i % 2];
+        float* dR = M.dR[i % 2];
+        float* dQKV = M.dQKV[i % 2];
+        float* dy_next = M.dx[(i + 1) % 3];
         // feed-forward
+        lanes.fork();
         gemm(M, dy, false, b.F1a, true, M.t[b.W2].g, d, ff, N);
         M.ck(jzhip_sum_rows(M.t[b.b2].g, dy, d, N, d));
+        lanes.back();
         // dF1 = (W2^T dy) .* act'(F1)
-        gemm_tail(M, M.t[b.W2].w, true, dy, M.dF1, ff, N, d, nullptr, c.gelu ? 4 : 3, b.F1, nullptr);
-        gemm(M, M.dF1, false, b.x2, true, M.t[b.W1].g, ff, d, N);
-        M.ck(jzhip_sum_rows(M.t[b.b1].g, M.dF1, ff, N, ff));
-        gemm(M, M.t[b.W1].w, true, M.dF1, false, M.dtmp, d, N, ff);      // dx2
-        M.ck(jzhip_layernorm_param_grads(M.t[b.g2].g, M.t[b.be2].g, M.dtmp, b.xhat2, d, N));
+        gemm_tail(M, M.t[b.W2].w, true, dy, dF1, ff, N, d, nullptr, c.gelu ? 4 : 3, b.F1, nullptr);
+        lanes.fork();
+        gemm(M, dF1, false, b.x2, true, M.t[b.W1].g, ff, d, N);
+        M.ck(jzhip_sum_rows(M.t[b.b1].g, dF1, ff, N, ff));
+        lanes.back();
+        gemm(M, M.t[b.W1].w, true, dF1, false, dx2, d, N, ff);
+        lanes.fork();
+        M.ck(jzhip_layernorm_param_grads(M.t[b.g2].g, M.t[b.be2].g, dx2, b.xhat2, d, N));
+        lanes.back();
         // dR = LN2'(dx2) + dy
-        M.ck(jzhip_layernorm_bwd_residual(M.dR, M.dtmp, M.t[b.g2].w, b.xhat2, b.inv2, dy, d, N));
+        M.ck(jzhip_layernorm_bwd_residual(dR, dx2, M.t[b.g2].w, b.xhat2, b.inv2, dy, d, N));
         // output projection
-        gemm(M, M.dR, false, b.H, true, M.t[b.Wo].g, d, d, N);
-        M.ck(jzhip_sum_rows(M.t[b.bo].g, M.dR, d, N, d));
-        gemm(M, M.t[b.Wo].w, true, M.dR, false, M.dH, d, N, d);
+        lanes.fork();
+        gemm(M, dR, false, b.H, true, M.t[b.Wo].g, d, d, N);
+        M.ck(jzhip_sum_rows(M.t[b.bo].g, dR, d, N, d));
+        lanes.back();
+        gemm(M, M.t[b.Wo].w, true, dR, false, M.dH, d, N, d);
         // attention core, gradients into the stacked (3d x N) buffer
-        M.ck(jzhip_attention_bwd_ld(M.dQKV, M.dQKV + d, M.dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
+        M.ck(jzhip_attention_bwd_ld(dQKV, dQKV + d, dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
                                     b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch, 1));
-        gemm(M, M.dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
-        gemm(M, M.t[b.Wq].w, true, M.dQKV, false, M.dtmp, d, N, 3 * d);        // dx1
-        M.ck(jzhip_layernorm_param_grads(M.t[b.g1].g, M.t[b.be1].g, M.dtmp, b.xhat1, d, N));
+        lanes.fork();
+        gemm(M, dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
+        lanes.back();
+        gemm(M, M.t[b.Wq].w, true, dQKV, false, dx1, d, N, 3 * d);
+        lanes.fork();
+        M.ck(jzhip_layernorm_param_grads(M.t[b.g1].g, M.t[b.be1].g, dx1, b.xhat1, d, N));
+        lanes.back();
+        lanes.mark(i);
         // dx = LN1'(dx1) + dR
-        M.ck(jzhip_layernorm_bwd_residual(dy, M.dtmp, M.t[b.g1].w, b.xhat1, b.inv1, M.dR, d, N));
+        M.ck(jzhip_layernorm_bwd_residual(dy_next, dx1, M.t[b.g1].w, b.xhat1, b.inv1, dR, d, N));
+        dy = dy_next;
     }
+    lanes.join();
     // embedding tables: dE (+)= dx0 * onehot_tok^T, dP = dx0 * onehot_pos^T
     gemm(M, dy, false, M.oh_tok, true, M.t[M.E].g, d, V, N, c.tied ? 1.0f : 0.0f);
     gemm(M, dy, false, M.oh_pos, true, M.t[M.P].g, d, c.seq, N);
@@ -299,12 +383,20 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
     M->dlogits = M->alloc(static_cast<size_t>(V) * N);
     M->targets = reinterpret_cast<int32_t*>(M->alloc(N));
     M->loss = M->alloc(1);
-    M->dx = M->alloc(dN); M->dR = M->alloc(dN); M->dtmp = M->alloc(dN);
-    M->dQKV = M->alloc(3 * dN); M->dH = M->alloc(dN);
-    M->dA = M->alloc(aN); M->dF1 = M->alloc(fN);
+    for (float*& p : M->dx) p = M->alloc(dN);
+    for (int k = 0; k < 2; ++k) {
+        M->dR[k] = M->alloc(dN); M->dtmp[k] = M->alloc(dN); M->dtmp1[k] = M->alloc(dN);
+        M->dQKV[k] = M->alloc(3 * dN); M->dF1[k] = M->alloc(fN);
+    }
+    M->dH = M->alloc(dN); M->dA = M->alloc(aN);
     if (M->rc != 0) {
         std::fprintf(stderr, "jzlm_create: device allocation failed (%s)\n", jzhip_error_string(M->rc));
+        return M;
     }
+    M->ck(jzhip_stream_create(&M->side));
+    for (void*& e : M->ev) M->ck(jzhip_event_create(&e));
+    for (void*& e : M->done) M->ck(jzhip_event_create(&e));
+    if (const char* env = std::getenv("JZLM_OVERLAP")) M->overlap = std::atoi(env) != 0;
     return M;
 }
 
@@ -312,9 +404,16 @@ JZLM_API void jzlm_destroy(void* h) {
     Model* M = static_cast<Model*>(h);
     if (!M) return;
     jzhip_synchronize();
+    for (void* e : M->ev) jzhip_event_destroy(e);
+    for (void* e : M->done) jzhip_event_destroy(e);
+    jzhip_stream_destroy(M->side);
     for (float* p : M->owned) jzhip_free(p);
     delete M;
 }
+
+// 1: weight-gradient work of the backward pass on a second stream (default);
+// 0: everything on the library's current stream in program order.
+JZLM_API void jzlm_set_overlap(void* h, int on) { static_cast<Model*>(h)->overlap = on != 0; }
 
 JZLM_API int jzlm_status(void* h) { return static_cast<Model*>(h)->rc; }
 JZLM_API int jzlm_num_tensors(void* h) { return static_cast<int>(static_cast<Model*>(h)->t.size()); }

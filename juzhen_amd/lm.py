@@ -56,6 +56,8 @@ def load():
         lib.jzlm_logits.restype = C.c_int
         lib.jzlm_logits.argtypes = [C.c_void_p, C.c_void_p]
         lib.jzlm_set_iteration.argtypes = [C.c_void_p, C.c_int]
+        lib.jzlm_set_overlap.argtypes = [C.c_void_p, C.c_int]
+        lib.jzlm_set_overlap.restype = None
         _lib = lib
     return _lib
 
@@ -65,7 +67,7 @@ class CharLM:
 
     def __init__(self, vocab=256, d_model=512, heads=8, d_ff=2048, layers=6, seq=256, batch=64,
                  gelu=True, tied=True, adamw=True, lr=3e-4, weight_decay=0.01, beta1=0.9, beta2=0.999,
-                 eps=1e-8):
+                 eps=1e-8, overlap=None):
         self.lib = load()
         self.cfg = Config(vocab, d_model, heads, d_ff, layers, seq, batch, int(gelu), int(tied), int(adamw),
                           lr, weight_decay, beta1, beta2, eps)
@@ -75,6 +77,13 @@ class CharLM:
         self._check("create", self.lib.jzlm_status(self.h))
         self.names = [self.lib.jzlm_tensor_name(self.h, i).decode() for i in range(self.lib.jzlm_num_tensors(self.h))]
         self.index = {n: i for i, n in enumerate(self.names)}
+        if overlap is not None:
+            self.set_overlap(overlap)
+
+    def set_overlap(self, on):
+        """Weight-gradient work of the backward pass on a second stream (the default)
+        or everything on one stream in program order."""
+        self.lib.jzlm_set_overlap(self.h, int(bool(on)))
 
     def _check(self, what, rc):
         if rc != 0:

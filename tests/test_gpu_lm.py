@@ -165,3 +165,35 @@ def test_gradients_against_float64_autograd(gpu):
         got, want = m.get(name, which=1), grads[name]
         assert np.linalg.norm(got - want) <= 1e-3 * np.linalg.norm(want), name
     m.close()
+
+
+@pytest.mark.parametrize("tied", [True, False])
+def test_two_stream_backward_is_bit_identical_to_program_order(gpu, tied):
+    """The backward pass issues weight, bias and LayerNorm-parameter gradients on a
+    second stream; every kernel and every accumulation order is the same as on one
+    stream, so losses, gradients and parameters must agree to the bit.  Four blocks
+    exercise the alternating scratch sets and the wait on the block two above."""
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 64, 128, 4, 512, 4, 64, 8
+    rng = np.random.default_rng(5)
+    tokens = make_tokens(rng, V, B, S)
+    runs = []
+    for overlap in (False, True):
+        m = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=tied, adamw=True, lr=1e-3, overlap=overlap)
+        m.init_random(3)
+        m.set_batch(tokens)
+        losses = []
+        for _ in range(6):
+            m.step()
+            losses.append(m.loss())
+        m.forward()
+        m.backward(update=False)
+        grads = {n: m.get(n, which=1) for n in m.names}
+        params = {n: m.get(n) for n in m.names}
+        runs.append((losses, grads, params))
+        m.close()
+    (l0, g0, p0), (l1, g1, p1) = runs
+    assert l0 == l1
+    for n in g0:
+        assert np.array_equal(g0[n], g1[n]), n
+        assert np.array_equal(p0[n], p1[n]), n
