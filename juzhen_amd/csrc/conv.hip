@@ -226,6 +226,34 @@ int transpose_batched(float* dst, const float* src, const float* bias, int R, in
 // HBM reads and the HBM writes are contiguous runs.
 constexpr int kPatchChunk = 256;   // k values per workgroup of im2col_rows: one float4 per lane
 
+// Workgroup order of the scatter row kernel.  Work items are (x, yz): x the
+// channel chunk, yz = row strip + strips*sample.  Workgroups are dealt round-robin to the 8
+// XCDs, so a 1-D grid of 8*per*gx is launched and XCD q takes yz in
+// [q*per, (q+1)*per), walking x fastest: the chunks of one strip, which read
+// neighbouring pieces of the same cache lines, and the strips above and below,
+// which share halo rows, run at the same time on the same L2.
+struct RowGrid {
+    int gx, gy, nyz, per;
+    unsigned blocks() const { return 8u * static_cast<unsigned>(per) * static_cast<unsigned>(gx); }
+};
+RowGrid make_rowgrid(int gx, int gy, int gz) {
+    RowGrid r;
+    r.gx = gx; r.gy = gy; r.nyz = gy * gz;
+    r.per = (r.nyz + 7) / 8;
+    return r;
+}
+// false: this workgroup is padding of the last XCD's range
+__device__ __forceinline__ bool rowgrid_item(const RowGrid& rg, int& x, int& y, int& z) {
+    const unsigned id = blockIdx.x;
+    const unsigned xcd = id % 8u, j = id / 8u;
+    x = static_cast<int>(j % static_cast<unsigned>(rg.gx));
+    const int yz = static_cast<int>(xcd) * rg.per + static_cast<int>(j / static_cast<unsigned>(rg.gx));
+    if (yz >= rg.nyz) return false;
+    y = yz % rg.gy;
+    z = yz / rg.gy;
+    return true;
+}
+
 // One workgroup = one row ph of the patch grid, one sample n, one chunk of 256
 // consecutive k.  The image rows that chunk touches (its channels x kH rows,
 // zero-filled where the window hangs over the border) are staged in LDS; then
@@ -236,6 +264,9 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
                                                              int WT, FastDiv dWT, FastDiv dkH) {
     extern __shared__ float tile[];   // [channels of the chunk][kH][WT]
     const int KK = g.kH * g.kW;
+    // (plain dispatch order, chunks of one patch row spread over the XCDs: the
+    // kernel is write-dominated and this order measured faster than the
+    // XCD-grouped one the scatter kernel uses)
     const int k0 = blockIdx.x * kPatchChunk;
     const int k1 = (k0 + kPatchChunk) < g.K ? (k0 + kPatchChunk) : g.K;
     const int ph = blockIdx.y, n = blockIdx.z;
@@ -295,20 +326,24 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
 // the ph rows involved) are staged in LDS with contiguous reads; the sums are
 // then formed in the CPU's order (kh, kw descending) out of LDS and written as
 // whole image rows.  The pitch is odd so that lanes walking along pw hit
-// distinct banks.
+// distinct banks.  S, KH, KW > 0 fix stride (both directions) and kernel extent
+// at compile time: the collection loop is index arithmetic per tap, and with
+// them known the divisions become shifts and the nine or sixteen taps unroll.
+template <int S, int KH, int KW>
 __global__ __launch_bounds__(kBlock) void col2im_rows_kernel(const float* __restrict__ col,
                                                              float* __restrict__ img,
                                                              const float* __restrict__ bias, PatchGeom g,
                                                              int CC, int R, int pitch, int vec4, FastDiv dL,
-                                                             FastDiv dR, FastDiv dsh, FastDiv dsw) {
+                                                             FastDiv dR, FastDiv dsh, FastDiv dsw, RowGrid rg) {
     extern __shared__ float tile[];   // [ph rows][Wp][pitch]
     const int KK = g.kH * g.kW;
     // (the launcher picks CC dividing C and R dividing H, so every workgroup is full)
-    const int c0 = blockIdx.x * CC;
+    int bx, by, n;
+    if (!rowgrid_item(rg, bx, by, n)) return;
+    const int c0 = bx * CC;
     const int cc = CC;
-    const int ih0 = blockIdx.y * R;
+    const int ih0 = by * R;
     const int rcnt = R;
-    const int n = blockIdx.z;
     // patch rows with ph*stride - pad + kh inside [ih0, ih0 + rcnt)
     int lo = ih0 + g.pad_h - (g.kH - 1);
     lo = lo <= 0 ? 0 : (lo + g.stride_h - 1) / g.stride_h;
@@ -377,18 +412,42 @@ __global__ __launch_bounds__(kBlock) void col2im_rows_kernel(const float* __rest
         const int cl = static_cast<int>(fdiv(t, dR));
         const int ih = ih0 + (static_cast<int>(t) - cl * rcnt);
         float val = bias ? bias[c0 + cl] : 0.0f;
-        for (int kh = g.kH - 1; kh >= 0; --kh) {
-            const int hn = ih + g.pad_h - kh;
-            if (hn < 0) continue;
-            const int ph = static_cast<int>(fdiv(static_cast<uint32_t>(hn), dsh));
-            if (ph * g.stride_h != hn || ph >= g.Hp) continue;
-            const float* row = tile + static_cast<size_t>(ph - lo) * g.Wp * pitch + cl * KK + kh * g.kW;
-            for (int kw = g.kW - 1; kw >= 0; --kw) {
-                const int wn = iw + g.pad_w - kw;
-                if (wn < 0) continue;
-                const int pw = static_cast<int>(fdiv(static_cast<uint32_t>(wn), dsw));
-                if (pw * g.stride_w != wn || pw >= g.Wp) continue;
-                val += row[pw * pitch + kw];
+        if constexpr (S > 0) {
+            // Only every S-th kernel row/column can reach this pixel (ih + pad - kh
+            // must be a multiple of S): start at the largest such kh, kw and step by
+            // S, the patch index going up by one each time; TH x TW taps instead of
+            // KH x KW, in the same descending (kh, kw) order.
+            constexpr int TH = (KH + S - 1) / S, TW = (KW + S - 1) / S;
+            const int hq = ih + g.pad_h, wq = iw + g.pad_w;
+            const int kh1 = (KH - 1) - ((KH - 1 - hq % S) + S) % S;   // may be negative: no tap then
+            const int kw1 = (KW - 1) - ((KW - 1 - wq % S) + S) % S;
+            const int ph1 = (hq - kh1) / S, pw1 = (wq - kw1) / S;      // exact divisions
+            const float* p0 = tile + cl * (KH * KW) + ((ph1 - lo) * g.Wp + pw1) * pitch + kh1 * KW + kw1;
+#pragma unroll
+            for (int a = 0; a < TH; ++a) {
+                const int kh = kh1 - a * S, ph = ph1 + a;
+                const bool okh = kh >= 0 && ph >= 0 && ph < g.Hp;
+                const float* row = p0 + a * (g.Wp * pitch - S * KW);
+#pragma unroll
+                for (int b = 0; b < TW; ++b) {
+                    const int kw = kw1 - b * S, pw = pw1 + b;
+                    if (okh && kw >= 0 && pw >= 0 && pw < g.Wp) val += row[b * (pitch - S)];
+                }
+            }
+        } else {
+            for (int kh = g.kH - 1; kh >= 0; --kh) {
+                const int hn = ih + g.pad_h - kh;
+                if (hn < 0) continue;
+                const int ph = static_cast<int>(fdiv(static_cast<uint32_t>(hn), dsh));
+                if (ph * g.stride_h != hn || ph >= g.Hp) continue;
+                const float* row = tile + static_cast<size_t>(ph - lo) * g.Wp * pitch + cl * KK + kh * g.kW;
+                for (int kw = g.kW - 1; kw >= 0; --kw) {
+                    const int wn = iw + g.pad_w - kw;
+                    if (wn < 0) continue;
+                    const int pw = static_cast<int>(fdiv(static_cast<uint32_t>(wn), dsw));
+                    if (pw * g.stride_w != wn || pw >= g.Wp) continue;
+                    val += row[pw * pitch + kw];
+                }
             }
         }
         img[static_cast<size_t>(n) * (g.C * g.H * g.W) + (static_cast<size_t>(c0 + cl) * g.H + ih) * g.W + iw] = val;
@@ -428,13 +487,13 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
     const size_t total = static_cast<size_t>(g.C) * g.H * g.W * g.N;
     if (total >= (size_t(1) << 31)) return -1;
     if (static_cast<size_t>(g.K) * g.P * g.N >= (size_t(1) << 31)) return -1;
-    if (g.N <= 65535 && g.W <= 1024) {
+    if (g.W <= 1024) {
         // channels and image rows per workgroup: as many as keep the staged strip
         // under 40 KB (four workgroups per CU), preferring a channel-chunk count
         // that is a multiple of 8 so that the workgroups sharing patch rows
         // (same chunk, neighbouring rows) meet in one XCD's L2
         const int KK = g.kH * g.kW;
-        int R = 4, CC = 8;
+        int R = 4, CC = 16;
         auto bytes = [&](int cc, int r) {
             const int nr = (r - 1 + g.kH - 1) / g.stride_h + 1;
             return static_cast<size_t>(nr) * g.Wp * ((cc * KK) | 1) * sizeof(float);
@@ -442,12 +501,22 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
         while (R > 1 && g.H % R != 0) R /= 2;
         while (CC > 1 && (g.C % CC != 0 || bytes(CC, R) > 40 * 1024)) CC /= 2;
         while (R > 1 && bytes(CC, R) > 40 * 1024) R /= 2;
-        if (bytes(CC, R) <= 40 * 1024 && g.H / R <= 65535) {
-            dim3 grid(g.C / CC, g.H / R, g.N);
+        if (bytes(CC, R) <= 40 * 1024) {
+            // (C/CC * H/R * N <= C*H*W*N < 2^31 workgroups)
+            const RowGrid rg = make_rowgrid(g.C / CC, g.H / R, g.N);
+            const unsigned grid = rg.blocks();
             const int vec4 = ((CC * KK) % 4 == 0 && g.K % 4 == 0 && aligned16(col)) ? 1 : 0;
-            col2im_rows_kernel<<<grid, kBlock, bytes(CC, R), stream()>>>(
-                col, img, bias, g, CC, R, (CC * KK) | 1, vec4, make_fastdiv(vec4 ? CC * KK / 4 : CC * KK), make_fastdiv(R),
-                make_fastdiv(g.stride_h), make_fastdiv(g.stride_w));
+            const int S = g.stride_h == g.stride_w ? g.stride_h : 0;
+#define JZ_COL2IM(S_, KH_, KW_)                                                                              \
+    col2im_rows_kernel<S_, KH_, KW_><<<grid, kBlock, bytes(CC, R), stream()>>>(                              \
+        col, img, bias, g, CC, R, (CC * KK) | 1, vec4, make_fastdiv(vec4 ? CC * KK / 4 : CC * KK), make_fastdiv(R), \
+        make_fastdiv(g.stride_h), make_fastdiv(g.stride_w), rg)
+            if (S == 1 && g.kH == 3 && g.kW == 3) JZ_COL2IM(1, 3, 3);
+            else if (S == 2 && g.kH == 3 && g.kW == 3) JZ_COL2IM(2, 3, 3);
+            else if (S == 2 && g.kH == 4 && g.kW == 4) JZ_COL2IM(2, 4, 4);
+            else if (S == 1 && g.kH == 5 && g.kW == 5) JZ_COL2IM(1, 5, 5);
+            else JZ_COL2IM(0, 1, 1);
+#undef JZ_COL2IM
             return launch_rc();
         }
     }

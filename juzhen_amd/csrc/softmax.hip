@@ -546,12 +546,21 @@ __global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, fl
     }
 }
 
-__global__ __launch_bounds__(kBlock) void neg_mean_kernel(float* out, const float* v, int n,
-                                                          float inv_n) {
-    __shared__ float red[kBlock / kWave];
-    float acc = 0.f;
-    for (int i = threadIdx.x; i < n; i += kBlock) acc += v[i];
-    const float s = block_allreduce<kBlock / kWave>(acc, SumOp{}, red, 0.f);
+// out = -mean(v): one block of sixteen waves, four independent loads in flight
+// per thread (the per-sample losses are few; a serial loop over them costs more
+// than the cross-entropy kernel itself)
+constexpr int kMeanBlock = 1024;
+__global__ __launch_bounds__(kMeanBlock) void neg_mean_kernel(float* out, const float* v, int n,
+                                                              float inv_n) {
+    __shared__ float red[kMeanBlock / kWave];
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int i = threadIdx.x;
+    for (; i + 3 * kMeanBlock < n; i += 4 * kMeanBlock) {
+        const float x0 = v[i], x1 = v[i + kMeanBlock], x2 = v[i + 2 * kMeanBlock], x3 = v[i + 3 * kMeanBlock];
+        a0 += x0; a1 += x1; a2 += x2; a3 += x3;
+    }
+    for (; i < n; i += kMeanBlock) a0 += v[i];
+    const float s = block_allreduce<kMeanBlock / kWave>((a0 + a1) + (a2 + a3), SumOp{}, red, 0.f);
     if (threadIdx.x == 0) out[0] = -s * inv_n;
 }
 
@@ -733,6 +742,6 @@ JZ_API int jzhip_softmax_xent(float* loss_out, float* dlogits, const float* logi
     if (!per_sample) return -2;
     int rc = dispatch_nv<XentL>(K, per_sample, dlogits, logits, labels, K, N, static_cast<size_t>(ld));
     if (rc) return rc;
-    neg_mean_kernel<<<1, kBlock, 0, stream()>>>(loss_out, per_sample, N, static_cast<float>(1.0 / N));
+    neg_mean_kernel<<<1, kMeanBlock, 0, stream()>>>(loss_out, per_sample, N, static_cast<float>(1.0 / N));
     return launch_rc();
 }
