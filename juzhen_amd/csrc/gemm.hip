@@ -636,10 +636,16 @@ int launch_tile(const GemmArgs& g) {
     const long long cus = num_cus();
     if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 1024 && !g.ep.any) {
         splits = static_cast<int>((cus * 2 + tiles - 1) / tiles);
+        // The K chunk is the fastest-varying part of the workgroup id and
+        // workgroups are dealt round-robin to 8 XCDs: with a count that divides 8
+        // or is a multiple of it, an XCD only ever sees chunks congruent to its
+        // index and the operand panels of a chunk are fetched into one L2.
+        auto xcd_friendly = [](int n) { return n <= 2 ? n : n <= 4 ? 4 : (n + 7) / 8 * 8; };
+        splits = xcd_friendly(splits);
         const int max_by_k = g.K / 256;
-        if (splits > max_by_k) splits = max_by_k;
         const size_t per = static_cast<size_t>(g.M) * g.N;
-        while (splits > 1 && per * splits > kWorkspaceFloats) --splits;
+        while (splits > 1 && (splits > max_by_k || per * splits > kWorkspaceFloats))
+            splits = splits > 8 ? splits - 8 : splits / 2;
         if (splits < 2) splits = 1;
     }
     int k_chunk = g.K;
