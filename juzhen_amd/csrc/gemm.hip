@@ -600,10 +600,60 @@ __global__ __launch_bounds__(kBlock) void splitk_reduce_kernel(float* C, const f
     const size_t total = static_cast<size_t>(M) * N;
     const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
     for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+        // eight partials requested at a time, summed in split order
+        const float* p = part + i;
         float acc = 0.f;
-        for (int s = 0; s < splits; ++s) acc += part[static_cast<size_t>(s) * total + i];
+        int s = 0;
+        for (; s + 8 <= splits; s += 8) {
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = p[static_cast<size_t>(s + u) * total];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += x[u];
+        }
+        for (; s < splits; ++s) acc += p[static_cast<size_t>(s) * total];
         float* dst = C + (i / M) * ldc + (i % M);
         float r = alpha * acc;
+        if (beta != 0.0f) r += beta * *dst;
+        *dst = r;
+    }
+}
+
+// The same sum for a small C cut into many chunks (convolution weight
+// gradients: a few tiles, K in the tens of thousands): 64 elements per
+// workgroup, its sixteen waves taking interleaved partials (four in flight
+// each) and meeting in LDS; wave w adds partials w, w+16, ... and the sixteen
+// sums are added in wave order, so the result is deterministic.
+constexpr int kTallBlock = 1024;
+__global__ __launch_bounds__(kTallBlock) void splitk_reduce_tall_kernel(float* C, const float* part, int M, int N,
+                                                                        size_t ldc, int splits, float alpha,
+                                                                        float beta) {
+    constexpr int NW = kTallBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const size_t total = static_cast<size_t>(M) * N;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const size_t i = static_cast<size_t>(blockIdx.x) * kWave + lane;
+    float acc = 0.f;
+    if (i < total) {
+        const float* p = part + i;
+        int s = wave;
+        for (; s + 3 * NW < splits; s += 4 * NW) {
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = p[static_cast<size_t>(s + u * NW) * total];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc += x[u];
+        }
+        for (; s < splits; s += NW) acc += p[static_cast<size_t>(s) * total];
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && i < total) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[w][lane];
+        float* dst = C + (i / M) * ldc + (i % M);
+        float r = alpha * sum;
         if (beta != 0.0f) r += beta * *dst;
         *dst = r;
     }
@@ -700,8 +750,12 @@ int launch_tile(const GemmArgs& g) {
     }
     if (splits > 1) {
         const size_t total = static_cast<size_t>(g.M) * g.N;
-        splitk_reduce_kernel<<<grid_for(total, kBlock, 4), kBlock, 0, s>>>(g.C, out, g.M, g.N, g.ldc, splits,
-                                                                           g.alpha, g.beta);
+        if (splits >= 32 && total <= (size_t(1) << 20))
+            splitk_reduce_tall_kernel<<<static_cast<unsigned>((total + kWave - 1) / kWave), kTallBlock, 0, s>>>(
+                g.C, out, g.M, g.N, g.ldc, splits, g.alpha, g.beta);
+        else
+            splitk_reduce_kernel<<<grid_for(total, kBlock, 4), kBlock, 0, s>>>(g.C, out, g.M, g.N, g.ldc, splits,
+                                                                               g.alpha, g.beta);
     }
     return launch_rc();
 }
@@ -722,6 +776,15 @@ int launch_shape(const GemmArgs& g) {
     // still fills the chip; otherwise fall back to 64 x 64 tiles
     // (only when at least cus/8 big tiles exist: more than ~16 partial sums per
     // output cost more in the reduction than the bigger tile saves)
+    // an extent that is a multiple of 64 but not of 128 (3x3 patches of 64 or 192
+    // channels) takes the half-size tile in that direction: full tiles stay on
+    // the unchecked float4 loaders
+    if (g.M % 128 != 0 && g.M % 64 == 0 && g.N % 128 == 0 && g.K % 32 == 0)
+        return launch_tile<1, 4, 2, 1, TA, TB>(g);   // 64 x 128
+    if (g.N % 128 != 0 && g.N % 64 == 0 && g.M % 128 == 0 && g.K % 32 == 0)
+        return launch_tile<4, 1, 1, 2, TA, TB>(g);   // 128 x 64
+    if (g.M % 64 != 0 && g.M % 32 == 0 && g.N % 256 == 0 && g.K % 32 == 0 && g.K <= 256)
+        return launch_tile<1, 4, 1, 2, TA, TB>(g);   // 32 x 256: short-K products are store-bound anyway
     const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && tiles(128, 128) * 8 >= cus && !g.ep.any;
     if (tiles(128, 128) < cus && !splittable) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
     return launch_tile<2, 2, 2, 2, TA, TB>(g);                  // 128 x 128
