@@ -73,7 +73,9 @@ size_t jzhip_workspace_bytes(void);
  * against the gradient chain).  `jzhip_stream_create` makes a non-blocking
  * stream of default priority; `jzhip_event_record` marks the current stream's
  * position and `jzhip_stream_wait_event` makes everything issued afterwards
- * on the current stream wait for that mark.  Neither blocks the host. */
+ * on the current stream wait for that mark.  Neither blocks the host.
+ * `jzhip_stream_destroy` waits for the stream, frees the workspace the stream
+ * may have acquired and restores the null stream if it was the current one. */
 int jzhip_stream_create(void** out_stream);
 int jzhip_stream_destroy(void* hip_stream);
 int jzhip_event_create(void** out_event);

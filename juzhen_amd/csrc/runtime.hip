@@ -12,14 +12,15 @@ namespace {
 std::atomic<hipStream_t> g_stream{nullptr};
 std::atomic<int> g_cus{0};
 // One workspace per stream that has asked for one: launches on different
-// streams may run concurrently and must not share partial-result storage.
-constexpr int kMaxWorkspaces = 16;
+// streams may run concurrently and must not share partial-result storage.  A
+// slot is given back when its stream is destroyed through jzhip_stream_destroy.
+constexpr int kMaxWorkspaces = 64;
 struct WorkspaceSlot {
-    std::atomic<float*> ptr{nullptr};
+    std::atomic<float*> ptr{nullptr};   // nullptr: slot free
     hipStream_t owner = nullptr;
 };
 WorkspaceSlot g_ws[kMaxWorkspaces];
-std::atomic<int> g_ws_count{0};
+std::atomic<int> g_ws_count{0};         // slots ever used (scan bound)
 std::mutex g_ws_mutex;
 }  // namespace
 
@@ -42,22 +43,55 @@ int num_cus() {
 float* workspace() {
     const hipStream_t s = stream();
     const int n = g_ws_count.load(std::memory_order_acquire);
-    for (int i = 0; i < n; ++i)
-        if (g_ws[i].owner == s) return g_ws[i].ptr.load(std::memory_order_relaxed);
+    for (int i = 0; i < n; ++i) {
+        float* p = g_ws[i].ptr.load(std::memory_order_acquire);
+        if (p && g_ws[i].owner == s) return p;
+    }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     const int m = g_ws_count.load(std::memory_order_acquire);
-    for (int i = n; i < m; ++i)
-        if (g_ws[i].owner == s) return g_ws[i].ptr.load(std::memory_order_relaxed);
-    if (m == kMaxWorkspaces) return nullptr;
+    int slot = -1;
+    for (int i = 0; i < m; ++i) {
+        float* p = g_ws[i].ptr.load(std::memory_order_acquire);
+        if (p && g_ws[i].owner == s) return p;
+        if (!p && slot < 0) slot = i;
+    }
+    if (slot < 0) {
+        if (m == kMaxWorkspaces) return nullptr;
+        slot = m;
+    }
     void* p = nullptr;
     if (hipMalloc(&p, kWorkspaceFloats * sizeof(float)) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
-    g_ws[m].owner = s;
-    g_ws[m].ptr.store(static_cast<float*>(p), std::memory_order_relaxed);
-    g_ws_count.store(m + 1, std::memory_order_release);
+    g_ws[slot].owner = s;
+    g_ws[slot].ptr.store(static_cast<float*>(p), std::memory_order_release);
+    if (slot == m) g_ws_count.store(m + 1, std::memory_order_release);
     return static_cast<float*>(p);
+}
+
+// The stream is going away: wait for it and free its workspace.
+int release_workspace(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    const int m = g_ws_count.load(std::memory_order_acquire);
+    for (int i = 0; i < m; ++i) {
+        float* p = g_ws[i].ptr.load(std::memory_order_acquire);
+        if (p && g_ws[i].owner == s) {
+            int rc = rc_of(hipStreamSynchronize(s));
+            g_ws[i].ptr.store(nullptr, std::memory_order_release);
+            const int rc2 = rc_of(hipFree(p));
+            return rc ? rc : rc2;
+        }
+    }
+    return 0;
+}
+
+size_t workspace_total_bytes() {
+    size_t n = 0;
+    const int m = g_ws_count.load(std::memory_order_acquire);
+    for (int i = 0; i < m; ++i)
+        if (g_ws[i].ptr.load(std::memory_order_acquire)) n += kWorkspaceFloats * sizeof(float);
+    return n;
 }
 
 }  // namespace jz
@@ -135,9 +169,7 @@ JZ_API void* jzhip_get_stream(void) { return jz::stream(); }
 
 JZ_API int jzhip_synchronize(void) { return jz::rc_of(hipStreamSynchronize(jz::stream())); }
 
-JZ_API size_t jzhip_workspace_bytes(void) {
-    return static_cast<size_t>(jz::g_ws_count.load(std::memory_order_acquire)) * jz::kWorkspaceFloats * sizeof(float);
-}
+JZ_API size_t jzhip_workspace_bytes(void) { return jz::workspace_total_bytes(); }
 
 JZ_API int jzhip_stream_create(void** out_stream) {
     if (!out_stream) return -1;
@@ -150,7 +182,9 @@ JZ_API int jzhip_stream_create(void** out_stream) {
 JZ_API int jzhip_stream_destroy(void* hip_stream) {
     if (!hip_stream) return 0;
     if (jz::stream() == static_cast<hipStream_t>(hip_stream)) jzhip_set_stream(nullptr);
-    return jz::rc_of(hipStreamDestroy(static_cast<hipStream_t>(hip_stream)));
+    const int rc = jz::release_workspace(static_cast<hipStream_t>(hip_stream));
+    const int rc2 = jz::rc_of(hipStreamDestroy(static_cast<hipStream_t>(hip_stream)));
+    return rc ? rc : rc2;
 }
 JZ_API int jzhip_event_create(void** out_event) {
     if (!out_event) return -1;

@@ -791,3 +791,66 @@ def test_attention_fwd_bwd(gpu, d_k, heads, S, B, causal):
     assert np.array_equal(got[:, 0].reshape(-1), to_host(oq))
     assert np.array_equal(got[:, 1].reshape(-1), to_host(ok_))
     assert np.array_equal(got[:, 2].reshape(-1), to_host(ov))
+
+
+def test_second_stream_workspace_and_event_order(gpu):
+    """Calls on two streams with no host synchronisation between them: each stream
+    has its own split-K / reduction workspace, so concurrent launches give the
+    one-stream results to the bit, and an event recorded on one stream orders a
+    consumer on the other."""
+    from juzhen_amd import capi
+    lib = capi.load()
+    r = rng(77)
+    m, n, k = 256, 128, 8192              # two tiles: K is split, partials go to the workspace
+    A = to_dev(r.normal(size=m * k).astype(np.float32))
+    B = to_dev(r.normal(size=k * n).astype(np.float32))
+    X = to_dev(r.normal(size=512 * 16384).astype(np.float32))   # row sums in chunks: workspace again
+    want_c, want_r = dev_empty(m * n), dev_empty(512)
+    gpu.gemm(dptr(A), dptr(B), dptr(want_c), m, n, k, 0, 1, m, n, m, 1.0, 0.0)
+    gpu.sum_rows(dptr(want_r), dptr(X), 512, 16384, 512)
+    gpu.synchronize()
+    want_c, want_r = to_host(want_c), to_host(want_r)
+
+    main = lib.jzhip_get_stream()
+    side, ev = C.c_void_p(), C.c_void_p()
+    assert lib.jzhip_stream_create(C.byref(side)) == 0 and side.value
+    assert lib.jzhip_event_create(C.byref(ev)) == 0 and ev.value
+    before = lib.jzhip_workspace_bytes()
+    c_main = [dev_empty(m * n) for _ in range(8)]
+    c_side = [dev_empty(m * n) for _ in range(8)]
+    r_side = [dev_empty(512) for _ in range(8)]
+    try:
+        for i in range(8):
+            gpu.gemm(dptr(A), dptr(B), dptr(c_main[i]), m, n, k, 0, 1, m, n, m, 1.0, 0.0)
+            gpu.set_stream(side)
+            gpu.sum_rows(dptr(r_side[i]), dptr(X), 512, 16384, 512)
+            gpu.gemm(dptr(A), dptr(B), dptr(c_side[i]), m, n, k, 0, 1, m, n, m, 1.0, 0.0)
+            gpu.set_stream(main)
+        # producer on the side stream, consumer on the main stream behind an event
+        buf, out = dev_empty(1 << 20), dev_empty(1 << 20)
+        gpu.fill(dptr(out), 1 << 20, -1.0)
+        gpu.set_stream(side)
+        gpu.fill(dptr(buf), 1 << 20, 3.0)
+        gpu.event_record(ev)
+        gpu.set_stream(main)
+        gpu.stream_wait_event(ev)
+        gpu.affine(dptr(out), dptr(buf), 1 << 20, 2.0, 1.0)
+        gpu.set_stream(side)
+        gpu.synchronize()
+        gpu.set_stream(main)
+        gpu.synchronize()
+    finally:
+        lib.jzhip_set_stream(main)
+    during = lib.jzhip_workspace_bytes()
+    assert during == before + (64 << 20)   # the side stream's own
+    for i in range(8):
+        assert np.array_equal(to_host(c_main[i]), want_c)
+        assert np.array_equal(to_host(c_side[i]), want_c)
+        assert np.array_equal(to_host(r_side[i]), want_r)
+    assert np.array_equal(to_host(out), np.full(1 << 20, 7.0, np.float32))
+    assert lib.jzhip_event_record(None) == -1
+    assert lib.jzhip_stream_wait_event(None) == -1
+    assert lib.jzhip_stream_create(None) == -1 and lib.jzhip_event_create(None) == -1
+    assert lib.jzhip_event_destroy(ev) == 0
+    assert lib.jzhip_stream_destroy(side) == 0
+    assert lib.jzhip_workspace_bytes() == before   # given back with the stream
