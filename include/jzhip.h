@@ -189,6 +189,18 @@ int jzhip_slice_assign(float* dst, size_t dst_numrow, int dst_transpose,
                        const float* src, size_t src_numrow, int src_transpose,
                        size_t rows, size_t cols);
 
+/* No reference counterpart as a kernel: the reference's language-model demo
+ * feeds one-hot matrices through dense layers (examples/demo_transformer.cu,
+ * LinearLayer ml/layer.hpp:83-105), i.e. x0 = E*onehot(tokens) +
+ * P*onehot(positions) + b*ones.  A product with a one-hot matrix copies one
+ * column per token, so this lookup gives the same bits:
+ * out(:, n) = E(:, tokens[n]) + P(:, n % S) (+ bias), all column-major with
+ * leading dimension d; an id outside [0, vocab) selects no column.  (The
+ * gradient of the position table is jzhip_sum_rows over the (d*S) x (N/S)
+ * view of the gradient; the token table keeps the one-hot product.) */
+int jzhip_embedding_fwd(float* out, const float* E, const float* P, const float* bias,
+                        const int32_t* tokens, int d, int vocab, int S, int N);
+
 /* ── reductions ──────────────────────────────────────────────────────── */
 
 /* Sums over a physical column-major numrow x numcol buffer; replace the

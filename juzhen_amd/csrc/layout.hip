@@ -217,6 +217,63 @@ JZ_API int jzhip_stack_copy_rows(float* dst, size_t dst_numrow, size_t dst_row_o
                         static_cast<int>(src_numrow), src_transpose, 0, 0, rows, cols);
 }
 
+// Token + position embedding lookup: out(:, n) = E(:, tok[n]) + P(:, n % S) (+ bias).
+// The product of a table with a one-hot matrix copies one column per token
+// (every other term is an exact zero), so this equals the two one-hot products
+// and the bias broadcast bit for bit; an id outside [0, vocab) selects no
+// column, as an all-zero one-hot column would.
+namespace jz {
+namespace {
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void embedding_fwd_kernel(float* __restrict__ out, const float* __restrict__ E,
+                                                               const float* __restrict__ P,
+                                                               const float* __restrict__ bias,
+                                                               const int32_t* __restrict__ tokens, int d, int vocab,
+                                                               FastDiv dS, int S, FastDiv dD, size_t total) {
+    const int dv = d / VEC;   // dD divides by dv
+    const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t n = fdiv(static_cast<uint32_t>(i), dD);
+    const uint32_t r = (static_cast<uint32_t>(i) - n * dv) * VEC;
+    const uint32_t pos = n - fdiv(n, dS) * S;
+    const int32_t tok = tokens[n];
+    const bool live = tok >= 0 && tok < vocab;
+    if constexpr (VEC == 4) {
+        float4 e = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) e = *reinterpret_cast<const float4*>(E + static_cast<size_t>(tok) * d + r);
+        const float4 p = *reinterpret_cast<const float4*>(P + static_cast<size_t>(pos) * d + r);
+        float4 v = make_float4(e.x + p.x, e.y + p.y, e.z + p.z, e.w + p.w);
+        if (bias) {
+            const float4 b = *reinterpret_cast<const float4*>(bias + r);
+            v = make_float4(v.x + b.x, v.y + b.y, v.z + b.z, v.w + b.w);
+        }
+        *reinterpret_cast<float4*>(out + static_cast<size_t>(n) * d + r) = v;
+    } else {
+        float v = (live ? E[static_cast<size_t>(tok) * d + r] : 0.0f) + P[static_cast<size_t>(pos) * d + r];
+        if (bias) v = v + bias[r];
+        out[static_cast<size_t>(n) * d + r] = v;
+    }
+}
+}  // namespace
+}  // namespace jz
+
+JZ_API int jzhip_embedding_fwd(float* out, const float* E, const float* P, const float* bias, const int32_t* tokens,
+                               int d, int vocab, int S, int N) {
+    if (!out || !E || !P || !tokens || d <= 0 || vocab <= 0 || S <= 0 || N <= 0) return -1;
+    const size_t elems = static_cast<size_t>(d) * N;
+    if (elems >= (size_t(1) << 31)) return -1;
+    const bool vec = d % 4 == 0 && aligned16(out) && aligned16(E) && aligned16(P) && (!bias || aligned16(bias));
+    if (vec) {
+        const size_t total = elems / 4;
+        embedding_fwd_kernel<4><<<grid_cover(total, kBlock), kBlock, 0, stream()>>>(
+            out, E, P, bias, tokens, d, vocab, make_fastdiv(S), S, make_fastdiv(d / 4), total);
+    } else {
+        embedding_fwd_kernel<1><<<grid_cover(elems, kBlock), kBlock, 0, stream()>>>(
+            out, E, P, bias, tokens, d, vocab, make_fastdiv(S), S, make_fastdiv(d), elems);
+    }
+    return launch_rc();
+}
+
 // slice get / set (cpp/hipmatrix.cpp:268-324).
 JZ_API int jzhip_slice_extract(float* dst, size_t dst_numrow, const float* src, size_t src_numrow,
                                int src_transpose, size_t rstart, size_t cstart, size_t rows,

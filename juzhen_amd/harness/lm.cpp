@@ -9,9 +9,12 @@
 // options it reproduces a stack built from the reference's own classes
 // (examples/demo_transformer.cu:214-383: one-hot token+position input into a
 // LinearLayer, TransformerLayers, a LinearLayer head, LogisticLayer loss).
-// Embedding, positional table and head are expressed as GEMMs against one-hot
-// matrices, the reference's formulation (demo_transformer.cu:133-149), which
-// keeps them deterministic and checkable against the CPU path.
+// The reference feeds one-hot token and position matrices through a dense layer
+// (demo_transformer.cu:133-149).  A product with a one-hot matrix copies one
+// column per token, so the forward embedding is a lookup with the same bits,
+// and the position-table gradient is a sum over sequences; the token-table
+// gradient and the head stay products (against the one-hot matrix and the
+// logits gradient), deterministic and checkable against the CPU path.
 //
 // Everything is preallocated at creation; a step issues only library calls
 // (no allocation, no host synchronisation).  The loss stays on the device until
@@ -75,8 +78,8 @@ struct Model {
     std::vector<float*> owned;
     Arena arena[kGroups];
     int E = -1, P = -1, be = -1, Wp = -1, bp = -1;
-    float *oh_tok = nullptr, *oh_pos = nullptr, *x0 = nullptr, *logits = nullptr, *dlogits = nullptr;
-    int32_t* targets = nullptr;
+    float *oh_tok = nullptr, *x0 = nullptr, *logits = nullptr, *dlogits = nullptr;
+    int32_t *tokens = nullptr, *targets = nullptr;
     float* loss = nullptr;
     // backward scratch shared by all blocks
     // (the ones the weight-gradient products read exist twice, alternating by
@@ -162,10 +165,9 @@ inline void gemm_tail(Model& M, const float* A, bool ta, const float* B, float* 
 void forward(Model& M) {
     const Config& c = M.c;
     const int d = c.d_model, N = M.N, ff = c.d_ff;
-    // x0 = E * onehot(tokens) + P * onehot(positions) [+ embedding bias]
-    gemm(M, M.t[M.E].w, false, M.oh_tok, false, M.x0, d, N, c.vocab);
-    gemm_tail(M, M.t[M.P].w, false, M.oh_pos, M.x0, d, N, c.seq, M.be >= 0 ? M.t[M.be].w : nullptr, 0, nullptr,
-              nullptr, 1.0f);
+    // x0 = E * onehot(tokens) + P * onehot(positions) [+ embedding bias], as a lookup
+    M.ck(jzhip_embedding_fwd(M.x0, M.t[M.E].w, M.t[M.P].w, M.be >= 0 ? M.t[M.be].w : nullptr, M.tokens, d, c.vocab,
+                             c.seq, N));
     const float* x = M.x0;
     for (Block& b : M.blocks) {
         M.ck(jzhip_layernorm_fwd(b.x1, b.xhat1, b.inv1, x, M.t[b.g1].w, M.t[b.be1].w, d, N));
@@ -316,7 +318,8 @@ void backward(Model& M, bool update) {
     lanes.join();
     // embedding tables: dE (+)= dx0 * onehot_tok^T, dP = dx0 * onehot_pos^T
     gemm(M, dy, false, M.oh_tok, true, M.t[M.E].g, d, V, N, c.tied ? 1.0f : 0.0f);
-    gemm(M, dy, false, M.oh_pos, true, M.t[M.P].g, d, c.seq, N);
+    // (token n = b*S + s: the (d, N) gradient is a (d*S) x B matrix whose row sums are dP)
+    M.ck(jzhip_sum_rows(M.t[M.P].g, dy, d * c.seq, c.batch, d * c.seq));
     if (M.be >= 0) M.ck(jzhip_sum_rows(M.t[M.be].g, dy, d, N, d));
     if (update) {
         step_group(M, kDecay);
@@ -377,7 +380,7 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
         b.F1 = M->alloc(fN); b.F1a = M->alloc(fN); b.out = M->alloc(dN);
     }
     M->oh_tok = M->alloc(static_cast<size_t>(V) * N);
-    M->oh_pos = M->alloc(static_cast<size_t>(S) * N);
+    M->tokens = reinterpret_cast<int32_t*>(M->alloc(N));
     M->x0 = M->alloc(dN);
     M->logits = M->alloc(static_cast<size_t>(V) * N);
     M->dlogits = M->alloc(static_cast<size_t>(V) * N);
@@ -450,8 +453,8 @@ JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
     Model* M = static_cast<Model*>(h);
     const Config& c = M->c;
     const int N = M->N;
-    std::vector<float> oh(static_cast<size_t>(c.vocab) * N, 0.0f), op(static_cast<size_t>(c.seq) * N, 0.0f);
-    std::vector<int32_t> tg(N);
+    std::vector<float> oh(static_cast<size_t>(c.vocab) * N, 0.0f);
+    std::vector<int32_t> tk(N), tg(N);
     for (int b = 0; b < c.batch; ++b)
         for (int s = 0; s < c.seq; ++s) {
             const int n = b * c.seq + s;
@@ -459,11 +462,11 @@ JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
             const int32_t nxt = tokens[static_cast<size_t>(b) * (c.seq + 1) + s + 1];
             if (tok < 0 || tok >= c.vocab || nxt < 0 || nxt >= c.vocab) return -1;
             oh[static_cast<size_t>(n) * c.vocab + tok] = 1.0f;
-            op[static_cast<size_t>(n) * c.seq + s] = 1.0f;
+            tk[n] = tok;
             tg[n] = nxt;
         }
     int rc = jzhip_memcpy_h2d(M->oh_tok, oh.data(), oh.size());
-    if (rc == 0) rc = jzhip_memcpy_h2d(M->oh_pos, op.data(), op.size());
+    if (rc == 0) rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->tokens), reinterpret_cast<const float*>(tk.data()), N);
     if (rc == 0) rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->targets), reinterpret_cast<const float*>(tg.data()), N);
     return rc;
 }

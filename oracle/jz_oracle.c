@@ -195,6 +195,25 @@ JZO_API void jzo_dgelu_mul(float* out, const float* pre, const float* up, size_t
     }
 }
 
+/* Embedding lookup, defined as the reference's one-hot formulation
+ * (examples/demo_transformer.cu:133-149 builds one-hot token and position
+ * columns; LinearLayer::eval ml/layer.hpp:83-86 is W*x + b*ones):
+ * out(:, n) = E*e_tok[n] + P*e_(n % S) + bias, where a product with a one-hot
+ * column copies the selected column.  An id outside [0, vocab) gives the zero
+ * column, as an all-zero one-hot column would. */
+JZO_API void jzo_embedding_fwd(float* out, const float* E, const float* P, const float* bias,
+                               const int32_t* tokens, int d, int vocab, int S, int N) {
+    for (int n = 0; n < N; n++) {
+        int tok = tokens[n], pos = n % S;
+        for (int i = 0; i < d; i++) {
+            float e = (tok >= 0 && tok < vocab) ? E[(size_t)tok * d + i] : 0.0f;
+            float v = e + P[(size_t)pos * d + i];
+            if (bias) v = v + bias[i];
+            out[(size_t)n * d + i] = v;
+        }
+    }
+}
+
 /* ── reductions ───────────────────────────────────────────────────────── */
 
 /* sum(M, dim) (cpp/matrix.hpp:74-91): GEMV with a ones vector on the physical

@@ -854,3 +854,42 @@ def test_second_stream_workspace_and_event_order(gpu):
     assert lib.jzhip_event_destroy(ev) == 0
     assert lib.jzhip_stream_destroy(side) == 0
     assert lib.jzhip_workspace_bytes() == before   # given back with the stream
+
+
+@pytest.mark.parametrize("d,V,S,B,with_bias", [(512, 256, 256, 4, 0), (64, 13, 8, 3, 1), (30, 5, 7, 2, 1), (4, 3, 1, 9, 0)])
+def test_embedding_fwd(gpu, oracle_lib, d, V, S, B, with_bias):
+    """Lookup against the oracle (bit-exact: one addition or two per element) and
+    against the one-hot products it replaces, through the library's own GEMM."""
+    r = rng(d + V)
+    N = S * B
+    E = r.normal(size=V * d).astype(np.float32)
+    Pm = r.normal(size=S * d).astype(np.float32)
+    bias = r.normal(size=d).astype(np.float32)
+    tok = r.integers(0, V, N).astype(np.int32)
+    if N > 2:
+        tok[1], tok[2] = -3, V + 5
+    want = np.empty(N * d, np.float32)
+    oracle_lib.jzo_embedding_fwd(hptr(want), hptr(E), hptr(Pm), hptr(bias) if with_bias else None, hptr(tok), d, V, S, N)
+    import torch
+    dtok = torch.from_numpy(tok).cuda()
+    dE, dP, db = to_dev(E), to_dev(Pm), to_dev(bias)
+    out = dev_empty(N * d)
+    gpu.embedding_fwd(dptr(out), dptr(dE), dptr(dP), dptr(db) if with_bias else None, dptr(dtok), d, V, S, N)
+    got = to_host(out)
+    assert np.array_equal(got, want)
+    # the two one-hot products (+ bias broadcast) on the GPU
+    oh = np.zeros((N, V), np.float32)
+    for n, t in enumerate(tok):
+        if 0 <= t < V:
+            oh[n, t] = 1.0
+    op = np.zeros((N, S), np.float32)
+    op[np.arange(N), np.arange(N) % S] = 1.0
+    x0 = dev_empty(N * d)
+    gpu.gemm(dptr(dE), dp(oh.ravel()), dptr(x0), d, N, V, 0, 0, d, V, d, 1.0, 0.0)
+    gpu.gemm(dptr(dP), dp(op.ravel()), dptr(x0), d, N, S, 0, 0, d, S, d, 1.0, 1.0)
+    if with_bias:
+        gpu.add_bias(dptr(x0), dptr(db), d, N)
+    assert np.array_equal(to_host(x0), got)
+    from juzhen_amd import capi
+    assert capi.load().jzhip_embedding_fwd(dptr(out), None, dptr(dP), None, dptr(dtok), d, V, S, N) == -1
+    assert capi.load().jzhip_embedding_fwd(dptr(out), dptr(dE), dptr(dP), None, dptr(dtok), 0, V, S, N) == -1

@@ -357,3 +357,34 @@ def test_gelu_closed_form(oracle_lib):
     num = [(0.5 * (v + eps) * (1 + erf((v + eps) / sqrt(2))) - 0.5 * (v - eps) * (1 + erf((v - eps) / sqrt(2)))) / (2 * eps)
            for v in x.astype(np.float64)]
     assert np.allclose(d, num, rtol=1e-4, atol=1e-6)
+
+
+def test_embedding_lookup_is_the_one_hot_product(oracle_lib):
+    """The lookup is defined by the reference's one-hot formulation
+    (examples/demo_transformer.cu:133-149): it must equal E*onehot(tok) +
+    P*onehot(pos) + bias computed by the oracle's own GEMM, bit for bit (every
+    product with a zero adds an exact zero), including ids outside the table."""
+    o = oracle_lib
+    r = np.random.default_rng(11)
+    d, V, S, B = 12, 7, 5, 3
+    N = S * B
+    E = r.normal(size=(V, d)).astype(np.float32)       # row v = column v of the (d, V) table
+    Pm = r.normal(size=(S, d)).astype(np.float32)
+    bias = r.normal(size=d).astype(np.float32)
+    tok = r.integers(0, V, N).astype(np.int32)
+    tok[3], tok[7] = -1, V                             # invalid ids: zero column
+    oh = np.zeros((N, V), np.float32)
+    for n, t in enumerate(tok):
+        if 0 <= t < V:
+            oh[n, t] = 1.0
+    op = np.zeros((N, S), np.float32)
+    op[np.arange(N), np.arange(N) % S] = 1.0
+    want = np.zeros((N, d), np.float32)
+    o.jzo_gemm(0, 0, d, N, V, 1.0, hptr(E), d, hptr(oh), V, 0.0, hptr(want), d)
+    o.jzo_gemm(0, 0, d, N, S, 1.0, hptr(Pm), d, hptr(op), S, 1.0, hptr(want), d)
+    got = np.empty((N, d), np.float32)
+    o.jzo_embedding_fwd(hptr(got), hptr(E), hptr(Pm), None, hptr(tok), d, V, S, N)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got[3], Pm[3 % S]) and np.array_equal(got[7], Pm[7 % S])
+    o.jzo_embedding_fwd(hptr(got), hptr(E), hptr(Pm), hptr(bias), hptr(tok), d, V, S, N)
+    assert np.array_equal(got, want + bias[None, :])
