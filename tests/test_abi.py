@@ -66,3 +66,24 @@ def test_argument_validation_without_gpu():
     assert lib.jzhip_fill(None, 0, 1.0) == 0          # empty input is a no-op
     assert lib.jzhip_error_string(-1).decode().startswith("jzhip")
     assert lib.jzhip_version() >= 100
+
+
+def test_product_code_never_reaches_into_the_oracle():
+    """The oracle is test infrastructure: nothing that ships (the package's Python,
+    the kernels, the C++ mirror, the train-step harness) may import, include or
+    link it.  (juzhen_amd/build.py only names oracle/_ref as the output directory
+    of the reference-program builds.)"""
+    import re
+    root = Path(__file__).resolve().parent.parent
+    bad = []
+    for p in (root / "juzhen_amd").rglob("*"):
+        if p.is_dir() or "build" in p.relative_to(root).parts[1:2] or p.suffix not in (
+                ".py", ".hip", ".hpp", ".cuh", ".cpp", ".cu", ".h"):
+            continue
+        text = p.read_text(errors="ignore")
+        if p.suffix == ".py":
+            if re.search(r"^\s*(import oracle|from oracle)", text, re.M):
+                bad.append(str(p))
+        elif re.search(r'#include\s*[<"][^>"]*(oracle|jz_oracle|ref_shim)', text) or "jzo_" in text or "jzref_" in text:
+            bad.append(str(p))
+    assert not bad, bad
