@@ -560,16 +560,40 @@ __global__ __launch_bounds__(kBlock) void gemv_n_partial_kernel(const float* A, 
     }
 }
 
-__global__ __launch_bounds__(kBlock) void gemv_n_combine_kernel(float* y, const float* part, int m,
-                                                                int chunks, size_t incy,
-                                                                float alpha, float beta) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= m) return;
+// y[i] = alpha * sum_c part[c*m + i] + beta*y[i]: 64 outputs per workgroup, its
+// sixteen waves taking interleaved chunks (four loads in flight each) and
+// meeting in LDS; fixed order, so the result is deterministic.
+constexpr int kGemvCombineBlock = 1024;
+__global__ __launch_bounds__(kGemvCombineBlock) void gemv_n_combine_kernel(float* y, const float* part, int m,
+                                                                           int chunks, size_t incy, float alpha,
+                                                                           float beta) {
+    constexpr int NW = kGemvCombineBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int i = blockIdx.x * kWave + lane;
     float acc = 0.f;
-    for (int c = 0; c < chunks; ++c) acc += part[static_cast<size_t>(c) * m + i];
-    float r = alpha * acc;
-    if (beta != 0.0f) r += beta * y[i * incy];
-    y[i * incy] = r;
+    if (i < m) {
+        const float* p = part + i;
+        int c = wave;
+        for (; c + 3 * NW < chunks; c += 4 * NW) {
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = p[static_cast<size_t>(c + u * NW) * m];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc += x[u];
+        }
+        for (; c < chunks; c += NW) acc += p[static_cast<size_t>(c) * m];
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && i < m) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[w][lane];
+        float r = alpha * sum;
+        if (beta != 0.0f) r += beta * y[i * incy];
+        y[i * incy] = r;
+    }
 }
 
 // y(rows x cols) += b[i]
@@ -684,7 +708,7 @@ int launch_tile(const GemmArgs& g) {
     int splits = 1;
     const long long tiles = static_cast<long long>(tiles_m) * tiles_n * g.batch * g.batch2;
     const long long cus = num_cus();
-    if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 1024 && !g.ep.any) {
+    if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 256 && !g.ep.any) {
         splits = static_cast<int>((cus * 2 + tiles - 1) / tiles);
         // The K chunk is the fastest-varying part of the workgroup id and
         // workgroups are dealt round-robin to 8 XCDs: with a count that divides 8
@@ -692,7 +716,10 @@ int launch_tile(const GemmArgs& g) {
         // index and the operand panels of a chunk are fetched into one L2.
         auto xcd_friendly = [](int n) { return n <= 2 ? n : n <= 4 ? 4 : (n + 7) / 8 * 8; };
         splits = xcd_friendly(splits);
-        const int max_by_k = g.K / 256;
+        // at least sixteen K steps per chunk; a short K (skinny first-layer
+        // gradients) is still cut, down to four steps, because a handful of
+        // workgroups walking it alone only wait for their loads
+        const int max_by_k = g.K >= 1024 ? g.K / 256 : g.K / 64;
         const size_t per = static_cast<size_t>(g.M) * g.N;
         while (splits > 1 && (splits > max_by_k || per * splits > kWorkspaceFloats))
             splits = splits > 8 ? splits - 8 : splits / 2;
@@ -815,7 +842,8 @@ int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans
     float* part = workspace();
     if (!part) return -2;
     gemv_n_partial_kernel<<<dim3(row_blocks, chunks), kBlock, 0, s>>>(A, x, part, m, n, lda, incx, chunk_len);
-    gemv_n_combine_kernel<<<(m + kBlock - 1) / kBlock, kBlock, 0, s>>>(y, part, m, chunks, incy, alpha, beta);
+    gemv_n_combine_kernel<<<(m + kWave - 1) / kWave, kGemvCombineBlock, 0, s>>>(y, part, m, chunks, incy, alpha,
+                                                                                beta);
     return launch_rc();
 }
 
