@@ -1,7 +1,8 @@
 // Batched causal self-attention core for TransformerLayer<ROCMfloat>: replaces
 // the reference's per-(head, sequence) slice loop with its host-side mask
-// writes (ml/layer.hpp:2967-3006, 3329-3363) by five batched launches forward
-// and backward.  Same mathematics and the same buffer layouts as the
+// writes (ml/layer.hpp:2967-3006, 3329-3363) by one fused launch forward and
+// three launches backward (batched products and softmax kernels for shapes the
+// fused kernel does not cover).  Same mathematics and the same buffer layouts as the
 // reference's CUDA path (ml/layer.hpp:2880-2927, 3214-3283):
 //   Q, K, V, H, dQ, dK, dV, dH : (d_k, S*B) column-major, head hh owns rows
 //                                [hh*d_h, (hh+1)*d_h), sequence b columns [b*S, (b+1)*S)

@@ -4,8 +4,9 @@
 // broadcasts, matrix-vector products) and a strided-batched form for attention.
 //
 // Tiled kernel: a workgroup of four wavefronts owns a BM x BN tile of C and
-// walks K in steps of BK=16 through two LDS buffers (global loads for step
-// t+1 are in flight while step t is multiplied).  Both operand tiles are kept
+// walks K in steps of BK=16 through two LDS buffers (the global loads of step
+// t+2 are in flight and step t+1 is being stored to LDS while step t is
+// multiplied).  Both operand tiles are kept
 // in LDS as [k][m] / [k][n] so one v_mfma_f32_32x32x2_f32 operand is a single
 // conflict-free 32-lane row read.  The MFMA is issued with B^T as its first
 // operand and A^T as its second, i.e. it produces C^T tiles: each accumulator
