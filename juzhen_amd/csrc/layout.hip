@@ -74,9 +74,15 @@ __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
     int rel_b, size_t R, size_t C, unsigned tiles_r, float s1, float s2) {
     __shared__ float ta[kTileV][kTileV + 1];
     __shared__ float tb[OP == kOpCopy ? 1 : kTileV][kTileV + 1];
+    // Diagonal tile order: consecutive workgroups step along the rows and the
+    // columns at once.  With a power-of-two leading dimension, tiles that differ
+    // in one index only are a multiple of 2 MB apart in the transposed operand
+    // and land on the same memory channels.
     const unsigned tile = blockIdx.x;
-    const size_t r0 = static_cast<size_t>(tile % tiles_r) * kTileV;
-    const size_t c0 = static_cast<size_t>(tile / tiles_r) * kTileV;
+    const unsigned ti = tile % tiles_r, tj0 = tile / tiles_r;
+    const unsigned tiles_c = gridDim.x / tiles_r;
+    const size_t r0 = static_cast<size_t>(ti) * kTileV;
+    const size_t c0 = static_cast<size_t>((tj0 + ti) % tiles_c) * kTileV;
     const int q = threadIdx.x % 16;    // float4 slot along the contiguous index
     const int l = threadIdx.x / 16;    // line inside a pass of 16
     auto stage = [&](float (*t)[kTileV + 1], const float* x, size_t ldx) {
