@@ -3,8 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--serial] [--no-cpu-baseline]
 
-Workload (BASELINE.json configs[3]): character-level LM, vocab 256 byte tokens
-drawn from Zipf(s=1.1), context 256, batch 64 (16 384 tokens per step), 6
+Workload (the character-level transformer configuration): language model over
+vocab 256 byte tokens drawn from Zipf(s=1.1), context 256, batch 64 (16 384 tokens per step), 6
 pre-LayerNorm decoder blocks, d_model 512, 8 heads, causal softmax attention,
 FFN 2048 with GELU, tied embeddings, learned positional table, cross-entropy,
 AdamW (lr 3e-4, wd 0.01), fp32 everywhere.  One step = forward + loss +
