@@ -259,6 +259,7 @@ __device__ __forceinline__ bool rowgrid_item(const RowGrid& rg, int& x, int& y, 
 // zero-filled where the window hangs over the border) are staged in LDS; then
 // every wave writes whole 1 KB pieces of patch columns: lane l owns k = k0+4l..k0+4l+3
 // for all pw, so its four LDS offsets are computed once.
+template <int NSUB>
 __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __restrict__ img,
                                                              float* __restrict__ col, PatchGeom g,
                                                              int WT, FastDiv dWT, FastDiv dkH) {
@@ -267,8 +268,11 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
     // (plain dispatch order, chunks of one patch row spread over the XCDs: the
     // kernel is write-dominated and this order measured faster than the
     // XCD-grouped one the scatter kernel uses)
+    // one 256-wide piece per workgroup; with NSUB = 2 the last workgroup also takes
+    // the short remainder that would otherwise leave a workgroup mostly idle
     const int k0 = blockIdx.x * kPatchChunk;
-    const int k1 = (k0 + kPatchChunk) < g.K ? (k0 + kPatchChunk) : g.K;
+    const int k1 = (NSUB == 2 && blockIdx.x == gridDim.x - 1) ? g.K
+                                                                : ((k0 + kPatchChunk) < g.K ? (k0 + kPatchChunk) : g.K);
     const int ph = blockIdx.y, n = blockIdx.z;
     const int c_lo = fdiv(static_cast<uint32_t>(k0), g.dKK);
     const int c_hi = fdiv(static_cast<uint32_t>(k1 - 1), g.dKK);
@@ -301,23 +305,36 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
     }
     __syncthreads();
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int kq = k0 + 4 * lane;
-    if (kq >= k1) return;
-    int off[4];
+    // lane l owns k = k0 + 256*u + 4l .. +3 of every 256-wide piece u
+    int off[NSUB][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t k = static_cast<uint32_t>(kq + j);
-        const uint32_t ch = fdiv(k, g.dKK);
-        const uint32_t rem = k - ch * KK;
-        const uint32_t kh = fdiv(rem, g.dkW);
-        const uint32_t kw = rem - kh * g.kW;
-        off[j] = static_cast<int>(((ch - c_lo) * g.kH + kh) * WT + kw);
+    for (int u = 0; u < NSUB; ++u) {
+        const int kq = k0 + u * kPatchChunk + 4 * lane;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            off[u][j] = -1;
+            if (kq < k1) {
+                const uint32_t k = static_cast<uint32_t>(kq + j);
+                const uint32_t ch = fdiv(k, g.dKK);
+                const uint32_t rem = k - ch * KK;
+                const uint32_t kh = fdiv(rem, g.dkW);
+                const uint32_t kw = rem - kh * g.kW;
+                off[u][j] = static_cast<int>(((ch - c_lo) * g.kH + kh) * WT + kw);
+            }
+        }
     }
-    float* dst = col + (static_cast<size_t>(n) * g.P + static_cast<size_t>(ph) * g.Wp) * g.K + kq;
+    float* dst = col + (static_cast<size_t>(n) * g.P + static_cast<size_t>(ph) * g.Wp) * g.K + k0 + 4 * lane;
     for (int pw = wave; pw < g.Wp; pw += kBlock / kWave) {
         const int w = pw * g.stride_w;
-        const float4 v = make_float4(tile[off[0] + w], tile[off[1] + w], tile[off[2] + w], tile[off[3] + w]);
-        *reinterpret_cast<float4*>(dst + static_cast<size_t>(pw) * g.K) = v;
+        float* d = dst + static_cast<size_t>(pw) * g.K;
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u) {
+            if (off[u][0] >= 0) {
+                const float4 v = make_float4(tile[off[u][0] + w], tile[off[u][1] + w], tile[off[u][2] + w],
+                                             tile[off[u][3] + w]);
+                *reinterpret_cast<float4*>(d + u * kPatchChunk) = v;
+            }
+        }
     }
 }
 
@@ -466,11 +483,18 @@ int gather_patches(const float* img, float* col, const PatchGeom& g) {
     if (static_cast<size_t>(g.C) * g.H * g.W * g.N >= (size_t(1) << 31)) return -1;
     if (g.K % 4 == 0 && g.K >= 64 && aligned16(col) && g.N <= 65535 && g.Hp <= 65535) {
         const int WT = (g.Wp - 1) * g.stride_w + g.kW;
-        const int nch_max = kPatchChunk / (g.kH * g.kW) + 2;
+        // a last piece of at most 64 k is folded into the workgroup before it (a
+        // workgroup of its own would run with a quarter of its lanes; folding a
+        // longer remainder costs more in LDS per workgroup than it saves)
+        const int pieces = (g.K + kPatchChunk - 1) / kPatchChunk;
+        const bool fold = pieces >= 2 && g.K - (pieces - 1) * kPatchChunk <= kPatchChunk / 4;
+        const int nch_max = (fold ? kPatchChunk + kPatchChunk / 4 : kPatchChunk) / (g.kH * g.kW) + 2;
         const size_t lds = static_cast<size_t>(nch_max) * g.kH * WT * sizeof(float);
         if (lds <= 48 * 1024) {
-            dim3 grid((g.K + kPatchChunk - 1) / kPatchChunk, g.Hp, g.N);
-            im2col_rows_kernel<<<grid, kBlock, lds, stream()>>>(img, col, g, WT, make_fastdiv(WT), make_fastdiv(g.kH));
+            dim3 grid(fold ? pieces - 1 : pieces, g.Hp, g.N);
+            const FastDiv dWT = make_fastdiv(WT), dkH = make_fastdiv(g.kH);
+            if (fold) im2col_rows_kernel<2><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, dkH);
+            else im2col_rows_kernel<1><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, dkH);
             return launch_rc();
         }
     }
