@@ -34,6 +34,20 @@ __global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const floa
         if constexpr (VEC == 4) {
             const int v_end = r_begin + ((r_end - r_begin) / 4) * 4;
             int r = r_begin + lane * 4;
+            // four float4 loads in flight per lane (4 KB per wave), then two
+            float acc2 = 0.f, acc3 = 0.f;
+            for (; r + 3 * kWave * 4 < v_end; r += 4 * kWave * 4) {
+                const float4 x = *reinterpret_cast<const float4*>(p + r);
+                const float4 y = *reinterpret_cast<const float4*>(p + r + kWave * 4);
+                const float4 z = *reinterpret_cast<const float4*>(p + r + 2 * kWave * 4);
+                const float4 w = *reinterpret_cast<const float4*>(p + r + 3 * kWave * 4);
+                acc0 += (x.x + x.y) + (x.z + x.w);
+                acc1 += (y.x + y.y) + (y.z + y.w);
+                acc2 += (z.x + z.y) + (z.z + z.w);
+                acc3 += (w.x + w.y) + (w.z + w.w);
+            }
+            acc0 += acc2;
+            acc1 += acc3;
             for (; r + kWave * 4 < v_end; r += 2 * kWave * 4) {
                 const float4 x = *reinterpret_cast<const float4*>(p + r);
                 const float4 y = *reinterpret_cast<const float4*>(p + r + kWave * 4);
