@@ -49,18 +49,6 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // [d][key], M2 as [key][d] (pitch DH+4); X1 fragments are read straight from
 // global memory (each lane DH/4 consecutive floats of its query's column: lane
 // group kq contracts d in [kq*DH/4, (kq+1)*DH/4)).
-// e^x for x <= 0 through the hardware exp2: x*log2(e) is formed with its
-// rounding error (fma) and the error is folded back in, which keeps the result
-// within about 2 ulp; libm's expf costs an order of magnitude more
-// instructions and made the softmax the longest phase of the kernel.
-__device__ __forceinline__ float exp_neg(float x) {
-    const float l2e = 1.44269504088896341f;
-    x = x > -100.0f ? x : -100.0f;   // masked scores (-1e9) end as an exact +0
-    const float t = x * l2e;
-    const float err = fmaf(x, l2e, -t) + x * 1.92596299112661746e-8f;   // low bits of the product and of log2(e)
-    return __builtin_amdgcn_exp2f(t) * (1.0f + 0.693147180559945309f * err);
-}
-
 constexpr int kMaxKeys = 256;      // S <= 256
 constexpr int kAttnThreads = 1024;  // sixteen waves, one group of 16 queries each, four per SIMD
 // pitch of the [d][key] staging, whatever S is: the four lane groups of a

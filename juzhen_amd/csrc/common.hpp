@@ -112,6 +112,19 @@ __device__ __forceinline__ size_t wave_end(size_t n, size_t w, size_t nw) {
     return e < n ? e : n;
 }
 
+// e^x for x <= 0 through the hardware exp2: x*log2(e) is formed with its
+// rounding error (fma) and the error is folded back in, which keeps the result
+// within about 2 ulp; libm's expf costs an order of magnitude more
+// instructions and made the softmax the longest phase of the attention kernel
+// (and a third of the time of the long-column softmax).
+__device__ __forceinline__ float exp_neg(float x) {
+    const float l2e = 1.44269504088896341f;
+    x = x > -100.0f ? x : -100.0f;   // masked scores (-1e9) end as an exact +0
+    const float t = x * l2e;
+    const float err = fmaf(x, l2e, -t) + x * 1.92596299112661746e-8f;   // low bits of the product and of log2(e)
+    return __builtin_amdgcn_exp2f(t) * (1.0f + 0.693147180559945309f * err);
+}
+
 // Unsigned division by a runtime-uniform divisor via multiply-high.
 // Valid for n < 2^31 and 1 <= d < 2^31.
 struct FastDiv {

@@ -6,7 +6,7 @@
 // kept in registers, and written once: 8 bytes per element.
 //
 // Arithmetic follows the reference expression: m = max(x) (floor -1e30f),
-// e = expf(x - m), p = e * (1.0f / (sum(e) + 1e-12f)).
+// e = exp(x - m) (hardware exp2 with the argument's rounding error folded back in), p = e * (1.0f / (sum(e) + 1e-12f)).
 #include "common.hpp"
 
 #include <cmath>
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_kernel(float* out, const 
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int r = lane + v * kWave;
-            x[v] = (r < numrow) ? expf(x[v] - m) : 0.f;
+            x[v] = (r < numrow) ? exp_neg(x[v] - m) : 0.f;
             s += x[v];
         }
         s = wave_sum(s);
@@ -84,10 +84,10 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_long_kernel(float* out, c
         for (int r = threadIdx.x; r < numrow; r += kBlock) m = m > p[r] ? m : p[r];
         m = block_allreduce<kBlock / kWave>(m, MaxOp{}, red, -1e30f);
         float s = 0.f;
-        for (int r = threadIdx.x; r < numrow; r += kBlock) s += expf(p[r] - m);
+        for (int r = threadIdx.x; r < numrow; r += kBlock) s += exp_neg(p[r] - m);
         s = block_allreduce<kBlock / kWave>(s, SumOp{}, red, 0.f);
         const float inv = 1.0f / (s + 1e-12f);
-        for (int r = threadIdx.x; r < numrow; r += kBlock) q[r] = expf(p[r] - m) * inv;
+        for (int r = threadIdx.x; r < numrow; r += kBlock) q[r] = exp_neg(p[r] - m) * inv;
     }
 }
 
@@ -121,8 +121,8 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_block_kernel(float* out, 
         for (int v = 0; v < NV4; ++v) {
             const int r = (threadIdx.x + v * kBlock) * 4;
             if (r < numrow) {
-                x[v].x = expf(x[v].x - m); x[v].y = expf(x[v].y - m);
-                x[v].z = expf(x[v].z - m); x[v].w = expf(x[v].w - m);
+                x[v].x = exp_neg(x[v].x - m); x[v].y = exp_neg(x[v].y - m);
+                x[v].z = exp_neg(x[v].z - m); x[v].w = exp_neg(x[v].w - m);
                 s += (x[v].x + x[v].y) + (x[v].z + x[v].w);
             }
         }
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(float* out, const 
     float* q = out + static_cast<size_t>(blockIdx.y) * batch_stride;
     const bool live = row < numrow;
     // with a causal mask only keys <= query (columns <= row) are unmasked;
-    // masked entries contribute expf(-1e9 - m) == 0 exactly and are written as 0
+    // masked entries contribute exp(-1e9 - m) == 0 exactly and are written as 0
     const int c_live = (xf.S && xf.causal) ? (row + 1 < numcol ? row + 1 : numcol) : numcol;
 
     float m = -1e30f;
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(float* out, const 
         for (int c = cp; c < c_live; c += CP) {
             float t = p[static_cast<size_t>(c) * ld + row];
             if (xf.S) t = t * xf.scale;
-            s += expf(t - m);
+            s += exp_neg(t - m);
         }
     }
     red[cp][rl] = s;
@@ -195,9 +195,9 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(float* out, const 
             if (c < c_live) {
                 float t = p[static_cast<size_t>(c) * ld + row];
                 if (xf.S) t = t * xf.scale;
-                r = expf(t - m) * inv;
+                r = exp_neg(t - m) * inv;
             } else {
-                r = expf(-1e9f - m) * inv;
+                r = exp_neg(-1e9f - m) * inv;
             }
             q[static_cast<size_t>(c) * ld + row] = r;
         }
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(float* out, co
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int c = cp + v * CP;
-        x[v] = (live && c < numcol) ? expf(x[v] - m) : 0.f;
+        x[v] = (live && c < numcol) ? exp_neg(x[v] - m) : 0.f;
         s += x[v];
     }
     red[cp][rl] = s;
@@ -294,11 +294,11 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* par
                 tm = tm > t[u] ? tm : t[u];
             }
             const float mn = m > tm ? m : tm;
-            float acc = s * expf(m - mn);
+            float acc = s * exp_neg(m - mn);
 #pragma unroll
             for (int u = 0; u < kRowUnroll; ++u) {
                 const int cc = c + u * CP;
-                if (cc < c1) acc += expf(t[u] - mn);
+                if (cc < c1) acc += exp_neg(t[u] - mn);
             }
             s = acc;
             m = mn;
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* par
         for (int k = 0; k < CP; ++k) M = M > redm[k][rl] ? M : redm[k][rl];
         float S = 0.f;
 #pragma unroll
-        for (int k = 0; k < CP; ++k) S += reds[k][rl] * expf(redm[k][rl] - M);
+        for (int k = 0; k < CP; ++k) S += reds[k][rl] * exp_neg(redm[k][rl] - M);
         const size_t o = static_cast<size_t>(blockIdx.y) * 2 * numrow + row;
         part[o] = M;
         part[o + numrow] = S;
@@ -343,9 +343,9 @@ __global__ __launch_bounds__(kFoldThreads) void softmax_rows_fold_kernel(float* 
                 tm = tm > mk[u] ? tm : mk[u];
             }
             const float mn = m > tm ? m : tm;
-            float acc = s * expf(m - mn);
+            float acc = s * exp_neg(m - mn);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) acc += sk[u] * expf(mk[u] - mn);
+            for (int u = 0; u < 4; ++u) acc += sk[u] * exp_neg(mk[u] - mn);
             s = acc;
             m = mn;
         }
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(kFoldThreads) void softmax_rows_fold_kernel(float* 
         for (int k = 0; k < CP; ++k) M = M > redm[k][rl] ? M : redm[k][rl];
         float S = 0.f;
 #pragma unroll
-        for (int k = 0; k < CP; ++k) S += reds[k][rl] * expf(redm[k][rl] - M);
+        for (int k = 0; k < CP; ++k) S += reds[k][rl] * exp_neg(redm[k][rl] - M);
         rowstat[row] = M;
         rowstat[numrow + row] = 1.0f / (S + 1e-12f);
     }
@@ -386,7 +386,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, 
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int cc = c + u * CP;
-            if (cc < c1) out[static_cast<size_t>(cc) * ld + row] = expf(t[u] - M) * inv;
+            if (cc < c1) out[static_cast<size_t>(cc) * ld + row] = exp_neg(t[u] - M) * inv;
         }
     }
 }
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kWideThreads) void softmax_rows_wide_kernel(float* 
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int c = cp + v * kWidePhases;
-        x[v] = (live && c < numcol) ? expf(x[v] - m) : 0.f;
+        x[v] = (live && c < numcol) ? exp_neg(x[v] - m) : 0.f;
         s += x[v];
     }
     red[cp][rl] = s;
@@ -523,7 +523,7 @@ __global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, fl
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int r = lane + v * kWave;
-            e[v] = r < K ? expf(x[v] - m) : 0.f;
+            e[v] = r < K ? exp_neg(x[v] - m) : 0.f;
             s += e[v];
             if (r == label) picked = x[v];
         }
