@@ -93,12 +93,13 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_long_kernel(float* out, c
 
 // Medium-long columns (1024 < numrow <= 16384): one block per column with the
 // column held in registers (NV4 float4 per thread), so it is still one read
-// and one write per element.
-template <int NV4>
-__global__ __launch_bounds__(kBlock) void softmax_cols_block_kernel(float* out, const float* in,
+// and one write per element.  Columns over 4096 rows take 1024 threads: a
+// quarter of the registers per thread, so more columns are in flight per CU.
+template <int NV4, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void softmax_cols_block_kernel(float* out, const float* in,
                                                                     int numrow, size_t numcol,
                                                                     size_t ld) {
-    __shared__ float red[kBlock / kWave];
+    __shared__ float red[BLOCK / kWave];
     for (size_t col = blockIdx.x; col < numcol; col += gridDim.x) {
         const float* p = in + col * ld;
         float* q = out + col * ld;
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_block_kernel(float* out, 
         float m = -1e30f;
 #pragma unroll
         for (int v = 0; v < NV4; ++v) {
-            const int r = (threadIdx.x + v * kBlock) * 4;
+            const int r = (threadIdx.x + v * BLOCK) * 4;
             if (r < numrow) {   // numrow % 4 == 0 on this path
                 x[v] = *reinterpret_cast<const float4*>(p + r);
                 const float a = x[v].x > x[v].y ? x[v].x : x[v].y;
@@ -115,22 +116,22 @@ __global__ __launch_bounds__(kBlock) void softmax_cols_block_kernel(float* out, 
                 m = m > c ? m : c;
             }
         }
-        m = block_allreduce<kBlock / kWave>(m, MaxOp{}, red, -1e30f);
+        m = block_allreduce<BLOCK / kWave>(m, MaxOp{}, red, -1e30f);
         float s = 0.f;
 #pragma unroll
         for (int v = 0; v < NV4; ++v) {
-            const int r = (threadIdx.x + v * kBlock) * 4;
+            const int r = (threadIdx.x + v * BLOCK) * 4;
             if (r < numrow) {
                 x[v].x = exp_neg(x[v].x - m); x[v].y = exp_neg(x[v].y - m);
                 x[v].z = exp_neg(x[v].z - m); x[v].w = exp_neg(x[v].w - m);
                 s += (x[v].x + x[v].y) + (x[v].z + x[v].w);
             }
         }
-        s = block_allreduce<kBlock / kWave>(s, SumOp{}, red, 0.f);
+        s = block_allreduce<BLOCK / kWave>(s, SumOp{}, red, 0.f);
         const float inv = 1.0f / (s + 1e-12f);
 #pragma unroll
         for (int v = 0; v < NV4; ++v) {
-            const int r = (threadIdx.x + v * kBlock) * 4;
+            const int r = (threadIdx.x + v * BLOCK) * 4;
             if (r < numrow) {
                 x[v].x *= inv; x[v].y *= inv; x[v].z *= inv; x[v].w *= inv;
                 *reinterpret_cast<float4*>(q + r) = x[v];
@@ -609,13 +610,13 @@ int softmax_cols_impl(float* out, const float* in, int numrow, size_t numcol, si
         const unsigned grid = static_cast<unsigned>(numcol);
         hipStream_t st = stream();
         if (numrow <= 2048)
-            softmax_cols_block_kernel<2><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+            softmax_cols_block_kernel<2, kBlock><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
         else if (numrow <= 4096)
-            softmax_cols_block_kernel<4><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+            softmax_cols_block_kernel<4, kBlock><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
         else if (numrow <= 8192)
-            softmax_cols_block_kernel<8><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+            softmax_cols_block_kernel<2, 1024><<<grid, 1024, 0, st>>>(out, in, numrow, numcol, ld);
         else
-            softmax_cols_block_kernel<16><<<grid, kBlock, 0, st>>>(out, in, numrow, numcol, ld);
+            softmax_cols_block_kernel<4, 1024><<<grid, 1024, 0, st>>>(out, in, numrow, numcol, ld);
         return launch_rc();
     }
     const unsigned grid = grid_for(numcol, 1, 8);

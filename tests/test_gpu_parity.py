@@ -448,7 +448,7 @@ def test_add_bias(gpu):
                                        # every kernel of the family: register, wide-block, chunked rows;
                                        # wave, block and three-sweep columns
                                        (1024, 1024), (520, 700), (2048, 1500), (64, 9000), (600, 2500),
-                                       (4096, 33), (16384, 7), (20000, 3), (1028, 40), (1030, 12)])
+                                       (4096, 33), (6000, 4), (16384, 7), (20000, 3), (1028, 40), (1030, 12)])
 def test_softmax_cols_rows(gpu, oracle_lib, rows, cols):
     x = rng(rows + cols).normal(0, 3, rows * cols).astype(np.float32)
     dx = to_dev(x)
