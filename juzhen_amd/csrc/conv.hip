@@ -517,7 +517,9 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
         // that is a multiple of 8 so that the workgroups sharing patch rows
         // (same chunk, neighbouring rows) meet in one XCD's L2
         const int KK = g.kH * g.kW;
-        int R = 4, CC = 16;
+        // (four rows at stride 1, where neighbouring strips share two of six
+        // patch rows; two at larger strides, where the smaller strip measured faster)
+        int R = g.stride_h >= 2 ? 2 : 4, CC = 16;
         auto bytes = [&](int cc, int r) {
             const int nr = (r - 1 + g.kH - 1) / g.stride_h + 1;
             return static_cast<size_t>(nr) * g.Wp * ((cc * KK) | 1) * sizeof(float);
