@@ -372,9 +372,10 @@ __global__ __launch_bounds__(kBlock) void col2im_rows_kernel(const float* __rest
         const size_t col0 = static_cast<size_t>(n) * g.P + static_cast<size_t>(lo) * g.Wp;
         const int ncols = NR * g.Wp;
         const float* base = col + col0 * g.K + static_cast<size_t>(c0) * KK;
-        // eight independent loads in flight per thread, then their LDS stores;
+        // four independent loads in flight per thread, then their LDS stores (eight
+        // cost more in registers, hence resident workgroups, than they hide);
         // float4 loads when the runs are 16-byte aligned (L and K multiples of 4)
-        constexpr int kBatch = 8;
+        constexpr int kBatch = 4;
         if (vec4) {
             const int L4 = L / 4;
             const int count = ncols * L4;
