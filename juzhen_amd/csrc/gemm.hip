@@ -23,6 +23,11 @@
 #include <vector>
 
 namespace jz {
+// matrix-vector forms (gemv.hip)
+int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda, size_t incx,
+              size_t incy, float alpha, float beta);
+int gemm_thin(const float* A, const float* B, float* C, int m, int n, int k, bool trans_a, bool trans_b, int lda,
+              int ldb, int ldc, float alpha, float beta, bool* taken);
 namespace {
 
 // Optional per-launch timing of the tiled kernel (jzhip_profile_gemm): HIP
@@ -512,91 +517,6 @@ __global__ __launch_bounds__(kBlock) void rank1_kernel(float* C, const float* a,
     }
 }
 
-// y[j] = alpha * <A[:,j], x> + beta*y[j]: one wavefront per column of the
-// physical m x n matrix (op = transpose).
-__global__ __launch_bounds__(kBlock) void gemv_t_kernel(const float* A, const float* x, float* y,
-                                                        int m, int n, size_t lda, size_t incx,
-                                                        size_t incy, float alpha, float beta) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
-    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
-    for (size_t j = wave0; j < static_cast<size_t>(n); j += nwaves) {
-        const float* col = A + j * lda;
-        float acc = 0.f;
-        for (int i = lane; i < m; i += kWave) acc += col[i] * x[i * incx];
-        acc = wave_sum(acc);
-        if (lane == 0) {
-            float r = alpha * acc;
-            if (beta != 0.0f) r += beta * y[j * incy];
-            y[j * incy] = r;
-        }
-    }
-}
-
-// y[i] = alpha * sum_j A[i,j]*x[j] + beta*y[i] (op = none): lanes along rows,
-// the block's waves split the columns, combined through LDS.  Partial results
-// over column chunks go to part[chunk*m + i].
-__global__ __launch_bounds__(kBlock) void gemv_n_partial_kernel(const float* A, const float* x,
-                                                                float* part, int m, int n,
-                                                                size_t lda, size_t incx,
-                                                                int chunk_len) {
-    constexpr int NW = kBlock / kWave;
-    __shared__ float red[NW][kWave];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave;
-    const int row = blockIdx.x * kWave + lane;
-    const int c_begin = blockIdx.y * chunk_len;
-    int c_end = c_begin + chunk_len;
-    if (c_end > n) c_end = n;
-    float acc = 0.f;
-    if (row < m)
-        for (int c = c_begin + wave; c < c_end; c += NW) acc += A[static_cast<size_t>(c) * lda + row] * x[c * incx];
-    red[wave][lane] = acc;
-    __syncthreads();
-    if (wave == 0 && row < m) {
-        float s = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) s += red[w][lane];
-        part[static_cast<size_t>(blockIdx.y) * m + row] = s;
-    }
-}
-
-// y[i] = alpha * sum_c part[c*m + i] + beta*y[i]: 64 outputs per workgroup, its
-// sixteen waves taking interleaved chunks (four loads in flight each) and
-// meeting in LDS; fixed order, so the result is deterministic.
-constexpr int kGemvCombineBlock = 1024;
-__global__ __launch_bounds__(kGemvCombineBlock) void gemv_n_combine_kernel(float* y, const float* part, int m,
-                                                                           int chunks, size_t incy, float alpha,
-                                                                           float beta) {
-    constexpr int NW = kGemvCombineBlock / kWave;
-    __shared__ float red[NW][kWave];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int i = blockIdx.x * kWave + lane;
-    float acc = 0.f;
-    if (i < m) {
-        const float* p = part + i;
-        int c = wave;
-        for (; c + 3 * NW < chunks; c += 4 * NW) {
-            float x[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) x[u] = p[static_cast<size_t>(c + u * NW) * m];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) acc += x[u];
-        }
-        for (; c < chunks; c += NW) acc += p[static_cast<size_t>(c) * m];
-    }
-    red[wave][lane] = acc;
-    __syncthreads();
-    if (wave == 0 && i < m) {
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) sum += red[w][lane];
-        float r = alpha * sum;
-        if (beta != 0.0f) r += beta * y[i * incy];
-        y[i * incy] = r;
-    }
-}
-
 // y(rows x cols) += b[i]
 __global__ __launch_bounds__(kBlock) void add_bias_kernel(float* y, const float* b, int rows,
                                                           size_t total4) {
@@ -798,6 +718,11 @@ int launch_shape(const GemmArgs& g) {
     };
     if (g.M <= 32) return launch_tile<1, 4, 1, 2, TA, TB>(g);   // 32 x 256
     if (g.N <= 32) return launch_tile<4, 1, 2, 1, TA, TB>(g);   // 256 x 32
+    // 64 against a multiple of 64 that is not one of 128 (576 x 64 x 131072, the
+    // weight gradient of a 3x3 convolution on 64 channels): 64 x 64 tiles are all
+    // full and stay on the unchecked loaders
+    if (g.M == 64 && g.N % 128 != 0 && g.N % 64 == 0 && g.K % BK == 0) return launch_tile<2, 2, 1, 1, TA, TB>(g);
+    if (g.N == 64 && g.M % 128 != 0 && g.M % 64 == 0 && g.K % BK == 0) return launch_tile<2, 2, 1, 1, TA, TB>(g);
     if (g.M <= 64) return launch_tile<1, 4, 2, 1, TA, TB>(g);   // 64 x 128
     if (g.N <= 64) return launch_tile<4, 1, 1, 2, TA, TB>(g);   // 128 x 64
     // a long K is split across workgroups by launch_tile, so the big tile
@@ -821,31 +746,6 @@ int launch_shape(const GemmArgs& g) {
 int gemm_dispatch(const GemmArgs& g, bool ta, bool tb) {
     if (ta) return tb ? launch_shape<true, true>(g) : launch_shape<true, false>(g);
     return tb ? launch_shape<false, true>(g) : launch_shape<false, false>(g);
-}
-
-int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda,
-              size_t incx, size_t incy, float alpha, float beta) {
-    hipStream_t s = stream();
-    if (trans) {
-        gemv_t_kernel<<<grid_cover(n, kBlock / kWave), kBlock, 0, s>>>(A, x, y, m, n, lda, incx, incy,
-                                                                         alpha, beta);
-        return launch_rc();
-    }
-    const int row_blocks = (m + kWave - 1) / kWave;
-    int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
-    if (chunks > n / 32) chunks = n / 32;
-    if (chunks < 1) chunks = 1;
-    if (chunks > 4096) chunks = 4096;
-    while (chunks > 1 && static_cast<size_t>(chunks) * m > kWorkspaceFloats) --chunks;
-    if (static_cast<size_t>(chunks) * m > kWorkspaceFloats) return -1;
-    const int chunk_len = (n + chunks - 1) / chunks;
-    chunks = (n + chunk_len - 1) / chunk_len;
-    float* part = workspace();
-    if (!part) return -2;
-    gemv_n_partial_kernel<<<dim3(row_blocks, chunks), kBlock, 0, s>>>(A, x, part, m, n, lda, incx, chunk_len);
-    gemv_n_combine_kernel<<<(m + kWave - 1) / kWave, kGemvCombineBlock, 0, s>>>(y, part, m, chunks, incy, alpha,
-                                                                                beta);
-    return launch_rc();
 }
 
 }  // namespace
@@ -947,6 +847,11 @@ JZ_API int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, in
         if (trans_b) return gemv_impl(B, A, C, n, k, false, ldb, incx, ldc, alpha, beta);
         return gemv_impl(B, A, C, k, n, true, ldb, incx, ldc, alpha, beta);
     }
+    {
+        bool taken = false;
+        const int rc = gemm_thin(A, B, C, m, n, k, trans_a != 0, trans_b != 0, lda, ldb, ldc, alpha, beta, &taken);
+        if (taken) return rc;
+    }
     GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
                static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
     return gemm_dispatch(g, trans_a != 0, trans_b != 0);
@@ -979,14 +884,6 @@ JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int
 JZ_API int jzhip_gemm_nn(const float* A, const float* B, float* C, int m, int n, int k, float alpha,
                          float beta) {
     return jzhip_gemm(A, B, C, m, n, k, 0, 0, m, k, m, alpha, beta);
-}
-
-JZ_API int jzhip_gemv(const float* A, const float* x, float* y, int m, int n, int trans_a, int lda,
-                      int incx, int incy, float alpha, float beta) {
-    if (m <= 0 || n <= 0 || lda < m) return -1;
-    if (!A || !x || !y) return -1;
-    if (incx <= 0 || incy <= 0) return -1;
-    return gemv_impl(A, x, y, m, n, trans_a != 0, lda, incx, incy, alpha, beta);
 }
 
 JZ_API int jzhip_add_bias(float* y, const float* b, int rows, int cols) {

@@ -1,0 +1,346 @@
+// Matrix-vector products and their few-vector generalisation, the
+// bandwidth-bound relatives of the tiled GEMM: y = alpha*op(A)*x + beta*y, and
+// C = op(A) op(B) where m or n is at most kThinMax.
+#include "common.hpp"
+
+namespace jz {
+namespace {
+
+// y[j] = alpha * <A[:,j], x> + beta*y[j]: one wavefront per column of the
+// physical m x n matrix (op = transpose).
+__global__ __launch_bounds__(kBlock) void gemv_t_kernel(const float* A, const float* x, float* y,
+                                                        int m, int n, size_t lda, size_t incx,
+                                                        size_t incy, float alpha, float beta) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t j = wave0; j < static_cast<size_t>(n); j += nwaves) {
+        const float* col = A + j * lda;
+        float acc = 0.f;
+        for (int i = lane; i < m; i += kWave) acc += col[i] * x[i * incx];
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            float r = alpha * acc;
+            if (beta != 0.0f) r += beta * y[j * incy];
+            y[j * incy] = r;
+        }
+    }
+}
+
+// y[i] = alpha * sum_j A[i,j]*x[j] + beta*y[i] (op = none): lanes along rows,
+// the block's waves split the columns, combined through LDS.  Partial results
+// over column chunks go to part[chunk*m + i].
+__global__ __launch_bounds__(kBlock) void gemv_n_partial_kernel(const float* A, const float* x,
+                                                                float* part, int m, int n,
+                                                                size_t lda, size_t incx,
+                                                                int chunk_len) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int row = blockIdx.x * kWave + lane;
+    const int c_begin = blockIdx.y * chunk_len;
+    int c_end = c_begin + chunk_len;
+    if (c_end > n) c_end = n;
+    float acc = 0.f;
+    if (row < m)
+        for (int c = c_begin + wave; c < c_end; c += NW) acc += A[static_cast<size_t>(c) * lda + row] * x[c * incx];
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && row < m) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += red[w][lane];
+        part[static_cast<size_t>(blockIdx.y) * m + row] = s;
+    }
+}
+
+// y[i] = alpha * sum_c part[c*m + i] + beta*y[i]: 64 outputs per workgroup, its
+// sixteen waves taking interleaved chunks (four loads in flight each) and
+// meeting in LDS; fixed order, so the result is deterministic.
+constexpr int kGemvCombineBlock = 1024;
+// Output i lives at y[(i % len)*s_in + (i / len)*s_out] (a plain vector has len = m).
+__global__ __launch_bounds__(kGemvCombineBlock) void gemv_n_combine_kernel(float* y, const float* part, int m,
+                                                                           int chunks, int len, size_t s_in,
+                                                                           size_t s_out, float alpha, float beta) {
+    constexpr int NW = kGemvCombineBlock / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int i = blockIdx.x * kWave + lane;
+    float acc = 0.f;
+    if (i < m) {
+        const float* p = part + i;
+        int c = wave;
+        for (; c + 3 * NW < chunks; c += 4 * NW) {
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = p[static_cast<size_t>(c + u * NW) * m];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc += x[u];
+        }
+        for (; c < chunks; c += NW) acc += p[static_cast<size_t>(c) * m];
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && i < m) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[w][lane];
+        float* dst = y + static_cast<size_t>(i % len) * s_in + static_cast<size_t>(i / len) * s_out;
+        float r = alpha * sum;
+        if (beta != 0.0f) r += beta * *dst;
+        *dst = r;
+    }
+}
+
+// ── thin products: one extent of C is at most kThinMax ───────────────────
+// C = op(A) op(B) with m or n <= kThinMax (a 3-channel output convolution:
+// 3 x 131072 x 576 forward, 576 x 3 x 131072 for its weight gradient) is a
+// handful of matrix-vector products over one big operand: bound by reading
+// that operand once, which an MFMA tile padded to 32 rows cannot approach.
+// The big operand X is L x K (element (l,k) at X[l*xs_l + k*xs_k], one of the
+// strides being 1), the thin one V is T x K (V[t*vs_t + k*vs_k]); output (l,t)
+// goes to C[l*cs_l + t*cs_t].
+constexpr int kThinMax = 8;
+constexpr int kThinRows = 4;   // rows of X a wavefront walks together in the dot form
+constexpr int kThinChunkMax = 1024;   // k per workgroup in the other form
+
+// k contiguous in X: a wavefront takes kThinRows rows, its lanes stride over k
+// in float4 steps against V staged in LDS (each LDS read serves all the rows).
+template <int TT>
+__global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restrict__ X, size_t xs_l,
+                                                          const float* __restrict__ V, size_t vs_t, size_t vs_k,
+                                                          float* C, size_t cs_l, size_t cs_t, int L, int K, int T,
+                                                          float alpha, float beta) {
+    extern __shared__ __attribute__((aligned(16))) float vlds[];   // [TT][K]
+    for (int i = threadIdx.x; i < TT * K; i += kBlock) {
+        const int t = i / K, k = i - t * K;
+        vlds[i] = t < T ? V[t * vs_t + k * vs_k] : 0.f;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    const int K4 = K / 4;
+    const float4* v4 = reinterpret_cast<const float4*>(vlds);
+    for (size_t l0 = wave0 * kThinRows; l0 < static_cast<size_t>(L); l0 += nwaves * kThinRows) {
+        float acc[kThinRows][TT];
+#pragma unroll
+        for (int u = 0; u < kThinRows; ++u)
+#pragma unroll
+            for (int t = 0; t < TT; ++t) acc[u][t] = 0.f;
+        for (int k4 = lane; k4 < K4; k4 += kWave) {
+            float4 x[kThinRows];
+#pragma unroll
+            for (int u = 0; u < kThinRows; ++u) {
+                const size_t l = l0 + u < static_cast<size_t>(L) ? l0 + u : L - 1;   // clamped, dropped at the store
+                x[u] = reinterpret_cast<const float4*>(X + l * xs_l)[k4];
+            }
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                const float4 v = v4[t * K4 + k4];
+#pragma unroll
+                for (int u = 0; u < kThinRows; ++u)
+                    acc[u][t] += x[u].x * v.x + x[u].y * v.y + x[u].z * v.z + x[u].w * v.w;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kThinRows; ++u)
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                const float r = wave_sum(acc[u][t]);
+                if (lane == u * TT + t && l0 + u < static_cast<size_t>(L) && t < T) {
+                    float* dst = C + (l0 + u) * cs_l + t * cs_t;
+                    float o = alpha * r;
+                    if (beta != 0.0f) o += beta * *dst;
+                    *dst = o;
+                }
+            }
+    }
+}
+
+// l contiguous in X: lanes hold four rows each (a wavefront reads 1 KB of one
+// column), the block's waves split the k of a chunk eight at a time, and the
+// chunk's slice of V sits in LDS as [t][chunk_len], zero-filled past the end
+// of K, read as broadcast float4.  Partial sums go to part[chunk][t*L + l].
+template <int TT>
+__global__ __launch_bounds__(kBlock) void thin_axpy_partial_kernel(const float* __restrict__ X, size_t xs_k,
+                                                                   const float* __restrict__ V, size_t vs_t,
+                                                                   size_t vs_k, float* part, int L, int K, int T,
+                                                                   int chunk_len) {
+    constexpr int NW = kBlock / kWave;
+    constexpr int U = 8;   // columns in flight per wavefront; chunk_len % U == 0
+    extern __shared__ __attribute__((aligned(16))) float vl[];   // [TT][chunk_len]
+    __shared__ float4 red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int l = (blockIdx.x * kWave + lane) * 4;
+    const bool live = l < L;
+    const int k_begin = blockIdx.y * chunk_len;
+    const int len = (K - k_begin) < chunk_len ? (K - k_begin) : chunk_len;
+    for (int i = threadIdx.x; i < TT * chunk_len; i += kBlock) {
+        const int t = i / chunk_len, kk = i - t * chunk_len;
+        vl[i] = (t < T && kk < len) ? V[t * vs_t + static_cast<size_t>(k_begin + kk) * vs_k] : 0.f;
+    }
+    __syncthreads();
+    float4 acc[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) acc[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float* xp = X + (live ? l : 0) + static_cast<size_t>(k_begin) * xs_k;
+    for (int kk = wave * U; kk < len; kk += NW * U) {
+        float4 x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = kk + u < len ? kk + u : len - 1;   // clamped; its V entry is zero
+            x[u] = *reinterpret_cast<const float4*>(xp + static_cast<size_t>(c) * xs_k);
+        }
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+#pragma unroll
+            for (int q = 0; q < U / 4; ++q) {
+                const float4 v = *reinterpret_cast<const float4*>(vl + t * chunk_len + kk + 4 * q);
+                const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[t].x += x[4 * q + e].x * vv[e]; acc[t].y += x[4 * q + e].y * vv[e];
+                    acc[t].z += x[4 * q + e].z * vv[e]; acc[t].w += x[4 * q + e].w * vv[e];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+        if (t < T) {   // T is uniform: every thread takes the same barriers
+            red[wave][lane] = acc[t];
+            __syncthreads();
+            if (wave == 0 && live) {
+                float4 sum = red[0][lane];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) {
+                    const float4 o = red[w][lane];
+                    sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
+                }
+                *reinterpret_cast<float4*>(part + (static_cast<size_t>(blockIdx.y) * T + t) * L + l) = sum;
+            }
+            __syncthreads();
+        }
+    }
+}
+
+}  // namespace
+
+int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda,
+              size_t incx, size_t incy, float alpha, float beta) {
+    hipStream_t s = stream();
+    if (trans) {
+        gemv_t_kernel<<<grid_cover(n, kBlock / kWave), kBlock, 0, s>>>(A, x, y, m, n, lda, incx, incy,
+                                                                         alpha, beta);
+        return launch_rc();
+    }
+    const int row_blocks = (m + kWave - 1) / kWave;
+    int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
+    if (chunks > n / 32) chunks = n / 32;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 4096) chunks = 4096;
+    while (chunks > 1 && static_cast<size_t>(chunks) * m > kWorkspaceFloats) --chunks;
+    if (static_cast<size_t>(chunks) * m > kWorkspaceFloats) return -1;
+    const int chunk_len = (n + chunks - 1) / chunks;
+    chunks = (n + chunk_len - 1) / chunk_len;
+    float* part = workspace();
+    if (!part) return -2;
+    gemv_n_partial_kernel<<<dim3(row_blocks, chunks), kBlock, 0, s>>>(A, x, part, m, n, lda, incx, chunk_len);
+    gemv_n_combine_kernel<<<(m + kWave - 1) / kWave, kGemvCombineBlock, 0, s>>>(y, part, m, chunks, m, incy, 0,
+                                                                                alpha, beta);
+    return launch_rc();
+}
+
+namespace {
+
+struct ThinArgs {
+    const float* X; size_t xs_l, xs_k;
+    const float* V; size_t vs_t, vs_k;
+    float* C; size_t cs_l, cs_t;
+    int L, K, T;
+    float alpha, beta;
+};
+
+template <int TT>
+int thin_launch(const ThinArgs& a) {
+    hipStream_t s = stream();
+    if (a.xs_k == 1) {
+        const size_t groups = (static_cast<size_t>(a.L) + kThinRows - 1) / kThinRows;
+        const unsigned grid = grid_for(groups, kBlock / kWave, 8);
+        thin_dot_kernel<TT><<<grid, kBlock, static_cast<size_t>(TT) * a.K * sizeof(float), s>>>(
+            a.X, a.xs_l, a.V, a.vs_t, a.vs_k, a.C, a.cs_l, a.cs_t, a.L, a.K, a.T, a.alpha, a.beta);
+        return launch_rc();
+    }
+    const int row_blocks = (a.L / 4 + kWave - 1) / kWave;
+    int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
+    if (chunks > a.K / 64) chunks = a.K / 64;
+    if (chunks < 1) chunks = 1;
+    int chunk_len = ((a.K + chunks - 1) / chunks + 7) / 8 * 8;
+    if (chunk_len > kThinChunkMax) chunk_len = kThinChunkMax;   // V's slice of a chunk stays within 32 KB of LDS
+    chunks = (a.K + chunk_len - 1) / chunk_len;
+    const size_t outs = static_cast<size_t>(a.T) * a.L;
+    if (outs * chunks > kWorkspaceFloats) return -1;            // thin_ok() rules this out
+    float* part = workspace();
+    if (!part) return -2;
+    thin_axpy_partial_kernel<TT><<<dim3(row_blocks, chunks), kBlock, static_cast<size_t>(TT) * chunk_len * sizeof(float),
+                                   s>>>(a.X, a.xs_k, a.V, a.vs_t, a.vs_k, part, a.L, a.K, a.T, chunk_len);
+    gemv_n_combine_kernel<<<static_cast<unsigned>((outs + kWave - 1) / kWave), kGemvCombineBlock, 0, s>>>(
+        a.C, part, static_cast<int>(outs), chunks, a.L, a.cs_l, a.cs_t, a.alpha, a.beta);
+    return launch_rc();
+}
+
+// Whether the thin forms apply: float4 access to X in its contiguous direction,
+// V small enough for LDS in the dot form, partial sums that fit the workspace.
+bool thin_ok(const ThinArgs& a) {
+    if (a.T > kThinMax || !aligned16(a.X)) return false;
+    if (a.xs_k == 1)
+        return a.L >= 256 && a.K % 4 == 0 && a.xs_l % 4 == 0 && a.K >= 64 &&
+               static_cast<size_t>(a.T <= 4 ? 4 : kThinMax) * a.K * sizeof(float) <= 48 * 1024;
+    if (a.L < 64) return false;
+    // partial sums of every chunk must fit the workspace even at the longest chunk
+    const size_t min_chunks = (static_cast<size_t>(a.K) + kThinChunkMax - 1) / kThinChunkMax;
+    const size_t row_blocks = (static_cast<size_t>(a.L) / 4 + kWave - 1) / kWave;
+    const size_t want = (static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks;
+    const size_t chunks = want > min_chunks ? want : min_chunks;
+    return a.xs_l == 1 && a.L % 4 == 0 && a.xs_k % 4 == 0 && a.K >= 256 &&
+           static_cast<size_t>(a.T) * a.L * (chunks + 1) <= kWorkspaceFloats;
+}
+
+int thin_impl(const ThinArgs& a) { return a.T <= 4 ? thin_launch<4>(a) : thin_launch<kThinMax>(a); }
+
+}  // namespace
+
+// C = alpha*op(A)*op(B) + beta*C through the thin forms when they apply;
+// *taken says whether they did.
+int gemm_thin(const float* A, const float* B, float* C, int m, int n, int k, bool trans_a, bool trans_b, int lda,
+              int ldb, int ldc, float alpha, float beta, bool* taken) {
+    *taken = false;
+    if (n <= kThinMax || m <= kThinMax) {
+        const size_t ula = static_cast<size_t>(lda), ulb = static_cast<size_t>(ldb), ulc = static_cast<size_t>(ldc);
+        // op(A)(i,p) and op(B)(p,j) as (extent stride, k stride) pairs
+        const size_t a_i = trans_a ? ula : 1, a_k = trans_a ? 1 : ula;
+        const size_t b_j = trans_b ? 1 : ulb, b_k = trans_b ? ulb : 1;
+        const ThinArgs t = n <= m ? ThinArgs{A, a_i, a_k, B, b_j, b_k, C, 1, ulc, m, k, n, alpha, beta}
+                                  : ThinArgs{B, b_j, b_k, A, a_i, a_k, C, ulc, 1, n, k, m, alpha, beta};
+        if (thin_ok(t)) {
+            *taken = true;
+            return thin_impl(t);
+        }
+    }
+    return 0;
+}
+
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_gemv(const float* A, const float* x, float* y, int m, int n, int trans_a, int lda,
+                      int incx, int incy, float alpha, float beta) {
+    if (m <= 0 || n <= 0 || lda < m) return -1;
+    if (!A || !x || !y) return -1;
+    if (incx <= 0 || incy <= 0) return -1;
+    return gemv_impl(A, x, y, m, n, trans_a != 0, lda, incx, incy, alpha, beta);
+}

@@ -4,6 +4,7 @@ maps and argmax; relative 1e-5 for elementwise ops; 1e-4 for reductions,
 softmax and LayerNorm; 1e-3 for GEMM.
 """
 import ctypes as C
+import math
 
 import numpy as np
 import pytest
@@ -301,6 +302,58 @@ def test_gemm_variants(gpu, oracle_lib, m, n, k, ta, tb):
             # rows m..ldc-1 of every column must be untouched (tests/testCpuLinalg.cu:152-172)
             g2 = got.reshape(n, ldc)
             assert np.array_equal(g2[:, m:], C0.reshape(n, ldc)[:, m:])
+
+
+# one extent of at most 8 against a long one: the matrix-vector forms (lanes along
+# k with the thin operand in LDS, or lanes along the long extent with partial sums
+# over k chunks), in both roles and all four layouts, with and without padded
+# leading dimensions; (64, 1216, 512) and (1216, 64, 512) take full 64 x 64 tiles
+THIN_SHAPES = [(3, 4100, 576), (576, 3, 5000), (8, 2052, 128), (1028, 5, 300), (4, 1024, 64),
+               (1500, 7, 257), (2, 1027, 512), (64, 1216, 512), (1216, 64, 512)]
+
+
+@pytest.mark.parametrize("m,n,k", THIN_SHAPES)
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_thin_products(gpu, oracle_lib, m, n, k, ta, tb):
+    r = rng(m * 7919 + n * 31 + k + 2 * ta + tb)
+    for pad, alpha, beta in ((0, 1.0, 0.0), (4, 0.75, -0.5), (8, 1.0, 1.0)):
+        lda = (k if ta else m) + pad
+        ldb = (n if tb else k) + pad
+        ldc = m + pad
+        A = r.normal(0, 1, lda * (m if ta else k)).astype(np.float32)
+        B = r.normal(0, 1, ldb * (k if tb else n)).astype(np.float32)
+        C0 = r.normal(0, 1, ldc * n).astype(np.float32)
+        exact = naive_gemm64(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C0, ldc)
+        ref = C0.copy()
+        oracle_lib.jzo_gemm(ta, tb, m, n, k, alpha, hptr(A), lda, hptr(B), ldb, beta, hptr(ref), ldc)
+        dC = to_dev(C0)
+        gpu.gemm(dp(A), dp(B), dptr(dC), m, n, k, ta, tb, lda, ldb, ldc, alpha, beta)
+        got = to_host(dC)
+        assert rel_err(got, exact) <= TOL_GEMM
+        assert rel_err(got, ref) <= TOL_GEMM
+        if pad:
+            g2 = got.reshape(n, ldc)
+            assert np.array_equal(g2[:, m:], C0.reshape(n, ldc)[:, m:])
+
+
+def test_gemm_thin_products_at_the_output_convolution_size(gpu):
+    """3 x 131072 x 576 (forward, TN) and 576 x 3 x 131072 (weight gradient, NT) of a
+    64 -> 3 channel 3x3 convolution on 128 images of 32 x 32, against float64."""
+    r = rng(99)
+    K, n, co = 576, 131072, 3
+    W = r.normal(0, 1 / math.sqrt(K), K * co).astype(np.float32)       # K x co
+    col = r.normal(0, 1, K * n).astype(np.float32)                     # K x n
+    dcol, dW = to_dev(col), to_dev(W)
+    out = dev_empty(co * n)
+    gpu.gemm(dptr(dW), dptr(dcol), dptr(out), co, n, K, 1, 0, K, K, co, 1.0, 0.0)
+    Wm, Cm = W.astype(np.float64).reshape(co, K), col.astype(np.float64).reshape(n, K)
+    want = Cm @ Wm.T                                                    # (n, co) == column-major co x n
+    got = to_host(out)
+    assert rel_err(got, want.reshape(-1)) <= TOL_GEMM
+    g = dev_empty(K * co)
+    gpu.gemm(dptr(dcol), dptr(out), dptr(g), K, co, n, 0, 1, K, co, K, 1.0, 0.0)
+    want_g = got.astype(np.float64).reshape(n, co).T @ Cm               # (co, K) == column-major K x co
+    assert rel_err(to_host(g), want_g.reshape(-1)) <= TOL_GEMM
 
 
 @pytest.mark.parametrize("m,n,k", [(3, 5, 7), (64, 64, 64), (129, 127, 17), (256, 512, 128), (128, 1024, 96)])
