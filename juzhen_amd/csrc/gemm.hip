@@ -16,6 +16,7 @@
 #include "activations.hpp"
 
 #include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <string>
