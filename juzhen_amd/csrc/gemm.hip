@@ -638,6 +638,24 @@ int launch_tile(const GemmArgs& g) {
         // index and the operand panels of a chunk are fetched into one L2.
         auto xcd_friendly = [](int n) { return n <= 2 ? n : n <= 4 ? 4 : (n + 7) / 8 * 8; };
         splits = xcd_friendly(splits);
+        // Rounding up can push the launch just past the 2 x CUs workgroups that are
+        // resident together (9 tiles x 64 chunks = 576 against 512): the extra
+        // workgroups then run as a second, nearly empty round.  Compare the
+        // neighbouring multiples of 8 with a small model: a resident round costs its
+        // chunk length (plus a fixed start and store cost of about eight K steps)
+        // twice when two workgroups share a CU, 1.2 times when they do not.
+        if (splits > 8) {
+            auto cost = [&](int sp) {
+                const long long wgs = tiles * sp, slots = cus * 2;
+                const long long full = wgs / slots, rem = wgs % slots;
+                const double per = static_cast<double>(g.K) / sp + 8.0 * BK;
+                return per * (2.0 * full + (rem == 0 ? 0.0 : rem > cus ? 2.0 : 1.2));
+            };
+            int best = splits;
+            for (int sp = splits - 8; sp <= splits + 8; sp += 8)
+                if (sp >= 8 && cost(sp) < cost(best) * 0.97) best = sp;
+            splits = best;
+        }
         // at least sixteen K steps per chunk; a short K (skinny first-layer
         // gradients) is still cut, down to four steps, because a handful of
         // workgroups walking it alone only wait for their loads

@@ -108,6 +108,12 @@ def bench_gemm(r):
         ("C4 dx TN", 2048, 16384, 512, 1, 0), ("C4 dW NT", 512, 512, 16384, 0, 1),
         ("C4 dW NT", 2048, 512, 16384, 0, 1), ("C4 dW NT", 512, 2048, 16384, 0, 1),
         ("C4 logits TN", 256, 16384, 512, 1, 0),
+        # C5 (UNet, 128 images of 32 x 32): 3x3 convolutions 64 -> 64, 128 -> 64 and the 64 -> 3 output layer
+        ("C5 conv 64>64 fwd TN", 64, 131072, 576, 1, 0), ("C5 conv 64>64 dW NT", 576, 64, 131072, 0, 1),
+        ("C5 conv 64>64 dcol NN", 576, 131072, 64, 0, 0), ("C5 conv 128>64 fwd TN", 64, 131072, 1152, 1, 0),
+        ("C5 conv 128>64 dW NT", 1152, 64, 131072, 0, 1), ("C5 conv 128>64 dcol NN", 1152, 131072, 64, 0, 0),
+        ("C5 conv 128>128 fwd TN", 128, 32768, 1152, 1, 0), ("C5 conv 128>128 dW NT", 1152, 128, 32768, 0, 1),
+        ("C5 up 256>128 fwd NN", 2048, 8192, 256, 0, 0),
         ("square NN", 4096, 4096, 4096, 0, 0), ("square NT", 4096, 4096, 4096, 0, 1),
         ("square TN", 4096, 4096, 4096, 1, 0), ("square TT", 4096, 4096, 4096, 1, 1),
         ("square NN", 8192, 8192, 8192, 0, 0), ("square TN", 8192, 8192, 8192, 1, 0),
@@ -117,6 +123,14 @@ def bench_gemm(r):
         lda, ldb = (k if ta else m), (n if tb else k)
         r.run("gemm", f"jzhip_gemm {label}", f"{m}x{n}x{k}",
               lambda: jz.gemm(P(A), P(B), P(Cm), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0), flops=2.0 * m * n * k)
+    # thin products (m or n <= 8) are bound by reading the big operand once
+    for label, m, n, k, ta, tb in (("C5 output conv fwd TN (thin)", 3, 131072, 576, 1, 0),
+                                   ("C5 output conv dW NT (thin)", 576, 3, 131072, 0, 1)):
+        A, B, Cm = dev(m * k), dev(k * n), dev(m * n, 0)
+        lda, ldb = (k if ta else m), (n if tb else k)
+        r.run("gemm", f"jzhip_gemm {label}", f"{m}x{n}x{k}",
+              lambda: jz.gemm(P(A), P(B), P(Cm), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0),
+              bytes_=4.0 * (m * k + k * n + m * n))
     # products with the layer's elementwise tail fused into the store (C4 shapes)
     for label, m, n, k, ta, act, use_res in (("C4 Wo: bias+residual NN", 512, 16384, 512, 0, 0, 1),
                                              ("C4 W2: bias+residual NN", 512, 16384, 2048, 0, 0, 1),
