@@ -1,7 +1,8 @@
 // fp32 GEMM on CDNA4 matrix cores: C = alpha*op(A)*op(B) + beta*C, column-major,
-// all four transpose variants, arbitrary leading dimensions, plus the
-// bandwidth-bound special cases the layers generate (rank-1 products for bias
-// broadcasts, matrix-vector products) and a strided-batched form for attention.
+// all four transpose variants, arbitrary leading dimensions, plus rank-1
+// products (the layers' bias broadcasts) and a strided-batched form for
+// attention.  Matrix-vector products and products with m or n of at most 8
+// are bandwidth-bound and live in gemv.hip.
 //
 // Tiled kernel: a workgroup of four wavefronts owns a BM x BN tile of C and
 // walks K in steps of BK=16 through two LDS buffers (the global loads of step
