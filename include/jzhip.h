@@ -201,6 +201,12 @@ int jzhip_slice_assign(float* dst, size_t dst_numrow, int dst_transpose,
 int jzhip_embedding_fwd(float* out, const float* E, const float* P, const float* bias,
                         const int32_t* tokens, int d, int vocab, int S, int N);
 
+/* The device form of one_hot (ml/util.cuh:295-303), which fills a k x n
+ * column-major matrix on the host (zeros, then elem(Y(0,j), j) = 1) and leaves
+ * the caller to upload k*n floats: here the labels are n int32 values already
+ * on the device.  A label outside [0, k) leaves its column zero. */
+int jzhip_one_hot(float* out, const int32_t* labels, int k, size_t n);
+
 /* ── reductions ──────────────────────────────────────────────────────── */
 
 /* Sums over a physical column-major numrow x numcol buffer; replace the

@@ -79,6 +79,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_sum_cols": (I, [P, P, I, I, I]),
     "jzhip_sum_rows": (I, [P, P, I, I, I]),
     "jzhip_embedding_fwd": (I, [P, P, P, P, P, I, I, I, I]),
+    "jzhip_one_hot": (I, [P, P, I, Z]),
     "jzhip_nrm2": (I, [P, P, Z]),
     "jzhip_max_cols": (I, [P, P, I, I, I]),
     "jzhip_argmax_cols": (I, [P, P, I, I, I]),

@@ -280,6 +280,45 @@ JZ_API int jzhip_embedding_fwd(float* out, const float* E, const float* P, const
     return launch_rc();
 }
 
+// One-hot columns from int32 labels on the device (one_hot, ml/util.cuh:295-303,
+// builds them on the host and uploads k*n floats): out is k x n column-major,
+// zero except out[labels[j] + j*k] = 1.  A label outside [0, k) leaves its
+// column zero.
+namespace jz {
+namespace {
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void one_hot_kernel(float* __restrict__ out, const int32_t* __restrict__ labels,
+                                                         int k, FastDiv dK, size_t total) {
+    const int kv = k / VEC;   // dK divides by kv
+    const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t j = fdiv(static_cast<uint32_t>(i), dK);
+    const int r = static_cast<int>(static_cast<uint32_t>(i) - j * kv) * VEC;
+    const int lab = labels[j];
+    if constexpr (VEC == 4) {
+        const float4 v = make_float4(lab == r ? 1.f : 0.f, lab == r + 1 ? 1.f : 0.f, lab == r + 2 ? 1.f : 0.f,
+                                     lab == r + 3 ? 1.f : 0.f);
+        *reinterpret_cast<float4*>(out + static_cast<size_t>(j) * k + r) = v;
+    } else {
+        out[static_cast<size_t>(j) * k + r] = lab == r ? 1.f : 0.f;
+    }
+}
+}  // namespace
+}  // namespace jz
+
+JZ_API int jzhip_one_hot(float* out, const int32_t* labels, int k, size_t n) {
+    if (!out || !labels || k <= 0 || n == 0) return -1;
+    const size_t elems = static_cast<size_t>(k) * n;
+    if (elems >= (size_t(1) << 31)) return -1;
+    if (k % 4 == 0 && aligned16(out)) {
+        const size_t total = elems / 4;
+        one_hot_kernel<4><<<grid_cover(total, kBlock), kBlock, 0, stream()>>>(out, labels, k, make_fastdiv(k / 4), total);
+    } else {
+        one_hot_kernel<1><<<grid_cover(elems, kBlock), kBlock, 0, stream()>>>(out, labels, k, make_fastdiv(k), elems);
+    }
+    return launch_rc();
+}
+
 // slice get / set (cpp/hipmatrix.cpp:268-324).
 JZ_API int jzhip_slice_extract(float* dst, size_t dst_numrow, const float* src, size_t src_numrow,
                                int src_transpose, size_t rstart, size_t cstart, size_t rows,

@@ -453,7 +453,6 @@ JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
     Model* M = static_cast<Model*>(h);
     const Config& c = M->c;
     const int N = M->N;
-    std::vector<float> oh(static_cast<size_t>(c.vocab) * N, 0.0f);
     std::vector<int32_t> tk(N), tg(N);
     for (int b = 0; b < c.batch; ++b)
         for (int s = 0; s < c.seq; ++s) {
@@ -461,13 +460,14 @@ JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
             const int32_t tok = tokens[static_cast<size_t>(b) * (c.seq + 1) + s];
             const int32_t nxt = tokens[static_cast<size_t>(b) * (c.seq + 1) + s + 1];
             if (tok < 0 || tok >= c.vocab || nxt < 0 || nxt >= c.vocab) return -1;
-            oh[static_cast<size_t>(n) * c.vocab + tok] = 1.0f;
             tk[n] = tok;
             tg[n] = nxt;
         }
-    int rc = jzhip_memcpy_h2d(M->oh_tok, oh.data(), oh.size());
-    if (rc == 0) rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->tokens), reinterpret_cast<const float*>(tk.data()), N);
+    // only the ids cross PCIe (2 x 4 bytes per token); the one-hot matrix the
+    // embedding gradient multiplies by is built on the device
+    int rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->tokens), reinterpret_cast<const float*>(tk.data()), N);
     if (rc == 0) rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->targets), reinterpret_cast<const float*>(tg.data()), N);
+    if (rc == 0) rc = jzhip_one_hot(M->oh_tok, M->tokens, c.vocab, static_cast<size_t>(N));
     return rc;
 }
 

@@ -48,6 +48,7 @@ SIGNATURES = {
     "jzo_gelu": (None, [P, P, Z]),
     "jzo_dgelu_mul": (None, [P, P, P, Z]),
     "jzo_embedding_fwd": (None, [P, P, P, P, P, I, I, I, I]),
+    "jzo_one_hot": (None, [P, P, I, Z]),
     "jzo_sum_phys": (None, [P, P, I, I, I, I]),
     "jzo_norm": (F, [P, Z]),
     "jzo_max_cols": (None, [P, P, I, I, I]),

@@ -214,6 +214,15 @@ JZO_API void jzo_embedding_fwd(float* out, const float* E, const float* P, const
     }
 }
 
+/* one_hot (ml/util.cuh:295-303): zeros, then elem(Y(0, j), j) = 1 for every
+ * sample j; k x n column-major.  The reference does not range-check a label;
+ * here a label outside [0, k) leaves its column zero (the device form's rule). */
+JZO_API void jzo_one_hot(float* out, const int32_t* labels, int k, size_t n) {
+    for (size_t i = 0; i < (size_t)k * n; i++) out[i] = 0.0f;
+    for (size_t j = 0; j < n; j++)
+        if (labels[j] >= 0 && labels[j] < k) out[j * (size_t)k + (size_t)labels[j]] = 1.0f;
+}
+
 /* ── reductions ───────────────────────────────────────────────────────── */
 
 /* sum(M, dim) (cpp/matrix.hpp:74-91): GEMV with a ones vector on the physical

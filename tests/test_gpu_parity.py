@@ -496,6 +496,20 @@ def test_add_bias(gpu):
         assert np.array_equal(to_host(dy), (y.reshape(cols, rows) + b[None, :]).reshape(-1))
 
 
+@pytest.mark.parametrize("k,n", [(10, 128), (7, 33), (256, 16384), (4, 1), (1, 5)])
+def test_one_hot(gpu, oracle_lib, k, n):
+    r = rng(k * 31 + n)
+    lab = r.integers(0, k, n).astype(np.int32)
+    if n > 4:
+        lab[1], lab[n - 2] = -1, k                      # outside the range: zero column
+    dl = to_dev(lab)
+    out = to_dev(np.full(k * n, 7.0, np.float32))
+    gpu.one_hot(dptr(out), dptr(dl), k, n)
+    ref = np.empty(k * n, np.float32)
+    oracle_lib.jzo_one_hot(hptr(ref), hptr(lab), k, n)
+    assert np.array_equal(to_host(out), ref)
+
+
 # ── softmax family ───────────────────────────────────────────────────────
 @pytest.mark.parametrize("rows,cols", [(1, 1), (10, 128), (64, 9), (100, 300), (256, 2048), (1024, 64), (3000, 5),
                                        # every kernel of the family: register, wide-block, chunked rows;

@@ -388,3 +388,20 @@ def test_embedding_lookup_is_the_one_hot_product(oracle_lib):
     assert np.array_equal(got[3], Pm[3 % S]) and np.array_equal(got[7], Pm[7 % S])
     o.jzo_embedding_fwd(hptr(got), hptr(E), hptr(Pm), hptr(bias), hptr(tok), d, V, S, N)
     assert np.array_equal(got, want + bias[None, :])
+
+
+def test_one_hot_is_the_identity_indexed_by_label(oracle_lib):
+    """one_hot (ml/util.cuh:295-303): column j is column Y(0,j) of the k x k
+    identity; a label outside [0, k) gives the zero column."""
+    r = np.random.default_rng(5)
+    for k, n in ((10, 128), (7, 33), (256, 300)):
+        lab = r.integers(0, k, n).astype(np.int32)
+        lab[1], lab[n - 2] = -1, k
+        out = np.full((n, k), 7.0, np.float32)          # row j of this array = column j of the k x n matrix
+        oracle_lib.jzo_one_hot(hptr(out), hptr(lab), k, n)
+        want = np.zeros((n, k), np.float32)
+        ok = (lab >= 0) & (lab < k)
+        want[ok] = np.eye(k, dtype=np.float32)[lab[ok]]
+        assert np.array_equal(out, want)
+        assert out.sum() == n - 2
+
