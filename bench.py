@@ -167,6 +167,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--serial", action="store_true",
                     help="one stream, program order, also in the timed steps (for per-kernel traces and counters)")
+    ap.add_argument("--fresh-batches", action="store_true",
+                    help="hand a new batch of host token ids to the model before every step (PCIe-inclusive rate); "
+                         "by default one batch is uploaded before the timed region and reused")
     ap.add_argument("--cpu-baseline-only", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain copy of 2^26 floats three times, so that a counter run of this "
@@ -209,7 +212,11 @@ def main():
         ev.sync()
         del src, dst
 
-    for _ in range(args.warmup):
+    fresh = ([zipf_tokens(rng, CFG["vocab"], CFG["batch"], CFG["seq"]) for _ in range(8)]
+             if args.fresh_batches else None)
+    for i in range(args.warmup):
+        if fresh:
+            model.set_batch(fresh[i % len(fresh)])
         model.step()
     ev.sync()
     first_loss = model.loss()
@@ -218,7 +225,9 @@ def main():
     ev.sync()
     t0 = time.perf_counter()
     ev.record(e0, stream)
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        if fresh:
+            model.set_batch(fresh[i % len(fresh)])
         model.step()
     ev.record(e1, stream)
     gpu_ms = ev.elapsed_ms(e0, e1)
@@ -275,6 +284,8 @@ def main():
                                "d_model 512, 8 heads, FFN 2048 GELU, tied embeddings, learned positions, AdamW "
                                "lr 3e-4 wd 0.01", "tokens_per_step": tokens_per_step,
                    "backward_streams": 1 if args.serial else 2,
+                   "batch_upload": "every step (host ids -> device inside the timed region)" if fresh
+                                   else "once, before the timed region",
                    "parameters": int(model.param_count), "loss_first": round(first_loss, 4),
                    "loss_last": round(last_loss, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 3)},
         "roofline": roofline,

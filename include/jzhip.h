@@ -82,6 +82,23 @@ int jzhip_event_create(void** out_event);
 int jzhip_event_destroy(void* event);
 int jzhip_event_record(void* event);
 int jzhip_stream_wait_event(void* event);
+/* Block the host until the work marked by `jzhip_event_record` has run. */
+int jzhip_event_synchronize(void* event);
+/* No reference counterpart: the reference reads a batch into pageable host
+ * memory and uploads it with a blocking copy in Matrix<ROCMfloat>'s converting
+ * constructor (ml/dataloader.hpp:88-113, cpp/hipmatrix.cpp:60-63), which drains
+ * the stream before every batch.  `jzhip_host_alloc` returns page-locked host
+ * memory; `jzhip_memcpy_h2d_async` / `_d2h_async` enqueue a copy of `bytes`
+ * bytes on the current stream and return at once when the host side is such
+ * memory (from pageable memory the copy is still ordered but may block; an
+ * upload of up to 1 MiB from page-locked memory is done by a kernel that reads
+ * the host buffer directly, so it never leaves the compute queue).  The
+ * host buffer must stay untouched until the stream has passed the copy: record
+ * an event after it and `jzhip_event_synchronize` before reusing the buffer. */
+int jzhip_host_alloc(void** ptr, size_t bytes);
+int jzhip_host_free(void* ptr);
+int jzhip_memcpy_h2d_async(void* dst_device, const void* src_host, size_t bytes);
+int jzhip_memcpy_d2h_async(void* dst_host, const void* src_device, size_t bytes);
 
 /* ── random numbers ──────────────────────────────────────────────────── */
 

@@ -41,6 +41,11 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_event_destroy": (I, [P]),
     "jzhip_event_record": (I, [P]),
     "jzhip_stream_wait_event": (I, [P]),
+    "jzhip_event_synchronize": (I, [P]),
+    "jzhip_host_alloc": (I, [P, Z]),
+    "jzhip_host_free": (I, [P]),
+    "jzhip_memcpy_h2d_async": (I, [P, P, Z]),
+    "jzhip_memcpy_d2h_async": (I, [P, P, Z]),
     "jzhip_rand_uniform": (I, [P, Z, U64]),
     "jzhip_rand_normal": (I, [P, Z, F, F, U64]),
     "jzhip_fill": (I, [P, Z, F]),

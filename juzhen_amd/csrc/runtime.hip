@@ -3,6 +3,8 @@
 // (cpp/hipkernels.cpp:463-569) without rocRAND/hipBLAS handles.
 #include "common.hpp"
 
+#include <cstdint>
+
 #include <atomic>
 #include <mutex>
 
@@ -139,6 +141,7 @@ JZ_API int jzhip_free(float* ptr) {
 }
 
 namespace {
+constexpr size_t kKernelCopyBytes = size_t(1) << 20;
 int sync_copy(void* dst, const void* src, size_t count, hipMemcpyKind kind) {
     if (count == 0) return 0;
     if (dst == nullptr || src == nullptr) return -1;
@@ -159,6 +162,47 @@ JZ_API int jzhip_memcpy_d2d(float* dst_device, const float* src_device, size_t c
     // Device-to-device copies stay asynchronous: a copy kernel keeps stream
     // order and does not stall the host the way hipMemcpy does.
     return jzhip_copy(dst_device, src_device, count);
+}
+
+JZ_API int jzhip_host_alloc(void** ptr, size_t bytes) {
+    if (ptr == nullptr) return -1;
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 1;
+    void* p = nullptr;
+    hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return static_cast<int>(e);
+    }
+    *ptr = p;
+    return 0;
+}
+JZ_API int jzhip_host_free(void* ptr) {
+    if (ptr == nullptr) return 0;
+    return jz::rc_of(hipHostFree(ptr));
+}
+JZ_API int jzhip_memcpy_h2d_async(void* dst_device, const void* src_host, size_t bytes) {
+    if (bytes == 0) return 0;
+    if (dst_device == nullptr || src_host == nullptr) return -1;
+    // A small copy from page-locked memory (a batch of ids) is done by a kernel
+    // that reads the host buffer through its device alias: it stays on the
+    // compute queue, where a DMA copy between kernels costs a hand-over to the
+    // copy engine and back that is far longer than the transfer.
+    if (bytes <= kKernelCopyBytes && bytes % sizeof(float) == 0 &&
+        reinterpret_cast<uintptr_t>(dst_device) % sizeof(float) == 0) {
+        hipPointerAttribute_t at;
+        if (hipPointerGetAttributes(&at, src_host) == hipSuccess && at.type == hipMemoryTypeHost &&
+            at.devicePointer != nullptr)
+            return jzhip_copy(static_cast<float*>(dst_device), static_cast<const float*>(at.devicePointer),
+                              bytes / sizeof(float));
+        (void)hipGetLastError();   // pageable memory is not known to the runtime: not an error here
+    }
+    return jz::rc_of(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, jz::stream()));
+}
+JZ_API int jzhip_memcpy_d2h_async(void* dst_host, const void* src_device, size_t bytes) {
+    if (bytes == 0) return 0;
+    if (dst_host == nullptr || src_device == nullptr) return -1;
+    return jz::rc_of(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, jz::stream()));
 }
 
 JZ_API int jzhip_set_stream(void* hip_stream) {
@@ -200,6 +244,10 @@ JZ_API int jzhip_event_destroy(void* event) {
 JZ_API int jzhip_event_record(void* event) {
     if (!event) return -1;
     return jz::rc_of(hipEventRecord(static_cast<hipEvent_t>(event), jz::stream()));
+}
+JZ_API int jzhip_event_synchronize(void* event) {
+    if (!event) return -1;
+    return jz::rc_of(hipEventSynchronize(static_cast<hipEvent_t>(event)));
 }
 JZ_API int jzhip_stream_wait_event(void* event) {
     if (!event) return -1;

@@ -95,6 +95,12 @@ struct Model {
     void* ev[kEvents] = {};
     void* done[kDone] = {};   // side stream finished a block's weight gradients
     int ev_next = 0;
+    // Batches are staged in two page-locked host buffers (ids, then targets) and
+    // copied asynchronously, so handing over the next batch does not wait for the
+    // step in flight; staged[k] marks the stream position after buffer k's copies.
+    int32_t* stage[2] = {};
+    void* staged[2] = {};
+    unsigned batches = 0;
     float* io = nullptr;  // dense staging for get/set of strided views
     size_t io_floats = 0;
     int iteration = 1;
@@ -380,11 +386,11 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
         b.F1 = M->alloc(fN); b.F1a = M->alloc(fN); b.out = M->alloc(dN);
     }
     M->oh_tok = M->alloc(static_cast<size_t>(V) * N);
-    M->tokens = reinterpret_cast<int32_t*>(M->alloc(N));
+    M->tokens = reinterpret_cast<int32_t*>(M->alloc(2 * static_cast<size_t>(N)));   // ids, then targets: one upload
+    M->targets = M->tokens + N;
     M->x0 = M->alloc(dN);
     M->logits = M->alloc(static_cast<size_t>(V) * N);
     M->dlogits = M->alloc(static_cast<size_t>(V) * N);
-    M->targets = reinterpret_cast<int32_t*>(M->alloc(N));
     M->loss = M->alloc(1);
     for (float*& p : M->dx) p = M->alloc(dN);
     for (int k = 0; k < 2; ++k) {
@@ -399,6 +405,12 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
     M->ck(jzhip_stream_create(&M->side));
     for (void*& e : M->ev) M->ck(jzhip_event_create(&e));
     for (void*& e : M->done) M->ck(jzhip_event_create(&e));
+    for (int k = 0; k < 2; ++k) {
+        void* p = nullptr;
+        M->ck(jzhip_host_alloc(&p, sizeof(int32_t) * 2 * static_cast<size_t>(N)));
+        M->stage[k] = static_cast<int32_t*>(p);
+        M->ck(jzhip_event_create(&M->staged[k]));
+    }
     if (const char* env = std::getenv("JZLM_OVERLAP")) M->overlap = std::atoi(env) != 0;
     return M;
 }
@@ -410,6 +422,10 @@ JZLM_API void jzlm_destroy(void* h) {
     for (void* e : M->ev) jzhip_event_destroy(e);
     for (void* e : M->done) jzhip_event_destroy(e);
     jzhip_stream_destroy(M->side);
+    for (int k = 0; k < 2; ++k) {
+        jzhip_event_destroy(M->staged[k]);
+        jzhip_host_free(M->stage[k]);
+    }
     for (float* p : M->owned) jzhip_free(p);
     delete M;
 }
@@ -453,7 +469,15 @@ JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
     Model* M = static_cast<Model*>(h);
     const Config& c = M->c;
     const int N = M->N;
-    std::vector<int32_t> tk(N), tg(N);
+    const int slot = static_cast<int>(M->batches & 1u);
+    if (!M->stage[slot]) return -1;
+    // the copies issued from this buffer two batches ago must have run
+    if (M->batches >= 2) {
+        const int rc0 = jzhip_event_synchronize(M->staged[slot]);
+        if (rc0 != 0) return rc0;
+    }
+    int32_t* tk = M->stage[slot];
+    int32_t* tg = tk + N;
     for (int b = 0; b < c.batch; ++b)
         for (int s = 0; s < c.seq; ++s) {
             const int n = b * c.seq + s;
@@ -465,9 +489,10 @@ JZLM_API int jzlm_set_batch(void* h, const int32_t* tokens) {
         }
     // only the ids cross PCIe (2 x 4 bytes per token); the one-hot matrix the
     // embedding gradient multiplies by is built on the device
-    int rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->tokens), reinterpret_cast<const float*>(tk.data()), N);
-    if (rc == 0) rc = jzhip_memcpy_h2d(reinterpret_cast<float*>(M->targets), reinterpret_cast<const float*>(tg.data()), N);
+    int rc = jzhip_memcpy_h2d_async(M->tokens, tk, sizeof(int32_t) * 2 * static_cast<size_t>(N));
+    if (rc == 0) rc = jzhip_event_record(M->staged[slot]);
     if (rc == 0) rc = jzhip_one_hot(M->oh_tok, M->tokens, c.vocab, static_cast<size_t>(N));
+    ++M->batches;
     return rc;
 }
 

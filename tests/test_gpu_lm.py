@@ -197,3 +197,36 @@ def test_two_stream_backward_is_bit_identical_to_program_order(gpu, tied):
     for n in g0:
         assert np.array_equal(g0[n], g1[n]), n
         assert np.array_equal(p0[n], p1[n]), n
+
+
+def test_fresh_batch_every_step_without_waiting_for_the_step_in_flight(gpu):
+    """Batches go through two page-locked staging buffers and asynchronous copies:
+    handing over batch i+1 while step i is still running must not disturb step i,
+    and a buffer is reused only after its copies have run.  Five different batches
+    handed over back to back give the losses of the same five batches handed over
+    with a full synchronisation before each."""
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 64, 128, 4, 512, 2, 64, 8
+    rng = np.random.default_rng(9)
+    batches = [make_tokens(rng, V, B, S) for _ in range(5)]
+    out = []
+    for drain in (True, False):
+        m = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=True, adamw=True, lr=1e-3)
+        m.init_random(4)
+        losses = []
+        for t in batches:
+            if drain:
+                gpu.synchronize()
+            m.set_batch(t)
+            m.step()
+            if drain:
+                losses.append(m.loss())
+        params = {n: m.get(n) for n in m.names}
+        out.append((losses, params, m.loss()))
+        m.close()
+    (l0, p0, last0), (_, p1, last1) = out
+    assert last0 == last1 == l0[-1]
+    for n in p0:
+        assert np.array_equal(p0[n], p1[n]), n
+    assert len(set(l0)) == len(l0)          # the batches really differ
+

@@ -960,3 +960,37 @@ def test_embedding_fwd(gpu, oracle_lib, d, V, S, B, with_bias):
     from juzhen_amd import capi
     assert capi.load().jzhip_embedding_fwd(dptr(out), None, dptr(dP), None, dptr(dtok), d, V, S, N) == -1
     assert capi.load().jzhip_embedding_fwd(dptr(out), dptr(dE), dptr(dP), None, dptr(dtok), 0, V, S, N) == -1
+
+
+def test_page_locked_host_memory_and_asynchronous_copies(gpu):
+    """jzhip_host_alloc / jzhip_memcpy_h2d_async / _d2h_async / jzhip_event_synchronize:
+    a round trip through the device behind a kernel on the same stream, with the
+    host waiting on an event instead of draining the stream."""
+    from juzhen_amd import capi
+    lib = capi.load()
+    n = 1 << 20
+    src, dst, ev = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert lib.jzhip_host_alloc(C.byref(src), 4 * n) == 0 and src.value
+    assert lib.jzhip_host_alloc(C.byref(dst), 4 * n) == 0 and dst.value
+    assert lib.jzhip_event_create(C.byref(ev)) == 0
+    try:
+        a = np.ctypeslib.as_array(C.cast(src, C.POINTER(C.c_float)), shape=(n,))
+        b = np.ctypeslib.as_array(C.cast(dst, C.POINTER(C.c_float)), shape=(n,))
+        a[:] = rng(1).normal(size=n).astype(np.float32)
+        b[:] = 0
+        d_in, d_out = dev_empty(n), dev_empty(n)
+        gpu.memcpy_h2d_async(dptr(d_in), src, 4 * n)
+        gpu.affine(dptr(d_out), dptr(d_in), n, 2.0, 1.0)          # 2*x + 1 behind the copy
+        gpu.memcpy_d2h_async(dst, dptr(d_out), 4 * n)
+        gpu.event_record(ev)
+        gpu.event_synchronize(ev)
+        assert np.array_equal(b, a * np.float32(2.0) + np.float32(1.0))
+        assert lib.jzhip_memcpy_h2d_async(None, src, 16) == -1
+        assert lib.jzhip_memcpy_h2d_async(dptr(d_in), src, 0) == 0
+        assert lib.jzhip_event_synchronize(None) == -1
+    finally:
+        gpu.synchronize()
+        lib.jzhip_event_destroy(ev)
+        assert lib.jzhip_host_free(src) == 0 and lib.jzhip_host_free(dst) == 0
+    assert lib.jzhip_host_alloc(None, 16) == -1 and lib.jzhip_host_free(None) == 0
+
