@@ -234,6 +234,14 @@ def bench_fused(r):
           lambda: jz.attention_fwd(P(H), P(A), P(Q), P(K), P(V), dk, heads, S, B, 1), flops=fl)
     r.run("fused", "jzhip_attention_bwd", f"S{S} d_k{dk} h{heads} B{B}",
           lambda: jz.attention_bwd(P(dQ), P(dK), P(dV), P(dA), P(H), P(Q), P(K), P(V), P(A), dk, heads, S, B), flops=2 * fl)
+    # token embedding and one-hot construction of C4 (vocab 256, d_model 512, 16384 tokens)
+    import torch
+    Vc, dm = 256, 512
+    tok = torch.randint(0, Vc, (N,), dtype=torch.int32, device="cuda")
+    E, Pt, x0, oh = dev(dm * Vc), dev(dm * S), dev(dm * N, 0), dev(Vc * N, 0)
+    r.run("fused", "jzhip_embedding_fwd", f"{dm}x{N} vocab {Vc}",
+          lambda: jz.embedding_fwd(P(x0), P(E), P(Pt), None, P(tok), dm, Vc, S, N), bytes_=4.0 * (dm * N + N))
+    r.run("fused", "jzhip_one_hot", f"{Vc}x{N}", lambda: jz.one_hot(P(oh), P(tok), Vc, N), bytes_=4.0 * (Vc * N + N))
 
 
 def bench_conv(r):
