@@ -758,8 +758,14 @@ int launch_shape(const GemmArgs& g) {
         return launch_tile<4, 1, 1, 2, TA, TB>(g);   // 128 x 64
     if (g.M % 64 != 0 && g.M % 32 == 0 && g.N % 256 == 0 && g.K % 32 == 0 && g.K <= 256)
         return launch_tile<1, 4, 1, 2, TA, TB>(g);   // 32 x 256: short-K products are store-bound anyway
-    const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && tiles(128, 128) * 8 >= cus && !g.ep.any;
-    if (tiles(128, 128) < cus && !splittable) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
+    // (fewer big tiles still pay when K is long enough that summing the partial
+    // results, 8 bytes per output and chunk, stays under a tenth of the product:
+    // 2304 x 128 x 32768 as 18 tiles x 24 chunks)
+    const long long t128 = tiles(128, 128);
+    const long long chunks_wanted = (2 * cus + t128 - 1) / t128;
+    const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && !g.ep.any &&
+                            (t128 * 8 >= cus || g.K >= 600 * chunks_wanted);
+    if (t128 < cus && !splittable) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
     return launch_tile<2, 2, 2, 2, TA, TB>(g);                  // 128 x 128
 }
 
