@@ -356,6 +356,11 @@ int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratch,
  * ld_qkv / ld_dqkv / ld_h / ld_dh are the leading dimensions of those buffers.
  * causal != 0 in the backward call states that A came from a causal forward
  * call (exact zeros above the diagonal), which lets it skip those key tiles.
+ * causal == 2 additionally states that the entries above the diagonal of the
+ * output score buffer (A forward, dA_scratch backward) already hold the zeros
+ * an earlier call with causal == 1 wrote into the same buffer, so the fused
+ * kernel does not write them again (a training loop reuses both buffers every
+ * step; nearly half of each is such zeros).
  * For head widths 32 and 64 with S a multiple of 32 up to 256 both calls run
  * as one fused kernel per pass (scores, softmax and the second product in
  * registers); other shapes take batched GEMMs and the softmax kernels. */

@@ -201,10 +201,12 @@ __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, 
             }
         }
     }
-    // key tiles past the causal range hold exact zeros
-    for (int t = nkt; t < S / 16; ++t)
+    // key tiles past the causal range hold exact zeros (causal == 2: the caller
+    // states that they already do, from an earlier call on the same buffer)
+    if (causal != 2)
+        for (int t = nkt; t < S / 16; ++t)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) ((BWD ? dSblk : Ablk) + static_cast<size_t>(16 * t + v) * S)[lane_off] = 0.0f;
+            for (int v = 0; v < 4; ++v) ((BWD ? dSblk : Ablk) + static_cast<size_t>(16 * t + v) * S)[lane_off] = 0.0f;
 
     // second product: Out[d][query] = sum_key M2[d][key] * sc[key][query]; the
     // skipped tiles are a suffix, so the fragment prefetch can run ahead freely
@@ -372,6 +374,7 @@ JZ_API int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q, 
                                   int causal) {
     if (d_k <= 0 || heads <= 0 || S <= 0 || B <= 0 || d_k % heads != 0) return -1;
     if (!H || !A || !Q || !K || !V || ld_h < d_k || ld_qkv < d_k) return -1;
+    if (causal < 0 || causal > 2) return -1;
     const int d_h = d_k / heads;
     const long long seq = static_cast<long long>(S) * ld_qkv;  // next sequence in Q/K/V
     const long long seq_h = static_cast<long long>(S) * ld_h;  // next sequence in H
@@ -389,7 +392,7 @@ JZ_API int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q, 
                                blk * B, heads, 1.0f, 0.0f);
     if (rc) return rc;
     // A = softmax over keys of (scores*scale, masked)
-    rc = jzhip_attn_softmax(A, A, S, B * heads, scale, causal, 0);
+    rc = jzhip_attn_softmax(A, A, S, B * heads, scale, causal != 0, 0);
     if (rc) return rc;
     // H_i = V_i * A_i^T
     return jz::gemm_batched2(V, A, H, d_h, S, S, false, true, ld_qkv, S, ld_h, seq, blk, seq_h, B, d_h,
@@ -408,6 +411,7 @@ JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, 
     if (d_k <= 0 || heads <= 0 || S <= 0 || B <= 0 || d_k % heads != 0) return -1;
     if (!dQ || !dK || !dV || !dA_scratch || !dH || !Q || !K || !V || !A) return -1;
     if (ld_dqkv < d_k || ld_dh < d_k || ld_qkv < d_k) return -1;
+    if (causal < 0 || causal > 2) return -1;
     const int d_h = d_k / heads;
     const long long seq = static_cast<long long>(S) * ld_qkv;
     const long long seq_d = static_cast<long long>(S) * ld_dqkv;

@@ -68,6 +68,7 @@ struct Arena {
 struct Block {
     int Wq, Wk, Wv, Wo, bo, W1, b1, W2, b2, g1, be1, g2, be2;           // tensor indices
     float *x1, *xhat1, *inv1, *QKV, *A, *H, *R, *x2, *xhat2, *inv2, *F1, *F1a, *out;  // cached activations
+    bool A_masked_zero = false;   // A's entries above the diagonal already hold the zeros of a first forward call
 };
 
 struct Model {
@@ -86,6 +87,7 @@ struct Model {
     // block, and the block-output gradient three times: see backward())
     float *dx[3] = {}, *dR[2] = {}, *dtmp[2] = {}, *dtmp1[2] = {}, *dQKV[2] = {}, *dF1[2] = {};
     float *dH = nullptr, *dA = nullptr;
+    bool dA_masked_zero = false;   // dA's entries above the diagonal already hold the zeros of a first backward call
     // Weight, bias and LayerNorm-parameter gradients are leaves of the backward
     // graph: with `overlap` they go to a second stream and fill the gaps the
     // gradient chain leaves (tile prologues and tails, bandwidth-bound kernels).
@@ -179,8 +181,11 @@ void forward(Model& M) {
         M.ck(jzhip_layernorm_fwd(b.x1, b.xhat1, b.inv1, x, M.t[b.g1].w, M.t[b.be1].w, d, N));
         // Q, K, V in one product against the stacked projection
         gemm(M, M.t[b.Wq].w, false, b.x1, false, b.QKV, 3 * d, N, d);
+        // the weights above the diagonal are zeros written by the first call; later
+        // calls leave them alone (a third of the kernel's stores)
         M.ck(jzhip_attention_fwd_ld(b.H, d, b.A, b.QKV, b.QKV + d, b.QKV + 2 * d, 3 * d, d, c.heads, c.seq,
-                                    c.batch, 1));
+                                    c.batch, b.A_masked_zero ? 2 : 1));
+        b.A_masked_zero = true;
         // R = x + (Wo*H + bo)
         gemm_tail(M, M.t[b.Wo].w, false, b.H, b.R, d, N, d, M.t[b.bo].w, 0, nullptr, x);
         M.ck(jzhip_layernorm_fwd(b.x2, b.xhat2, b.inv2, b.R, M.t[b.g2].w, M.t[b.be2].w, d, N));
@@ -308,7 +313,8 @@ void backward(Model& M, bool update) {
         gemm(M, M.t[b.Wo].w, true, dR, false, M.dH, d, N, d);
         // attention core, gradients into the stacked (3d x N) buffer
         M.ck(jzhip_attention_bwd_ld(dQKV, dQKV + d, dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
-                                    b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch, 1));
+                                    b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch, M.dA_masked_zero ? 2 : 1));
+        M.dA_masked_zero = true;   // the score-gradient scratch is shared by all blocks and only ever used here
         lanes.fork();
         gemm(M, dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
         lanes.back();

@@ -858,6 +858,24 @@ def test_attention_fwd_bwd(gpu, d_k, heads, S, B, causal):
     assert np.array_equal(got[:, 0].reshape(-1), to_host(oq))
     assert np.array_equal(got[:, 1].reshape(-1), to_host(ok_))
     assert np.array_equal(got[:, 2].reshape(-1), to_host(ov))
+    if causal:
+        # causal == 2: a second call on the same score buffers (new operands) leaves the
+        # entries above the diagonal, zeros since the first call, unwritten: same bits as
+        # a first call on fresh buffers
+        q2 = to_dev(rng(5).normal(0, 1, 3 * N * d_k).astype(np.float32))
+        b2 = q2.data_ptr()
+        p2 = [C.c_void_p(b2 + 4 * i * d_k) for i in range(3)]
+        g2 = to_dev(rng(6).normal(0, 1, N * d_k).astype(np.float32))
+        Hf, Af, sf, of = dev_empty(N * d_k), dev_empty(S * S * B * heads), dev_empty(S * S * B * heads), dev_empty(3 * N * d_k)
+        gpu.attention_fwd_ld(dptr(Hf), d_k, dptr(Af), *p2, ld, d_k, heads, S, B, 1)
+        gpu.attention_bwd_ld(C.c_void_p(of.data_ptr()), C.c_void_p(of.data_ptr() + 4 * d_k),
+                             C.c_void_p(of.data_ptr() + 8 * d_k), ld, dptr(sf), dptr(g2), d_k, *p2, ld, dptr(Af),
+                             d_k, heads, S, B, 1)
+        gpu.attention_fwd_ld(dptr(Hs), d_k, dptr(As), *p2, ld, d_k, heads, S, B, 2)
+        gpu.attention_bwd_ld(C.c_void_p(ob), C.c_void_p(ob + 4 * d_k), C.c_void_p(ob + 8 * d_k), ld, dptr(scratch),
+                             dptr(g2), d_k, *p2, ld, dptr(As), d_k, heads, S, B, 2)
+        assert np.array_equal(to_host(Hs), to_host(Hf)) and np.array_equal(to_host(As), to_host(Af))
+        assert np.array_equal(to_host(scratch), to_host(sf)) and np.array_equal(to_host(dqkv), to_host(of))
 
 
 def test_second_stream_workspace_and_event_order(gpu):
