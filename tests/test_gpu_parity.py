@@ -336,6 +336,33 @@ def test_gemm_thin_products(gpu, oracle_lib, m, n, k, ta, tb):
             assert np.array_equal(g2[:, m:], C0.reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("m,n,k,ta,tb", [
+    (256, 512, 128, 0, 0),        # full tiles, unchecked loaders
+    (129, 127, 17, 0, 1),         # ragged edges, checked loaders
+    (256, 128, 8192, 0, 1),       # split along K: partial sums and their reduction
+    (64, 1216, 512, 1, 0),        # 64 x 64 tiles
+    (3, 4100, 576, 1, 0),         # thin, k contiguous in the big operand
+    (576, 3, 5000, 0, 1),         # thin, long extent contiguous, k chunks
+    (300, 1, 70, 0, 0), (1, 300, 70, 1, 0),   # matrix-vector forms
+    (40, 50, 1, 0, 0),            # rank-1
+])
+def test_gemm_with_beta_zero_never_reads_c(gpu, m, n, k, ta, tb):
+    """dot() hands the product a fresh block from the pool (cpp/hipmatrix.cpp:134-152,
+    cpp/memory.hpp:50-97): whatever bits it holds, NaN included, must not reach the
+    result when beta == 0."""
+    r = rng(m + 3 * n + 7 * k)
+    lda, ldb = (k if ta else m), (n if tb else k)
+    A = r.normal(0, 1, m * k).astype(np.float32)
+    B = r.normal(0, 1, k * n).astype(np.float32)
+    C0 = np.full(m * n, np.nan, np.float32)
+    exact = naive_gemm64(ta, tb, m, n, k, 1.0, A, lda, B, ldb, 0.0, np.zeros(m * n, np.float32), m)
+    dC = to_dev(C0)
+    gpu.gemm(dp(A), dp(B), dptr(dC), m, n, k, ta, tb, lda, ldb, m, 1.0, 0.0)
+    got = to_host(dC)
+    assert np.isfinite(got).all()
+    assert rel_err(got, exact) <= TOL_GEMM
+
+
 def test_gemm_thin_products_at_the_output_convolution_size(gpu):
     """3 x 131072 x 576 (forward, TN) and 576 x 3 x 131072 (weight gradient, NT) of a
     64 -> 3 channel 3x3 convolution on 128 images of 32 x 32, against float64."""
