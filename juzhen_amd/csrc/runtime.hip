@@ -189,7 +189,8 @@ JZ_API int jzhip_memcpy_h2d_async(void* dst_device, const void* src_host, size_t
     // compute queue, where a DMA copy between kernels costs a hand-over to the
     // copy engine and back that is far longer than the transfer.
     if (bytes <= kKernelCopyBytes && bytes % sizeof(float) == 0 &&
-        reinterpret_cast<uintptr_t>(dst_device) % sizeof(float) == 0) {
+        reinterpret_cast<uintptr_t>(dst_device) % sizeof(float) == 0 &&
+        reinterpret_cast<uintptr_t>(src_host) % sizeof(float) == 0) {
         hipPointerAttribute_t at;
         if (hipPointerGetAttributes(&at, src_host) == hipSuccess && at.type == hipMemoryTypeHost &&
             at.devicePointer != nullptr)
