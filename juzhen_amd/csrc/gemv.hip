@@ -102,10 +102,42 @@ __global__ __launch_bounds__(kGemvCombineBlock) void gemv_n_combine_kernel(float
 // strides being 1), the thin one V is T x K (V[t*vs_t + k*vs_k]); output (l,t)
 // goes to C[l*cs_l + t*cs_t].
 constexpr int kThinMax = 8;
-constexpr int kThinRows = 4;   // rows of X a wavefront walks together in the dot form
+// rows of X a wavefront walks together in the dot form: two with up to four thin
+// vectors (measured 55 against 58 us at 3 x 131072 x 576), four with more, where
+// each LDS read of V should serve more rows
+template <int TT> constexpr int kThinRows = TT <= 4 ? 2 : 4;
 constexpr int kThinChunkMax = 1024;   // k per workgroup in the other form
 
-// k contiguous in X: a wavefront takes kThinRows rows, its lanes stride over k
+// Sums NV (a power of two, at most 64) values per lane over the 64 lanes.  On
+// return v[0] of lane i holds the total of value i >> log2(64 / NV); the lane
+// whose low bits are zero gets that index back, the others -1.
+template <int N>
+__device__ __forceinline__ void fold_half(float* v, int lane, int mask) {
+    const bool upper = (lane & mask) != 0;
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i) {
+        const float keep = upper ? v[i + N / 2] : v[i];
+        const float send = upper ? v[i] : v[i + N / 2];
+        v[i] = keep + __shfl_xor(send, mask, kWave);
+    }
+}
+template <int NV>
+__device__ __forceinline__ int wave_sum_many(float (&v)[NV], int lane) {
+    static_assert(NV >= 1 && NV <= kWave && (NV & (NV - 1)) == 0, "power of two");
+    int mask = kWave / 2;
+    if constexpr (NV >= 64) { fold_half<64>(v, lane, mask); mask >>= 1; }
+    if constexpr (NV >= 32) { fold_half<32>(v, lane, mask); mask >>= 1; }
+    if constexpr (NV >= 16) { fold_half<16>(v, lane, mask); mask >>= 1; }
+    if constexpr (NV >= 8) { fold_half<8>(v, lane, mask); mask >>= 1; }
+    if constexpr (NV >= 4) { fold_half<4>(v, lane, mask); mask >>= 1; }
+    if constexpr (NV >= 2) { fold_half<2>(v, lane, mask); mask >>= 1; }
+    const int rest = 2 * mask;   // lanes that now hold the same value index, a power of two (or 0 when NV == 64)
+    for (int m = mask; m >= 1; m >>= 1) v[0] += __shfl_xor(v[0], m, kWave);
+    if (rest == 0) return lane;
+    return (lane & (rest - 1)) == 0 ? lane / rest : -1;
+}
+
+// k contiguous in X: a wavefront takes kThinRows<TT> rows, its lanes stride over k
 // in float4 steps against V staged in LDS (each LDS read serves all the rows).
 template <int TT>
 __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restrict__ X, size_t xs_l,
@@ -123,16 +155,17 @@ __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restric
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
     const int K4 = K / 4;
     const float4* v4 = reinterpret_cast<const float4*>(vlds);
-    for (size_t l0 = wave0 * kThinRows; l0 < static_cast<size_t>(L); l0 += nwaves * kThinRows) {
-        float acc[kThinRows][TT];
+    constexpr int R = kThinRows<TT>;
+    for (size_t l0 = wave0 * R; l0 < static_cast<size_t>(L); l0 += nwaves * R) {
+        float acc[R][TT];
 #pragma unroll
-        for (int u = 0; u < kThinRows; ++u)
+        for (int u = 0; u < R; ++u)
 #pragma unroll
             for (int t = 0; t < TT; ++t) acc[u][t] = 0.f;
         for (int k4 = lane; k4 < K4; k4 += kWave) {
-            float4 x[kThinRows];
+            float4 x[R];
 #pragma unroll
-            for (int u = 0; u < kThinRows; ++u) {
+            for (int u = 0; u < R; ++u) {
                 const size_t l = l0 + u < static_cast<size_t>(L) ? l0 + u : L - 1;   // clamped, dropped at the store
                 x[u] = reinterpret_cast<const float4*>(X + l * xs_l)[k4];
             }
@@ -140,22 +173,28 @@ __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restric
             for (int t = 0; t < TT; ++t) {
                 const float4 v = v4[t * K4 + k4];
 #pragma unroll
-                for (int u = 0; u < kThinRows; ++u)
+                for (int u = 0; u < R; ++u)
                     acc[u][t] += x[u].x * v.x + x[u].y * v.y + x[u].z * v.z + x[u].w * v.w;
             }
         }
+        // R*TT sums over the wavefront at once: each exchange halves the number of
+        // values a lane carries (the upper half of the lanes keeps the upper half of
+        // the values), so 64 lanes x NV values cost NV - 1 + log2(64 / NV) exchanges
+        // instead of 6 per value
+        constexpr int NV = R * TT;
+        float v[NV];
 #pragma unroll
-        for (int u = 0; u < kThinRows; ++u)
+        for (int u = 0; u < R; ++u)
 #pragma unroll
-            for (int t = 0; t < TT; ++t) {
-                const float r = wave_sum(acc[u][t]);
-                if (lane == u * TT + t && l0 + u < static_cast<size_t>(L) && t < T) {
-                    float* dst = C + (l0 + u) * cs_l + t * cs_t;
-                    float o = alpha * r;
-                    if (beta != 0.0f) o += beta * *dst;
-                    *dst = o;
-                }
-            }
+            for (int t = 0; t < TT; ++t) v[u * TT + t] = acc[u][t];
+        const int idx = wave_sum_many<NV>(v, lane);
+        const int u = idx / TT, t = idx - u * TT;
+        if (idx >= 0 && l0 + u < static_cast<size_t>(L) && t < T) {
+            float* dst = C + (l0 + u) * cs_l + t * cs_t;
+            float o = alpha * v[0];
+            if (beta != 0.0f) o += beta * *dst;
+            *dst = o;
+        }
     }
 }
 
@@ -268,7 +307,7 @@ template <int TT>
 int thin_launch(const ThinArgs& a) {
     hipStream_t s = stream();
     if (a.xs_k == 1) {
-        const size_t groups = (static_cast<size_t>(a.L) + kThinRows - 1) / kThinRows;
+        const size_t groups = (static_cast<size_t>(a.L) + kThinRows<TT> - 1) / kThinRows<TT>;
         const unsigned grid = grid_for(groups, kBlock / kWave, 8);
         thin_dot_kernel<TT><<<grid, kBlock, static_cast<size_t>(TT) * a.K * sizeof(float), s>>>(
             a.X, a.xs_l, a.V, a.vs_t, a.vs_k, a.C, a.cs_l, a.cs_t, a.L, a.K, a.T, a.alpha, a.beta);
