@@ -6,8 +6,9 @@
  *   - plain C: device pointers are `float*`, element counts `size_t`, matrix
  *     dimensions `int`, flags `int` (0/1).  No C++ or torch types cross it.
  *   - return value: 0 = success, -1 = invalid argument (null pointer,
- *     non-positive dimension, unsupported flag), otherwise a positive
- *     hipError_t value.  `jzhip_error_string` turns it into text.
+ *     non-positive dimension, unsupported flag), -2 = the workspace could not
+ *     be created, -3 = a size beyond the fixed scratch of a no-allocation
+ *     entry point, otherwise a positive hipError_t value.  `jzhip_error_string` turns it into text.
  *   - matrices are fp32, column-major: element (i,j) of a matrix with
  *     physical row count `ld` lives at `p[j*ld + i]`.  A "trans" flag means
  *     the logical matrix is the transpose of the physical one
@@ -233,6 +234,16 @@ int jzhip_one_hot(float* out, const int32_t* labels, int k, size_t n);
  *   jzhip_sum_rows: out[i] = sum_j a[j*ld+i]   (numrow outputs) */
 int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, int ld);
 int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, int ld);
+/* No counterpart in the reference.  For callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  Same result as jzhip_sum_rows (the column-chunk partial
+ * sums are combined in the same fixed order), but the partials live in a fixed
+ * 4 MiB array inside the library's code object instead of the lazily created
+ * workspace, so the call performs no hipMalloc/hipFree at all.  Limit:
+ * numrow <= 65536, otherwise rc -3 (any numcol).  Every call on one GPU shares
+ * that GPU's array: calls that may overlap on one GPU (different streams, or
+ * different host threads) race and must be ordered by the caller. */
+int jzhip_sum_rows_noalloc(float* out, const float* a, int numrow, int numcol, int ld);
 /* out[0] = sqrt(sum x^2): replaces hipblasSnrm2 in norm()
  * (cpp/hipmatrix.cpp:232-254; oracle cpp/core.hpp:337-344). */
 int jzhip_nrm2(float* out_device, const float* x, size_t count);

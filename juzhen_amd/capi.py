@@ -83,6 +83,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_slice_assign": (I, [P, Z, I, Z, Z, P, Z, I, Z, Z]),
     "jzhip_sum_cols": (I, [P, P, I, I, I]),
     "jzhip_sum_rows": (I, [P, P, I, I, I]),
+    "jzhip_sum_rows_noalloc": (I, [P, P, I, I, I]),
     "jzhip_embedding_fwd": (I, [P, P, P, P, P, I, I, I, I]),
     "jzhip_one_hot": (I, [P, P, I, Z]),
     "jzhip_nrm2": (I, [P, P, Z]),

@@ -6,6 +6,7 @@
 // atomics on global memory).
 #include "common.hpp"
 
+#include <atomic>
 #include <cmath>
 
 namespace jz {
@@ -323,9 +324,15 @@ JZ_API int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, in
     return launch_rc();
 }
 
-JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, int ld) {
-    if (numrow <= 0 || numcol <= 0 || ld < numrow) return -1;
-    if (!out || !a) return -1;
+namespace jz {
+namespace {
+
+// Row sums with the partial results of the column chunks in `scratch`
+// (capacity `cap` floats).  `scratch` is a callable so that the shared
+// workspace is only created when a launch really needs partials.
+template <class GetScratch>
+int sum_rows_impl(float* out, const float* a, int numrow, int numcol, int ld, size_t cap,
+                  GetScratch scratch) {
     hipStream_t s = stream();
     if (numrow <= kWave && ld == numrow) {
         // short contiguous matrix: flat stream
@@ -333,16 +340,16 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
         const int active = (kBlock / numrow) * numrow;
         // columns per block so that there are a few blocks per CU
         size_t blocks = (total + static_cast<size_t>(active) * 16 - 1) / (static_cast<size_t>(active) * 16);
-        const size_t cap = static_cast<size_t>(num_cus()) * 8;
-        if (blocks > cap) blocks = cap;
+        const size_t limit = static_cast<size_t>(num_cus()) * 8;
+        if (blocks > limit) blocks = limit;
         if (blocks < 1) blocks = 1;
-        while (blocks > 1 && blocks * numrow > kWorkspaceFloats) blocks /= 2;
+        while (blocks > 1 && blocks * numrow > cap) blocks /= 2;
         size_t cols_per_block = (numcol + blocks - 1) / blocks;
         blocks = (numcol + cols_per_block - 1) / cols_per_block;
         const size_t span = cols_per_block * numrow;
         float* dst = out;
         if (blocks > 1) {
-            dst = workspace();
+            dst = scratch();
             if (!dst) return -2;
         }
         sum_rows_short_kernel<<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(dst, a, numrow, total,
@@ -357,13 +364,13 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
     const int rows_per_block = kWave * (vec ? 4 : 1);
     const int row_blocks = (numrow + rows_per_block - 1) / rows_per_block;
     int chunks = pick_chunks(row_blocks * (kBlock / kWave), numcol, 64);
-    while (chunks > 1 && static_cast<size_t>(chunks) * numrow > kWorkspaceFloats) --chunks;
+    while (chunks > 1 && static_cast<size_t>(chunks) * numrow > cap) --chunks;
     if (chunks > 65535) chunks = 65535;
     const int chunk_len = (numcol + chunks - 1) / chunks;
     chunks = (numcol + chunk_len - 1) / chunk_len;
     float* dst = out;
     if (chunks > 1) {
-        dst = workspace();
+        dst = scratch();
         if (!dst) return -2;
     }
     dim3 grid(row_blocks, chunks);
@@ -375,6 +382,15 @@ JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, in
         combine_partials_kernel<<<(numrow + kWave - 1) / kWave, kCombineBlock, 0, s>>>(out, dst, numrow, chunks);
     }
     return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
+JZ_API int jzhip_sum_rows(float* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow) return -1;
+    if (!out || !a) return -1;
+    return sum_rows_impl(out, a, numrow, numcol, ld, kWorkspaceFloats, [] { return workspace(); });
 }
 
 JZ_API int jzhip_nrm2(float* out_device, const float* x, size_t count) {
@@ -402,4 +418,54 @@ JZ_API int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numco
     const unsigned grid = grid_cover(numcol, kBlock / kWave);
     max_cols_kernel<true><<<grid, kBlock, 0, stream()>>>(nullptr, out, a, numrow, numcol, ld);
     return launch_rc();
+}
+
+// ── row sums without any allocation ──────────────────────────────────────
+// Callers that may not allocate device memory (code under HIP graph capture,
+// serving loops, harnesses that forbid hipMalloc) cannot use the lazily
+// created workspace.  This variant keeps the column-chunk partial sums in a
+// fixed array that is part of the code object: every GPU the library runs on
+// holds its own 4 MiB copy from the first launch until the process ends.
+namespace {
+constexpr size_t kFixedScratchFloats = size_t(1) << 20;   // 4 MiB
+constexpr int kFixedScratchMaxRows = 65536;               // leaves room for >= 16 column chunks
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float scratch[kFixedScratchFloats];
+// Device address of `scratch` per device ordinal.  In host code the array's
+// name is only a handle for hipGetSymbolAddress, never a pointer a kernel may
+// be given.
+std::atomic<float*> g_fixed_scratch[kMaxDevices];
+
+int fixed_scratch(float** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return -1;
+    float* p = g_fixed_scratch[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* addr = nullptr;
+        e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return static_cast<int>(e);
+        }
+        if (!addr) return -2;
+        p = static_cast<float*>(addr);
+        g_fixed_scratch[dev].store(p, std::memory_order_release);   // same value from any thread
+    }
+    *out = p;
+    return 0;
+}
+}  // namespace
+
+JZ_API int jzhip_sum_rows_noalloc(float* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow) return -1;
+    if (!out || !a) return -1;
+    if (numrow > kFixedScratchMaxRows) return -3;
+    float* fixed = nullptr;
+    const int rc = fixed_scratch(&fixed);
+    if (rc) return rc;
+    // Every partial the combine kernel reads is written by the launch before
+    // it, so nothing in the array has to start at zero.
+    return sum_rows_impl(out, a, numrow, numcol, ld, kFixedScratchFloats, [fixed] { return fixed; });
 }

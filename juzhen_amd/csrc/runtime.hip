@@ -113,6 +113,7 @@ JZ_API const char* jzhip_error_string(int rc) {
     if (rc == 0) return "success";
     if (rc == -1) return "jzhip: invalid argument";
     if (rc == -2) return "jzhip: workspace allocation failed";
+    if (rc == -3) return "jzhip: size exceeds the fixed scratch of the no-allocation entry point";
     return hipGetErrorString(static_cast<hipError_t>(rc));
 }
 
