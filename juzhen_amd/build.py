@@ -104,6 +104,10 @@ REFERENCE_PROGRAMS = [
     "tests/testUNet.cu",
     "tests/testTransformerRef.cu",
     "tests/testTransformer.cu",
+    "tests/testUNetLearning.cu",
+    "tests/testTransformerTorchDump.cu",
+    "tests/testRectifiedFlowTinyUNetParity.cu",
+    "tests/testRectifiedPathParity.cu",
 ]
 
 HOST_FLAGS = [
@@ -190,7 +194,13 @@ def build_host(force: bool = False, jobs: int = 6):
     cfg_obj = hostobj / "configs_rocm.o"
     if force or _stale(cfg_obj, [cfg_src, *ours, ROOT / "include" / "jzhip.h"]):
         _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(cfg_src), "-o", str(cfg_obj)], "compile configs.cu (rocm)")
-    REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj)]
+    # transpose-flag / ownership semantics of the mirror against Matrix<float>, one binary
+    sem_src = PKG / "harness" / "semantics.cu"
+    sem_obj = hostobj / "semantics_rocm.o"
+    if force or _stale(sem_obj, [sem_src, *ours, ROOT / "include" / "jzhip.h"]):
+        _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(sem_src), "-o", str(sem_obj)], "compile semantics.cu")
+    REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj),
+                                                                         ("harness/semantics_rocm.cu", sem_obj)]
     cpu_bin = REF_BIN / "configs_cpu"
     if force or _stale(cpu_bin, [cfg_src]):
         blas = sorted(Path("/usr/local/lib").glob("python3*/dist-packages/scipy.libs/libscipy_openblas*.so"))

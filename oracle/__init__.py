@@ -174,3 +174,34 @@ def load_ref():
         lib.jzref_init()
         _ref = lib
     return _ref
+
+
+REF_LIB_OPENBLAS = REF_DIR / "libjzref_openblas.so"
+_ref_blas = None
+
+
+def load_ref_openblas(threads: int | None = None):
+    """The same reference CPU path linked against OpenBLAS (the reference's default
+    configuration, cpp/helper.hpp:190-250), for model-sized checks the BLAS-free
+    build would take minutes over.  None if it was never built.  Returns
+    (library, BLAS thread count)."""
+    global _ref_blas
+    if _ref_blas is None:
+        if not REF_LIB_OPENBLAS.exists():
+            return None
+        lib = C.CDLL(str(REF_LIB_OPENBLAS))
+        for name, (res, args) in REF_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        lib.jzref_init()
+        cores = 1
+        for dep in sorted(Path("/usr/local/lib").glob("python3*/dist-packages/scipy.libs/libscipy_openblas*.so")):
+            blas = C.CDLL(str(dep))
+            want = threads or min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+            blas.scipy_openblas_set_num_threads(C.c_int(want))
+            blas.scipy_openblas_get_num_threads.restype = C.c_int
+            cores = int(blas.scipy_openblas_get_num_threads())
+            break
+        _ref_blas = (lib, cores)
+    return _ref_blas

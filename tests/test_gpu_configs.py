@@ -13,6 +13,8 @@ from pathlib import Path
 import numpy as np
 import pytest
 
+from util import need_ref_binary
+
 pytestmark = pytest.mark.gpu
 
 ROOT = Path(__file__).resolve().parent.parent
@@ -22,9 +24,7 @@ BIN = ROOT / "oracle" / "_ref" / "bin"
 def run_both(tmp_path, config, scale, steps):
     out = {}
     for backend in ("cpu", "rocm"):
-        exe = BIN / f"configs_{backend}"
-        if not exe.exists():
-            pytest.skip(f"{exe} not built (needs the reference tree at build time)")
+        exe = need_ref_binary(BIN / f"configs_{backend}")
         env = dict(os.environ, JZ_CONFIG=config, JZ_SCALE=scale, JZ_STEPS=str(steps), JZ_OUT=str(tmp_path))
         print(f"running configs_{backend} {config} {scale} steps={steps}", flush=True)
         r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=900, env=env)

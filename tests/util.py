@@ -58,3 +58,23 @@ def hp(a):
     a = np.ascontiguousarray(a)
     _KEEP.append(a)
     return hptr(a)
+
+
+def need_ref_binary(exe):
+    """Programs built from the reference tree live under oracle/_ref (never
+    committed).  A missing one is a failure wherever a reference build was
+    possible or has happened (the tree is mounted, or oracle/_ref exists), and
+    a skip only in a checkout that never saw the reference."""
+    import os
+    from pathlib import Path
+
+    import pytest
+    exe = Path(exe)
+    if exe.exists():
+        return exe
+    ref_root = Path(os.environ.get("JUZHEN_REFERENCE", "/root/reference"))
+    ref_out = Path(__file__).resolve().parent.parent / "oracle" / "_ref"
+    if ref_root.exists() or ref_out.exists():
+        pytest.fail(f"{exe} is missing although a reference build is expected here: "
+                    "run `python -m juzhen_amd.build --host` where the reference tree is mounted")
+    pytest.skip(f"{exe} not built (this checkout has never seen the reference tree)")
