@@ -199,8 +199,14 @@ def build_host(force: bool = False, jobs: int = 6):
     sem_obj = hostobj / "semantics_rocm.o"
     if force or _stale(sem_obj, [sem_src, *ours, ROOT / "include" / "jzhip.h"]):
         _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(sem_src), "-o", str(sem_obj)], "compile semantics.cu")
+    # the character LM written with the reference's own layer classes (drop-in API measurement)
+    dro_src = PKG / "harness" / "lm_dropin.cu"
+    dro_obj = hostobj / "lm_dropin_rocm.o"
+    if force or _stale(dro_obj, [dro_src, *ours, ROOT / "include" / "jzhip.h"]):
+        _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(dro_src), "-o", str(dro_obj)], "compile lm_dropin.cu")
     REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj),
-                                                                         ("harness/semantics_rocm.cu", sem_obj)]
+                                                                         ("harness/semantics_rocm.cu", sem_obj),
+                                                                         ("harness/lm_dropin_rocm.cu", dro_obj)]
     cpu_bin = REF_BIN / "configs_cpu"
     if force or _stale(cpu_bin, [cfg_src]):
         blas = sorted(Path("/usr/local/lib").glob("python3*/dist-packages/scipy.libs/libscipy_openblas*.so"))

@@ -401,16 +401,22 @@ MR col_softmax(const MR& M) {
     return JzRocmFused::materialise(tmp);
 }
 
-// row_softmax(M) = col_softmax(M.T()).T()  (ml/layer.hpp:2364-2367)
+// row_softmax(M) = col_softmax(M.T()).T()  (ml/layer.hpp:2364-2367): the result
+// is always a transposed view of a plain (cols x rows) buffer, like the CPU's.
 MR row_softmax(const MR& M) {
-    if (M.num_row() == 0 || M.num_col() == 0) return JzRocmFused::make("softmax", M.num_row(), M.num_col(), 0);
-    const int pr = as_int(JzRocmFused::phys_rows(M)), pc = as_int(JzRocmFused::phys_cols(M));
-    MR out = JzRocmFused::like("softmax", M);  // same layout and flag as M
-    if (!M.get_transpose())
-        ok(jzhip_softmax_rows(JzRocmFused::ptr(out), JzRocmFused::ptr(M), pr, pc, pr), "softmax_rows");
-    else
+    if (M.num_row() == 0 || M.num_col() == 0) return MR(JzRocmFused::make("softmax", M.num_col(), M.num_row(), 0).T());
+    if (M.get_transpose()) {
+        // logical rows are contiguous physical columns already
+        const int pr = as_int(JzRocmFused::phys_rows(M)), pc = as_int(JzRocmFused::phys_cols(M));
+        MR out = JzRocmFused::like("softmax", M);
         ok(jzhip_softmax_cols(JzRocmFused::ptr(out), JzRocmFused::ptr(M), pr, pc, pr), "softmax_cols");
-    return out;
+        return out;
+    }
+    // plain input: lay the rows out contiguously, then the column kernel in place
+    MR t = JzRocmFused::materialise(M.T());
+    const int pr = as_int(JzRocmFused::phys_rows(t)), pc = as_int(JzRocmFused::phys_cols(t));
+    ok(jzhip_softmax_cols(JzRocmFused::ptr(t), JzRocmFused::ptr(t), pr, pc, pr), "softmax_cols");
+    return MR(t.T());
 }
 
 }  // namespace Juzhen
