@@ -403,6 +403,12 @@ int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma,
 int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float* gamma,
                                  const float* xhat, const float* inv_std,
                                  const float* res, int dim, int N);
+/* Tangent through the normalisation at the point cached by the forward call:
+ * out = gamma .* inv*(dx - mean(dx) - xhat*mean(dx*xhat)), LayerNorm<D>::jvp
+ * (ml/layer.hpp:2690-2702: two sums, three rank-1 products and four Hadamard
+ * products there). */
+int jzhip_layernorm_jvp(float* out, const float* dx, const float* gamma,
+                        const float* xhat, const float* inv_std, int dim, int N);
 /* dgamma[i] = sum_c dy*xhat, dbeta[i] = sum_c dy in one pass over dy/xhat:
  * the two sum(...,1) calls of ml/layer.hpp:2683-2686. */
 int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,

@@ -204,7 +204,13 @@ def build_host(force: bool = False, jobs: int = 6):
     dro_obj = hostobj / "lm_dropin_rocm.o"
     if force or _stale(dro_obj, [dro_src, *ours, ROOT / "include" / "jzhip.h"]):
         _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(dro_src), "-o", str(dro_obj)], "compile lm_dropin.cu")
+    # forward-mode tangents on the device against the CPU (the reference's testJVP skips on ROCm)
+    jvp_src = PKG / "harness" / "jvp_check.cu"
+    jvp_obj = hostobj / "jvp_check_rocm.o"
+    if force or _stale(jvp_obj, [jvp_src, *ours, ROOT / "include" / "jzhip.h"]):
+        _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(jvp_src), "-o", str(jvp_obj)], "compile jvp_check.cu")
     REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj),
+                                                                         ("harness/jvp_check_rocm.cu", jvp_obj),
                                                                          ("harness/semantics_rocm.cu", sem_obj),
                                                                          ("harness/lm_dropin_rocm.cu", dro_obj)]
     cpu_bin = REF_BIN / "configs_cpu"

@@ -109,6 +109,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_layernorm_fwd": (I, [P, P, P, P, P, P, I, I]),
     "jzhip_layernorm_bwd": (I, [P, P, P, P, P, I, I]),
     "jzhip_layernorm_bwd_residual": (I, [P, P, P, P, P, P, I, I]),
+    "jzhip_layernorm_jvp": (I, [P, P, P, P, P, I, I]),
     "jzhip_layernorm_param_grads": (I, [P, P, P, P, I, I]),
     "jzhip_adam_update": (I, [P, P, P, Z, F, F, F, F, I]),
     "jzhip_adamw_step": (I, [P, P, P, P, Z, F, F, F, F, F, I]),

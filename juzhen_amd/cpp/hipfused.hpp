@@ -75,6 +75,19 @@ inline Matrix<ROCMfloat> LayerNorm<ROCMfloat>::backward(Matrix<ROCMfloat>&& dy, 
     return dx;
 }
 
+// Tangent through the normalisation at the point cached by forward()
+// (ml/layer.hpp:2690-2702): one kernel instead of two sums, three rank-1
+// products and four Hadamard products.
+template <>
+inline Matrix<ROCMfloat> LayerNorm<ROCMfloat>::jvp(const Matrix<ROCMfloat>& dx) const {
+    using namespace rocm_detail;
+    if (dx.get_transpose()) return jvp(JzRocmFused::materialise(dx));
+    const int N = (int)dx.num_col();
+    Matrix<ROCMfloat> out("ln_jvp", dim, N);
+    must(jzhip_layernorm_jvp(p(out), p(dx), p(gamma), p(cached_xhat), p(cached_inv), dim, N), "layernorm_jvp");
+    return out;
+}
+
 // ── TransformerLayer ─────────────────────────────────────────────────────────
 
 template <>
@@ -158,6 +171,62 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
         b2 -= adam_update(std::move(db2), adam_b2);
     }
     return dx;
+}
+
+// Tangent of the whole block at the point cached by eval() (ml/layer.hpp:3034-3178).
+// The attention part follows the structure of the reference's batched CUDA
+// branch (:3061-3142): per head two strided-batched products for the score
+// tangent dS = dQ^T K + Q^T dK, one softmax-tangent kernel over all blocks
+// (the softmax Jacobian is symmetric, so it is the backward kernel), two
+// products for dH = dV A^T + V dA^T -- instead of about fifteen launches per
+// (head, sequence) block of the generic slice loop.
+template <>
+inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::jvp(const Matrix<ROCMfloat>&, const Matrix<ROCMfloat>& tangent_in) {
+    using namespace rocm_detail;
+    using MD = Matrix<ROCMfloat>;
+    const int N = seq_len * batchN;
+    const float scale = 1.0f / sqrtf((float)d_h);
+    const MD tangent = plain(tangent_in);
+
+    MD dx1 = ln1.jvp(tangent);
+    MD dQ = Wq * dx1;
+    MD dK = Wk * dx1;
+    MD dV = Wv * dx1;
+
+    const long long stride_qkv = (long long)d_k * seq_len;
+    const long long stride_attn = (long long)seq_len * seq_len;
+    const long long head_attn = stride_attn * batchN;
+    float* ds = p(attn_dS_scratch);
+    MD dH("jvp_dH", d_k, N);
+    for (int hh = 0; hh < num_heads; ++hh) {
+        // dS_h[query, key] = <dQ[:, query], K[:, key]> + <Q[:, query], dK[:, key]>, unscaled
+        must(jzhip_gemm_strided_batched(p(dQ) + hh * d_h, p(cached_K) + hh * d_h, ds + hh * head_attn, seq_len, seq_len,
+                                        d_h, 1, 0, d_k, d_k, seq_len, stride_qkv, stride_qkv, stride_attn, batchN,
+                                        1.0f, 0.0f),
+             "jvp scores (dQ)");
+        must(jzhip_gemm_strided_batched(p(cached_Q) + hh * d_h, p(dK) + hh * d_h, ds + hh * head_attn, seq_len, seq_len,
+                                        d_h, 1, 0, d_k, d_k, seq_len, stride_qkv, stride_qkv, stride_attn, batchN,
+                                        1.0f, 1.0f),
+             "jvp scores (dK)");
+    }
+    // dA = A .* (scale*dS - rowsum(A .* scale*dS)), in place
+    must(jzhip_attn_softmax_bwd(ds, p(cached_A), ds, seq_len, batchN * num_heads, scale, 0), "jvp softmax");
+    for (int hh = 0; hh < num_heads; ++hh) {
+        // dH_h = dV_h A_h^T + V_h dA_h^T
+        must(jzhip_gemm_strided_batched(p(dV) + hh * d_h, p(cached_A) + hh * head_attn, p(dH) + hh * d_h, d_h, seq_len,
+                                        seq_len, 0, 1, d_k, seq_len, d_k, stride_qkv, stride_attn, stride_qkv, batchN,
+                                        1.0f, 0.0f),
+             "jvp dH (dV)");
+        must(jzhip_gemm_strided_batched(p(cached_V) + hh * d_h, ds + hh * head_attn, p(dH) + hh * d_h, d_h, seq_len,
+                                        seq_len, 0, 1, d_k, seq_len, d_k, stride_qkv, stride_attn, stride_qkv, batchN,
+                                        1.0f, 1.0f),
+             "jvp dH (dA)");
+    }
+    MD dR = tangent + Wo * dH;
+    MD dx2 = ln2.jvp(dR);
+    MD dF1 = W1 * dx2;
+    must(jzhip_drelu_mul(p(dF1), p(cached_F1), p(dF1), (size_t)d_ff * N), "drelu_mul");
+    return dR + W2 * dF1;
 }
 
 }  // namespace Juzhen

@@ -34,6 +34,52 @@ inline int as_int(size_t v) { return static_cast<int>(v); }
 
 void pool_release(ROCMfloat* p) { Memory<ROCMfloat>::free(p); }
 
+// Host -> device uploads.  The reference's converting constructor is a blocking
+// copy from pageable memory (cpp/hipmatrix.cpp:60-63): it waits for everything
+// in flight, so a training loop that uploads a batch per step
+// (ml/dataloader.hpp:88-113, examples/demo_transformer.cu:378-380) drains the
+// device once per step.  Here the host data is copied into one of two
+// page-locked staging buffers and an asynchronous copy is enqueued behind the
+// work in flight; the call returns once the staging buffer holds the data, so
+// the caller may reuse or free its buffer at once, as with the blocking copy.
+// A staging buffer is reused only after the event behind its last copy has
+// passed.  Uploads beyond the staging cap take the blocking copy.
+struct Staging {
+    void* buf = nullptr;
+    size_t cap = 0;
+    void* event = nullptr;
+    bool busy = false;
+};
+constexpr size_t kStagingCap = size_t(64) << 20;
+Staging g_staging[2];
+int g_staging_next = 0;
+
+void upload(float* dst, const float* src, size_t count) {
+    const size_t bytes = count * sizeof(float);
+    if (bytes == 0) return;
+    if (bytes > kStagingCap) {
+        ok(jzhip_memcpy_h2d(dst, src, count), "upload");
+        return;
+    }
+    Staging& st = g_staging[g_staging_next];
+    g_staging_next ^= 1;
+    if (st.busy) {
+        ok(jzhip_event_synchronize(st.event), "upload (staging wait)");
+        st.busy = false;
+    }
+    if (st.cap < bytes) {
+        if (st.buf) ok(jzhip_host_free(st.buf), "upload (staging free)");
+        st.buf = nullptr;
+        st.cap = (bytes + (size_t(1) << 20) - 1) >> 20 << 20;
+        ok(jzhip_host_alloc(&st.buf, st.cap), "upload (staging alloc)");
+    }
+    if (!st.event) ok(jzhip_event_create(&st.event), "upload (event)");
+    std::memcpy(st.buf, src, bytes);
+    ok(jzhip_memcpy_h2d_async(dst, st.buf, bytes), "upload");
+    ok(jzhip_event_record(st.event), "upload (event record)");
+    st.busy = true;
+}
+
 }  // namespace
 
 using MR = Matrix<ROCMfloat>;
@@ -52,7 +98,7 @@ MR::Matrix(const char* name, size_t numrow, size_t numcol, int trans)
 MR::Matrix(const Matrix<float>& M)
     : MR(M.get_name().c_str(), M.numrow, M.numcol, M.transpose) {
     // physical dims and the flag travel unchanged (cpp/hipmatrix.cpp:60-63)
-    ok(jzhip_memcpy_h2d(dev(), M.data(), count()), "upload");
+    upload(dev(), M.data(), count());
 }
 
 MR::Matrix(const MR& M) : MR(M.name.c_str(), M.numrow, M.numcol, M.transpose) {
@@ -461,7 +507,7 @@ void read(FILE* fp, MR& M) {
     M.numrow = tmp.numrow;
     M.numcol = tmp.numcol;
     M.transpose = tmp.transpose;
-    ok(jzhip_memcpy_h2d(M.dev(), tmp.elements.get(), M.count()), "upload");
+    upload(M.dev(), tmp.elements.get(), M.count());
 }
 
 #endif  // ROCM_HIP

@@ -234,27 +234,26 @@ inline Matrix<ROCMfloat> adam_update(Matrix<ROCMfloat>&& g, adam_state<ROCMfloat
 
 // ── user-functor templates ──────────────────────────────────────────────────
 // elemwise<F> and reduce<F> take arbitrary device functors, so they have to be
-// header templates that launch from the user's translation unit.  elemwise is
-// a grid-stride kernel over float4 (the functor is applied per lane, so its
-// semantics are unchanged); reduce keeps the reference contract "one functor
-// call per reduced vector, on a contiguous vector the functor may overwrite".
+// header templates that launch from the user's translation unit.  elemwise
+// applies the functor per lane over float4 loads, one float4 per thread with
+// the grid covering the data once (workgroups are dispatched in id order, so
+// the resident ones stream one compact window of memory).  reduce keeps the
+// reference contract "one functor call per reduced vector, on a contiguous
+// vector the functor may overwrite" (cpp/matrix.hpp:202-250) but moves the
+// data with the whole workgroup: a group of vectors is read into LDS in
+// coalesced rows, each vector's functor call then runs on its LDS copy, and
+// whatever the functor changed is written back the same way, so the caller
+// sees the same overwritten input as on the CPU (examples/knn.cu:61-78 relies
+// on overwriting its input while it selects minima).
 
 namespace jzrocm {
 constexpr int kThreads = 256;
 inline hipStream_t stream() { return static_cast<hipStream_t>(jzhip_get_stream()); }
-inline unsigned grid_for(size_t items) {
-    static int cus = 0;
-    if (cus == 0) {
-        hipDeviceProp_t prop;
-        int dev = 0;
-        cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-                  ? prop.multiProcessorCount
-                  : 256;
-    }
+inline unsigned grid_cover(size_t items) {
     size_t need = (items + kThreads - 1) / kThreads;
-    size_t cap = static_cast<size_t>(cus) * 8;
     if (need < 1) need = 1;
-    return static_cast<unsigned>(need < cap ? need : cap);
+    if (need > 0x7fffffffull) need = 0x7fffffffull;   // the kernels keep a stride loop for the excess
+    return static_cast<unsigned>(need);
 }
 
 template <class Function>
@@ -279,6 +278,8 @@ __global__ __launch_bounds__(kThreads) void elemwise_kernel(Function func, float
     }
 }
 
+// One thread per vector, straight from global memory: vectors too long for
+// the staged form below.
 template <class Function>
 __global__ __launch_bounds__(kThreads) void reduce_kernel(Function func, float* vecdes, float* vec,
                                                           size_t lenvec, size_t lenvecdes,
@@ -287,6 +288,75 @@ __global__ __launch_bounds__(kThreads) void reduce_kernel(Function func, float* 
     for (size_t i = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; i < numvecs; i += stride)
         func(&vec[i * lenvec], &vecdes[i * lenvecdes], lenvec, lenvecdes);
 }
+
+// Staged form: a workgroup takes `group` consecutive vectors (group * lenvec
+// floats, contiguous in memory), keeps two copies in LDS with an odd pitch
+// (lanes that walk their own vectors in step hit distinct banks), runs one
+// functor call per vector on the first copy, then compares the copies and
+// writes the group back only when a call changed its vector.
+constexpr int kReduceLdsFloats = 8128;   // per copy: two copies fill the 64 KiB a workgroup may declare
+template <class Function>
+__global__ __launch_bounds__(kThreads) void reduce_staged_kernel(Function func, float* vecdes, float* vec,
+                                                                 int lenvec, int lenvecdes,
+                                                                 size_t numvecs, int group, int pitch) {
+    __shared__ float work[kReduceLdsFloats];
+    __shared__ float keep[kReduceLdsFloats];
+    __shared__ int changed;
+    // element e = threadIdx.x + i*kThreads of the group is (vector v, row r): stepped without divisions
+    const int v0 = threadIdx.x / lenvec, r0 = threadIdx.x % lenvec;
+    const int dv = kThreads / lenvec, dr = kThreads % lenvec;
+    for (size_t first = static_cast<size_t>(blockIdx.x) * group; first < numvecs;
+         first += static_cast<size_t>(gridDim.x) * group) {
+        const int nv = numvecs - first < static_cast<size_t>(group) ? static_cast<int>(numvecs - first) : group;
+        const int total = nv * lenvec;
+        float* base = vec + first * lenvec;
+        if (threadIdx.x == 0) changed = 0;
+        for (int e = threadIdx.x, v = v0, r = r0; e < total; e += kThreads) {
+            const float x = base[e];
+            work[v * pitch + r] = x;
+            keep[v * pitch + r] = x;
+            v += dv; r += dr;
+            if (r >= lenvec) { r -= lenvec; ++v; }
+        }
+        __syncthreads();
+        if (threadIdx.x < nv)
+            func(&work[threadIdx.x * pitch], &vecdes[(first + threadIdx.x) * lenvecdes], lenvec, lenvecdes);
+        __syncthreads();
+        int diff = 0;
+        for (int e = threadIdx.x, v = v0, r = r0; e < total; e += kThreads) {
+            // bit comparison: a functor that writes the same value, or a NaN, counts as it should
+            diff |= __float_as_uint(work[v * pitch + r]) != __float_as_uint(keep[v * pitch + r]);
+            v += dv; r += dr;
+            if (r >= lenvec) { r -= lenvec; ++v; }
+        }
+        if (diff) changed = 1;
+        __syncthreads();
+        if (changed) {
+            for (int e = threadIdx.x, v = v0, r = r0; e < total; e += kThreads) {
+                base[e] = work[v * pitch + r];
+                v += dv; r += dr;
+                if (r >= lenvec) { r -= lenvec; ++v; }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <class Function>
+inline void launch_reduce(Function func, float* dst, float* src, size_t lenvec, size_t k, size_t numvecs) {
+    if (numvecs == 0) return;
+    if (lenvec >= 1 && lenvec <= static_cast<size_t>(kReduceLdsFloats) / 2) {
+        const int pitch = static_cast<int>(lenvec | 1);                       // odd: conflict-free column walks
+        int group = kReduceLdsFloats / pitch;
+        if (group > kThreads) group = kThreads;
+        const size_t blocks = (numvecs + group - 1) / group;
+        reduce_staged_kernel<<<static_cast<unsigned>(blocks < 0x7fffffffull ? blocks : 0x7fffffffull), kThreads, 0,
+                               stream()>>>(func, dst, src, static_cast<int>(lenvec), static_cast<int>(k), numvecs,
+                                           group, pitch);
+        return;
+    }
+    reduce_kernel<<<grid_cover(numvecs), kThreads, 0, stream()>>>(func, dst, src, lenvec, k, numvecs);
+}
 }  // namespace jzrocm
 
 template <class Function>
@@ -294,7 +364,7 @@ Matrix<ROCMfloat> elemwise(Function func, const Matrix<ROCMfloat>& M) {
     Matrix<ROCMfloat> result("resM", M.numrow, M.numcol, M.transpose);
     const size_t n = M.count();
     const int vec = ((reinterpret_cast<uintptr_t>(M.dev()) | reinterpret_cast<uintptr_t>(result.dev())) & 15) == 0;
-    jzrocm::elemwise_kernel<<<jzrocm::grid_for(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+    jzrocm::elemwise_kernel<<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
         func, result.dev(), M.dev(), n, vec);
     return result;
 }
@@ -303,7 +373,7 @@ template <class Function>
 Matrix<ROCMfloat> elemwise(Function func, Matrix<ROCMfloat>&& M) {
     const size_t n = M.count();
     const int vec = (reinterpret_cast<uintptr_t>(M.dev()) & 15) == 0;
-    jzrocm::elemwise_kernel<<<jzrocm::grid_for(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+    jzrocm::elemwise_kernel<<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
         func, M.dev(), M.dev(), n, vec);
     return std::move(M);
 }
@@ -316,15 +386,13 @@ Matrix<ROCMfloat> reduce(Function func, const Matrix<ROCMfloat>& M, int dim, int
     const bool direct = (dim == 0) == !M.transpose;
     if (direct) {
         Matrix<ROCMfloat> result("resM", k, M.numcol);
-        jzrocm::reduce_kernel<<<jzrocm::grid_for(M.numcol), jzrocm::kThreads, 0, jzrocm::stream()>>>(
-            func, result.dev(), M.dev(), M.numrow, k, M.numcol);
+        jzrocm::launch_reduce(func, result.dev(), M.dev(), M.numrow, k, M.numcol);
         return M.transpose ? Matrix<ROCMfloat>(result.T()) : result;
     }
     // physical transpose of the buffer: its columns are the vectors to reduce
     Matrix<ROCMfloat> t = JzRocmFused::materialise(M.transpose ? M : M.T());
     Matrix<ROCMfloat> result("resM", k, t.numcol);
-    jzrocm::reduce_kernel<<<jzrocm::grid_for(t.numcol), jzrocm::kThreads, 0, jzrocm::stream()>>>(
-        func, result.dev(), t.dev(), t.numrow, k, t.numcol);
+    jzrocm::launch_reduce(func, result.dev(), t.dev(), t.numrow, k, t.numcol);
     return M.transpose ? result : Matrix<ROCMfloat>(result.T());
 }
 

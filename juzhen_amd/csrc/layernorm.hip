@@ -104,7 +104,10 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic_kernel(float* y, float*
     }
 }
 
-template <int NV>
+// JVP = false: dx = P(gamma .* dy) (+ res), the backward pass.  JVP = true:
+// out = gamma .* P(dy), the tangent through the same standardisation operator
+// P(v) = inv .* (v - mean(v) - xhat .* mean(xhat .* v)) (ml/layer.hpp:2690-2702).
+template <int NV, bool JVP>
 __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const float* dy,
                                                             const float* gamma, const float* xhat,
                                                             const float* inv_std, const float* res,
@@ -129,7 +132,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
             if (r < dim) {
                 d[v] = *reinterpret_cast<const float4*>(dy + base + r);
                 h[v] = *reinterpret_cast<const float4*>(xhat + base + r);
-                d[v].x *= g[v].x; d[v].y *= g[v].y; d[v].z *= g[v].z; d[v].w *= g[v].w;
+                if constexpr (!JVP) { d[v].x *= g[v].x; d[v].y *= g[v].y; d[v].z *= g[v].z; d[v].w *= g[v].w; }
                 s1 += (d[v].x + d[v].y) + (d[v].z + d[v].w);
                 s2 += (d[v].x * h[v].x + d[v].y * h[v].y) + (d[v].z * h[v].z + d[v].w * h[v].w);
             }
@@ -146,6 +149,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
                 o.y = inv * (d[v].y - m1 - h[v].y * m2);
                 o.z = inv * (d[v].z - m1 - h[v].z * m2);
                 o.w = inv * (d[v].w - m1 - h[v].w * m2);
+                if constexpr (JVP) { o.x *= g[v].x; o.y *= g[v].y; o.z *= g[v].z; o.w *= g[v].w; }
                 if (res) {  // dx = LN'(dy) + res, rounded like a separate add
                     const float4 rr = *reinterpret_cast<const float4*>(res + base + r);
                     o.x += rr.x; o.y += rr.y; o.z += rr.z; o.w += rr.w;
@@ -156,6 +160,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
     }
 }
 
+template <bool JVP>
 __global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const float* dy,
                                                                 const float* gamma,
                                                                 const float* xhat,
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const
         const size_t base = col * dim;
         float s1 = 0.f, s2 = 0.f;
         for (int r = lane; r < dim; r += kWave) {
-            const float d = dy[base + r] * gamma[r];
+            const float d = JVP ? dy[base + r] : dy[base + r] * gamma[r];
             s1 += d;
             s2 += d * xhat[base + r];
         }
@@ -177,8 +182,9 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_generic_kernel(float* dx, const
         const float m2 = wave_sum(s2) * invdim;
         const float inv = inv_std[col];
         for (int r = lane; r < dim; r += kWave) {
-            const float d = dy[base + r] * gamma[r];
+            const float d = JVP ? dy[base + r] : dy[base + r] * gamma[r];
             float o = inv * (d - m1 - xhat[base + r] * m2);
+            if constexpr (JVP) o *= gamma[r];
             if (res) o += res[base + r];
             dx[base + r] = o;
         }
@@ -334,23 +340,36 @@ JZ_API int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const floa
     return launch_rc();
 }
 
-JZ_API int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float* gamma,
-                                        const float* xhat, const float* inv_std, const float* res,
-                                        int dim, int N) {
+namespace {
+template <bool JVP>
+int launch_ln_bwd(float* dx, const float* dy, const float* gamma, const float* xhat, const float* inv_std,
+                  const float* res, int dim, int N) {
     if (dim <= 0 || N <= 0 || !dx || !dy || !gamma || !xhat || !inv_std) return -1;
     const bool vec = (dim % 4 == 0) && dim <= 1024 && aligned16(dx) && aligned16(dy) &&
                      aligned16(xhat) && aligned16(gamma) && (!res || aligned16(res));
     const unsigned grid = grid_cover(N, kBlock / kWave);
     hipStream_t s = stream();
     if (vec && dim <= 256)
-        ln_bwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+        ln_bwd_vec_kernel<1, JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     else if (vec && dim <= 512)
-        ln_bwd_vec_kernel<2><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+        ln_bwd_vec_kernel<2, JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     else if (vec)
-        ln_bwd_vec_kernel<4><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+        ln_bwd_vec_kernel<4, JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     else
-        ln_bwd_generic_kernel<<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+        ln_bwd_generic_kernel<JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     return launch_rc();
+}
+}  // namespace
+
+JZ_API int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float* gamma,
+                                        const float* xhat, const float* inv_std, const float* res,
+                                        int dim, int N) {
+    return launch_ln_bwd<false>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+}
+
+JZ_API int jzhip_layernorm_jvp(float* out, const float* dx, const float* gamma, const float* xhat,
+                               const float* inv_std, int dim, int N) {
+    return launch_ln_bwd<true>(out, dx, gamma, xhat, inv_std, nullptr, dim, N);
 }
 
 JZ_API int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma, const float* xhat,

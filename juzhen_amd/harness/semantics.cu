@@ -210,6 +210,23 @@ void battery(std::vector<Rec>& out, int r, int c, const std::string& tag) {
         out.push_back(rec(N("reduce(stats,At,1,2)"), reduce(stats_f, A.T(), 1, 2)));
         // the input of a reduce is left as it was
         out.push_back(rec(N("A after reduce"), A));
+        // a functor that overwrites its vector (the selection of examples/knn.cu:61-78): when the
+        // vectors are the matrix's own columns the caller sees them overwritten, on both backends;
+        // along the other dimension the functor works on a private transposed copy
+        auto min2_f = [] __GPU_CPU__(float* src, float* dst, int n, int k) {
+            for (int j = 0; j < k; ++j) {
+                int at = 0;
+                for (int i = 1; i < n; ++i)
+                    if (src[i] < src[at]) at = i;
+                dst[j] = (float)at;
+                src[at] = 1e30f;
+            }
+        };
+        Matrix<D> X(A), Y(A);
+        out.push_back(rec(N("reduce(min2,X,0,2)"), reduce(min2_f, X, 0, 2)));
+        out.push_back(rec(N("X after overwriting reduce"), X));
+        out.push_back(rec(N("reduce(min2,Y,1,2)"), reduce(min2_f, Y, 1, 2)));
+        out.push_back(rec(N("Y after overwriting reduce"), Y));
     }
     // elemwise<F> keeps layout and flag; rvalue reuses the buffer
     {
@@ -319,6 +336,96 @@ int exceptions(const char* what) {
     return caught == wanted ? 0 : 1;
 }
 
+// write/read of the .matrix layout (three ints numrow, numcol, transpose, then the
+// physical payload; cpp/core.hpp:484-525) through Matrix<D>: the file a device
+// matrix writes must be byte-identical to the CPU writer's, for both transpose
+// flags, and read back into a device matrix must give the same matrix.
+template <class D>
+int io_roundtrip(const char* what) {
+    D* const sel = nullptr;
+    int bad = 0;
+    const std::string dir = std::string(PROJECT_DIR) + "/res/";
+    for (int flag = 0; flag < 2; ++flag) {
+        const Matrix<float> base = quarters(7, 5, 77 + flag);
+        const Matrix<float> Mh = flag ? deep(base.T()) : base;
+        const Matrix<D> Md = up(Mh, sel);
+        const std::string f_cpu = dir + "io_cpu.matrix", f_dev = dir + "io_dev.matrix";
+        FILE* fp = std::fopen(f_cpu.c_str(), "wb");
+        if (!fp) { std::printf("%s io: cannot write %s\n", what, f_cpu.c_str()); return 1; }
+        write(fp, Mh);
+        std::fclose(fp);
+        fp = std::fopen(f_dev.c_str(), "wb");
+        write(fp, Md);
+        std::fclose(fp);
+        auto slurp = [](const std::string& p) {
+            std::vector<unsigned char> b;
+            if (FILE* f = std::fopen(p.c_str(), "rb")) {
+                unsigned char buf[4096];
+                size_t n;
+                while ((n = std::fread(buf, 1, sizeof buf, f)) > 0) b.insert(b.end(), buf, buf + n);
+                std::fclose(f);
+            }
+            return b;
+        };
+        const auto a = slurp(f_cpu), b = slurp(f_dev);
+        int hdr[3] = {0, 0, 0};
+        if (a.size() >= 12) std::memcpy(hdr, a.data(), 12);
+        const bool header_ok = a.size() == 12 + 35 * sizeof(float) && hdr[0] == 7 && hdr[1] == 5 &&
+                               hdr[2] == flag;   // physical dims travel, the flag beside them
+        if (!header_ok || a != b) {
+            std::printf("FAIL %s io flag %d: files differ or header wrong (%zu vs %zu bytes, header %d %d %d)\n", what,
+                        flag, a.size(), b.size(), hdr[0], hdr[1], hdr[2]);
+            ++bad;
+        }
+        Matrix<D> R("r", 2, 2);
+        fp = std::fopen(f_dev.c_str(), "rb");
+        read(fp, R);
+        std::fclose(fp);
+        const Rec want = rec("io", Mh), got = rec("io", R);
+        if (want.rows != got.rows || want.cols != got.cols || want.flag != got.flag || want.v != got.v) {
+            std::printf("FAIL %s io flag %d: read back %zux%zu flag %d\n", what, flag, got.rows, got.cols, got.flag);
+            ++bad;
+        }
+    }
+    std::printf("%s .matrix round trip: %d failures\n", what, bad);
+    return bad;
+}
+
+// Uploads must not disturb work in flight and must deliver the host values as
+// they were at the call: the converting constructor copies through page-locked
+// staging buffers and returns before the device has run the copy.
+template <class D>
+int uploads_in_flight(const char* what) {
+    D* const sel = nullptr;
+    int bad = 0;
+    const Matrix<float> Wh = quarters(256, 256, 3);
+    const Matrix<D> W = up(Wh, sel);
+    Matrix<D> acc = W * W;                               // work in flight while batches are uploaded
+    std::vector<Matrix<D>> kept;
+    std::vector<Matrix<float>> want;
+    Matrix<float> batch = quarters(300, 41, 9);
+    for (int i = 0; i < 12; ++i) {
+        float* p = const_cast<float*>(batch.data());
+        for (int j = 0; j < 300 * 41; ++j) p[j] += 0.25f;   // the host buffer is reused right after each upload
+        kept.push_back(up(batch, sel));
+        want.push_back(batch);
+        acc = acc * W * (1.0 / 4096.0);
+    }
+    for (size_t i = 0; i < kept.size(); ++i)
+        if (rec("u", kept[i]).v != rec("u", want[i]).v) {
+            std::printf("FAIL %s upload %zu differs from the host values at the call\n", what, i);
+            ++bad;
+        }
+    // one larger than a staging buffer is expected to hold
+    const Matrix<float> big = quarters(4096, 5000, 5);
+    if (rec("u", up(big, sel)).v != rec("u", big).v) {
+        std::printf("FAIL %s large upload\n", what);
+        ++bad;
+    }
+    std::printf("%s uploads beside work in flight: %d failures\n", what, bad);
+    return bad;
+}
+
 int compare(const std::vector<Rec>& cpu, const std::vector<Rec>& gpu) {
     int bad = 0;
     if (cpu.size() != gpu.size()) {
@@ -372,6 +479,8 @@ int compute() {
     }
     bad += golden_chain<float>("cpu");
     bad += golden_chain<Dev>("rocm");
+    bad += io_roundtrip<Dev>("rocm");
+    bad += uploads_in_flight<Dev>("rocm");
     bad += exceptions<float>("cpu");
     bad += exceptions<Dev>("rocm");
     std::printf("%s: %zu cases, %d failures\n", bad ? "FAILED" : "PASSED", checks, bad);

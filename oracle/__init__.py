@@ -60,6 +60,7 @@ SIGNATURES = {
     "jzo_softmax_xent": (F, [P, P, P, I, I, I]),
     "jzo_layernorm_fwd": (None, [P, P, P, P, P, P, I, I]),
     "jzo_layernorm_bwd": (None, [P, P, P, P, P, I, I]),
+    "jzo_layernorm_jvp": (None, [P, P, P, P, P, I, I]),
     "jzo_layernorm_param_grads": (None, [P, P, P, P, I, I]),
     "jzo_adam_update": (None, [P, P, P, Z, F, F, F, F, I]),
     "jzo_adamw_step": (None, [P, P, P, P, Z, F, F, F, F, F, I]),
@@ -138,6 +139,7 @@ REF_SIGNATURES = {
     "jzref_adam_update": (None, [P, P, P, I, F, F, F, F, I]),
     "jzref_layernorm_fwd": (None, [P, P, P, P, P, P, I, I]),
     "jzref_layernorm_bwd": (None, [P, P, P, P, P, P, P, I, I]),
+    "jzref_layernorm_jvp": (None, [P, P, P, P, P, I, I]),
     "jzref_logistic": (F, [P, P, P, I, I]),
     "jzref_conv_eval": (None, [P, P, P, P] + [I] * 10),
     "jzref_conv_backward": (None, [P, P, P, P, P] + [I] * 10),

@@ -418,6 +418,26 @@ JZO_API void jzo_layernorm_bwd(float* dx, const float* dy, const float* gamma, c
     }
 }
 
+/* LayerNorm<D>::jvp (ml/layer.hpp:2695-2702): m1 = sum(dx,0)/dim, m2 =
+ * sum(dx .* xhat,0)/dim, out = gamma .* (inv .* (dx - m1 - xhat .* m2)). */
+JZO_API void jzo_layernorm_jvp(float* out, const float* dx, const float* gamma, const float* xhat,
+                               const float* inv_std, int dim, int N) {
+    const float invdim = 1.0f / (float)dim;
+    for (int c = 0; c < N; c++) {
+        size_t base = (size_t)c * dim;
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int i = 0; i < dim; i++) {
+            s1 += dx[base + i];
+            s2 += dx[base + i] * xhat[base + i];
+        }
+        float m1 = s1 * invdim, m2 = s2 * invdim;
+        for (int i = 0; i < dim; i++) {
+            float t = (dx[base + i] - m1) - xhat[base + i] * m2;
+            out[base + i] = gamma[i] * (inv_std[c] * t);
+        }
+    }
+}
+
 JZO_API void jzo_layernorm_param_grads(float* dgamma, float* dbeta, const float* dy,
                                        const float* xhat, int dim, int N) {
     for (int i = 0; i < dim; i++) {

@@ -189,6 +189,16 @@ API void jzref_layernorm_bwd(float* dx, float* dgamma, float* dbeta, const float
     out_logical(dbeta, sum(g, 1));
 }
 
+// LayerNorm<float>::jvp at the point x (ml/layer.hpp:2690-2702)
+API void jzref_layernorm_jvp(float* out, const float* dx, const float* x, const float* gamma,
+                             const float* beta, int dim, int N) {
+    Juzhen::LayerNorm<float> ln(dim, N);
+    ln.set_gamma(mk(gamma, dim, 1, 0));
+    ln.set_beta(mk(beta, dim, 1, 0));
+    ln.forward(mk(x, dim, N, 0));
+    out_logical(out, ln.jvp(mk(dx, dim, N, 0)));
+}
+
 // LogisticLayer value and gradient (ml/layer.hpp:232-284); targets one-hot K x N
 API float jzref_logistic(float* grad, const float* logits, const float* onehot, int K, int N) {
     Juzhen::LogisticLayer<float> L(N, mk(onehot, K, N, 0));

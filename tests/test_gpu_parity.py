@@ -644,6 +644,13 @@ def test_layernorm(gpu, oracle_lib, dim, N):
     assert np.array_equal(to_host(dfused), to_host(ddx))
     assert rel_err(to_host(dfused), dx.astype(np.float64) + res) <= TOL_RED
 
+    # tangent through the same point (LayerNorm::jvp)
+    jv = np.empty(dim * N, np.float32)
+    oracle_lib.jzo_layernorm_jvp(hptr(jv), hptr(g), hptr(gamma), hptr(xh), hptr(inv), dim, N)
+    djv = dev_empty(dim * N)
+    gpu.layernorm_jvp(dptr(djv), dp(g), dptr(dg), dp(xh), dp(inv), dim, N)
+    assert rel_err(to_host(djv), jv) <= TOL_RED
+
     rg, rb = np.empty(dim, np.float32), np.empty(dim, np.float32)
     oracle_lib.jzo_layernorm_param_grads(hptr(rg), hptr(rb), hptr(g), hptr(xh), dim, N)
     og, ob = dev_empty(dim), dev_empty(dim)

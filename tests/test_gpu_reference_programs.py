@@ -64,6 +64,20 @@ def test_mirror_transpose_and_ownership_semantics(gpu, project_dir):
     assert any(l.startswith("PASSED") for l in lines)
 
 
+def test_forward_mode_tangents(gpu, project_dir):
+    """juzhen_amd/harness/jvp_check.cu: LayerNorm, dense-stack and TransformerLayer
+    tangents on Matrix<ROCMfloat> against the CPU tangents of layers with the same
+    weights (1e-3; 1e-4 for the dense stack and LayerNorm), adjoint consistency with
+    backprop on the device (1e-4) and central differences (5e-2, the criteria of
+    tests/testJVP.cu:60-95, which itself skips on ROCm)."""
+    exe = need_ref_binary(BIN / "jvp_check_rocm")
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300, cwd=str(project_dir))
+    lines = [l for l in (r.stdout + r.stderr).splitlines() if l.startswith(("ok", "FAIL", "PASSED"))]
+    print("\n".join(lines))
+    assert r.returncode == 0, (r.stdout + r.stderr)[-3000:]
+    assert any(l.startswith("PASSED") for l in lines)
+
+
 def test_transformer_dump_against_float64_autograd(gpu, project_dir):
     """tests/testTransformerTorchDump.cu run on Matrix<ROCMfloat> writes weights,
     input, upstream gradient, forward output and input gradient of one

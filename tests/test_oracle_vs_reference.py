@@ -214,6 +214,38 @@ def test_layernorm(oracle_lib):
     assert np.allclose(dg2, dg1, rtol=1e-5, atol=1e-6) and np.allclose(db2, db1, rtol=1e-5, atol=1e-6)
 
 
+def test_layernorm_jvp(oracle_lib):
+    """LayerNorm<float>::jvp (ml/layer.hpp:2690-2702) of the compiled reference, the
+    restatement, and central differences of the reference's own forward pass along
+    the tangent (float64 differences of a float32 forward: 1e-3)."""
+    dim, N = 24, 7
+    r = R(12)
+    x = r.normal(0.4, 2, dim * N).astype(np.float32)
+    g = r.normal(1, .2, dim).astype(np.float32)
+    b = r.normal(0, .2, dim).astype(np.float32)
+    u = r.normal(size=dim * N).astype(np.float32)
+    y, h, inv = np.empty_like(x), np.empty_like(x), np.empty(N, np.float32)
+    ref.jzref_layernorm_fwd(hptr(y), hptr(h), hptr(inv), hptr(x), hptr(g), hptr(b), dim, N)
+    j1, j2 = np.empty_like(x), np.empty_like(x)
+    ref.jzref_layernorm_jvp(hptr(j1), hptr(u), hptr(x), hptr(g), hptr(b), dim, N)
+    oracle_lib.jzo_layernorm_jvp(hptr(j2), hptr(u), hptr(g), hptr(h), hptr(inv), dim, N)
+    assert np.allclose(j2, j1, rtol=1e-5, atol=1e-6)
+    # closed form in float64: d/de LN(x + e u) at e = 0
+    X, U = x.reshape(N, dim).astype(np.float64), u.reshape(N, dim).astype(np.float64)
+
+    def ln(z):
+        mu = z.mean(1, keepdims=True)
+        var = ((z - mu) ** 2).mean(1, keepdims=True)
+        return (z - mu) / np.sqrt(var + 1e-5) * g + b
+    e = 1e-6
+    fd = (ln(X + e * U) - ln(X - e * U)) / (2 * e)
+    assert np.allclose(j2.reshape(N, dim), fd, rtol=1e-4, atol=1e-5)
+    # the tangent is not the backward pass: gamma multiplies outside the projection
+    bw = np.empty_like(x)
+    oracle_lib.jzo_layernorm_bwd(hptr(bw), hptr(u), hptr(g), hptr(h), hptr(inv), dim, N)
+    assert not np.allclose(bw, j2, rtol=1e-3, atol=1e-4)
+
+
 def test_logistic(oracle_lib):
     K, N = 10, 33
     r = R(3)
