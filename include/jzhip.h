@@ -429,6 +429,23 @@ int jzhip_adamw_step(float* w, const float* g, float* m, float* v, size_t count,
                      float alpha, float beta1, float beta2, float eps,
                      float weight_decay, int iteration);
 
+/* The same step for several tensors in one launch: a layer's weights and bias
+ * (the two adam_update calls plus two in-place subtractions of Layer::update,
+ * ml/layer.hpp:108-111), or all parameter tensors of a small model, where one
+ * launch per tensor costs more than the arithmetic.  Each tensor carries its
+ * own hyper-parameters and step counter; element for element the result is
+ * that of jzhip_adamw_step. */
+typedef struct jzhip_adam_tensor {
+    float* w;
+    const float* g;
+    float* m;
+    float* v;
+    size_t count;
+    float alpha, beta1, beta2, eps, weight_decay;
+    int iteration;
+} jzhip_adam_tensor;
+int jzhip_adamw_step_multi(const jzhip_adam_tensor* tensors, int n_tensors);
+
 /* ── convolution data movement ───────────────────────────────────────── */
 
 /* Juzhen::RocmIm2col / RocmCol2im (cpp/hipbackend.hpp:99-111; oracle

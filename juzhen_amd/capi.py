@@ -20,6 +20,13 @@ D = C.c_double
 U64 = C.c_uint64
 LL = C.c_longlong
 
+class AdamTensor(C.Structure):
+    """struct jzhip_adam_tensor of include/jzhip.h"""
+    _fields_ = [("w", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("count", C.c_size_t),
+                ("alpha", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("eps", C.c_float),
+                ("weight_decay", C.c_float), ("iteration", C.c_int)]
+
+
 # name -> (restype, argtypes); mirrors include/jzhip.h one to one
 SIGNATURES: dict[str, tuple] = {
     "jzhip_runtime_available": (I, []),
@@ -113,6 +120,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_layernorm_param_grads": (I, [P, P, P, P, I, I]),
     "jzhip_adam_update": (I, [P, P, P, Z, F, F, F, F, I]),
     "jzhip_adamw_step": (I, [P, P, P, P, Z, F, F, F, F, F, I]),
+    "jzhip_adamw_step_multi": (I, [C.POINTER(AdamTensor), I]),
     "jzhip_im2col": (I, [P, P] + [I] * 12),
     "jzhip_col2im": (I, [P, P] + [I] * 12),
     "jzhip_conv_forward_reshape_bias": (I, [P, P, P, I, I, I]),

@@ -22,6 +22,9 @@
 #ifndef JZ_HIPFUSED_HPP
 #define JZ_HIPFUSED_HPP
 
+#include <initializer_list>
+#include <typeinfo>
+
 #include "jzhip.h"
 
 namespace Juzhen {
@@ -39,7 +42,121 @@ inline void must(int rc, const char* what) {
 inline Matrix<ROCMfloat> plain(const Matrix<ROCMfloat>& m) {
     return m.get_transpose() ? JzRocmFused::materialise(m) : Matrix<ROCMfloat>(m);
 }
+
+// `W -= adam_update(g, state)` for several parameter tensors in one launch
+// (ml/layer.hpp:108-111, 2683-2686, 3377-3387 issue an Adam kernel and an
+// in-place subtraction per tensor).  Element for element the arithmetic is the
+// same; tensors held as transposed views take the per-tensor path.
+struct AdamItem {
+    Matrix<ROCMfloat>* w;
+    Matrix<ROCMfloat>* g;
+    adam_state<ROCMfloat>* st;
+};
+inline void fused_update(std::initializer_list<AdamItem> items) {
+    bool all_plain = items.size() <= 16;
+    for (const AdamItem& it : items) {
+        const size_t n = it.w->num_row() * it.w->num_col();
+        all_plain = all_plain && !it.w->get_transpose() && !it.g->get_transpose() && !it.st->m.get_transpose() &&
+                    !it.st->v.get_transpose() && it.g->num_row() * it.g->num_col() == n &&
+                    it.st->m.num_row() * it.st->m.num_col() == n && it.st->v.num_row() * it.st->v.num_col() == n &&
+                    it.g->num_row() == it.w->num_row();
+    }
+    if (!all_plain) {
+        for (const AdamItem& it : items) *it.w -= adam_update(std::move(*it.g), *it.st);
+        return;
+    }
+    jzhip_adam_tensor t[16];
+    int n = 0;
+    for (const AdamItem& it : items) {
+        t[n].w = p(*it.w); t[n].g = p(*it.g); t[n].m = p(it.st->m); t[n].v = p(it.st->v);
+        t[n].count = it.w->num_row() * it.w->num_col();
+        t[n].alpha = it.st->alpha; t[n].beta1 = it.st->beta1; t[n].beta2 = it.st->beta2; t[n].eps = it.st->eps;
+        t[n].weight_decay = 0.0f;
+        t[n].iteration = it.st->iteration;
+        ++n;
+    }
+    must(jzhip_adamw_step_multi(t, n), "adamw_step_multi");
+    for (const AdamItem& it : items) it.st->iteration++;
+}
+
+// weights * input + bias * ones(1, n) (+ ReLU) in one launch: the chain every
+// dense layer's eval() and grad() issues as a product, a rank-1 product, an
+// addition and an activation (ml/layer.hpp:77-80, 118-121, 174-177, 189-195).
+// Each step rounds as the separate kernels do.
+inline Matrix<ROCMfloat> dense_affine(const Matrix<ROCMfloat>& W, const Matrix<ROCMfloat>& x,
+                                      const Matrix<ROCMfloat>& b, int act) {
+    const size_t m = W.num_row(), k = W.num_col(), n = x.num_col();
+    if (k != x.num_row() || b.num_row() != m || b.num_col() != 1)
+        throw std::invalid_argument("Matrix dimensions are not compatible");
+    Matrix<ROCMfloat> out = JzRocmFused::make("affine", m, n, 0);
+    if (m == 0 || n == 0) return out;
+    if (k == 0) {   // empty contraction: the bias alone
+        out.zeros();
+        must(jzhip_add_bias(p(out), p(b), (int)m, (int)n), "add_bias");
+        if (act == 1) must(jzhip_relu(p(out), p(out), m * n), "relu");
+        return out;
+    }
+    must(jzhip_gemm_fused(p(W), p(x), p(out), (int)m, (int)n, (int)k, (int)W.get_transpose(), (int)x.get_transpose(),
+                          (int)JzRocmFused::phys_rows(W), (int)JzRocmFused::phys_rows(x), (int)m, 1.0f, 0.0f, p(b), act,
+                          nullptr, (int)m, nullptr, (int)m),
+         "gemm_fused");
+    return out;
+}
 }  // namespace rocm_detail
+
+// ── dense layers (ml/layer.hpp:52-196) ───────────────────────────────────────
+
+template <>
+inline void Layer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+    val = tanh(rocm_detail::dense_affine(weights, input, bias, 0));
+}
+template <>
+inline Matrix<ROCMfloat> Layer<ROCMfloat>::grad(const Matrix<ROCMfloat>& input) const {
+    return d_tanh(rocm_detail::dense_affine(weights, input, bias, 0));
+}
+template <>
+inline void LinearLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+    Layer<ROCMfloat>::val = rocm_detail::dense_affine(Layer<ROCMfloat>::weights, input, Layer<ROCMfloat>::bias, 0);
+}
+template <>
+inline void ReluLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+    Layer<ROCMfloat>::val = rocm_detail::dense_affine(Layer<ROCMfloat>::weights, input, Layer<ROCMfloat>::bias, 1);
+}
+template <>
+inline Matrix<ROCMfloat> ReluLayer<ROCMfloat>::grad(const Matrix<ROCMfloat>& input) const {
+    return d_relu(rocm_detail::dense_affine(Layer<ROCMfloat>::weights, input, Layer<ROCMfloat>::bias, 0));
+}
+
+// Layer::backward (ml/layer.hpp:96-105) with the same statements in the same
+// order; what changes is how many launches they take.  The activation
+// derivative times the upstream gradient is one pass for the two layer kinds
+// whose derivative is known here (all ones for LinearLayer: the product with
+// ones is the upstream gradient itself; the ReLU mask for ReluLayer); any other
+// subclass goes through its own grad().  Weights and bias take one optimiser
+// launch together.  As in the reference, the returned input gradient is formed
+// with the weights after their update.
+template <>
+inline Matrix<ROCMfloat> Layer<ROCMfloat>::backward(const Matrix<ROCMfloat>& input, Matrix<ROCMfloat>&& upstream_grad) {
+    using namespace rocm_detail;
+    using MD = Matrix<ROCMfloat>;
+    MD t = [&]() -> MD {
+        if (typeid(*this) == typeid(LinearLayer<ROCMfloat>)) return std::move(upstream_grad);
+        if (typeid(*this) == typeid(ReluLayer<ROCMfloat>) && !upstream_grad.get_transpose()) {
+            MD pre = dense_affine(weights, input, bias, 0);
+            if (pre.num_row() != upstream_grad.num_row() || pre.num_col() != upstream_grad.num_col())
+                throw std::invalid_argument("Matrix dimensions are not compatible");
+            must(jzhip_drelu_mul(p(upstream_grad), p(pre), p(upstream_grad), pre.num_row() * pre.num_col()), "drelu_mul");
+            return std::move(upstream_grad);
+        }
+        return hadmd(grad(input), std::move(upstream_grad));
+    }();
+    MD gW = t * input.T();
+    MD gb = sum(t, 1);
+    // (Layer::update itself cannot be specialised here: the ROCm ConvLayer bodies earlier in
+    // ml/layer.hpp have already instantiated it)
+    if (need_update) fused_update({{&weights, &gW, &adamW}, {&bias, &gb, &adamb}});
+    return W().T() * t;
+}
 
 // ── LayerNorm ────────────────────────────────────────────────────────────────
 
@@ -69,8 +186,7 @@ inline Matrix<ROCMfloat> LayerNorm<ROCMfloat>::backward(Matrix<ROCMfloat>&& dy, 
     if (update) {
         Matrix<ROCMfloat> dg("ln_dgamma", dim, 1), db("ln_dbeta", dim, 1);
         must(jzhip_layernorm_param_grads(p(dg), p(db), p(dy), p(cached_xhat), dim, N), "layernorm_param_grads");
-        gamma -= adam_update(std::move(dg), adam_g);
-        beta -= adam_update(std::move(db), adam_b);
+        fused_update({{&gamma, &dg, &adam_g}, {&beta, &db, &adam_b}});
     }
     return dx;
 }
@@ -160,15 +276,9 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
     MD dx = ln1.backward(std::move(dx1), this->need_update) + dR;
 
     if (this->need_update) {
-        Wq -= adam_update(std::move(dWq), adam_Wq);
-        Wk -= adam_update(std::move(dWk), adam_Wk);
-        Wv -= adam_update(std::move(dWv), adam_Wv);
-        Wo -= adam_update(std::move(dWo), adam_Wo);
-        bo -= adam_update(std::move(dbo), adam_bo);
-        W1 -= adam_update(std::move(dW1), adam_W1);
-        b1 -= adam_update(std::move(db1), adam_b1);
-        W2 -= adam_update(std::move(dW2), adam_W2);
-        b2 -= adam_update(std::move(db2), adam_b2);
+        fused_update({{&Wq, &dWq, &adam_Wq}, {&Wk, &dWk, &adam_Wk}, {&Wv, &dWv, &adam_Wv}, {&Wo, &dWo, &adam_Wo},
+                      {&bo, &dbo, &adam_bo}, {&W1, &dW1, &adam_W1}, {&b1, &db1, &adam_b1}, {&W2, &dW2, &adam_W2},
+                      {&b2, &db2, &adam_b2}});
     }
     return dx;
 }

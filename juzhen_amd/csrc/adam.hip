@@ -127,10 +127,108 @@ int launch_adam(float* w, float* g, float* m, float* v, size_t n, const AdamCons
     return launch_rc();
 }
 
+// Several tensors in one launch (a layer's weights and bias, or every tensor
+// of a small model): a workgroup owns 1024 consecutive elements of one tensor
+// and finds its tensor by walking the table of first-block indices.
+constexpr int kMultiMax = 16;
+constexpr int kMultiPerBlock = kBlock * 4;
+struct AdamMulti {
+    float* w[kMultiMax];
+    const float* g[kMultiMax];
+    float* m[kMultiMax];
+    float* v[kMultiMax];
+    unsigned long long n[kMultiMax];
+    unsigned first_block[kMultiMax + 1];
+    AdamConst c[kMultiMax];
+    int vec[kMultiMax];
+    int count;
+};
+
+__global__ __launch_bounds__(kBlock) void adam_multi_kernel(AdamMulti p) {
+    int t = 0;
+    while (t + 1 < p.count && blockIdx.x >= p.first_block[t + 1]) ++t;
+    const AdamConst c = p.c[t];
+    float* w = p.w[t];
+    const float* g = p.g[t];
+    float* m = p.m[t];
+    float* v = p.v[t];
+    const size_t n = p.n[t];
+    const size_t base = (static_cast<size_t>(blockIdx.x - p.first_block[t]) * kBlock + threadIdx.x) * 4;
+    if (base >= n) return;
+    if (p.vec[t] && base + 3 < n) {
+        const float4 gv = *reinterpret_cast<const float4*>(g + base);
+        float4 mv = *reinterpret_cast<float4*>(m + base);
+        float4 vv = *reinterpret_cast<float4*>(v + base);
+        float4 st;
+        st.x = adam_one(gv.x, mv.x, vv.x, c);
+        st.y = adam_one(gv.y, mv.y, vv.y, c);
+        st.z = adam_one(gv.z, mv.z, vv.z, c);
+        st.w = adam_one(gv.w, mv.w, vv.w, c);
+        *reinterpret_cast<float4*>(m + base) = mv;
+        *reinterpret_cast<float4*>(v + base) = vv;
+        float4 wv = *reinterpret_cast<float4*>(w + base);
+        if (c.use_decay) {
+            wv.x *= c.decay; wv.y *= c.decay; wv.z *= c.decay; wv.w *= c.decay;
+        }
+        wv.x = 1.0f * wv.x + -1.0f * st.x;
+        wv.y = 1.0f * wv.y + -1.0f * st.y;
+        wv.z = 1.0f * wv.z + -1.0f * st.z;
+        wv.w = 1.0f * wv.w + -1.0f * st.w;
+        *reinterpret_cast<float4*>(w + base) = wv;
+        return;
+    }
+    for (size_t j = base; j < n && j < base + 4; ++j) {
+        float mi = m[j], vi = v[j];
+        const float st = adam_one(g[j], mi, vi, c);
+        m[j] = mi;
+        v[j] = vi;
+        float wj = w[j];
+        if (c.use_decay) wj *= c.decay;
+        w[j] = 1.0f * wj + -1.0f * st;
+    }
+}
+
 }  // namespace
 }  // namespace jz
 
 using namespace jz;
+
+JZ_API int jzhip_adamw_step_multi(const jzhip_adam_tensor* tensors, int n_tensors) {
+    if (n_tensors < 0 || (n_tensors > 0 && !tensors)) return -1;
+    for (int i = 0; i < n_tensors; ++i) {
+        const jzhip_adam_tensor& t = tensors[i];
+        if (t.count && (!t.w || !t.g || !t.m || !t.v)) return -1;
+        if (t.iteration < 1) return -1;
+    }
+    hipStream_t s = stream();
+    for (int at = 0; at < n_tensors;) {
+        AdamMulti p;
+        p.count = 0;
+        unsigned blocks = 0;
+        for (; at < n_tensors && p.count < kMultiMax; ++at) {
+            const jzhip_adam_tensor& t = tensors[at];
+            if (t.count == 0) continue;
+            const size_t nb = (t.count + kMultiPerBlock - 1) / kMultiPerBlock;
+            if (nb > 0x7fffffffull - blocks) {   // a tensor this large goes alone
+                if (p.count > 0) break;
+            }
+            const int k = p.count++;
+            p.w[k] = t.w; p.g[k] = t.g; p.m[k] = t.m; p.v[k] = t.v;
+            p.n[k] = t.count;
+            p.first_block[k] = blocks;
+            p.c[k] = make_const(t.alpha, t.beta1, t.beta2, t.eps, t.weight_decay, t.iteration);
+            p.vec[k] = aligned16(t.w) && aligned16(t.g) && aligned16(t.m) && aligned16(t.v);
+            if (nb > 0x7fffffffull) return -1;
+            blocks += static_cast<unsigned>(nb);
+        }
+        if (p.count == 0) continue;
+        p.first_block[p.count] = blocks;
+        adam_multi_kernel<<<blocks, kBlock, 0, s>>>(p);
+        const int rc = launch_rc();
+        if (rc) return rc;
+    }
+    return 0;
+}
 
 JZ_API int jzhip_adam_update(float* g, float* m, float* v, size_t count, float alpha, float beta1,
                              float beta2, float eps, int iteration) {

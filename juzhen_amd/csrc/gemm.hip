@@ -894,6 +894,33 @@ JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int
     if ((act == 3 || act == 4) && !aux) return -1;
     if (aux && ld_aux < m) return -1;
     if (residual && ldr < m) return -1;
+    // A product that the plain entry point serves with a special form (rank-1,
+    // matrix-vector, thin, or K split across workgroups because the output alone
+    // cannot fill the chip) keeps that form; its tail then runs as the separate
+    // kernels the fused store is defined to equal.
+    {
+        const long long cus = num_cus();
+        const long long t128 = static_cast<long long>((m + 127) / 128) * ((n + 127) / 128);
+        const bool special = k == 1 || m <= 8 || n <= 8 || (t128 * 2 <= cus && k >= 1024);
+        const bool flat = ldc == m && (!aux || ld_aux == m) && (!residual || (ldr == m && residual != C));
+        if (special && flat) {
+            const size_t total = static_cast<size_t>(m) * n;
+            int rc = jzhip_gemm(A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta);
+            if (rc) return rc;
+            if (bias && (rc = jzhip_add_bias(C, bias, m, n))) return rc;
+            if (act == 1 || act == 2) {
+                if (aux && (rc = jzhip_copy(aux, C, total))) return rc;
+                rc = act == 1 ? jzhip_relu(C, C, total) : jzhip_gelu(C, C, total);
+            } else if (act == 3) {
+                rc = jzhip_drelu_mul(C, aux, C, total);
+            } else if (act == 4) {
+                rc = jzhip_dgelu_mul(C, aux, C, total);
+            }
+            if (rc) return rc;
+            if (residual) return jzhip_axpby(C, C, residual, total, 1.0f, 1.0f);
+            return 0;
+        }
+    }
     GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
                static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
     g.ep.bias = bias;

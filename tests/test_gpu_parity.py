@@ -383,7 +383,10 @@ def test_gemm_thin_products_at_the_output_convolution_size(gpu):
     assert rel_err(to_host(g), want_g.reshape(-1)) <= TOL_GEMM
 
 
-@pytest.mark.parametrize("m,n,k", [(3, 5, 7), (64, 64, 64), (129, 127, 17), (256, 512, 128), (128, 1024, 96)])
+# (10, 128, 2560): the split-K form; (5, 300, 64): thin; (40, 50, 1): rank-1; (300, 1, 70): matrix-vector --
+# the fused entry point keeps those forms and runs the tail as separate kernels
+@pytest.mark.parametrize("m,n,k", [(3, 5, 7), (64, 64, 64), (129, 127, 17), (256, 512, 128), (128, 1024, 96),
+                                   (10, 128, 2560), (5, 300, 64), (40, 50, 1), (300, 1, 70)])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1)])
 @pytest.mark.parametrize("act", [0, 1, 2, 3, 4])
 def test_gemm_fused_epilogue(gpu, m, n, k, ta, tb, act):
@@ -704,6 +707,51 @@ def test_adamw_step(gpu, oracle_lib, wd):
     assert np.array_equal(to_host(dm), m)
     assert np.array_equal(to_host(dv), v)
     assert np.array_equal(to_host(dg), g)
+
+
+def test_adamw_step_multi_equals_single_tensor_steps(gpu):
+    """Seven tensors of awkward sizes (one unaligned, one empty, different
+    hyper-parameters and step counters) in one launch against jzhip_adamw_step per
+    tensor: parameters and both moments bit for bit, over three steps."""
+    from juzhen_amd.capi import AdamTensor
+    r = rng(31)
+    sizes = [1, 5, 1024, 4099, 0, 256 * 256, 70001]
+    hyper = [(1e-3, 0.9, 0.999, 1e-8, 0.0, 1), (3e-4, 0.8, 0.99, 1e-6, 0.01, 4), (1e-2, 0.9, 0.999, 1e-8, 0.0, 2),
+             (1e-3, 0.9, 0.999, 1e-8, 0.1, 1), (1e-3, 0.9, 0.999, 1e-8, 0.0, 1), (2e-4, 0.95, 0.999, 1e-8, 0.0, 7),
+             (1e-3, 0.9, 0.98, 1e-7, 0.02, 3)]
+    import torch
+    def fresh():
+        rr = rng(5)
+        out = []
+        for n in sizes:
+            pad = 1 if n == 4099 else 0          # a view that is not 16-byte aligned
+            w = to_dev(rr.normal(0, 1, n + pad).astype(np.float32))
+            m = to_dev(rr.normal(0, 0.1, n + pad).astype(np.float32))
+            v = to_dev(rr.uniform(0, 0.1, n + pad).astype(np.float32))
+            out.append((w, m, v, pad))
+        return out
+    A, B = fresh(), fresh()
+    for step in range(3):
+        grads = [to_dev(r.normal(0, 1, n + (1 if n == 4099 else 0)).astype(np.float32)) for n in sizes]
+        arr = (AdamTensor * len(sizes))()
+        for i, n in enumerate(sizes):
+            w, m, v, pad = A[i]
+            al, b1, b2, eps, wd, it = hyper[i]
+            o = 4 * pad
+            gpu.adamw_step(C.c_void_p(w.data_ptr() + o), C.c_void_p(grads[i].data_ptr() + o),
+                           C.c_void_p(m.data_ptr() + o), C.c_void_p(v.data_ptr() + o), n, al, b1, b2, eps, wd, it + step)
+            w2, m2, v2, _ = B[i]
+            arr[i] = AdamTensor(w2.data_ptr() + o, grads[i].data_ptr() + o, m2.data_ptr() + o, v2.data_ptr() + o, n,
+                                al, b1, b2, eps, wd, it + step)
+        gpu.adamw_step_multi(arr, len(sizes))
+        gpu.synchronize()
+        for i in range(len(sizes)):
+            for a, b in zip(A[i][:3], B[i][:3]):
+                assert torch.equal(a, b), (step, i)
+    from juzhen_amd import capi
+    lib = capi.load()
+    assert lib.jzhip_adamw_step_multi(None, 0) == 0
+    assert lib.jzhip_adamw_step_multi(None, 2) == -1
 
 
 # ── convolution data movement (bit-exact) ────────────────────────────────
