@@ -68,6 +68,12 @@ void dump(const std::string& dir, const std::string& name, const Matrix<float>& 
     std::fclose(f);
 }
 
+// Wait for everything issued so far (reading any device value does): timing marks only.
+template <class M>
+void sync_device(const std::vector<M>& kept) {
+    if (!kept.empty()) (void)item(kept.back());
+}
+
 double now_ms() {
     return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
@@ -133,18 +139,24 @@ int run_c2(const std::string& out, bool small, int steps) {
     }
     const Matrix<D> X(Xh), Y(Yh);
     Matrix<float> losses("losses", 1, steps);
+    // Losses stay on the device while the loop runs and are read after it: reading one
+    // per step (item(), ml/util.cuh:112-124) would drain the device once per step.
+    std::vector<Matrix<D>> loss_dev;
+    loss_dev.reserve(steps);
     double t0 = 0;
     for (int it = 0; it < steps; ++it) {
-        if (it == 3) t0 = now_ms();
+        if (it == 3) { sync_device(loss_dev); t0 = now_ms(); }
         forward(net, X);
         LossLayer<D> loss(nb, Y);
         loss.eval(L2.value());
-        losses.elem(0, it) = item(loss.value());
+        loss_dev.push_back(loss.value());
         net.push_front(&loss);
         backprop(net, X);
         net.pop_front();
     }
+    sync_device(loss_dev);
     if (steps > 3) std::printf("RESULT c2_ms_per_step %.4f\n", (now_ms() - t0) / (steps - 3));
+    for (int it = 0; it < steps; ++it) losses.elem(0, it) = item(loss_dev[it]);
     std::printf("RESULT c2_loss_first %.8g\nRESULT c2_loss_last %.8g\n", losses.elem(0, 0), losses.elem(0, steps - 1));
     dump(out, "c2_losses", losses);
     dump(out, "c2_W0", host(L0.W()));
@@ -176,18 +188,22 @@ int run_c3(const std::string& out, bool small, int steps) {
     }
     const Matrix<D> X(Xh), Y(Yh);
     Matrix<float> losses("losses", 1, steps);
+    std::vector<Matrix<D>> loss_dev;
+    loss_dev.reserve(steps);
     double t0 = 0;
     for (int it = 0; it < steps; ++it) {
-        if (it == 2) t0 = now_ms();
+        if (it == 2) { sync_device(loss_dev); t0 = now_ms(); }
         forward(net, X);
         LogisticLayer<D> loss(nb, Y);
         loss.eval(fc.value());
-        losses.elem(0, it) = item(loss.value());
+        loss_dev.push_back(loss.value());
         net.push_front(&loss);
         backprop(net, X);
         net.pop_front();
     }
+    sync_device(loss_dev);
     if (steps > 2) std::printf("RESULT c3_ms_per_step %.4f\n", (now_ms() - t0) / (steps - 2));
+    for (int it = 0; it < steps; ++it) losses.elem(0, it) = item(loss_dev[it]);
     std::printf("RESULT c3_loss_first %.8g\nRESULT c3_loss_last %.8g\n", losses.elem(0, 0), losses.elem(0, steps - 1));
     dump(out, "c3_losses", losses);
     dump(out, "c3_conv1_W", host(conv1.W()));
@@ -318,17 +334,21 @@ int run_c5(const std::string& out, bool small, int steps) {
     const Matrix<D> xt(xth), vt(vth);
     net.set_time(t);
     Matrix<float> losses("losses", 1, steps);
+    std::vector<Matrix<D>> loss_dev;
+    loss_dev.reserve(steps);
     double t0 = 0;
     for (int it = 0; it < steps; ++it) {
-        if (it == 1) t0 = now_ms();
+        if (it == 1) { sync_device(loss_dev); t0 = now_ms(); }
         const Matrix<D>& pred = net.fwd(xt);
         if (it == 0) dump(out, "c5_pred0", host(pred));
         Matrix<D> diff = pred - vt;
-        losses.elem(0, it) = item(sum(sum(square(Matrix<D>(diff)), 0), 1)) / (float)nb;   // demo_cnn_rectified.cu:531-534
+        loss_dev.push_back(sum(sum(square(Matrix<D>(diff)), 0), 1));   // demo_cnn_rectified.cu:531-534
         Matrix<D> grad = 2.0f * diff / (float)nb;
         net.bwd(xt, std::move(grad));
     }
+    sync_device(loss_dev);
     if (steps > 1) std::printf("RESULT c5_ms_per_step %.4f\n", (now_ms() - t0) / (steps - 1));
+    for (int it = 0; it < steps; ++it) losses.elem(0, it) = item(loss_dev[it]) / (float)nb;
     std::printf("RESULT c5_loss_first %.8g\nRESULT c5_loss_last %.8g\n", losses.elem(0, 0), losses.elem(0, steps - 1));
     dump(out, "c5_losses", losses);
     dump(out, "c5_head_W", host(net.head.W()));
