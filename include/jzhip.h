@@ -475,6 +475,39 @@ int jzhip_convtrans_gather(const float* t, float* tp, int C_out, int H_out,
 int jzhip_convtrans_reshape(const float* src, float* dst, int C, int spatial,
                             int N, int direction);
 
+/* ── convolution without the patch matrix ─────────────────────────────── */
+
+/* The three products of ConvLayer (ml/layer.hpp:1611-1719) with the patch
+ * matrix formed on the fly inside the product (implicit GEMM) instead of being
+ * written by RocmIm2col and read back.  Layouts are the layer's own: input
+ * (C_in*H_in*W_in, N), weights the stored (K, C_out) column-major matrix with
+ * K = C_in*kH*kW (ml/layer.hpp:1566-1569), out and t (C_out*H_out*W_out, N).
+ *   jzhip_conv2d_forward          replaces RocmIm2col + RocmGemm(W^T col) +
+ *                                 RocmConvForwardReshapeBias (+ relu when relu != 0;
+ *                                 bias may be NULL)                          (:1611-1637)
+ *   jzhip_conv2d_backward_weights replaces RocmConvBackwardReshape + RocmIm2col +
+ *                                 RocmGemm(col t2d^T): dW in the stored (K, C_out)
+ *                                 layout, t the upstream gradient after the
+ *                                 activation derivative                       (:1679-1696)
+ *   jzhip_conv2d_backward_data    replaces RocmGemm(W t2d) + RocmCol2im for stride 1
+ *                                 (returns -1 for other strides: those keep the
+ *                                 patch-matrix route); the taps of one input
+ *                                 pixel are summed inside the product, so the
+ *                                 result agrees with the col2im order to
+ *                                 rounding, not bit for bit                   (:1698-1709) */
+int jzhip_conv2d_forward(const float* input, const float* weights, const float* bias,
+                         float* out, int C_in, int H_in, int W_in, int C_out, int kH,
+                         int kW, int pad_h, int pad_w, int stride_h, int stride_w,
+                         int H_out, int W_out, int N, int relu);
+int jzhip_conv2d_backward_weights(const float* input, const float* t, float* dW, int C_in,
+                                  int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
+                                  int pad_w, int stride_h, int stride_w, int H_out,
+                                  int W_out, int N);
+int jzhip_conv2d_backward_data(const float* t, const float* weights, float* dx, int C_in,
+                               int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
+                               int pad_w, int stride_h, int stride_w, int H_out, int W_out,
+                               int N);
+
 #ifdef __cplusplus
 }
 #endif

@@ -143,16 +143,25 @@ def make_overlay() -> Path:
     for extra in HOST_SRC.glob("hipfused*.hpp"):
         _relink(OVERLAY / "cpp" / extra.name, extra)
     _link_tree(REFERENCE_ROOT / "ml", OVERLAY / "ml", {})
-    hooks = {"util.cuh": "hipfused_util.hpp", "layer.hpp": "hipfused.hpp"}
-    for fname, hook in hooks.items():
-        if not (HOST_SRC / hook).exists():
-            continue
+    # ml/util.cuh: upstream file followed by the one hook include.  ml/layer.hpp: the same, and
+    # the ROCm ConvLayer block of the upstream file (ml/layer.hpp:1562-1725) is replaced by
+    # cpp/hipconv.hpp -- the maintainer swaps the block for an #include; here the upstream class
+    # is compiled under another name so that the reference file itself stays untouched.
+    wrappers = {
+        "util.cuh": '#include "./upstream_util.cuh"\n#ifdef ROCM_HIP\n#include "../cpp/hipfused_util.hpp"\n#endif\n',
+        "layer.hpp": '#ifdef ROCM_HIP\n#define ConvLayer ConvLayer_patch_matrix_route\n#endif\n'
+                     '#include "./upstream_layer.hpp"\n'
+                     '#ifdef ROCM_HIP\n#undef ConvLayer\n#include "../cpp/hipfused.hpp"\n'
+                     '#include "../cpp/hipconv.hpp"\n#endif\n',
+    }
+    for extra in HOST_SRC.glob("hipconv*.hpp"):
+        _relink(OVERLAY / "cpp" / extra.name, extra)
+    for fname, text in wrappers.items():
         upstream = OVERLAY / "ml" / ("upstream_" + fname)
         _relink(upstream, REFERENCE_ROOT / "ml" / fname)
         wrapper = OVERLAY / "ml" / fname
         wrapper.unlink()
-        wrapper.write_text(f'#include "./{upstream.name}"\n'
-                           f'#ifdef ROCM_HIP\n#include "../cpp/{hook}"\n#endif\n')
+        wrapper.write_text(text)
     _link_tree(REFERENCE_ROOT / "tests", OVERLAY / "tests", {})
     _link_tree(REFERENCE_ROOT / "examples", OVERLAY / "examples", {})
     _relink(OVERLAY / "external", REFERENCE_ROOT / "external")

@@ -128,6 +128,9 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_convtrans_scatter": (I, [P, P, P] + [I] * 12),
     "jzhip_convtrans_gather": (I, [P, P] + [I] * 12),
     "jzhip_convtrans_reshape": (I, [P, P, I, I, I, I]),
+    "jzhip_conv2d_forward": (I, [P, P, P, P] + [I] * 14),
+    "jzhip_conv2d_backward_weights": (I, [P, P, P] + [I] * 13),
+    "jzhip_conv2d_backward_data": (I, [P, P, P] + [I] * 13),
 }
 
 

@@ -1,0 +1,577 @@
+// Convolution as an implicit GEMM on the fp32 matrix cores: the patch matrix
+// col(K, P*N) of the im2col formulation (ml/layer.hpp:1611-1719) is never
+// written.  Its elements are formed while an operand tile is staged into LDS,
+//     col(k, j) = input(c, oh*s - pad + ky, ow*s - pad + kx; image n)   or 0 outside,
+//     k = (c, ky, kx),  j = n*P + oh*W_out + ow,
+// so the three products of a convolution layer read the image (and the upstream
+// gradient) directly:
+//   forward        out(j, co)  = sum_k col(k, j) W(k, co) + bias(co)  [relu]
+//                  stored straight into the layer's (C_out*P, N) layout
+//   weight grads   dW(k, co)   = sum_j col(k, j) t(co, j)     (K split across workgroups)
+//   input grads    dx = the forward product of t with the flipped weights
+//                  (stride 1; strided layers keep the patch-matrix route)
+// The tile machinery (LDS layout, fragment reads, software pipeline) is the one
+// of gemm.hip; only the global -> register side of the loaders differs.
+// HBM traffic per forward call: input + output + weights instead of
+// input + 2 * patches + 2 * (C_out x P*N) + output.
+#include "common.hpp"
+#include "gemm_tile.hpp"
+
+namespace jz {
+void launch_splitk_reduce(float* C, const float* part, int M, int N, size_t ldc, int splits, float alpha,
+                          float beta);
+namespace {
+
+struct ConvGeom {
+    int C, H, W;          // image the patches are taken from
+    int kH, kW, pad_h, pad_w, sh, sw;
+    int Ho, Wo;           // patch grid
+    int N;                // images
+    int Cout;             // columns of the weight matrix
+    int K, P, HW, CHW, khw;
+    long long J;          // P * N
+    FastDiv dP, dWo, dkhw, dkW;
+};
+
+ConvGeom make_geom(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int sh, int sw, int Ho, int Wo, int N,
+                   int Cout) {
+    ConvGeom g;
+    g.C = C; g.H = H; g.W = W; g.kH = kH; g.kW = kW; g.pad_h = pad_h; g.pad_w = pad_w; g.sh = sh; g.sw = sw;
+    g.Ho = Ho; g.Wo = Wo; g.N = N; g.Cout = Cout;
+    g.khw = kH * kW;
+    g.K = C * g.khw;
+    g.P = Ho * Wo;
+    g.HW = H * W;
+    g.CHW = C * g.HW;
+    g.J = static_cast<long long>(g.P) * N;
+    g.dP = make_fastdiv(g.P);
+    g.dWo = make_fastdiv(Wo);
+    g.dkhw = make_fastdiv(g.khw);
+    g.dkW = make_fastdiv(kW);
+    return g;
+}
+
+// A patch-row index k = (c, ky, kx) as an offset into one image and its tap
+struct Tap {
+    int off;   // c*H*W + ky*W + kx
+    int ky, kx;
+};
+__device__ __forceinline__ Tap tap_of(int k, const ConvGeom& g) {
+    const int c = static_cast<int>(fdiv(static_cast<uint32_t>(k), g.dkhw));
+    const int r = k - c * g.khw;
+    const int ky = static_cast<int>(fdiv(static_cast<uint32_t>(r), g.dkW));
+    const int kx = r - ky * g.kW;
+    return Tap{c * g.HW + ky * g.W + kx, ky, kx};
+}
+__device__ __forceinline__ void tap_next(Tap& t, const ConvGeom& g) {
+    ++t.kx;
+    ++t.off;
+    if (t.kx == g.kW) {
+        t.kx = 0;
+        ++t.ky;
+        t.off += g.W - g.kW;
+        if (t.ky == g.kH) {
+            t.ky = 0;
+            t.off += g.HW - g.kH * g.W;
+        }
+    }
+}
+// A patch-column index j = (n, oh, ow): where its patch starts in the input
+struct Site {
+    long long base;   // n*C*H*W + ih0*W + iw0 (ih0, iw0 may be negative)
+    int ih0, iw0;
+    int oh, ow;
+    int n;
+};
+__device__ __forceinline__ Site site_of(long long j, const ConvGeom& g) {
+    const int n = static_cast<int>(fdiv(static_cast<uint32_t>(j), g.dP));
+    const int p = static_cast<int>(j - static_cast<long long>(n) * g.P);
+    const int oh = static_cast<int>(fdiv(static_cast<uint32_t>(p), g.dWo));
+    const int ow = p - oh * g.Wo;
+    Site s;
+    s.n = n; s.oh = oh; s.ow = ow;
+    s.ih0 = oh * g.sh - g.pad_h;
+    s.iw0 = ow * g.sw - g.pad_w;
+    s.base = static_cast<long long>(n) * g.CHW + static_cast<long long>(s.ih0) * g.W + s.iw0;
+    return s;
+}
+__device__ __forceinline__ void site_next(Site& s, const ConvGeom& g) {
+    ++s.ow;
+    s.iw0 += g.sw;
+    s.base += g.sw;
+    if (s.ow == g.Wo) {
+        s.ow = 0;
+        ++s.oh;
+        s.iw0 = -g.pad_w;
+        s.ih0 += g.sh;
+        s.base += static_cast<long long>(g.sh) * g.W - static_cast<long long>(g.Wo) * g.sw;
+        if (s.oh == g.Ho) {
+            s.oh = 0;
+            ++s.n;
+            s.ih0 = -g.pad_h;
+            s.base = static_cast<long long>(s.n) * g.CHW + static_cast<long long>(s.ih0) * g.W + s.iw0;
+        }
+    }
+}
+__device__ __forceinline__ float patch_value(const float* __restrict__ in, const Site& s, const Tap& t,
+                                             const ConvGeom& g) {
+    const bool ok = static_cast<unsigned>(s.ih0 + t.ky) < static_cast<unsigned>(g.H) &&
+                    static_cast<unsigned>(s.iw0 + t.kx) < static_cast<unsigned>(g.W);
+    return ok ? in[s.base + t.off] : 0.0f;
+}
+
+constexpr int kWGM = 2, kWGN = 2, kTM = 2;   // 128 rows per workgroup tile
+
+// ── forward: out(j, co) = sum_k col(k, j) W(k, co) ───────────────────────────
+// Rows of the tile are patch columns j (so that a register of the transposed
+// MFMA result holds 32 consecutive output pixels of one channel: the store into
+// the (C_out*P, N) layout is coalesced), columns are output channels.
+// The A loader takes one j and four consecutive k per thread and pass.
+template <int TM, int TN, bool FASTB>
+__global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __restrict__ in, const float* __restrict__ Wt,
+                                                             const float* __restrict__ bias, float* __restrict__ out,
+                                                             ConvGeom g, int relu, int tiles_n) {
+    constexpr int BM = kWGM * TM * 32;
+    constexpr int BN = kWGN * TN * 32;
+    using LA = TileLoader<BM, false, TM>;
+    using LB = TileLoader<BN, false, TN>;
+    constexpr int LDA_S = LA::LD, LDB_S = LB::LD;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA_S];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB_S];
+
+    // consecutive workgroups share a row tile (the same image patches) and differ in
+    // the channel tile; the 8 XCDs each take a contiguous run of row tiles
+    const int ntiles = gridDim.x;
+    int pid = blockIdx.x;
+    {
+        constexpr int kXcd = 8;
+        if (ntiles % kXcd == 0) pid = (pid % kXcd) * (ntiles / kXcd) + pid / kXcd;
+    }
+    const int tile_m = pid / tiles_n, tile_n = pid % tiles_n;
+    const long long m0 = static_cast<long long>(tile_m) * BM;
+    const int n0 = tile_n * BN;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int wm = wave % kWGM, wn = wave / kWGM;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // this thread's patch columns (one per pass), fixed for the whole K walk
+    Site site[LA::kPasses];
+    bool row_ok[LA::kPasses];
+    int kq;   // k offset of this thread inside a stage: 0, 4, 8 or 12
+    {
+        int x, k;
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps) {
+            LA::coords(ps, x, k);
+            const long long j = m0 + x;
+            row_ok[ps] = j < g.J;
+            site[ps] = site_of(row_ok[ps] ? j : 0, g);
+        }
+        LA::coords(0, x, kq);
+    }
+    floatx4 ra[LA::kPasses], rb[LB::kPasses];
+    unsigned offb[LB::kPasses];
+    if constexpr (FASTB) LB::offsets(offb, static_cast<unsigned>(g.K));
+    auto load_stage = [&](int k0) {
+        Tap t = tap_of(k0 + kq, g);
+        Tap taps[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            taps[e] = t;
+            tap_next(t, g);
+        }
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps) {
+            floatx4 r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                r[e] = (row_ok[ps] && k0 + kq + e < g.K) ? patch_value(in, site[ps], taps[e], g) : 0.0f;
+            ra[ps] = r;
+        }
+        if constexpr (FASTB)
+            LB::load_fast(rb, LB::origin(Wt, g.K, n0, k0), offb);
+        else
+            LB::load_checked(rb, Wt, g.K, n0, k0, g.Cout, g.K);
+    };
+
+    const int nk = (g.K + BK - 1) / BK;
+    load_stage(0);
+    LA::store(ra, As[0]);
+    LB::store(rb, Bs[0]);
+    __syncthreads();
+    if (nk > 1) load_stage(BK);
+
+    constexpr int KS = BK / 2;
+    constexpr int kStorePasses = LA::kPasses + LB::kPasses;
+    static_assert(kStorePasses <= KS - 2, "staging stores must fit the MFMA steps of a stage");
+    Frag<TM> af[2];
+    Frag<TN> bf[2];
+    const int a_off = wm * LA::kGroup + l32 * TM + h * LDA_S;
+    const int b_off = wn * LB::kGroup + l32 * TN + h * LDB_S;
+    auto read_frags = [&](int slot, const float* as, const float* bs, int kk) {
+        af[slot].read(as + 2 * kk * LDA_S);
+        bf[slot].read(bs + 2 * kk * LDB_S);
+    };
+    auto mfma_step = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
+    };
+    int cur = 0;
+    read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
+    for (int kt = 0; kt < nk; ++kt) {
+        const bool more = kt + 1 < nk;
+        const float* as = As[cur] + a_off;
+        const float* bs = Bs[cur] + b_off;
+#pragma unroll
+        for (int kk = 0; kk < KS - 1; ++kk) {
+            read_frags((kk + 1) & 1, as, bs, kk + 1);
+            if (more) {
+                if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
+                else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
+            }
+            if (kk == kStorePasses && kt + 2 < nk) load_stage((kt + 2) * BK);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step(kk & 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+        cur ^= 1;
+        if (more) read_frags(0, As[cur] + a_off, Bs[cur] + b_off, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step((KS - 1) & 1);
+    }
+
+    // store: register v of lane (h, l32) is (row l32, column 8*(v/4) + 4*h + v%4) of a 32x32 tile
+    const long long CoP = static_cast<long long>(g.Cout) * g.P;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const long long j = m0 + (wm * TM + i) * 32 + l32;
+        if (j >= g.J) continue;
+        const int n = static_cast<int>(fdiv(static_cast<uint32_t>(j), g.dP));
+        const int p = static_cast<int>(j - static_cast<long long>(n) * g.P);
+        float* dst = out + static_cast<long long>(n) * CoP + p;
+#pragma unroll
+        for (int jn = 0; jn < TN; ++jn) {
+            const int cbase = n0 + (wn * TN + jn) * 32 + 4 * h;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int co = cbase + 8 * (v / 4) + (v % 4);
+                if (co < g.Cout) {
+                    float r = acc[i][jn][v];
+                    if (bias) r += bias[co];
+                    if (relu) r = r > 0.0f ? r : 0.0f;
+                    dst[static_cast<long long>(co) * g.P] = r;
+                }
+            }
+        }
+    }
+}
+
+// ── weight gradients: dW(k, co) = sum_j col(k, j) t(co, j) ───────────────────
+// Rows of the tile are patch rows k, columns are output channels, the
+// contraction runs over patch columns j and is cut into chunks across
+// workgroups (partial results in `part`, summed afterwards in a fixed order).
+// t is the upstream gradient in the layer's own (C_out*P, N) layout.  Both
+// loaders take four consecutive j per thread: image pixels along a row for the
+// patch operand, one float4 of t for the other.
+template <int TN>
+__global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restrict__ in, const float* __restrict__ t,
+                                                            float* __restrict__ part, ConvGeom g, int tiles_n,
+                                                            long long j_chunk, int t_vec) {
+    constexpr int BM = kWGM * kTM * 32;
+    constexpr int BN = kWGN * TN * 32;
+    using LA = TileLoader<BM, false, kTM>;
+    using LB = TileLoader<BN, false, TN>;
+    constexpr int LDA_S = LA::LD, LDB_S = LB::LD;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA_S];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB_S];
+
+    // the chunk is the fastest-varying part of the dispatch order: an XCD (ids congruent
+    // mod 8) then keeps to its own chunks of the image
+    const int splits = gridDim.y;
+    const int lin = blockIdx.x + blockIdx.y * gridDim.x;
+    const int chunk = lin % splits;
+    const int pid = lin / splits;
+    const int tile_m = pid / tiles_n, tile_n = pid % tiles_n;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+    const long long j_lo = static_cast<long long>(chunk) * j_chunk;
+    const long long j_hi = (j_lo + j_chunk) < g.J ? (j_lo + j_chunk) : g.J;
+    float* C = part + static_cast<long long>(chunk) * g.K * g.Cout;
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int wm = wave % kWGM, wn = wave / kWGM;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    floatx16 acc[kTM][TN];
+#pragma unroll
+    for (int i = 0; i < kTM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // this thread's patch rows (one per pass of the A loader) and channels (B loader)
+    Tap tap[LA::kPasses];
+    bool k_ok[LA::kPasses];
+    int co_b[LB::kPasses];
+    int jq;   // j offset of this thread inside a stage: 0, 4, 8 or 12
+    {
+        int x, k;
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps) {
+            LA::coords(ps, x, k);
+            k_ok[ps] = m0 + x < g.K;
+            tap[ps] = tap_of(k_ok[ps] ? m0 + x : 0, g);
+        }
+#pragma unroll
+        for (int ps = 0; ps < LB::kPasses; ++ps) {
+            LB::coords(ps, x, k);
+            co_b[ps] = n0 + x;
+        }
+        LA::coords(0, x, jq);
+    }
+    const long long CoP = static_cast<long long>(g.Cout) * g.P;
+    floatx4 ra[LA::kPasses], rb[LB::kPasses];
+    auto load_stage = [&](long long jst) {
+        const long long j = jst + jq;
+        Site s = site_of(j < g.J ? j : 0, g);
+        Site sites[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            sites[e] = s;
+            site_next(s, g);
+        }
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps) {
+            floatx4 r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                r[e] = (k_ok[ps] && j + e < j_hi) ? patch_value(in, sites[e], tap[ps], g) : 0.0f;
+            ra[ps] = r;
+        }
+#pragma unroll
+        for (int ps = 0; ps < LB::kPasses; ++ps) {
+            if (!LB::active(ps)) continue;
+            floatx4 r = {0.f, 0.f, 0.f, 0.f};
+            if (co_b[ps] < g.Cout) {
+                if (t_vec && j + 3 < j_hi) {
+                    // P % 4 == 0 and j % 4 == 0: the four pixels are consecutive in one image
+                    const int p = sites[0].oh * g.Wo + sites[0].ow;
+                    r = *reinterpret_cast<const floatx4*>(t + sites[0].n * CoP + static_cast<long long>(co_b[ps]) * g.P + p);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (j + e < j_hi)
+                            r[e] = t[sites[e].n * CoP + static_cast<long long>(co_b[ps]) * g.P +
+                                     sites[e].oh * g.Wo + sites[e].ow];
+                }
+            }
+            rb[ps] = r;
+        }
+    };
+
+    const int nk = static_cast<int>((j_hi - j_lo + BK - 1) / BK);
+    if (nk > 0) {
+        load_stage(j_lo);
+        LA::store(ra, As[0]);
+        LB::store(rb, Bs[0]);
+        __syncthreads();
+        if (nk > 1) load_stage(j_lo + BK);
+
+        constexpr int KS = BK / 2;
+        constexpr int kStorePasses = LA::kPasses + LB::kPasses;
+        static_assert(kStorePasses <= KS - 2, "staging stores must fit the MFMA steps of a stage");
+        Frag<kTM> af[2];
+        Frag<TN> bf[2];
+        const int a_off = wm * LA::kGroup + l32 * kTM + h * LDA_S;
+        const int b_off = wn * LB::kGroup + l32 * TN + h * LDB_S;
+        auto read_frags = [&](int slot, const float* as, const float* bs, int kk) {
+            af[slot].read(as + 2 * kk * LDA_S);
+            bf[slot].read(bs + 2 * kk * LDB_S);
+        };
+        auto mfma_step = [&](int slot) {
+#pragma unroll
+            for (int i = 0; i < kTM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[slot][j], af[slot][i], acc[i][j], 0, 0, 0);
+        };
+        int cur = 0;
+        read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
+        for (int kt = 0; kt < nk; ++kt) {
+            const bool more = kt + 1 < nk;
+            const float* as = As[cur] + a_off;
+            const float* bs = Bs[cur] + b_off;
+#pragma unroll
+            for (int kk = 0; kk < KS - 1; ++kk) {
+                read_frags((kk + 1) & 1, as, bs, kk + 1);
+                if (more) {
+                    if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
+                    else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
+                }
+                if (kk == kStorePasses && kt + 2 < nk) load_stage(j_lo + static_cast<long long>(kt + 2) * BK);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_step(kk & 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            __syncthreads();
+            cur ^= 1;
+            if (more) read_frags(0, As[cur] + a_off, Bs[cur] + b_off, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step((KS - 1) & 1);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kTM; ++i) {
+        const int row = m0 + (wm * kTM + i) * 32 + l32;
+#pragma unroll
+        for (int jn = 0; jn < TN; ++jn) {
+            const int cbase = n0 + (wn * TN + jn) * 32 + 4 * h;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int col = cbase + 8 * (v / 4) + (v % 4);
+                if (row < g.K && col < g.Cout) C[static_cast<long long>(col) * g.K + row] = acc[i][jn][v];
+            }
+        }
+    }
+}
+
+// flipped weights for the input-gradient product: F(k', c) with k' = (co, ky', kx')
+// holds W((c, kH-1-ky', kW-1-kx'), co); F is (C_out*kH*kW) x C_in, column-major
+__global__ __launch_bounds__(kBlock) void conv_flip_weights_kernel(float* __restrict__ F, const float* __restrict__ Wt,
+                                                                   int C_in, int C_out, int kH, int kW) {
+    const int khw = kH * kW;
+    const int K = C_in * khw, Kp = C_out * khw;
+    const long long total = static_cast<long long>(Kp) * C_in;
+    for (long long i = static_cast<long long>(blockIdx.x) * kBlock + threadIdx.x; i < total;
+         i += static_cast<long long>(gridDim.x) * kBlock) {
+        const int c = static_cast<int>(i / Kp);
+        const int kp = static_cast<int>(i - static_cast<long long>(c) * Kp);
+        const int co = kp / khw, r = kp - co * khw;
+        const int ky = r / kW, kx = r - ky * kW;
+        F[i] = Wt[static_cast<long long>(co) * K + c * khw + (kH - 1 - ky) * kW + (kW - 1 - kx)];
+    }
+}
+
+bool dims_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int sh, int sw, int H_out,
+             int W_out, int N) {
+    if (C_in <= 0 || H_in <= 0 || W_in <= 0 || C_out <= 0 || kH <= 0 || kW <= 0 || pad_h < 0 || pad_w < 0 || sh <= 0 ||
+        sw <= 0 || H_out <= 0 || W_out <= 0 || N <= 0)
+        return false;
+    // every index product must stay inside the 32-bit arithmetic the kernels use per image
+    const long long chw = static_cast<long long>(C_in) * H_in * W_in, cop = static_cast<long long>(C_out) * H_out * W_out;
+    const long long j = static_cast<long long>(H_out) * W_out * N, k = static_cast<long long>(C_in) * kH * kW;
+    return chw < (1ll << 30) && cop < (1ll << 30) && j < (1ll << 31) && k < (1ll << 24);
+}
+
+int launch_fwd(const float* in, const float* Wt, const float* bias, float* out, const ConvGeom& g, int relu) {
+    // the largest tile that still gives every CU two workgroups; 64-row tiles for layers
+    // with few output pixels (8x8 grids), 64-channel tiles when that is not enough
+    const long long want = 2ll * num_cus();
+    auto tiles = [&](int bm, int bn) { return ((g.J + bm - 1) / bm) * ((g.Cout + bn - 1) / bn); };
+    int TM = 2, TN = g.Cout > 64 ? 2 : 1;
+    if (tiles(64 * TM, 64 * TN) < want) TM = 1;
+    if (tiles(64 * TM, 64 * TN) < want) TN = 1;
+    const int BM = 64 * TM, BN = 64 * TN;
+    const int tiles_n = (g.Cout + BN - 1) / BN;
+    const long long total = tiles(BM, BN);
+    if (total > 0x7fffffffll) return -1;
+    const bool fastb = g.K % BK == 0 && g.Cout % BN == 0 && aligned16(Wt);
+    const unsigned grid = static_cast<unsigned>(total);
+    hipStream_t s = stream();
+#define JZ_CONV_FWD(TMV, TNV)                                                                                   \
+    do {                                                                                                        \
+        if (fastb) conv_fwd_kernel<TMV, TNV, true><<<grid, kBlock, 0, s>>>(in, Wt, bias, out, g, relu, tiles_n); \
+        else conv_fwd_kernel<TMV, TNV, false><<<grid, kBlock, 0, s>>>(in, Wt, bias, out, g, relu, tiles_n);      \
+    } while (0)
+    if (TM == 2 && TN == 2) JZ_CONV_FWD(2, 2);
+    else if (TM == 2) JZ_CONV_FWD(2, 1);
+    else if (TN == 2) JZ_CONV_FWD(1, 2);
+    else JZ_CONV_FWD(1, 1);
+#undef JZ_CONV_FWD
+    return launch_rc();
+}
+
+}  // namespace
+}  // namespace jz
+
+using namespace jz;
+
+JZ_API int jzhip_conv2d_forward(const float* input, const float* weights, const float* bias, float* out, int C_in,
+                                int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int stride_h,
+                                int stride_w, int H_out, int W_out, int N, int relu) {
+    if (!input || !weights || !out) return -1;
+    if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    const ConvGeom g = make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N, C_out);
+    return launch_fwd(input, weights, bias, out, g, relu ? 1 : 0);
+}
+
+JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, float* dW, int C_in, int H_in, int W_in,
+                                         int C_out, int kH, int kW, int pad_h, int pad_w, int stride_h, int stride_w,
+                                         int H_out, int W_out, int N) {
+    if (!input || !t || !dW) return -1;
+    if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    const ConvGeom g = make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N, C_out);
+    const bool wide = C_out > 64;
+    const int BN = wide ? 128 : 64;
+    const int tiles_n = (C_out + BN - 1) / BN, tiles_m = (g.K + 127) / 128;
+    const long long tiles = static_cast<long long>(tiles_m) * tiles_n;
+    // chunks of the patch-column range: enough workgroups for two per CU, a multiple of 8
+    // so that an XCD keeps to its own chunks, at least 16 stages each
+    const long long cus = num_cus();
+    long long splits = (2 * cus + tiles - 1) / tiles;
+    splits = splits <= 2 ? splits : splits <= 4 ? 4 : (splits + 7) / 8 * 8;
+    const long long per = static_cast<long long>(g.K) * C_out;
+    while (splits > 1 && (g.J / splits < 16 * BK || per * splits > static_cast<long long>(kWorkspaceFloats)))
+        splits = splits > 8 ? splits - 8 : splits / 2;
+    if (splits < 1) splits = 1;
+    long long j_chunk = ((g.J + splits - 1) / splits + BK - 1) / BK * BK;
+    splits = (g.J + j_chunk - 1) / j_chunk;
+    if (splits > 65535 || tiles > 0x7fffffffll) return -1;
+    float* part = dW;
+    if (splits > 1) {
+        part = workspace();
+        if (!part) return -2;
+    }
+    const int t_vec = (g.P % 4 == 0) && aligned16(t);
+    dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits));
+    hipStream_t s = stream();
+    if (wide) conv_dw_kernel<2><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec);
+    else conv_dw_kernel<1><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec);
+    if (splits > 1) launch_splitk_reduce(dW, part, g.K, C_out, static_cast<size_t>(g.K), static_cast<int>(splits), 1.0f, 0.0f);
+    return launch_rc();
+}
+
+JZ_API int jzhip_conv2d_backward_data(const float* t, const float* weights, float* dx, int C_in, int H_in, int W_in,
+                                      int C_out, int kH, int kW, int pad_h, int pad_w, int stride_h, int stride_w,
+                                      int H_out, int W_out, int N) {
+    if (!t || !weights || !dx) return -1;
+    if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    if (stride_h != 1 || stride_w != 1) return -1;
+    if (pad_h > kH - 1 || pad_w > kW - 1) return -1;
+    const size_t wcount = static_cast<size_t>(C_out) * kH * kW * C_in;
+    if (wcount > kWorkspaceFloats) return -1;
+    float* flipped = workspace();
+    if (!flipped) return -2;
+    hipStream_t s = stream();
+    conv_flip_weights_kernel<<<grid_for(wcount, kBlock, 4), kBlock, 0, s>>>(flipped, weights, C_in, C_out, kH, kW);
+    // a stride-1 convolution of t (C_out channels on the H_out x W_out grid) with the
+    // flipped taps and padding k-1-pad lands on the H_in x W_in grid
+    const ConvGeom g = make_geom(C_out, H_out, W_out, kH, kW, kH - 1 - pad_h, kW - 1 - pad_w, 1, 1, H_in, W_in, N, C_in);
+    return launch_fwd(t, flipped, nullptr, dx, g, 0);
+}

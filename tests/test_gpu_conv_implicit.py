@@ -1,0 +1,182 @@
+"""Convolution products without the patch matrix (jzhip_conv2d_forward,
+_backward_weights, _backward_data) through the C ABI.
+
+Small cases are compared with the CPU oracle's restatement of the layer's own
+chain (make_im2col + gemm + reshape/bias, ml/layer.hpp:1897-1999 and the ROCm
+ConvLayer :1611-1719) within the GEMM tolerance 1e-3, and with a float64
+direct convolution (the method of tests/testConvBackendParity.cu:46-124).
+Layer-sized cases (the CNN and UNet configurations) are compared with the
+patch-matrix route on the device, jzhip_im2col + jzhip_gemm + the reshape
+kernels, which the other GPU tests pin to the oracle.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from util import dev_empty, dp, dptr, hptr, rel_err, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+TOL_GEMM = 1e-3
+
+
+def dims(H, W, kH, kW, pad, stride):
+    return (H + 2 * pad - kH) // stride + 1, (W + 2 * pad - kW) // stride + 1
+
+
+def direct_conv64(x, w, b, N, Ci, H, W, Co, kH, kW, pad, stride, relu):
+    """x: (N, Ci, H, W) float64, w stored (K, Co) column-major -> (Co, Ci, kH, kW)."""
+    Ho, Wo = dims(H, W, kH, kW, pad, stride)
+    wk = w.astype(np.float64).reshape(Co, Ci, kH, kW)
+    xp = np.zeros((N, Ci, H + 2 * pad, W + 2 * pad))
+    xp[:, :, pad:pad + H, pad:pad + W] = x
+    out = np.zeros((N, Co, Ho, Wo))
+    for ky in range(kH):
+        for kx in range(kW):
+            patch = xp[:, :, ky:ky + stride * (Ho - 1) + 1:stride, kx:kx + stride * (Wo - 1) + 1:stride]
+            out += np.einsum("nchw,oc->nohw", patch, wk[:, :, ky, kx])
+    if b is not None:
+        out += b.astype(np.float64)[None, :, None, None]
+    return np.maximum(out, 0) if relu else out
+
+
+SMALL = [
+    # N, Ci, H, W, Co, kH, kW, pad, stride
+    (2, 1, 5, 5, 3, 3, 3, 1, 1),
+    (3, 3, 8, 8, 5, 3, 3, 1, 2),
+    (2, 4, 7, 9, 70, 3, 3, 1, 1),     # channel tile with a masked edge, odd pixel count
+    (1, 2, 6, 6, 130, 3, 3, 0, 1),    # two channel tiles
+    (4, 5, 10, 10, 8, 5, 5, 2, 1),
+    (2, 11, 12, 12, 16, 3, 3, 1, 1),  # K = 99: not a multiple of the K stage
+    (5, 6, 9, 7, 4, 1, 1, 0, 1),
+    (2, 3, 9, 9, 6, 4, 4, 1, 2),
+]
+
+
+@pytest.mark.parametrize("case", SMALL)
+@pytest.mark.parametrize("relu", [0, 1])
+def test_forward_small(gpu, oracle_lib, case, relu):
+    N, Ci, H, W, Co, kH, kW, pad, stride = case
+    Ho, Wo = dims(H, W, kH, kW, pad, stride)
+    K, P = Ci * kH * kW, Ho * Wo
+    r = np.random.default_rng(sum(case))
+    x = r.normal(0, 1, N * Ci * H * W).astype(np.float32)
+    w = r.normal(0, 1 / np.sqrt(K), K * Co).astype(np.float32)
+    b = r.normal(0, 0.5, Co).astype(np.float32)
+    # oracle: the layer's own chain
+    col = np.empty(K * P * N, np.float32)
+    oracle_lib.jzo_im2col(hptr(x), hptr(col), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    y2d = np.zeros(Co * P * N, np.float32)
+    oracle_lib.jzo_gemm(1, 0, Co, P * N, K, 1.0, hptr(w), K, hptr(col), K, 0.0, hptr(y2d), Co)
+    want = np.empty(Co * P * N, np.float32)
+    oracle_lib.jzo_conv_forward_reshape_bias(hptr(y2d), hptr(want), hptr(b), Co, P, N)
+    if relu:
+        oracle_lib.jzo_relu(hptr(want), hptr(want), want.size)
+    out = to_dev(np.full(Co * P * N, np.nan, np.float32))
+    gpu.conv2d_forward(dp(x), dp(w), dp(b), dptr(out), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N, relu)
+    got = to_host(out)
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) <= TOL_GEMM
+    exact = direct_conv64(x.reshape(N, Ci, H, W), w, b, N, Ci, H, W, Co, kH, kW, pad, stride, relu)
+    assert rel_err(got, exact.reshape(-1)) <= TOL_GEMM
+    # without a bias
+    gpu.conv2d_forward(dp(x), dp(w), None, dptr(out), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N, 0)
+    exact0 = direct_conv64(x.reshape(N, Ci, H, W), w, None, N, Ci, H, W, Co, kH, kW, pad, stride, 0)
+    assert rel_err(to_host(out), exact0.reshape(-1)) <= TOL_GEMM
+
+
+@pytest.mark.parametrize("case", SMALL)
+def test_backward_small(gpu, oracle_lib, case):
+    N, Ci, H, W, Co, kH, kW, pad, stride = case
+    Ho, Wo = dims(H, W, kH, kW, pad, stride)
+    K, P = Ci * kH * kW, Ho * Wo
+    r = np.random.default_rng(sum(case) + 1)
+    x = r.normal(0, 1, N * Ci * H * W).astype(np.float32)
+    w = r.normal(0, 1 / np.sqrt(K), K * Co).astype(np.float32)
+    t = r.normal(0, 1, Co * P * N).astype(np.float32)
+    # oracle chain of ConvLayer::backward (ml/layer.hpp:1679-1709)
+    t2d = np.empty(Co * P * N, np.float32)
+    oracle_lib.jzo_conv_backward_reshape(hptr(t), hptr(t2d), Co, P, N)
+    col = np.empty(K * P * N, np.float32)
+    oracle_lib.jzo_im2col(hptr(x), hptr(col), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    dW = np.zeros(K * Co, np.float32)
+    oracle_lib.jzo_gemm(0, 1, K, Co, P * N, 1.0, hptr(col), K, hptr(t2d), Co, 0.0, hptr(dW), K)
+    got = to_dev(np.full(K * Co, np.nan, np.float32))
+    gpu.conv2d_backward_weights(dp(x), dp(t), dptr(got), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    assert rel_err(to_host(got), dW) <= TOL_GEMM
+    if stride == 1:
+        dcol = np.zeros(K * P * N, np.float32)
+        oracle_lib.jzo_gemm(0, 0, K, P * N, Co, 1.0, hptr(w), K, hptr(t2d), Co, 0.0, hptr(dcol), K)
+        dx = np.empty(Ci * H * W * N, np.float32)
+        oracle_lib.jzo_col2im(hptr(dcol), hptr(dx), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+        gdx = to_dev(np.full(Ci * H * W * N, np.nan, np.float32))
+        gpu.conv2d_backward_data(dp(t), dp(w), dptr(gdx), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+        assert rel_err(to_host(gdx), dx) <= TOL_GEMM
+    else:
+        from juzhen_amd import capi
+        lib = capi.load()
+        d = dev_empty(4)
+        assert lib.jzhip_conv2d_backward_data(dptr(d), dptr(d), dptr(d), Ci, H, W, Co, kH, kW, pad, pad, stride, stride,
+                                              Ho, Wo, N) == -1
+
+
+LAYERS = [
+    # the CNN configuration (batch 128) and the UNet configuration's 3x3 layers
+    (128, 1, 28, 28, 32, 3, 3, 1, 1), (128, 32, 28, 28, 64, 3, 3, 1, 2),
+    (128, 3, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 128, 3, 3, 1, 2),
+    (128, 128, 16, 16, 128, 3, 3, 1, 1), (128, 128, 16, 16, 256, 3, 3, 1, 2), (128, 256, 8, 8, 256, 3, 3, 1, 1),
+    (128, 256, 16, 16, 128, 3, 3, 1, 1), (128, 128, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 3, 3, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", LAYERS)
+def test_layer_sizes_against_the_patch_matrix_route(gpu, case):
+    import torch
+    N, Ci, H, W, Co, kH, kW, pad, stride = case
+    Ho, Wo = dims(H, W, kH, kW, pad, stride)
+    K, P = Ci * kH * kW, Ho * Wo
+    g = torch.Generator(device="cuda")
+    g.manual_seed(sum(case))
+    x = torch.randn(N * Ci * H * W, generator=g, device="cuda")
+    w = torch.randn(K * Co, generator=g, device="cuda") / np.sqrt(K)
+    b = torch.randn(Co, generator=g, device="cuda")
+    t = torch.randn(Co * P * N, generator=g, device="cuda")
+    col = torch.empty(K * P * N, device="cuda")
+    gpu.im2col(dptr(x), dptr(col), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    y2d = torch.empty(Co * P * N, device="cuda")
+    gpu.gemm(dptr(w), dptr(col), dptr(y2d), Co, P * N, K, 1, 0, K, K, Co, 1.0, 0.0)
+    want = torch.empty(Co * P * N, device="cuda")
+    gpu.conv_forward_reshape_bias(dptr(y2d), dptr(want), dptr(b), Co, P, N)
+    gpu.relu(dptr(want), dptr(want), Co * P * N)
+    got = torch.full((Co * P * N,), float("nan"), device="cuda")
+    gpu.conv2d_forward(dptr(x), dptr(w), dptr(b), dptr(got), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N, 1)
+    gpu.synchronize()
+    assert bool(torch.isfinite(got).all())
+    assert float((got - want).norm() / want.norm()) <= 1e-5
+    # weight gradients
+    t2d = torch.empty(Co * P * N, device="cuda")
+    gpu.conv_backward_reshape(dptr(t), dptr(t2d), Co, P, N)
+    dW = torch.empty(K * Co, device="cuda")
+    gpu.gemm(dptr(col), dptr(t2d), dptr(dW), K, Co, P * N, 0, 1, K, Co, K, 1.0, 0.0)
+    gW = torch.full((K * Co,), float("nan"), device="cuda")
+    gpu.conv2d_backward_weights(dptr(x), dptr(t), dptr(gW), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    gpu.synchronize()
+    assert float((gW - dW).norm() / dW.norm()) <= 1e-4
+    if stride == 1:
+        dcol = col                       # reuse the buffer
+        gpu.gemm(dptr(w), dptr(t2d), dptr(dcol), K, P * N, Co, 0, 0, K, Co, K, 1.0, 0.0)
+        dx = torch.empty(Ci * H * W * N, device="cuda")
+        gpu.col2im(dptr(dcol), dptr(dx), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+        gdx = torch.full((Ci * H * W * N,), float("nan"), device="cuda")
+        gpu.conv2d_backward_data(dptr(t), dptr(w), dptr(gdx), Ci, H, W, Co, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+        gpu.synchronize()
+        assert float((gdx - dx).norm() / dx.norm()) <= 1e-5
+
+
+def test_rejects_bad_arguments(gpu):
+    from juzhen_amd import capi
+    lib = capi.load()
+    d = dev_empty(64)
+    assert lib.jzhip_conv2d_forward(None, dptr(d), None, dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1, 0) == -1
+    assert lib.jzhip_conv2d_forward(dptr(d), dptr(d), None, dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 0, 1, 4, 4, 1, 0) == -1
+    assert lib.jzhip_conv2d_backward_weights(dptr(d), dptr(d), None, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
