@@ -218,7 +218,13 @@ def build_host(force: bool = False, jobs: int = 6):
     jvp_obj = hostobj / "jvp_check_rocm.o"
     if force or _stale(jvp_obj, [jvp_src, *ours, ROOT / "include" / "jzhip.h"]):
         _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(jvp_src), "-o", str(jvp_obj)], "compile jvp_check.cu")
+    # timing of the header templates elemwise<F> / reduce<F>
+    tpl_src = PKG / "harness" / "templates_bench.cu"
+    tpl_obj = hostobj / "templates_bench_rocm.o"
+    if force or _stale(tpl_obj, [tpl_src, *ours, ROOT / "include" / "jzhip.h"]):
+        _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(tpl_src), "-o", str(tpl_obj)], "compile templates_bench.cu")
     REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj),
+                                                                         ("harness/templates_bench_rocm.cu", tpl_obj),
                                                                          ("harness/jvp_check_rocm.cu", jvp_obj),
                                                                          ("harness/semantics_rocm.cu", sem_obj),
                                                                          ("harness/lm_dropin_rocm.cu", dro_obj)]

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel roofline report for the MI355X backend.
 
-    python -m juzhen_amd.opbench [--groups gemm,ew,reduce,fused,conv] [--out FILE]
+    python -m juzhen_amd.opbench [--groups gemm,ew,reduce,fused,conv,broadcast,conv_implicit] [--out FILE]
 
 Every line is one C-ABI entry point at one shape: median and p95 launch time
 over 20 samples after 3 warm-ups (the reference's convention,
@@ -264,7 +264,103 @@ def bench_conv(r):
               lambda: jz.conv_backward_reshape(P(out), P(y2d), Co, Pp, N), bytes_=8 * y2d.numel())
 
 
-GROUPS = {"gemm": bench_gemm, "ew": bench_ew, "reduce": bench_reduce, "fused": bench_fused, "conv": bench_conv}
+def bench_broadcast(r):
+    """Bandwidth-bound members of the product family (rank-1 products and bias
+    broadcasts, matrix-vector products) and the copy kernels behind slices and stacks."""
+    jz = r.jz
+    for m, n in ((256, 4096), (512, 16384), (2048, 16384), (16384, 16384)):
+        a, b, c = dev(m), dev(n), dev(m * n, 0)
+        s = f"{m}x{n}"
+        # bias * ones(1, n): the layers' broadcast idiom (ml/layer.hpp:79,120,2797)
+        r.run("broadcast", "jzhip_gemm k=1 (rank-1)", s, lambda: jz.gemm(P(a), P(b), P(c), m, n, 1, 0, 0, m, 1, m, 1.0, 0.0),
+              bytes_=4.0 * (m * n + m + n))
+        r.run("broadcast", "jzhip_add_bias", s, lambda: jz.add_bias(P(c), P(a), m, n), bytes_=8.0 * m * n + 4.0 * m)
+    for m, n in ((4096, 4096), (16384, 16384), (256, 1 << 20)):
+        A, x, y = dev(m * n), dev(max(m, n)), dev(max(m, n), 0)
+        s = f"{m}x{n}"
+        r.run("broadcast", "jzhip_gemv N", s, lambda: jz.gemv(P(A), P(x), P(y), m, n, 0, m, 1, 1, 1.0, 0.0),
+              bytes_=4.0 * (m * n + m + n))
+        r.run("broadcast", "jzhip_gemv T", s, lambda: jz.gemv(P(A), P(x), P(y), m, n, 1, m, 1, 1, 1.0, 0.0),
+              bytes_=4.0 * (m * n + m + n))
+    # slices and stacks: UNet skip concat / split (131072 + 65536 rows x 128 columns) and an attention-sized block
+    for rows, cols in ((131072, 128), (8192, 8192)):
+        src, dst = dev(rows * cols), dev(2 * rows * cols, 0)
+        s = f"{rows}x{cols}"
+        half = rows // 2
+        r.run("broadcast", "jzhip_slice_extract (rows)", s,
+              lambda: jz.slice_extract(P(dst), half, P(src), rows, 0, rows // 4, 0, half, cols), bytes_=8.0 * half * cols)
+        r.run("broadcast", "jzhip_slice_extract (transposed source)", s,
+              lambda: jz.slice_extract(P(dst), cols, P(src), rows, 1, 0, rows // 4, cols, half), bytes_=8.0 * half * cols)
+        r.run("broadcast", "jzhip_slice_assign", s,
+              lambda: jz.slice_assign(P(dst), rows, 0, rows // 4, 0, P(src), half, 0, half, cols), bytes_=8.0 * half * cols)
+        r.run("broadcast", "jzhip_stack_copy_rows (vstack)", s,
+              lambda: jz.stack_copy_rows(P(dst), 2 * rows, rows, P(src), rows, cols, 0), bytes_=8.0 * rows * cols)
+        r.run("broadcast", "jzhip_stack_copy_cols (hstack)", s,
+              lambda: jz.stack_copy_cols(P(dst), rows, cols, P(src), rows, cols, 0), bytes_=8.0 * rows * cols)
+    a = dev(512 * 16384)
+    o = dev(512, 0)
+    r.run("broadcast", "jzhip_sum_rows_noalloc", "512x16384", lambda: jz.sum_rows_noalloc(P(o), P(a), 512, 16384, 512),
+          bytes_=4.0 * (512 * 16384 + 512))
+    x, xh, inv, g, out = dev(512 * 16384), dev(512 * 16384), dev(16384, 1), dev(512, 1), dev(512 * 16384, 0)
+    r.run("broadcast", "jzhip_layernorm_jvp", "512x16384", lambda: jz.layernorm_jvp(P(out), P(x), P(g), P(xh), P(inv), 512, 16384),
+          bytes_=4.0 * (3 * 512 * 16384 + 16384 + 512))
+    from juzhen_amd.capi import AdamTensor
+    sizes = [512 * 512] * 4 + [2048 * 512] * 2 + [512, 2048, 512]      # one transformer block
+    bufs = [(dev(n), dev(n), dev(n, 0), dev(n, 0)) for n in sizes]
+    arr = (AdamTensor * len(sizes))()
+    for i, (n, (w, gr, m, v)) in enumerate(zip(sizes, bufs)):
+        arr[i] = AdamTensor(w.data_ptr(), gr.data_ptr(), m.data_ptr(), v.data_ptr(), n, 1e-3, 0.9, 0.999, 1e-8, 0.0, 3)
+    r.run("broadcast", "jzhip_adamw_step_multi", "9 tensors of one transformer block (3.15 M parameters)",
+          lambda: jz.adamw_step_multi(arr, len(sizes)), bytes_=28.0 * sum(sizes))
+
+
+def bench_conv_implicit(r):
+    """The three products of a convolution layer without the patch matrix against the
+    patch-matrix route (im2col, product, reshape / col2im), per layer of the CNN and UNet
+    configurations.  flops = 2*K*C_out*P*N for each product."""
+    jz = r.jz
+    layers = (("C3 conv1", 128, 1, 28, 32, 1), ("C3 conv2", 128, 32, 28, 64, 2), ("C5 in", 128, 3, 32, 64, 1),
+              ("C5 e1b", 128, 64, 32, 64, 1), ("C5 e2a", 128, 64, 32, 128, 2), ("C5 e2b", 128, 128, 16, 128, 1),
+              ("C5 mid", 128, 256, 8, 256, 1), ("C5 d2a", 128, 256, 16, 128, 1), ("C5 d1a", 128, 128, 32, 64, 1))
+    for label, N, Ci, H, Co, s in layers:
+        k, pad = 3, 1
+        Ho = (H + 2 * pad - k) // s + 1
+        K, Pp = Ci * k * k, Ho * Ho
+        x, w, b, t = dev(N * Ci * H * H), dev(K * Co), dev(Co), dev(Co * Pp * N)
+        col, y2d, out, dW, dx = dev(K * Pp * N, 0), dev(Co * Pp * N, 0), dev(Co * Pp * N, 0), dev(K * Co, 0), dev(N * Ci * H * H, 0)
+        dims = (Ci, H, H, Co, k, k, pad, pad, s, s, Ho, Ho, N)
+        cargs = (Ci, H, H, k, k, pad, pad, s, s, Ho, Ho, N)
+        fl = 2.0 * K * Co * Pp * N
+        shape = f"{label} N{N} {Ci}>{Co} {H}x{H} s{s}"
+
+        def fwd_patch():
+            jz.im2col(P(x), P(col), *cargs)
+            jz.gemm(P(w), P(col), P(y2d), Co, Pp * N, K, 1, 0, K, K, Co, 1.0, 0.0)
+            jz.conv_forward_reshape_bias(P(y2d), P(out), P(b), Co, Pp, N)
+            jz.relu(P(out), P(out), Co * Pp * N)
+
+        def dw_patch():
+            jz.conv_backward_reshape(P(t), P(y2d), Co, Pp, N)
+            jz.im2col(P(x), P(col), *cargs)
+            jz.gemm(P(col), P(y2d), P(dW), K, Co, Pp * N, 0, 1, K, Co, K, 1.0, 0.0)
+
+        def dx_patch():
+            jz.gemm(P(w), P(y2d), P(col), K, Pp * N, Co, 0, 0, K, Co, K, 1.0, 0.0)
+            jz.col2im(P(col), P(dx), *cargs)
+
+        r.run("conv", "forward, patch-matrix route (4 launches)", shape, fwd_patch, flops=fl)
+        r.run("conv", "jzhip_conv2d_forward", shape, lambda: jz.conv2d_forward(P(x), P(w), P(b), P(out), *dims, 1), flops=fl)
+        r.run("conv", "weight gradients, patch-matrix route (3 launches)", shape, dw_patch, flops=fl)
+        r.run("conv", "jzhip_conv2d_backward_weights", shape, lambda: jz.conv2d_backward_weights(P(x), P(t), P(dW), *dims), flops=fl)
+        r.run("conv", "input gradients, patch-matrix route (2 launches)", shape, dx_patch, flops=fl)
+        if s == 1:
+            r.run("conv", "jzhip_conv2d_backward_data", shape, lambda: jz.conv2d_backward_data(P(t), P(w), P(dx), *dims), flops=fl)
+        del x, w, b, t, col, y2d, out, dW, dx
+        torch.cuda.empty_cache()
+
+
+GROUPS = {"gemm": bench_gemm, "ew": bench_ew, "reduce": bench_reduce, "fused": bench_fused, "conv": bench_conv,
+          "broadcast": bench_broadcast, "conv_implicit": bench_conv_implicit}
 
 
 def main():
