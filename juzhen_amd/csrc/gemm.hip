@@ -358,6 +358,37 @@ __global__ __launch_bounds__(kBlock) void rank1_kernel(float* C, const float* a,
         *dst = r;
     }
 }
+// The same with contiguous a, M % 4 == 0 and 16-byte aligned C columns: a wavefront
+// writes 1 KB runs of a column (one float4 per lane), a workgroup sixteen columns,
+// four per wave, the grid covering C once.
+constexpr int kRank1Cols = 16;
+template <bool BETA>
+__global__ __launch_bounds__(kBlock) void rank1_vec_kernel(float* C, const float* __restrict__ a,
+                                                           const float* __restrict__ b, size_t sb, int rows4,
+                                                           int N, size_t ldc, float alpha, float beta) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int r4 = blockIdx.x * kWave + lane;
+    if (r4 >= rows4) return;
+    float4 av = reinterpret_cast<const float4*>(a)[r4];
+    // alpha*a_i first, then times b_j: the rounding order of the scalar kernel
+    av.x *= alpha; av.y *= alpha; av.z *= alpha; av.w *= alpha;
+    for (int j0 = blockIdx.y * kRank1Cols; j0 < N; j0 += gridDim.y * kRank1Cols) {
+#pragma unroll
+        for (int u = 0; u < kRank1Cols / 4; ++u) {
+            const int j = j0 + u * 4 + wave;
+            if (j < N) {
+                const float bj = b[j * sb];
+                float4* dst = reinterpret_cast<float4*>(C + static_cast<size_t>(j) * ldc) + r4;
+                float4 r = make_float4(av.x * bj, av.y * bj, av.z * bj, av.w * bj);
+                if constexpr (BETA) {
+                    const float4 c = *dst;
+                    r.x += beta * c.x; r.y += beta * c.y; r.z += beta * c.z; r.w += beta * c.w;
+                }
+                *dst = r;
+            }
+        }
+    }
+}
 
 // y(rows x cols) += b[i]
 __global__ __launch_bounds__(kBlock) void add_bias_kernel(float* y, const float* b, int rows,
@@ -705,6 +736,16 @@ JZ_API int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, in
         // rank-1 update: the layers' broadcast idiom (bias * ones(1,N))
         const size_t sa = trans_a ? lda : 1;   // op(A)(i,0)
         const size_t sb = trans_b ? 1 : ldb;   // op(B)(0,j)
+        if (sa == 1 && m % 4 == 0 && ldc % 4 == 0 && aligned16(A) && aligned16(C)) {
+            const int rows4 = m / 4;
+            const int col_groups = (n + kRank1Cols - 1) / kRank1Cols;
+            const dim3 grid((rows4 + kWave - 1) / kWave, col_groups < 65535 ? col_groups : 65535);
+            if (beta != 0.0f)
+                rank1_vec_kernel<true><<<grid, kBlock, 0, s>>>(C, A, B, sb, rows4, n, ldc, alpha, beta);
+            else
+                rank1_vec_kernel<false><<<grid, kBlock, 0, s>>>(C, A, B, sb, rows4, n, ldc, alpha, beta);
+            return launch_rc();
+        }
         int gy = n < 1024 ? n : 1024;
         rank1_kernel<<<dim3((m + kBlock - 1) / kBlock, gy), kBlock, 0, s>>>(C, A, sa, B, sb, m, n, ldc,
                                                                             alpha, beta);

@@ -105,7 +105,8 @@ constexpr int kThinMax = 8;
 // rows of X a wavefront walks together in the dot form: two with up to four thin
 // vectors (measured 55 against 58 us at 3 x 131072 x 576), four with more, where
 // each LDS read of V should serve more rows
-template <int TT> constexpr int kThinRows = TT <= 4 ? 2 : 4;
+template <int TT> constexpr int kThinRows = TT == 1 ? 4 : (TT <= 4 ? 2 : 4);
+constexpr int thin_tt(int T) { return T == 1 ? 1 : (T <= 4 ? 4 : 8); }   // template width serving T vectors
 constexpr int kThinChunkMax = 1024;   // k per workgroup in the other form
 
 // Sums NV (a power of two, at most 64) values per lane over the 64 lanes.  On
@@ -268,8 +269,9 @@ __global__ __launch_bounds__(kBlock) void thin_axpy_partial_kernel(const float* 
 
 }  // namespace
 
-int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda,
-              size_t incx, size_t incy, float alpha, float beta) {
+namespace {
+int gemv_plain(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda,
+               size_t incx, size_t incy, float alpha, float beta) {
     hipStream_t s = stream();
     if (trans) {
         gemv_t_kernel<<<grid_cover(n, kBlock / kWave), kBlock, 0, s>>>(A, x, y, m, n, lda, incx, incy,
@@ -292,6 +294,7 @@ int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans
                                                                                 alpha, beta);
     return launch_rc();
 }
+}  // namespace
 
 namespace {
 
@@ -337,7 +340,7 @@ bool thin_ok(const ThinArgs& a) {
     if (a.T > kThinMax || !aligned16(a.X)) return false;
     if (a.xs_k == 1)
         return a.L >= 256 && a.K % 4 == 0 && a.xs_l % 4 == 0 && a.K >= 64 &&
-               static_cast<size_t>(a.T <= 4 ? 4 : kThinMax) * a.K * sizeof(float) <= 48 * 1024;
+               static_cast<size_t>(thin_tt(a.T)) * a.K * sizeof(float) <= 64 * 1024;
     if (a.L < 64) return false;
     // partial sums of every chunk must fit the workspace even at the longest chunk
     const size_t min_chunks = (static_cast<size_t>(a.K) + kThinChunkMax - 1) / kThinChunkMax;
@@ -348,9 +351,89 @@ bool thin_ok(const ThinArgs& a) {
            static_cast<size_t>(a.T) * a.L * (chunks + 1) <= kWorkspaceFloats;
 }
 
-int thin_impl(const ThinArgs& a) { return a.T <= 4 ? thin_launch<4>(a) : thin_launch<kThinMax>(a); }
+int thin_impl(const ThinArgs& a) {
+    if (a.T == 1) return thin_launch<1>(a);
+    return a.T <= 4 ? thin_launch<4>(a) : thin_launch<kThinMax>(a);
+}
 
 }  // namespace
+
+namespace {
+// y[j] = alpha*<A[:,j], x> + beta*y[j] for long columns (m >= 1024, m % 4 == 0, lda % 4 == 0,
+// aligned A and x, incx == 1): a workgroup takes four columns, its four waves a quarter
+// of the rows each, eight float4 loads of A in flight per lane; x comes through the caches.
+constexpr int kGemvTCols = 4;
+__global__ __launch_bounds__(kBlock) void gemv_t_split_kernel(const float* __restrict__ A,
+                                                              const float* __restrict__ x, float* y, int m,
+                                                              int n, size_t lda, size_t incy, float alpha,
+                                                              float beta) {
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][kGemvTCols];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const size_t j0 = static_cast<size_t>(blockIdx.x) * kGemvTCols;
+    const float4* col[kGemvTCols];
+#pragma unroll
+    for (int c = 0; c < kGemvTCols; ++c) {
+        const size_t j = j0 + c < static_cast<size_t>(n) ? j0 + c : n - 1;   // clamped, dropped at the store
+        col[c] = reinterpret_cast<const float4*>(A + j * lda);
+    }
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const int m4 = m / 4;
+    float acc[kGemvTCols] = {0.f, 0.f, 0.f, 0.f};
+    int i = wave * kWave + lane;
+    for (; i + kBlock < m4; i += 2 * kBlock) {
+        float4 a[2][kGemvTCols];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int c = 0; c < kGemvTCols; ++c) a[u][c] = col[c][i + u * kBlock];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const float4 xv = x4[i + u * kBlock];
+#pragma unroll
+            for (int c = 0; c < kGemvTCols; ++c)
+                acc[c] += a[u][c].x * xv.x + a[u][c].y * xv.y + a[u][c].z * xv.z + a[u][c].w * xv.w;
+        }
+    }
+    for (; i < m4; i += kBlock) {
+        const float4 xv = x4[i];
+#pragma unroll
+        for (int c = 0; c < kGemvTCols; ++c) {
+            const float4 av = col[c][i];
+            acc[c] += av.x * xv.x + av.y * xv.y + av.z * xv.z + av.w * xv.w;
+        }
+    }
+    const int idx = wave_sum_many<kGemvTCols>(acc, lane);
+    if (idx >= 0) red[wave][idx] = acc[0];
+    __syncthreads();
+    if (threadIdx.x < kGemvTCols && j0 + threadIdx.x < static_cast<size_t>(n)) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += red[w][threadIdx.x];
+        float* dst = y + (j0 + threadIdx.x) * incy;
+        float r = alpha * sum;
+        if (beta != 0.0f) r += beta * *dst;
+        *dst = r;
+    }
+}
+}  // namespace
+
+// y = alpha*op(A)*x + beta*y, A the physical m x n matrix.  A matrix-vector product is the
+// thin product with one vector: those kernels keep several float4 loads of A in flight per
+// lane, which the plain kernels do not; the plain ones take what the thin forms exclude
+// (unaligned or short operands).
+int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans, size_t lda,
+              size_t incx, size_t incy, float alpha, float beta) {
+    const ThinArgs t = trans ? ThinArgs{A, lda, 1, x, 0, incx, y, incy, 0, n, m, 1, alpha, beta}
+                             : ThinArgs{A, 1, lda, x, 0, incx, y, incy, 0, m, n, 1, alpha, beta};
+    if (trans && incx == 1 && m >= 1024 && m % 4 == 0 && lda % 4 == 0 && aligned16(A) && aligned16(x)) {
+        const unsigned grid = static_cast<unsigned>((static_cast<size_t>(n) + kGemvTCols - 1) / kGemvTCols);
+        gemv_t_split_kernel<<<grid, kBlock, 0, stream()>>>(A, x, y, m, n, lda, incy, alpha, beta);
+        return launch_rc();
+    }
+    if (thin_ok(t)) return thin_impl(t);
+    return gemv_plain(A, x, y, m, n, trans, lda, incx, incy, alpha, beta);
+}
 
 // C = alpha*op(A)*op(B) + beta*C through the thin forms when they apply;
 // *taken says whether they did.
