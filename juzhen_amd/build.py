@@ -144,14 +144,17 @@ def make_overlay() -> Path:
         _relink(OVERLAY / "cpp" / extra.name, extra)
     _link_tree(REFERENCE_ROOT / "ml", OVERLAY / "ml", {})
     # ml/util.cuh: upstream file followed by the one hook include.  ml/layer.hpp: the same, and
-    # the ROCm ConvLayer block of the upstream file (ml/layer.hpp:1562-1725) is replaced by
+    # the ROCm ConvLayer and convtransLayer blocks of the upstream file (ml/layer.hpp:1562-1872) are replaced by
     # cpp/hipconv.hpp -- the maintainer swaps the block for an #include; here the upstream class
     # is compiled under another name so that the reference file itself stays untouched.
     wrappers = {
         "util.cuh": '#include "./upstream_util.cuh"\n#ifdef ROCM_HIP\n#include "../cpp/hipfused_util.hpp"\n#endif\n',
-        "layer.hpp": '#ifdef ROCM_HIP\n#define ConvLayer ConvLayer_patch_matrix_route\n#endif\n'
+        "layer.hpp": '#ifdef ROCM_HIP\n#define ConvLayer ConvLayer_patch_matrix_route\n'
+                     '#define convtransLayer convtransLayer_patch_matrix_route\n'
+                     '#define ConvTransLayer ConvTransLayer_patch_matrix_route\n#endif\n'
                      '#include "./upstream_layer.hpp"\n'
-                     '#ifdef ROCM_HIP\n#undef ConvLayer\n#include "../cpp/hipfused.hpp"\n'
+                     '#ifdef ROCM_HIP\n#undef ConvLayer\n#undef convtransLayer\n#undef ConvTransLayer\n'
+                     '#include "../cpp/hipfused.hpp"\n'
                      '#include "../cpp/hipconv.hpp"\n#endif\n',
     }
     for extra in HOST_SRC.glob("hipconv*.hpp"):

@@ -15,7 +15,7 @@
 //   * the patch-matrix route of the reference (im2col, product, reshape or
 //     col2im) for layers with few output pixels per image or very few
 //     channels, where the implicit form cannot fill the matrix cores.
-// Integration: replace the ROCm ConvLayer block of ml/layer.hpp by
+// Integration: replace the ROCm ConvLayer and convtransLayer blocks of ml/layer.hpp by
 // `#include "../cpp/hipconv.hpp"`; nothing else in the file refers to it.
 #ifndef JZ_HIPCONV_HPP
 #define JZ_HIPCONV_HPP
@@ -159,10 +159,118 @@ class ConvLayer : public Layer<ROCMfloat> {
             must(jzhip_sum_rows(ptr(db), ptr(per_image), C_out, batchN, C_out), "sum_rows");
         }
 
-        if (this->need_update) this->update(std::move(dW), std::move(db));
+        // weights and bias in one optimiser launch (Layer::update, ml/layer.hpp:108-112, is two
+        // adam_update chains and two subtractions)
+        if (this->need_update)
+            rocm_detail::fused_update({{&this->weights, &dW, &this->adamW}, {&this->bias, &db, &this->adamb}});
         return dx;
     }
 };
+
+// Transposed convolution for the ROCm backend: drop-in for convtransLayer of the
+// `#if defined(ROCM_HIP)` block of ml/layer.hpp (:1728-1870); same constructor, members,
+// layouts (weights the (C_out*kH*kW, C_in) column-major matrix stored as a column) and
+// order of operations.  eval() and jvp() keep the reference's route (pack, product,
+// scatter).  backward() differs: the reference gathers the upstream gradient into
+// tp(C_out*kH*kW, P_in*N), which is the patch matrix of a convolution over t seen as a
+// (C_out, H_out, W_out) image on the H_in x W_in patch grid, so
+//   dx = W^T tp       is jzhip_conv2d_forward of t with the stored weights, landing in
+//                     the layer's (C_in*P_in, N) layout without the unpack step, and
+//   dW = tp x2d^T     is jzhip_conv2d_backward_weights with the layer input as the
+//                     "upstream" operand;
+// the gathered matrix is never written.
+class convtransLayer : public Layer<ROCMfloat> {
+    using D = ROCMfloat;
+
+    int C_in, H_in, W_in;
+    int C_out, kH, kW;
+    int pad_h, pad_w, stride_h, stride_w;
+    int H_out, W_out;
+    int batchN;
+    bool use_relu = true;
+
+    static float* ptr(const Matrix<D>& m) { return JzRocmFused::ptr(m); }
+    static void must(int rc, const char* what) { rocm_detail::must(rc, what); }
+
+    // out(C_out*H_out*W_out, N) = scatter(W x2d) + bias
+    void deconv_into(Matrix<D>& out, const Matrix<D>& x, const Matrix<D>& b) const {
+        const int P_in = H_in * W_in, rows = C_out * kH * kW;
+        Matrix<D> x2d("deconv_x2d", C_in, (size_t)P_in * batchN);
+        must(jzhip_convtrans_reshape(ptr(x), ptr(x2d), C_in, P_in, batchN, 0), "convtrans reshape");
+        Matrix<D> patches("deconv_patches", rows, (size_t)P_in * batchN);
+        must(jzhip_gemm(ptr(this->weights), ptr(x2d), ptr(patches), rows, P_in * batchN, C_in, 0, 0, rows, C_in, rows,
+                        1.0f, 0.0f),
+             "gemm");
+        must(jzhip_convtrans_scatter(ptr(patches), ptr(out), ptr(b), C_out, H_out, W_out, H_in, W_in, kH, kW, pad_h, pad_w,
+                                     stride_h, stride_w, batchN),
+             "convtrans scatter");
+    }
+
+   public:
+    convtransLayer(int N, int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad = 0, int stride = 1,
+                   bool relu = true)
+        : Layer<D>(C_out * ((H_in - 1) * stride - 2 * pad + kH) * ((W_in - 1) * stride - 2 * pad + kW), 1, N),
+          C_in(C_in), H_in(H_in), W_in(W_in), C_out(C_out), kH(kH), kW(kW), pad_h(pad), pad_w(pad), stride_h(stride),
+          stride_w(stride), H_out((H_in - 1) * stride - 2 * pad + kH), W_out((W_in - 1) * stride - 2 * pad + kW),
+          batchN(N), use_relu(relu) {
+        if (H_out <= 0 || W_out <= 0) {
+            LOG_ERROR("Invalid transposed-conv output shape: H_out={}, W_out={}", H_out, W_out);
+            ERROR_OUT;
+        }
+        const size_t wcount = (size_t)C_in * C_out * kH * kW;
+        this->weights = Matrix<D>::randn(wcount, 1) * 0.001f;
+        this->bias = Matrix<D>::zeros(C_out, 1);
+        this->val = Matrix<D>("convtrans_out", (size_t)C_out * H_out * W_out, N);
+        this->adamW = adam_state<D>(0.0001, wcount, 1);
+        this->adamb = adam_state<D>(0.0001, C_out, 1);
+    }
+
+    void eval(const Matrix<D>& input) override {
+        deconv_into(this->val, input, this->bias);
+        if (use_relu)
+            must(jzhip_relu(ptr(this->val), ptr(this->val), (size_t)C_out * H_out * W_out * batchN), "relu");
+    }
+
+    Matrix<D> jvp(const Matrix<D>&, const Matrix<D>& tangent) override {
+        const size_t count = (size_t)C_out * H_out * W_out * batchN;
+        Matrix<D> out("convtrans_jvp", (size_t)C_out * H_out * W_out, batchN);
+        deconv_into(out, tangent, Matrix<D>::zeros(C_out, 1));
+        if (use_relu) must(jzhip_drelu_mul(ptr(out), ptr(this->val), ptr(out), count), "drelu_mul");
+        return out;
+    }
+
+    Matrix<D> grad(const Matrix<D>&) const override { return Matrix<D>::ones(1, 1); }
+
+    Matrix<D> backward(const Matrix<D>& input, Matrix<D>&& upstream_grad) override {
+        const int P_in = H_in * W_in, P_out = H_out * W_out, rows = C_out * kH * kW;
+        Matrix<D> t = std::move(upstream_grad);
+        if (use_relu)
+            must(jzhip_drelu_mul(ptr(t), ptr(this->val), ptr(t), (size_t)C_out * P_out * batchN), "drelu_mul");
+
+        // weight gradients in the stored (rows, C_in) layout
+        Matrix<D> dW("deconv_dW", (size_t)rows * C_in, 1);
+        must(jzhip_conv2d_backward_weights(ptr(t), ptr(input), ptr(dW), C_out, H_out, W_out, C_in, kH, kW, pad_h, pad_w,
+                                           stride_h, stride_w, H_in, W_in, batchN),
+             "conv2d_backward_weights");
+        // input gradients with the weights as they were in the forward pass
+        Matrix<D> dx("deconv_dx", (size_t)C_in * P_in, batchN);
+        must(jzhip_conv2d_forward(ptr(t), ptr(this->weights), nullptr, ptr(dx), C_out, H_out, W_out, C_in, kH, kW, pad_h,
+                                  pad_w, stride_h, stride_w, H_in, W_in, batchN, 0),
+             "conv2d_forward");
+        // bias gradients: t read as a (P_out, C_out*N) matrix, column sums, then the N images
+        Matrix<D> db("deconv_db", C_out, 1);
+        {
+            Matrix<D> per_image("deconv_db_n", C_out, batchN);
+            must(jzhip_sum_cols(ptr(per_image), ptr(t), P_out, C_out * batchN, P_out), "sum_cols");
+            must(jzhip_sum_rows(ptr(db), ptr(per_image), C_out, batchN, C_out), "sum_rows");
+        }
+        if (this->need_update)
+            rocm_detail::fused_update({{&this->weights, &dW, &this->adamW}, {&this->bias, &db, &this->adamb}});
+        return dx;
+    }
+};
+
+using ConvTransLayer = convtransLayer;
 
 }  // namespace Juzhen
 

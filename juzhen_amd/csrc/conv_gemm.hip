@@ -120,6 +120,19 @@ __device__ __forceinline__ float patch_value(const float* __restrict__ in, const
     return ok ? in[s.base + t.off] : 0.0f;
 }
 
+// Bounds-checked loads through a raw buffer resource over the whole input (at most 2 GiB):
+// an element that falls in the padding gets the offset kOutside, which the hardware range
+// check answers with 0, so a padded element costs a select on the offset instead of a
+// branch around the load.
+constexpr unsigned kOutside = 0x80000000u;
+constexpr long long kBufferMaxBytes = 1ll << 31;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t input_resource(const float* in, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(in), 0, static_cast<int>(bytes), 0x00020000);
+}
+__device__ __forceinline__ float load_or_zero(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+
 constexpr int kWGM = 2, kWGN = 2, kTM = 2;   // 128 rows per workgroup tile
 
 // ── forward: out(j, co) = sum_k col(k, j) W(k, co) ───────────────────────────
@@ -127,10 +140,15 @@ constexpr int kWGM = 2, kWGN = 2, kTM = 2;   // 128 rows per workgroup tile
 // MFMA result holds 32 consecutive output pixels of one channel: the store into
 // the (C_out*P, N) layout is coalesced), columns are output channels.
 // The A loader takes one j and four consecutive k per thread and pass.
-template <int TM, int TN, bool FASTB>
+// TAB (kH*kW <= 32 and a table of K entries that fits LDS): the patch-row index k is
+// decoded once per workgroup into a table {offset inside an image, one-hot tap bit}, and
+// each of a thread's pixels carries a 32-bit mask of the taps that fall inside the image,
+// so an element costs a table read, an AND and an address add instead of two divisions
+// and four comparisons.
+template <int TM, int TN, bool FASTB, bool TAB>
 __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __restrict__ in, const float* __restrict__ Wt,
                                                              const float* __restrict__ bias, float* __restrict__ out,
-                                                             ConvGeom g, int relu, int tiles_n) {
+                                                             ConvGeom g, int relu, int tiles_n, unsigned in_bytes) {
     constexpr int BM = kWGM * TM * 32;
     constexpr int BN = kWGN * TN * 32;
     using LA = TileLoader<BM, false, TM>;
@@ -138,6 +156,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
     constexpr int LDA_S = LA::LD, LDB_S = LB::LD;
     __shared__ __attribute__((aligned(16))) float As[2][BK * LDA_S];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB_S];
+    extern __shared__ __attribute__((aligned(16))) int2 tap_table[];   // TAB: K rounded up to BK entries
 
     // consecutive workgroups share a row tile (the same image patches) and differ in
     // the channel tile; the 8 XCDs each take a contiguous run of row tiles
@@ -167,6 +186,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
     // this thread's patch columns (one per pass), fixed for the whole K walk
     Site site[LA::kPasses];
     bool row_ok[LA::kPasses];
+    unsigned tap_ok[LA::kPasses];   // TAB: bit ky*kW + kx set when that tap of the pixel is inside the image
     int kq;   // k offset of this thread inside a stage: 0, 4, 8 or 12
     {
         int x, k;
@@ -176,32 +196,88 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
             const long long j = m0 + x;
             row_ok[ps] = j < g.J;
             site[ps] = site_of(row_ok[ps] ? j : 0, g);
+            tap_ok[ps] = 0;
+            if constexpr (TAB) {
+                if (row_ok[ps]) {
+                    for (int ky = 0; ky < g.kH; ++ky)
+                        for (int kx = 0; kx < g.kW; ++kx)
+                            if (static_cast<unsigned>(site[ps].ih0 + ky) < static_cast<unsigned>(g.H) &&
+                                static_cast<unsigned>(site[ps].iw0 + kx) < static_cast<unsigned>(g.W))
+                                tap_ok[ps] |= 1u << (ky * g.kW + kx);
+                }
+            }
         }
         LA::coords(0, x, kq);
+    }
+    if constexpr (TAB) {
+        const int kpad = (g.K + BK - 1) / BK * BK;
+        for (int k = threadIdx.x; k < kpad; k += kBlock) {
+            int2 e = make_int2(0, 0);   // rows past K match no pixel
+            if (k < g.K) {
+                const Tap t = tap_of(k, g);
+                e = make_int2(t.off * 4, 1 << (t.ky * g.kW + t.kx));   // byte offset inside an image
+            }
+            tap_table[k] = e;
+        }
+        // (the barrier after the first stage's LDS stores also publishes the table; the
+        // first two stages decode their taps directly)
     }
     floatx4 ra[LA::kPasses], rb[LB::kPasses];
     unsigned offb[LB::kPasses];
     if constexpr (FASTB) LB::offsets(offb, static_cast<unsigned>(g.K));
-    auto load_stage = [&](int k0) {
-        Tap t = tap_of(k0 + kq, g);
-        Tap taps[4];
+    // The loads of a stage are issued in pieces between the MFMA steps of the stage two
+    // before it (the four taps, then one loader pass per step), so that their index
+    // arithmetic runs in the shadow of the matrix pipe instead of in one burst.
+    Tap taps[4];
+    int kcur = 0;
+    auto stage_taps = [&](int k0) {
+        kcur = k0 + kq;
+        Tap t = tap_of(kcur, g);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             taps[e] = t;
             tap_next(t, g);
         }
+    };
+    auto load_a = [&](int ps) {
+        floatx4 r;
 #pragma unroll
-        for (int ps = 0; ps < LA::kPasses; ++ps) {
-            floatx4 r;
+        for (int e = 0; e < 4; ++e)
+            r[e] = (row_ok[ps] && kcur + e < g.K) ? patch_value(in, site[ps], taps[e], g) : 0.0f;
+        ra[ps] = r;
+    };
+    // table forms, used from the third stage on
+    int4 tq[2];   // the thread's four table entries of the stage: {off0, bit0, off1, bit1}, {off2, ...}
+    auto stage_taps_tab = [&](int k0) {
+        const int4* src = reinterpret_cast<const int4*>(tap_table + k0 + kq);
+        tq[0] = src[0];
+        tq[1] = src[1];
+    };
+    const __amdgpu_buffer_rsrc_t in_rsrc = input_resource(in, in_bytes);
+    unsigned site_byte[LA::kPasses];   // byte offset of the pixel's patch origin (wraps when the origin is in the padding)
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                r[e] = (row_ok[ps] && k0 + kq + e < g.K) ? patch_value(in, site[ps], taps[e], g) : 0.0f;
-            ra[ps] = r;
-        }
+    for (int ps = 0; ps < LA::kPasses; ++ps) site_byte[ps] = static_cast<unsigned>(site[ps].base) * 4u;
+    auto load_a_tab = [&](int ps) {
+        const int off[4] = {tq[0].x, tq[0].z, tq[1].x, tq[1].z};
+        const unsigned bit[4] = {static_cast<unsigned>(tq[0].y), static_cast<unsigned>(tq[0].w),
+                                 static_cast<unsigned>(tq[1].y), static_cast<unsigned>(tq[1].w)};
+        floatx4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            r[e] = load_or_zero(in_rsrc, (tap_ok[ps] & bit[e]) ? site_byte[ps] + static_cast<unsigned>(off[e]) : kOutside);
+        ra[ps] = r;
+    };
+    auto load_b = [&](int k0) {
         if constexpr (FASTB)
             LB::load_fast(rb, LB::origin(Wt, g.K, n0, k0), offb);
         else
             LB::load_checked(rb, Wt, g.K, n0, k0, g.Cout, g.K);
+    };
+    auto load_stage = [&](int k0) {
+        stage_taps(k0);
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps) load_a(ps);
+        load_b(k0);
     };
 
     const int nk = (g.K + BK - 1) / BK;
@@ -242,7 +318,17 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
                 if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
                 else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
             }
-            if (kk == kStorePasses && kt + 2 < nk) load_stage((kt + 2) * BK);
+            // pass p of the patch operand is requested one step after its registers went to LDS
+            if (kt + 2 < nk) {
+                if constexpr (TAB) {
+                    if (kk == 0) stage_taps_tab((kt + 2) * BK);
+                    if (kk >= 1 && kk - 1 < LA::kPasses) load_a_tab(kk - 1);
+                } else {
+                    if (kk == 1) stage_taps((kt + 2) * BK);
+                    if (kk >= 1 && kk - 1 < LA::kPasses) load_a(kk - 1);
+                }
+                if (kk == kStorePasses) load_b((kt + 2) * BK);
+            }
             __builtin_amdgcn_sched_barrier(0);
             mfma_step(kk & 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -287,10 +373,10 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
 // t is the upstream gradient in the layer's own (C_out*P, N) layout.  Both
 // loaders take four consecutive j per thread: image pixels along a row for the
 // patch operand, one float4 of t for the other.
-template <int TN>
+template <int TN, bool QUAD>
 __global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restrict__ in, const float* __restrict__ t,
                                                             float* __restrict__ part, ConvGeom g, int tiles_n,
-                                                            long long j_chunk, int t_vec) {
+                                                            long long j_chunk, int t_vec, unsigned in_bytes) {
     constexpr int BM = kWGM * kTM * 32;
     constexpr int BN = kWGN * TN * 32;
     using LA = TileLoader<BM, false, kTM>;
@@ -347,42 +433,93 @@ __global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restr
     }
     const long long CoP = static_cast<long long>(g.Cout) * g.P;
     floatx4 ra[LA::kPasses], rb[LB::kPasses];
-    auto load_stage = [&](long long jst) {
-        const long long j = jst + jq;
-        Site s = site_of(j < g.J ? j : 0, g);
-        Site sites[4];
+    // The loads of a stage are issued in pieces between the MFMA steps of the stage two
+    // before it (stage_sites, then one loader pass per step), so that their index
+    // arithmetic runs in the shadow of the matrix pipe instead of in one burst.
+    // QUAD (W_out % 4 == 0): the four patch columns of a thread are consecutive pixels of
+    // one output row, so one site and one row test serve all four.
+    const __amdgpu_buffer_rsrc_t in_rsrc = input_resource(in, in_bytes);   // used by the QUAD form
+    Site sites[QUAD ? 1 : 4];
+    long long jcur = 0;
+    bool quad_live = false;   // QUAD: the thread's four columns are inside this workgroup's chunk
+    auto stage_sites = [&](long long jst) {
+        jcur = jst + jq;
+        if constexpr (QUAD) {
+            // stages are visited in order, BK columns apart: the site moves along its row
+            // and wraps into the next row or image (J % 4 == 0, so a quad is inside the
+            // chunk or outside it as a whole)
+            if (jst == j_lo) {
+                sites[0] = site_of(jcur < g.J ? jcur : 0, g);
+            } else {
+                Site& q = sites[0];
+                q.ow += BK;
+                while (q.ow >= g.Wo) {
+                    q.ow -= g.Wo;
+                    if (++q.oh == g.Ho) {
+                        q.oh = 0;
+                        ++q.n;
+                    }
+                }
+                q.ih0 = q.oh * g.sh - g.pad_h;
+                q.iw0 = q.ow * g.sw - g.pad_w;
+                q.base = static_cast<long long>(q.n) * g.CHW + (q.ih0 * g.W + q.iw0);
+            }
+            quad_live = jcur < j_hi;
+        } else {
+            Site s0 = site_of(jcur < g.J ? jcur : 0, g);
+            sites[0] = s0;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            sites[e] = s;
-            site_next(s, g);
+            for (int e = 1; e < 4; ++e) {
+                site_next(s0, g);
+                sites[e] = s0;
+            }
         }
+    };
+    auto load_a = [&](int ps) {
+        floatx4 r;
+        if constexpr (QUAD) {
+            const Site& s0 = sites[0];
+            const bool row = k_ok[ps] && quad_live &&
+                             static_cast<unsigned>(s0.ih0 + tap[ps].ky) < static_cast<unsigned>(g.H);
+            const int iw = s0.iw0 + tap[ps].kx;
+            const unsigned byte0 = (static_cast<unsigned>(s0.base) + static_cast<unsigned>(tap[ps].off)) * 4u;
 #pragma unroll
-        for (int ps = 0; ps < LA::kPasses; ++ps) {
-            floatx4 r;
+            for (int e = 0; e < 4; ++e) {
+                const bool ok = row && static_cast<unsigned>(iw + e * g.sw) < static_cast<unsigned>(g.W);
+                r[e] = load_or_zero(in_rsrc, ok ? byte0 + static_cast<unsigned>(e * g.sw) * 4u : kOutside);
+            }
+        } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                r[e] = (k_ok[ps] && j + e < j_hi) ? patch_value(in, sites[e], tap[ps], g) : 0.0f;
-            ra[ps] = r;
+                r[e] = (k_ok[ps] && jcur + e < j_hi) ? patch_value(in, sites[e], tap[ps], g) : 0.0f;
         }
+        ra[ps] = r;
+    };
+    auto load_b = [&](int ps) {
+        if (!LB::active(ps)) return;
+        floatx4 r = {0.f, 0.f, 0.f, 0.f};
+        if (co_b[ps] < g.Cout) {
+            if (t_vec && jcur + 3 < j_hi) {
+                // P % 4 == 0 and j % 4 == 0: the four pixels are consecutive in one image
+                const int p = sites[0].oh * g.Wo + sites[0].ow;
+                r = *reinterpret_cast<const floatx4*>(t + sites[0].n * CoP + static_cast<long long>(co_b[ps]) * g.P + p);
+            } else {
+                Site se = sites[0];
 #pragma unroll
-        for (int ps = 0; ps < LB::kPasses; ++ps) {
-            if (!LB::active(ps)) continue;
-            floatx4 r = {0.f, 0.f, 0.f, 0.f};
-            if (co_b[ps] < g.Cout) {
-                if (t_vec && j + 3 < j_hi) {
-                    // P % 4 == 0 and j % 4 == 0: the four pixels are consecutive in one image
-                    const int p = sites[0].oh * g.Wo + sites[0].ow;
-                    r = *reinterpret_cast<const floatx4*>(t + sites[0].n * CoP + static_cast<long long>(co_b[ps]) * g.P + p);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (j + e < j_hi)
-                            r[e] = t[sites[e].n * CoP + static_cast<long long>(co_b[ps]) * g.P +
-                                     sites[e].oh * g.Wo + sites[e].ow];
+                for (int e = 0; e < 4; ++e) {
+                    if (jcur + e < j_hi) r[e] = t[se.n * CoP + static_cast<long long>(co_b[ps]) * g.P + se.oh * g.Wo + se.ow];
+                    site_next(se, g);
                 }
             }
-            rb[ps] = r;
         }
+        rb[ps] = r;
+    };
+    auto load_stage = [&](long long jst) {
+        stage_sites(jst);
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps) load_a(ps);
+#pragma unroll
+        for (int ps = 0; ps < LB::kPasses; ++ps) load_b(ps);
     };
 
     const int nk = static_cast<int>((j_hi - j_lo + BK - 1) / BK);
@@ -424,7 +561,12 @@ __global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restr
                     if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
                     else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
                 }
-                if (kk == kStorePasses && kt + 2 < nk) load_stage(j_lo + static_cast<long long>(kt + 2) * BK);
+                // pass p of an operand is requested one step after its registers went to LDS
+                if (kt + 2 < nk) {
+                    if (kk == 1) stage_sites(j_lo + static_cast<long long>(kt + 2) * BK);
+                    if (kk >= 1 && kk - 1 < LA::kPasses) load_a(kk - 1);
+                    else if (kk - 1 >= LA::kPasses && kk - 1 < kStorePasses) load_b(kk - 1 - LA::kPasses);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_step(kk & 1);
                 __builtin_amdgcn_sched_barrier(0);
@@ -494,15 +636,26 @@ int launch_fwd(const float* in, const float* Wt, const float* bias, float* out, 
     const bool fastb = g.K % BK == 0 && g.Cout % BN == 0 && aligned16(Wt);
     const unsigned grid = static_cast<unsigned>(total);
     hipStream_t s = stream();
-#define JZ_CONV_FWD(TMV, TNV)                                                                                   \
-    do {                                                                                                        \
-        if (fastb) conv_fwd_kernel<TMV, TNV, true><<<grid, kBlock, 0, s>>>(in, Wt, bias, out, g, relu, tiles_n); \
-        else conv_fwd_kernel<TMV, TNV, false><<<grid, kBlock, 0, s>>>(in, Wt, bias, out, g, relu, tiles_n);      \
+    // tap table: kH*kW one-hot bits in a word, K (rounded up to a stage) entries of 8 bytes in LDS
+    const size_t tab_bytes = static_cast<size_t>((g.K + BK - 1) / BK * BK) * sizeof(int2);
+    const long long in_bytes = static_cast<long long>(g.N) * g.CHW * static_cast<long long>(sizeof(float));
+    const bool tab = g.khw <= 32 && tab_bytes <= 24 * 1024 && g.K > 2 * BK && in_bytes <= kBufferMaxBytes;
+    const unsigned in_b = tab ? static_cast<unsigned>(in_bytes) : 0u;
+#define JZ_CONV_FWD_T(TMV, TNV, FB)                                                                              \
+    do {                                                                                                         \
+        if (tab) conv_fwd_kernel<TMV, TNV, FB, true><<<grid, kBlock, tab_bytes, s>>>(in, Wt, bias, out, g, relu, tiles_n, in_b); \
+        else conv_fwd_kernel<TMV, TNV, FB, false><<<grid, kBlock, 0, s>>>(in, Wt, bias, out, g, relu, tiles_n, in_b);  \
+    } while (0)
+#define JZ_CONV_FWD(TMV, TNV)                \
+    do {                                     \
+        if (fastb) JZ_CONV_FWD_T(TMV, TNV, true); \
+        else JZ_CONV_FWD_T(TMV, TNV, false); \
     } while (0)
     if (TM == 2 && TN == 2) JZ_CONV_FWD(2, 2);
     else if (TM == 2) JZ_CONV_FWD(2, 1);
     else if (TN == 2) JZ_CONV_FWD(1, 2);
     else JZ_CONV_FWD(1, 1);
+#undef JZ_CONV_FWD_T
 #undef JZ_CONV_FWD
     return launch_rc();
 }
@@ -531,10 +684,13 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
     const int BN = wide ? 128 : 64;
     const int tiles_n = (C_out + BN - 1) / BN, tiles_m = (g.K + 127) / 128;
     const long long tiles = static_cast<long long>(tiles_m) * tiles_n;
-    // chunks of the patch-column range: enough workgroups for two per CU, a multiple of 8
+    // chunks of the patch-column range: enough workgroups for two to four per CU, a multiple of 8
     // so that an XCD keeps to its own chunks, at least 16 stages each
     const long long cus = num_cus();
-    long long splits = (2 * cus + tiles - 1) / tiles;
+    // (four per CU while the partial results stay small: 167 against 202 us at 576 x 64;
+    // with larger outputs the extra partial sums cost more than the occupancy gains)
+    const long long per_cu = static_cast<long long>(g.K) * C_out <= 100000 ? 4 : 2;
+    long long splits = (per_cu * cus + tiles - 1) / tiles;
     splits = splits <= 2 ? splits : splits <= 4 ? 4 : (splits + 7) / 8 * 8;
     const long long per = static_cast<long long>(g.K) * C_out;
     while (splits > 1 && (g.J / splits < 16 * BK || per * splits > static_cast<long long>(kWorkspaceFloats)))
@@ -551,8 +707,13 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
     const int t_vec = (g.P % 4 == 0) && aligned16(t);
     dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits));
     hipStream_t s = stream();
-    if (wide) conv_dw_kernel<2><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec);
-    else conv_dw_kernel<1><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec);
+    const long long in_bytes = static_cast<long long>(N) * g.CHW * static_cast<long long>(sizeof(float));
+    const bool quad = W_out % 4 == 0 && in_bytes <= kBufferMaxBytes;
+    const unsigned in_b = quad ? static_cast<unsigned>(in_bytes) : 0u;
+    if (wide && quad) conv_dw_kernel<2, true><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
+    else if (wide) conv_dw_kernel<2, false><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
+    else if (quad) conv_dw_kernel<1, true><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
+    else conv_dw_kernel<1, false><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
     if (splits > 1) launch_splitk_reduce(dW, part, g.K, C_out, static_cast<size_t>(g.K), static_cast<int>(splits), 1.0f, 0.0f);
     return launch_rc();
 }

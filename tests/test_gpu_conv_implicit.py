@@ -50,6 +50,9 @@ SMALL = [
     (2, 11, 12, 12, 16, 3, 3, 1, 1),  # K = 99: not a multiple of the K stage
     (5, 6, 9, 7, 4, 1, 1, 0, 1),
     (2, 3, 9, 9, 6, 4, 4, 1, 2),
+    (3, 7, 8, 8, 20, 3, 3, 1, 1),     # K = 63 > two stages: tap table with a ragged last stage, W_out % 4 == 0
+    (2, 5, 16, 16, 9, 4, 4, 1, 2),    # 4x4 stride 2 (the transposed layers' backward), W_out = 8
+    (1, 40, 4, 4, 8, 3, 3, 1, 1),     # W_out = 4: a stage of 16 columns spans four rows
 ]
 
 
@@ -126,6 +129,9 @@ LAYERS = [
     (128, 3, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 128, 3, 3, 1, 2),
     (128, 128, 16, 16, 128, 3, 3, 1, 1), (128, 128, 16, 16, 256, 3, 3, 1, 2), (128, 256, 8, 8, 256, 3, 3, 1, 1),
     (128, 256, 16, 16, 128, 3, 3, 1, 1), (128, 128, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 3, 3, 3, 1, 1),
+    # the backward pass of the UNet's 4x4 stride-2 transposed convolutions is a convolution over the
+    # upstream gradient: image = (C_out, H_out, W_out), patch grid = (H_in, W_in), "channels out" = C_in
+    (128, 128, 16, 16, 256, 4, 4, 1, 2), (128, 64, 32, 32, 128, 4, 4, 1, 2),
 ]
 
 
