@@ -18,6 +18,13 @@
  *     synchronising; issue order is execution order, exactly as the
  *     reference's null-stream launches (cpp/hipkernels.cpp:610-622).  Only
  *     the memcpy calls and `jzhip_synchronize` block the host.
+ *   - threads: the current stream is one setting for the whole process, as the
+ *     reference's null stream is (cpp/hipkernels.cpp:458-461).  Drive the library
+ *     from one host thread, or serialise `jzhip_set_stream` plus the calls that
+ *     depend on it under a lock of your own: two threads that select different
+ *     streams at the same time would enqueue on each other's stream and share
+ *     its workspace.  The internal tables themselves (workspaces, one-time
+ *     kernel attributes) tolerate concurrent callers.
  *   - no entry point allocates device memory behind the caller's back except
  *     `jzhip_malloc` and the lazily created reduction workspace, one per
  *     stream that needs it (see `jzhip_workspace_bytes`).
@@ -59,7 +66,8 @@ int jzhip_memcpy_d2d(float* dst_device, const float* src_device, size_t count);
 
 /* No reference counterpart (the reference uses the null stream only,
  * cpp/hipkernels.cpp:458-461): select the hipStream_t every later call of
- * this thread's process enqueues on; NULL restores the null stream. */
+ * this process enqueues on (one setting for all host threads, see "threads"
+ * above); NULL restores the null stream. */
 int jzhip_set_stream(void* hip_stream);
 void* jzhip_get_stream(void);
 /* Block until the current stream is idle. */

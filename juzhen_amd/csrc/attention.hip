@@ -11,6 +11,7 @@
 #include "common.hpp"
 
 #include <cmath>
+#include <mutex>
 #include <type_traits>
 
 namespace jz {
@@ -354,13 +355,13 @@ template <int DH, bool BWD>
 int launch_attn_core(float* Out, int ld_out, float* Aio, float* dS, const float* X1, int ld_x1, const float* M1,
                      const float* M2, int ld_m, int heads, int S, int B, float scale, int causal) {
     const size_t lds = attn_core_lds_bytes(DH, S);
-    static bool configured = false;   // per instantiation
-    if (!configured) {
-        int rc = rc_of(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_core_kernel<DH, BWD>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        if (rc) return rc;
-        configured = true;
-    }
+    static std::once_flag once;   // per instantiation
+    static int configure_rc = 0;
+    std::call_once(once, [] {
+        configure_rc = rc_of(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_core_kernel<DH, BWD>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    });
+    if (configure_rc) return configure_rc;
     attn_core_kernel<DH, BWD><<<heads * B, kAttnThreads, lds, stream()>>>(Out, ld_out, Aio, dS, X1, ld_x1, M1, M2, ld_m,
                                                                    heads, S, B, scale, causal);
     return launch_rc();

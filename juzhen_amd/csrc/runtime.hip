@@ -19,7 +19,7 @@ std::atomic<int> g_cus{0};
 constexpr int kMaxWorkspaces = 64;
 struct WorkspaceSlot {
     std::atomic<float*> ptr{nullptr};   // nullptr: slot free
-    hipStream_t owner = nullptr;
+    std::atomic<hipStream_t> owner{nullptr};   // read by the lock-free scan while a slot is being reused
 };
 WorkspaceSlot g_ws[kMaxWorkspaces];
 std::atomic<int> g_ws_count{0};         // slots ever used (scan bound)
@@ -47,14 +47,14 @@ float* workspace() {
     const int n = g_ws_count.load(std::memory_order_acquire);
     for (int i = 0; i < n; ++i) {
         float* p = g_ws[i].ptr.load(std::memory_order_acquire);
-        if (p && g_ws[i].owner == s) return p;
+        if (p && g_ws[i].owner.load(std::memory_order_acquire) == s) return p;
     }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     const int m = g_ws_count.load(std::memory_order_acquire);
     int slot = -1;
     for (int i = 0; i < m; ++i) {
         float* p = g_ws[i].ptr.load(std::memory_order_acquire);
-        if (p && g_ws[i].owner == s) return p;
+        if (p && g_ws[i].owner.load(std::memory_order_acquire) == s) return p;
         if (!p && slot < 0) slot = i;
     }
     if (slot < 0) {
@@ -66,7 +66,7 @@ float* workspace() {
         (void)hipGetLastError();
         return nullptr;
     }
-    g_ws[slot].owner = s;
+    g_ws[slot].owner.store(s, std::memory_order_release);
     g_ws[slot].ptr.store(static_cast<float*>(p), std::memory_order_release);
     if (slot == m) g_ws_count.store(m + 1, std::memory_order_release);
     return static_cast<float*>(p);
@@ -78,7 +78,7 @@ int release_workspace(hipStream_t s) {
     const int m = g_ws_count.load(std::memory_order_acquire);
     for (int i = 0; i < m; ++i) {
         float* p = g_ws[i].ptr.load(std::memory_order_acquire);
-        if (p && g_ws[i].owner == s) {
+        if (p && g_ws[i].owner.load(std::memory_order_acquire) == s) {
             int rc = rc_of(hipStreamSynchronize(s));
             g_ws[i].ptr.store(nullptr, std::memory_order_release);
             const int rc2 = rc_of(hipFree(p));
