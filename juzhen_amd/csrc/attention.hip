@@ -367,133 +367,6 @@ int launch_attn_core(float* Out, int ld_out, float* Aio, float* dS, const float*
     return launch_rc();
 }
 
-// ── dV and dK in one launch ──────────────────────────────────────────────────
-//     dV[d, key] = sum_q dH[d, q] P[q, key],    dK[d, key] = sum_q Q[d, q] dS[q, key]
-// Both reduce over the queries, which the core kernel spreads over its waves, so they
-// are a second launch: one workgroup per (head, sequence) block and tile of 64 keys,
-// waves 0-1 forming dV and waves 2-3 dK (32 rows of d each, 32x32x2 MFMA), walking the
-// queries in chunks of 32 through LDS.  With the causal mask P and dS are zero for
-// key > q, so the walk starts at the tile's first key: 62 % of the full sum at S = 256,
-// and the zeros above the diagonal are never read.
-constexpr int kKvKeys = 64, kKvChunk = 32;
-template <int DH>
-__global__ __launch_bounds__(kBlock) void attn_kv_grad_kernel(float* __restrict__ dV, float* __restrict__ dK,
-                                                              int ld_out, const float* __restrict__ dH, int ld_dh,
-                                                              const float* __restrict__ Q, int ld_q,
-                                                              const float* __restrict__ P,
-                                                              const float* __restrict__ dS, int S, int B,
-                                                              int nblk, int causal) {
-    static_assert(DH == 64, "two waves of 32 rows cover the head");
-    constexpr int LDX = DH + 4;           // [q][d], float4 stores
-    constexpr int LDP = kKvChunk + 1;     // [key][q], odd pitch: lanes along keys hit distinct banks
-    constexpr int XV = kKvChunk * DH / 4 / kBlock;        // float4 per thread and operand: 2
-    constexpr int PV = kKvKeys * kKvChunk / 4 / kBlock;   // 2
-    __shared__ __attribute__((aligned(16))) float Xs[2][kKvChunk * LDX];
-    __shared__ float Ps[2][kKvKeys * LDP];
-
-    // Workgroups are dealt round-robin to the 8 XCDs: the key tiles of one block are given
-    // ids 8 apart so that they run on one XCD and share its L2 copy of dH and Q.
-    const int tiles = S / kKvKeys;
-    int blk, tile;   // blk = hh*B + b
-    if (nblk % 8 == 0) {
-        const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
-        tile = j % tiles;
-        blk = (j / tiles) * 8 + xcd;
-    } else {
-        tile = blockIdx.x % tiles;
-        blk = blockIdx.x / tiles;
-    }
-    const int hh = blk / B, b = blk % B;
-    const int key0 = tile * kKvKeys;
-    const size_t col0 = static_cast<size_t>(b) * S;
-    const float* xsrc[2] = {dH + col0 * ld_dh + hh * DH, Q + col0 * ld_q + hh * DH};
-    const int ldx[2] = {ld_dh, ld_q};
-    const size_t blk_off = static_cast<size_t>(blk) * S * S + static_cast<size_t>(key0) * S;
-    const float* psrc[2] = {P + blk_off, dS + blk_off};
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int which = wave >> 1, dhalf = wave & 1;
-    const int l32 = lane & 31, h = lane >> 5;
-
-    floatx16 acc[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
-
-    floatx4 rx[2][XV], rp[2][PV];
-    auto load = [&](int q0) {
-#pragma unroll
-        for (int w = 0; w < 2; ++w) {
-#pragma unroll
-            for (int i = 0; i < XV; ++i) {
-                const int idx = threadIdx.x + i * kBlock;
-                const int q = idx / (DH / 4), d4 = idx % (DH / 4);
-                rx[w][i] = *reinterpret_cast<const floatx4*>(xsrc[w] + static_cast<size_t>(q0 + q) * ldx[w] + 4 * d4);
-            }
-#pragma unroll
-            for (int i = 0; i < PV; ++i) {
-                const int idx = threadIdx.x + i * kBlock;
-                const int key = idx / (kKvChunk / 4), q4 = idx % (kKvChunk / 4);
-                rp[w][i] = *reinterpret_cast<const floatx4*>(psrc[w] + static_cast<size_t>(key) * S + q0 + 4 * q4);
-            }
-        }
-    };
-    auto stash = [&]() {
-#pragma unroll
-        for (int w = 0; w < 2; ++w) {
-#pragma unroll
-            for (int i = 0; i < XV; ++i) {
-                const int idx = threadIdx.x + i * kBlock;
-                const int q = idx / (DH / 4), d4 = idx % (DH / 4);
-                *reinterpret_cast<floatx4*>(&Xs[w][q * LDX + 4 * d4]) = rx[w][i];
-            }
-#pragma unroll
-            for (int i = 0; i < PV; ++i) {
-                const int idx = threadIdx.x + i * kBlock;
-                const int key = idx / (kKvChunk / 4), q4 = idx % (kKvChunk / 4);
-                float* d = &Ps[w][key * LDP + 4 * q4];
-                d[0] = rp[w][i].x; d[1] = rp[w][i].y; d[2] = rp[w][i].z; d[3] = rp[w][i].w;
-            }
-        }
-    };
-
-    const int q_lo = causal ? key0 : 0;
-    load(q_lo);
-    for (int q0 = q_lo; q0 < S; q0 += kKvChunk) {
-        __syncthreads();   // the previous chunk's fragments have been read
-        stash();
-        __syncthreads();
-        if (q0 + kKvChunk < S) load(q0 + kKvChunk);
-        const float* xa = &Xs[which][h * LDX + dhalf * 32 + l32];
-        const float* pb = &Ps[which][l32 * LDP + h];
-#pragma unroll
-        for (int kk = 0; kk < kKvChunk / 2; ++kk) {
-            const float a = xa[2 * kk * LDX];
-            const float b0 = pb[2 * kk], b1 = pb[32 * LDP + 2 * kk];
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(b0, a, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(b1, a, acc[1], 0, 0, 0);
-        }
-    }
-    // register v of lane (h, l32) is (row d = l32, key = 8*(v/4) + 4*h + v%4) of a 32x32 tile
-    float* out = (which ? dK : dV) + col0 * ld_out + hh * DH + dhalf * 32 + l32;
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int key = key0 + j * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-            out[static_cast<size_t>(key) * ld_out] = acc[j][v];
-        }
-}
-
-bool attn_kv_ok(int d_h, int S, int heads, int B, const void* p0, const void* p1, const void* p2, const void* p3,
-                int ld_dh, int ld_q) {
-    return d_h == 64 && S % kKvKeys == 0 && static_cast<long long>(heads) * B * (S / kKvKeys) <= 0x7fffffffLL &&
-           ld_dh % 4 == 0 &&
-           ld_q % 4 == 0 && aligned16(p0) && aligned16(p1) && aligned16(p2) && aligned16(p3);
-}
-
 }  // namespace
 }  // namespace jz
 
@@ -546,16 +419,11 @@ JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, 
     const long long seq_h = static_cast<long long>(S) * ld_dh;
     const long long blk = static_cast<long long>(S) * S;
     const float scale = 1.0f / sqrtf(static_cast<float>(d_h));
-    const bool core = jz::attn_core_ok(d_h, S, heads, B, dQ, dH, K, V, ld_dqkv, ld_dh, ld_qkv);
-    const bool kv = core && jz::attn_kv_ok(d_h, S, heads, B, dH, Q, A, dA_scratch, ld_dh, ld_qkv);
-    int rc = 0;
-    if (!kv) {
-        // dV_i = dH_i * A_i
-        rc = jz::gemm_batched2(dH, A, dV, d_h, S, S, false, false, ld_dh, S, ld_dqkv, seq_h, blk, seq_d, B, d_h, blk * B,
-                               d_h, heads, 1.0f, 0.0f);
-        if (rc) return rc;
-    }
-    if (core) {
+    // dV_i = dH_i * A_i
+    int rc = jz::gemm_batched2(dH, A, dV, d_h, S, S, false, false, ld_dh, S, ld_dqkv, seq_h, blk, seq_d, B, d_h,
+                               blk * B, d_h, heads, 1.0f, 0.0f);
+    if (rc) return rc;
+    if (jz::attn_core_ok(d_h, S, heads, B, dQ, dH, K, V, ld_dqkv, ld_dh, ld_qkv)) {
         // dA, dS and dQ in one launch; with causal set the key tiles above the
         // diagonal (exact zeros in A) are skipped
         rc = d_h == 64 ? jz::launch_attn_core<64, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, dH, ld_dh, V,
@@ -563,12 +431,6 @@ JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, 
                        : jz::launch_attn_core<32, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, dH, ld_dh, V,
                                                         K, ld_qkv, heads, S, B, scale, causal);
         if (rc) return rc;
-        if (kv) {
-            // dV_i = dH_i * A_i and dK_i = Q_i * dS_i together
-            jz::attn_kv_grad_kernel<64><<<(S / jz::kKvKeys) * heads * B, jz::kBlock, 0, jz::stream()>>>(
-                dV, dK, ld_dqkv, dH, ld_dh, Q, ld_qkv, A, dA_scratch, S, B, heads * B, causal ? 1 : 0);
-            return jz::launch_rc();
-        }
         // dK_i = Q_i * dS_i
         return jz::gemm_batched2(Q, dA_scratch, dK, d_h, S, S, false, false, ld_qkv, S, ld_dqkv, seq, blk, seq_d, B,
                                  d_h, blk * B, d_h, heads, 1.0f, 0.0f);
