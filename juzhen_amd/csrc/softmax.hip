@@ -392,109 +392,6 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, 
     }
 }
 
-// float4 forms of the two passes for numrow % 4 == 0, ld % 4 == 0 and 16-byte aligned
-// operands: a lane owns four consecutive rows, so a wavefront reads 1 KB runs of a
-// column instead of 256 B ones; four columns in flight per thread.
-constexpr int kRowUnrollV = 4;
-// exp(x), x <= 0, for the row sums only: one multiply and the hardware exp2.  Its
-// relative error grows like 1e-7*|x|, on terms whose weight in the sum falls like
-// exp(x), so the sum keeps full float accuracy; the values written use exp_neg.
-__device__ __forceinline__ float exp_stat(float x) {
-    x = x > -100.0f ? x : -100.0f;
-    return __builtin_amdgcn_exp2f(x * 1.44269504088896341f);
-}
-__device__ __forceinline__ float& comp(float4& v, int i) { return reinterpret_cast<float*>(&v)[i]; }
-
-__global__ __launch_bounds__(kBlock) void softmax_rows_partial_vec_kernel(float* part, const float* in,
-                                                                          int numrow, int numcol,
-                                                                          size_t ld, int chunk_len) {
-    constexpr int RPB = kWave, CP = kBlock / kWave;
-    __shared__ float4 redm[CP][RPB], reds[CP][RPB];
-    const int rl = threadIdx.x % RPB, cp = threadIdx.x / RPB;
-    const int row = (blockIdx.x * RPB + rl) * 4;
-    const int c0 = blockIdx.y * chunk_len;
-    const int c1 = (c0 + chunk_len) < numcol ? (c0 + chunk_len) : numcol;
-    float4 m = make_float4(-1e30f, -1e30f, -1e30f, -1e30f), s = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (row < numrow) {
-        for (int c = c0 + cp; c < c1; c += CP * kRowUnrollV) {
-            float4 t[kRowUnrollV];
-#pragma unroll
-            for (int u = 0; u < kRowUnrollV; ++u) {
-                const int cc = c + u * CP;
-                t[u] = cc < c1 ? *reinterpret_cast<const float4*>(in + static_cast<size_t>(cc) * ld + row)
-                               : make_float4(-1e30f, -1e30f, -1e30f, -1e30f);
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float tm = -1e30f;
-#pragma unroll
-                for (int u = 0; u < kRowUnrollV; ++u) tm = tm > comp(t[u], e) ? tm : comp(t[u], e);
-                const float mo = comp(m, e);
-                const float mn = mo > tm ? mo : tm;
-                float acc = comp(s, e) * exp_stat(mo - mn);
-#pragma unroll
-                for (int u = 0; u < kRowUnrollV; ++u)
-                    if (c + u * CP < c1) acc += exp_stat(comp(t[u], e) - mn);
-                comp(s, e) = acc;
-                comp(m, e) = mn;
-            }
-        }
-    }
-    redm[cp][rl] = m;
-    reds[cp][rl] = s;
-    __syncthreads();
-    if (cp == 0 && row < numrow) {
-        float4 M, S;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float mm = -1e30f;
-#pragma unroll
-            for (int k = 0; k < CP; ++k) mm = mm > comp(redm[k][rl], e) ? mm : comp(redm[k][rl], e);
-            float ss = 0.f;
-#pragma unroll
-            for (int k = 0; k < CP; ++k) ss += comp(reds[k][rl], e) * exp_stat(comp(redm[k][rl], e) - mm);
-            comp(M, e) = mm;
-            comp(S, e) = ss;
-        }
-        const size_t o = static_cast<size_t>(blockIdx.y) * 2 * numrow + row;
-        *reinterpret_cast<float4*>(part + o) = M;
-        *reinterpret_cast<float4*>(part + o + numrow) = S;
-    }
-}
-
-__global__ __launch_bounds__(kBlock) void softmax_rows_apply_vec_kernel(float* out, const float* in,
-                                                                        const float* rowstat, int numrow,
-                                                                        int numcol, size_t ld,
-                                                                        int chunk_len) {
-    constexpr int RPB = kWave, CP = kBlock / kWave;
-    const int rl = threadIdx.x % RPB, cp = threadIdx.x / RPB;
-    const int row = (blockIdx.x * RPB + rl) * 4;
-    if (row >= numrow) return;
-    const float4 M = *reinterpret_cast<const float4*>(rowstat + row);
-    const float4 inv = *reinterpret_cast<const float4*>(rowstat + numrow + row);
-    const int c0 = blockIdx.y * chunk_len;
-    const int c1 = (c0 + chunk_len) < numcol ? (c0 + chunk_len) : numcol;
-    for (int c = c0 + cp; c < c1; c += CP * kRowUnrollV) {
-        float4 t[kRowUnrollV];
-#pragma unroll
-        for (int u = 0; u < kRowUnrollV; ++u) {
-            const int cc = c + u * CP;
-            t[u] = cc < c1 ? *reinterpret_cast<const float4*>(in + static_cast<size_t>(cc) * ld + row)
-                           : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-#pragma unroll
-        for (int u = 0; u < kRowUnrollV; ++u) {
-            const int cc = c + u * CP;
-            if (cc < c1) {
-                float4 r;
-                r.x = exp_neg(t[u].x - M.x) * inv.x; r.y = exp_neg(t[u].y - M.y) * inv.y;
-                r.z = exp_neg(t[u].z - M.z) * inv.z; r.w = exp_neg(t[u].w - M.w) * inv.w;
-                *reinterpret_cast<float4*>(out + static_cast<size_t>(cc) * ld + row) = r;
-            }
-        }
-    }
-}
-
 // Rows of up to 2048 columns held in registers by a 1024-thread block: 16 row
 // lanes x 64 column phases, NV columns per thread.  One read and one write per
 // element with numrow/16 workgroups (the 64-row form above leaves most of the
@@ -758,45 +655,26 @@ int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_
             return launch_rc();
         }
         // long rows: two passes with the columns split over grid.y so that
-        // row_blocks x chunks fills the chip.  (Walking the matrix in 64 MB strips of rows,
-        // so that the second pass would find its strip in the memory-side cache, measured
-        // slower: 899 against 680 us at 16384 x 16384.)
-        const bool vec = numrow % 4 == 0 && ld % 4 == 0 && aligned16(in) && aligned16(out) && numrow >= 1024;
-        const int strip = numrow;
-        auto plan = [&](int rows, int& row_blocks, int& chunks, int& chunk_len) {
-            row_blocks = vec ? (rows / 4 + kWave - 1) / kWave : (rows + kWave - 1) / kWave;
-            chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 8 + row_blocks - 1) / row_blocks);
-            if (chunks > numcol / 32) chunks = numcol / 32;
-            if (chunks < 1) chunks = 1;
-            if (chunks > 512) chunks = 512;   // the fold walks them once per row
-            auto need = [&](int ch) { return (static_cast<size_t>(ch) + 1) * rows * 2; };
-            while (chunks > 1 && need(chunks) > kWorkspaceFloats) --chunks;
-            chunk_len = (numcol + chunks - 1) / chunks;
-            chunks = (numcol + chunk_len - 1) / chunk_len;
-            return need(chunks) <= kWorkspaceFloats;
-        };
-        int rb, ch, cl;
-        if (plan(strip < numrow ? strip : numrow, rb, ch, cl)) {
+        // row_blocks x chunks fills the chip.  (Measured and dropped: four rows per lane with
+        // float4 loads, 672 against 680 us at 16384 x 16384 and slower below; walking the
+        // matrix in 64 MB strips of rows so that the second pass would find its strip in the
+        // memory-side cache, 899 us.)
+        int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 8 + row_blocks - 1) / row_blocks);
+        if (chunks > numcol / 32) chunks = numcol / 32;
+        if (chunks < 1) chunks = 1;
+        if (chunks > 512) chunks = 512;   // the fold walks them once per row
+        auto need = [&](int ch) { return (static_cast<size_t>(ch) + 1) * numrow * 2; };
+        while (chunks > 1 && need(chunks) > kWorkspaceFloats) --chunks;
+        const int chunk_len = (numcol + chunks - 1) / chunks;
+        chunks = (numcol + chunk_len - 1) / chunk_len;
+        if (need(chunks) <= kWorkspaceFloats) {
             float* part = workspace();
             if (!part) return -2;
-            for (int r0 = 0; r0 < numrow; r0 += strip) {
-                const int rows = (numrow - r0) < strip ? (numrow - r0) : strip;
-                if (!plan(rows, rb, ch, cl)) return -1;   // a shorter last strip needs no more room
-                float* rowstat = part + static_cast<size_t>(ch) * rows * 2;
-                const dim3 grid(rb, ch);
-                const unsigned fold_grid = (rows + kWave - 1) / kWave;
-                const float* src = in + r0;
-                float* dst = out + r0;
-                if (vec) {
-                    softmax_rows_partial_vec_kernel<<<grid, kBlock, 0, s>>>(part, src, rows, numcol, ld, cl);
-                    softmax_rows_fold_kernel<<<fold_grid, kFoldThreads, 0, s>>>(rowstat, part, rows, ch);
-                    softmax_rows_apply_vec_kernel<<<grid, kBlock, 0, s>>>(dst, src, rowstat, rows, numcol, ld, cl);
-                } else {
-                    softmax_rows_partial_kernel<<<grid, kBlock, 0, s>>>(part, src, rows, numcol, ld, cl);
-                    softmax_rows_fold_kernel<<<fold_grid, kFoldThreads, 0, s>>>(rowstat, part, rows, ch);
-                    softmax_rows_apply_kernel<<<grid, kBlock, 0, s>>>(dst, src, rowstat, rows, numcol, ld, cl);
-                }
-            }
+            float* rowstat = part + static_cast<size_t>(chunks) * numrow * 2;
+            dim3 grid(row_blocks, chunks);
+            softmax_rows_partial_kernel<<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
+            softmax_rows_fold_kernel<<<row_blocks, kFoldThreads, 0, s>>>(rowstat, part, numrow, chunks);
+            softmax_rows_apply_kernel<<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
             return launch_rc();
         }
     }
