@@ -216,10 +216,60 @@ inline void TransformerLayer<ROCMfloat>::add_bias(Matrix<ROCMfloat>& y, const Ma
     y += b * ones_1N;
 }
 
+// op(W) * x with the rest of the statement it belongs to in the product's store:
+//   out = act(op(W) x + bias) + residual,   act 0 none, 1 ReLU (pre-activation kept in *aux),
+//                                           3 multiply by ReLU'(*aux) instead
+// Every step rounds as the separate kernel it replaces (add_bias, relu / drelu_mul,
+// operator+), so the block computes the same bits as the statement-by-statement form.
+// x, aux and residual must be plain (callers materialise transposed views first).
+namespace rocm_detail {
+inline Matrix<ROCMfloat> fused_product(const Matrix<ROCMfloat>& W, bool transpose_w, const Matrix<ROCMfloat>& x,
+                                       const Matrix<ROCMfloat>* bias, int act, Matrix<ROCMfloat>* aux,
+                                       const Matrix<ROCMfloat>* residual) {
+    const bool tw = transpose_w != (bool)W.get_transpose();
+    const size_t m = transpose_w ? W.num_col() : W.num_row(), k = transpose_w ? W.num_row() : W.num_col();
+    const size_t n = x.num_col();
+    if (k != x.num_row() || x.get_transpose() || (bias && (bias->num_row() * bias->num_col() != m)) ||
+        (aux && (aux->get_transpose() || aux->num_row() != m || aux->num_col() != n)) ||
+        (residual && (residual->get_transpose() || residual->num_row() != m || residual->num_col() != n)))
+        throw std::invalid_argument("Matrix dimensions are not compatible");
+    Matrix<ROCMfloat> out = JzRocmFused::make("fused_product", m, n, 0);
+    must(jzhip_gemm_fused(p(W), p(x), p(out), (int)m, (int)n, (int)k, tw ? 1 : 0, 0, (int)JzRocmFused::phys_rows(W),
+                          (int)k, (int)m, 1.0f, 0.0f, bias ? p(*bias) : nullptr, act, aux ? p(*aux) : nullptr, (int)m,
+                          residual ? p(*residual) : nullptr, (int)m),
+         "gemm_fused");
+    return out;
+}
+// LayerNorm::backward followed by `+ residual` (ml/layer.hpp:3309, 3371) as one pass over dy
+inline Matrix<ROCMfloat> ln_backward_plus(LayerNorm<ROCMfloat>& ln, Matrix<ROCMfloat>&& dy,
+                                          const Matrix<ROCMfloat>& residual, bool update) {
+    if (dy.get_transpose() || residual.get_transpose()) return ln.backward(std::move(dy), update) + residual;
+    const int N = (int)dy.num_col();
+    Matrix<ROCMfloat> dx("ln_dx", ln.dim, N);
+    must(jzhip_layernorm_bwd_residual(p(dx), p(dy), p(ln.gamma), p(ln.cached_xhat), p(ln.cached_inv), p(residual),
+                                      ln.dim, N),
+         "layernorm_bwd_residual");
+    // dx reads gamma, so the parameter step comes second (ml/layer.hpp:2682-2686)
+    if (update) {
+        Matrix<ROCMfloat> dg("ln_dgamma", ln.dim, 1), db("ln_dbeta", ln.dim, 1);
+        must(jzhip_layernorm_param_grads(p(dg), p(db), p(dy), p(ln.cached_xhat), ln.dim, N), "layernorm_param_grads");
+        fused_update({{&ln.gamma, &dg, &ln.adam_g}, {&ln.beta, &db, &ln.adam_b}});
+    }
+    return dx;
+}
+}  // namespace rocm_detail
+
+// TransformerLayer::eval (ml/layer.hpp:2946-3031) with the same statements in the same
+// order; biases, ReLU and the two residual additions ride in the stores of the products
+// they follow instead of being passes of their own over (d, N) and (d_ff, N) matrices.
 template <>
-inline void TransformerLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+inline void TransformerLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input_in) {
     using namespace rocm_detail;
     using MD = Matrix<ROCMfloat>;
+    MD held;
+    if (input_in.get_transpose()) held = JzRocmFused::materialise(input_in);
+    const MD& input = input_in.get_transpose() ? held : input_in;
+    const int N = seq_len * batchN;
     // pre-norm attention
     cached_x1 = ln1.forward(input);
     cached_Q = Wq * cached_x1;
@@ -228,17 +278,15 @@ inline void TransformerLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
     must(jzhip_attention_fwd(p(cached_H), p(cached_A), p(cached_Q), p(cached_K), p(cached_V), d_k, num_heads,
                              seq_len, batchN, causal ? 1 : 0),
          "attention_fwd");
-    MD O = Wo * cached_H;
-    add_bias(O, bo);
-    cached_R = input + O;
-    // pre-norm feed-forward
+    // R = input + (Wo H + bo)
+    cached_R = fused_product(Wo, false, cached_H, &bo, 0, nullptr, &input);
+    // pre-norm feed-forward: F1 = W1 x2 + b1 kept beside relu(F1)
     cached_x2 = ln2.forward(cached_R);
-    cached_F1 = W1 * cached_x2;
-    add_bias(cached_F1, b1);
-    cached_F1_relu = relu(MD(cached_F1));
-    MD F = W2 * cached_F1_relu;
-    add_bias(F, b2);
-    this->val = cached_R + F;
+    if (cached_F1.get_transpose() || (int)cached_F1.num_row() != d_ff || (int)cached_F1.num_col() != N)
+        cached_F1 = MD("cached_F1", d_ff, N);
+    cached_F1_relu = fused_product(W1, false, cached_x2, &b1, 1, &cached_F1, nullptr);
+    // val = R + (W2 relu(F1) + b2)
+    this->val = fused_product(W2, false, cached_F1_relu, &b2, 0, nullptr, &cached_R);
 }
 
 template <>
@@ -247,16 +295,16 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
     using namespace rocm_detail;
     using MD = Matrix<ROCMfloat>;
     const int N = seq_len * batchN;
-    MD dout = plain(upstream_grad);  // read three times below; also the residual gradient
+    // read three times below; also the residual gradient
+    MD dout = upstream_grad.get_transpose() ? JzRocmFused::materialise(upstream_grad) : std::move(upstream_grad);
 
     // feed-forward: F = W2 relu(W1 x2 + b1) + b2
     MD dW2 = dout * cached_F1_relu.T();
     MD db2 = sum(dout, 1);
-    MD dF1 = W2.T() * dout;
-    must(jzhip_drelu_mul(p(dF1), p(cached_F1), p(dF1), (size_t)d_ff * N), "drelu_mul");
+    MD dF1 = fused_product(W2, true, dout, nullptr, 3, &cached_F1, nullptr);   // (W2^T dout) .* relu'(F1)
     MD dW1 = dF1 * cached_x2.T();
     MD db1 = sum(dF1, 1);
-    MD dR = ln2.backward(W1.T() * dF1, this->need_update) + dout;
+    MD dR = ln_backward_plus(ln2, W1.T() * dF1, dout, this->need_update);
 
     // output projection: O = Wo H + bo
     MD dWo = dR * cached_H.T();
@@ -272,8 +320,16 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
     MD dWq = dQ * cached_x1.T();
     MD dWk = dK * cached_x1.T();
     MD dWv = dV * cached_x1.T();
-    MD dx1 = Wq.T() * dQ + Wk.T() * dK + Wv.T() * dV;
-    MD dx = ln1.backward(std::move(dx1), this->need_update) + dR;
+    // dx1 = Wq^T dQ + Wk^T dK + Wv^T dV: the second and third products add into the first
+    MD dx1 = Wq.T() * dQ;
+    auto add_product = [&](const MD& W, const MD& g) {
+        must(jzhip_gemm(p(W), p(g), p(dx1), d_model, N, d_k, W.get_transpose() ? 0 : 1, 0, (int)JzRocmFused::phys_rows(W),
+                        d_k, d_model, 1.0f, 1.0f),
+             "gemm");
+    };
+    add_product(Wk, dK);
+    add_product(Wv, dV);
+    MD dx = ln_backward_plus(ln1, std::move(dx1), dR, this->need_update);
 
     if (this->need_update) {
         fused_update({{&Wq, &dWq, &adam_Wq}, {&Wk, &dWk, &adam_Wk}, {&Wv, &dWv, &adam_Wv}, {&Wo, &dWo, &adam_Wo},
