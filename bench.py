@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: transformer train-step tokens/s on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--serial] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--serial] [--no-cpu-baseline] [--no-dropin]
 
 Workload (the character-level transformer configuration): language model over
 vocab 256 byte tokens drawn from Zipf(s=1.1), context 256, batch 64 (16 384 tokens per step), 6
@@ -22,7 +22,10 @@ launch time, measured with HIP events around every launch in separate
 instrumented steps after the timed region; those steps always run on one
 stream.  `cpu_baseline` times the
 reference's own CPU path (oracle/_ref, OpenBLAS build when available) on a
-bounded sample of the same workload.
+bounded sample of the same workload.  `dropin_api` is the same model written on
+the reference's layer classes and run through the drop-in Matrix<ROCMfloat> API
+(a prebuilt program started after the timed region; `--no-dropin` skips it, as
+the profiler commands do).
 """
 from __future__ import annotations
 
@@ -170,6 +173,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dropin", action="store_true",
+                    help="skip the run of the same model on the reference's layer classes (dropin_api key)")
     ap.add_argument("--serial", action="store_true",
                     help="one stream, program order, also in the timed steps (for per-kernel traces and counters)")
     ap.add_argument("--fresh-batches", action="store_true",
@@ -281,6 +286,27 @@ def main():
         except Exception as exc:  # the baseline must never take the GPU number down with it
             cpu = {"value": None, "unit": "tokens/s", "cores": 0, "kind": "reference", "sample": f"failed: {exc}"}
 
+    # The same model written on the reference's own layer classes (LinearLayer + 6 x
+    # TransformerLayer<ROCMfloat> + LogisticLayer, ReLU FFN, Adam) through the drop-in API:
+    # what a user of Matrix<ROCMfloat> gets without the harness.  A prebuilt program; run
+    # after the timed region, reported beside the headline number, never part of it.
+    dropin = None
+    dropin_bin = Path(__file__).resolve().parent / "oracle" / "_ref" / "bin" / "lm_dropin_rocm"
+    if not args.no_dropin and dropin_bin.exists():
+        try:
+            import re
+            import subprocess
+            r = subprocess.run([str(dropin_bin)], capture_output=True, text=True, timeout=200)
+            line = next(l for l in r.stdout.splitlines() if l.startswith("RESULT dropin"))
+            kv = dict(re.findall(r"(\w+)=(\S+)", line))
+            dropin = {"tokens_per_s": float(kv["tokens_per_second"]), "ms_per_step": float(kv["mean_ms"]),
+                      "steps": int(kv["steps"]), "warmup": int(kv["warmup"]),
+                      "model": "LinearLayer + 6 x TransformerLayer<ROCMfloat> + LinearLayer + LogisticLayer "
+                               "(ml/layer.hpp), d_model 512, 8 heads, FFN 2048 ReLU, context 256, batch 64, Adam",
+                      "program": "oracle/_ref/bin/lm_dropin_rocm (juzhen_amd/harness/lm_dropin.cu)"}
+        except Exception as exc:
+            dropin = {"tokens_per_s": None, "error": str(exc)}
+
     out = {
         "metric": "transformer train-step tokens/s", "value": round(value, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3),
@@ -295,6 +321,7 @@ def main():
                    "loss_last": round(last_loss, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 3)},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "dropin_api": dropin,
     }
     if cpu and cpu.get("value"):
         out["speedup_vs_cpu_baseline"] = round(value / cpu["value"], 1)
