@@ -91,7 +91,8 @@ class ConvLayer : public Layer<ROCMfloat> {
         // forward: the implicit form needs enough output pixels to fill the chip with 64-row tiles
         fwd_implicit = J >= 16384 && (P >= 256 || K <= 64);
         // weight gradients: wins when the patch matrix is cheap to form relative to the product
-        dw_implicit = (K <= 288) || (stride == 1 && C_out >= 32 && K <= 1152);
+        // (and always with at most four output channels on a 3x3 kernel: a direct kernel streams the input once)
+        dw_implicit = (K <= 288) || (stride == 1 && C_out >= 32 && K <= 1152) || (C_out <= 4 && kH == 3 && kW == 3);
         // input gradients: stride 1 only; needs channels on both sides and a grid of 16 x 16 or more
         dx_implicit = stride == 1 && pad <= kH - 1 && pad <= kW - 1 && C_in >= 32 && (long long)H_in * W_in >= 256 &&
                       (long long)H_in * W_in * N >= 16384;

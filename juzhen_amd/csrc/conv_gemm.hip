@@ -610,6 +610,142 @@ __global__ __launch_bounds__(kBlock) void conv_flip_weights_kernel(float* __rest
     }
 }
 
+// ── at most four output channels (the 3-channel output layer of the UNet) ────
+// A 64-wide MFMA tile for three channels wastes twenty MFMA columns in twenty-one, and
+// the weight gradients took the patch-matrix route (302 MB written and read).  With so few
+// channels both products are a stream over the input, so they are plain vector code:
+// forward 92 -> 57 us, weight gradients 204 -> 37 us at 64 -> 3 channels, 32 x 32,
+// batch 128 (and the input gradients of a 3 -> 64 layer, which are a forward product
+// with three output channels, 99 -> 58 us).
+constexpr int kThinCout = 4;
+constexpr int kThinPixels = 64;   // pixels per workgroup in the forward kernel: one wavefront wide
+
+// Forward: a workgroup takes 64 consecutive output pixels; its four waves take a quarter
+// of the input channels each (lanes along the pixels: 256-byte runs of an image row) and
+// meet in LDS in a fixed order.  The weights sit in LDS as one float4 per patch row
+// (the channels of that row, zero-filled), read as a broadcast.
+__global__ __launch_bounds__(kBlock) void conv_thin_fwd_kernel(const float* __restrict__ in,
+                                                               const float* __restrict__ Wt,
+                                                               const float* __restrict__ bias,
+                                                               float* __restrict__ out, ConvGeom g, int relu) {
+    extern __shared__ __attribute__((aligned(16))) float thin_lds[];
+    floatx4* wl = reinterpret_cast<floatx4*>(thin_lds);                 // [K]
+    floatx4* red = wl + g.K;                                            // [3][64]
+    for (int k = threadIdx.x; k < g.K; k += kBlock) {
+        floatx4 w = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int co = 0; co < kThinCout; ++co)
+            if (co < g.Cout) w[co] = Wt[static_cast<long long>(co) * g.K + k];
+        wl[k] = w;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const long long j = static_cast<long long>(blockIdx.x) * kThinPixels + lane;
+    const bool live = j < g.J;
+    const Site s = site_of(live ? j : 0, g);
+    constexpr int NW = kBlock / kWave;
+    const int c_per = (g.C + NW - 1) / NW;
+    const int c_lo = wave * c_per, c_hi = (c_lo + c_per) < g.C ? (c_lo + c_per) : g.C;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        for (int c = c_lo; c < c_hi; ++c) {
+            const float* plane = in + s.base + static_cast<long long>(c) * g.HW;
+            const floatx4* wc = wl + c * g.khw;
+            for (int ky = 0; ky < g.kH; ++ky) {
+                const bool row = static_cast<unsigned>(s.ih0 + ky) < static_cast<unsigned>(g.H);
+                for (int kx = 0; kx < g.kW; ++kx) {
+                    const bool ok = row && static_cast<unsigned>(s.iw0 + kx) < static_cast<unsigned>(g.W);
+                    const float v = ok ? plane[ky * g.W + kx] : 0.0f;
+                    const floatx4 w = wc[ky * g.kW + kx];
+                    acc[0] += v * w[0]; acc[1] += v * w[1]; acc[2] += v * w[2]; acc[3] += v * w[3];
+                }
+            }
+        }
+    }
+    if (wave > 0) red[(wave - 1) * kWave + lane] = acc;
+    __syncthreads();
+    if (wave == 0 && live) {
+#pragma unroll
+        for (int w = 0; w < NW - 1; ++w) {
+            const floatx4 o = red[w * kWave + lane];
+            acc[0] += o[0]; acc[1] += o[1]; acc[2] += o[2]; acc[3] += o[3];
+        }
+        const int p = s.oh * g.Wo + s.ow;
+        float* dst = out + static_cast<long long>(s.n) * g.Cout * g.P + p;
+#pragma unroll
+        for (int co = 0; co < kThinCout; ++co) {
+            if (co < g.Cout) {
+                float r = acc[co];
+                if (bias) r += bias[co];
+                if (relu) r = r > 0.0f ? r : 0.0f;
+                dst[static_cast<long long>(co) * g.P] = r;
+            }
+        }
+    }
+}
+
+// Weight gradients for a KH x KW kernel: a workgroup takes one input channel and a
+// chunk of the patch columns; a thread walks its pixels and keeps KH*KW*4 sums
+// (tap x channel), which the workgroup adds up at the end; one partial result per
+// chunk, summed afterwards in a fixed order.
+template <int KH, int KW>
+__global__ __launch_bounds__(kBlock) void conv_thin_dw_kernel(const float* __restrict__ in,
+                                                              const float* __restrict__ t,
+                                                              float* __restrict__ part, ConvGeom g,
+                                                              long long j_chunk) {
+    constexpr int KHW = KH * KW;
+    constexpr int NW = kBlock / kWave;
+    __shared__ float red[NW][KHW * kThinCout];
+    const int c = blockIdx.x;
+    const long long j_lo = static_cast<long long>(blockIdx.y) * j_chunk;
+    const long long j_hi = (j_lo + j_chunk) < g.J ? (j_lo + j_chunk) : g.J;
+    const long long CoP = static_cast<long long>(g.Cout) * g.P;
+    float acc[KHW][kThinCout];
+#pragma unroll
+    for (int a = 0; a < KHW; ++a)
+#pragma unroll
+        for (int co = 0; co < kThinCout; ++co) acc[a][co] = 0.0f;
+    for (long long j = j_lo + threadIdx.x; j < j_hi; j += kBlock) {
+        const Site s = site_of(j, g);
+        const float* tp = t + s.n * CoP + s.oh * g.Wo + s.ow;
+        float tv[kThinCout];
+#pragma unroll
+        for (int co = 0; co < kThinCout; ++co) tv[co] = co < g.Cout ? tp[static_cast<long long>(co) * g.P] : 0.0f;
+        const float* plane = in + s.base + static_cast<long long>(c) * g.HW;
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky) {
+            const bool row = static_cast<unsigned>(s.ih0 + ky) < static_cast<unsigned>(g.H);
+#pragma unroll
+            for (int kx = 0; kx < KW; ++kx) {
+                const bool ok = row && static_cast<unsigned>(s.iw0 + kx) < static_cast<unsigned>(g.W);
+                const float v = ok ? plane[ky * g.W + kx] : 0.0f;
+#pragma unroll
+                for (int co = 0; co < kThinCout; ++co) acc[ky * KW + kx][co] += v * tv[co];
+            }
+        }
+    }
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int a = 0; a < KHW; ++a)
+#pragma unroll
+        for (int co = 0; co < kThinCout; ++co) {
+            const float v = wave_sum(acc[a][co]);
+            if (lane == 0) red[wave][a * kThinCout + co] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < KHW * kThinCout) {
+        const int a = threadIdx.x / kThinCout, co = threadIdx.x % kThinCout;
+        if (co < g.Cout) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += red[w][threadIdx.x];
+            // partial result of this chunk: (K, C_out) column-major, row k = c*KHW + a
+            part[static_cast<long long>(blockIdx.y) * g.K * g.Cout + static_cast<long long>(co) * g.K + c * KHW + a] = sum;
+        }
+    }
+}
+
 bool dims_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int sh, int sw, int H_out,
              int W_out, int N) {
     if (C_in <= 0 || H_in <= 0 || W_in <= 0 || C_out <= 0 || kH <= 0 || kW <= 0 || pad_h < 0 || pad_w < 0 || sh <= 0 ||
@@ -622,6 +758,14 @@ bool dims_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
 }
 
 int launch_fwd(const float* in, const float* Wt, const float* bias, float* out, const ConvGeom& g, int relu) {
+    if (g.Cout <= kThinCout && g.C >= 8) {
+        const size_t lds = (static_cast<size_t>(g.K) + 3 * kWave) * sizeof(floatx4);
+        const long long blocks = (g.J + kThinPixels - 1) / kThinPixels;
+        if (lds <= 48 * 1024 && blocks <= 0x7fffffffll) {
+            conv_thin_fwd_kernel<<<static_cast<unsigned>(blocks), kBlock, lds, stream()>>>(in, Wt, bias, out, g, relu);
+            return launch_rc();
+        }
+    }
     // the largest tile that still gives every CU two workgroups; 64-row tiles for layers
     // with few output pixels (8x8 grids), 64-channel tiles when that is not enough
     const long long want = 2ll * num_cus();
@@ -680,6 +824,29 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
     if (!input || !t || !dW) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
     const ConvGeom g = make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N, C_out);
+    if (C_out <= kThinCout && kH == 3 && kW == 3 && C_in <= 65535) {
+        // chunks of the patch columns so that channels x chunks gives every CU several workgroups
+        const long long cus = num_cus();
+        long long chunks = (8 * cus + C_in - 1) / C_in;
+        if (chunks > g.J / 1024) chunks = g.J / 1024;
+        if (chunks < 1) chunks = 1;
+        const long long per = static_cast<long long>(g.K) * C_out;
+        while (chunks > 1 && per * chunks > static_cast<long long>(kWorkspaceFloats)) --chunks;
+        const long long j_chunk = (g.J + chunks - 1) / chunks;
+        chunks = (g.J + j_chunk - 1) / j_chunk;
+        if (chunks <= 65535) {
+            float* part = dW;
+            if (chunks > 1) {
+                part = workspace();
+                if (!part) return -2;
+            }
+            conv_thin_dw_kernel<3, 3><<<dim3(C_in, static_cast<unsigned>(chunks)), kBlock, 0, stream()>>>(input, t, part, g,
+                                                                                                           j_chunk);
+            if (chunks > 1)
+                launch_splitk_reduce(dW, part, g.K, C_out, static_cast<size_t>(g.K), static_cast<int>(chunks), 1.0f, 0.0f);
+            return launch_rc();
+        }
+    }
     const bool wide = C_out > 64;
     const int BN = wide ? 128 : 64;
     const int tiles_n = (C_out + BN - 1) / BN, tiles_m = (g.K + 127) / 128;

@@ -53,6 +53,10 @@ SMALL = [
     (3, 7, 8, 8, 20, 3, 3, 1, 1),     # K = 63 > two stages: tap table with a ragged last stage, W_out % 4 == 0
     (2, 5, 16, 16, 9, 4, 4, 1, 2),    # 4x4 stride 2 (the transposed layers' backward), W_out = 8
     (1, 40, 4, 4, 8, 3, 3, 1, 1),     # W_out = 4: a stage of 16 columns spans four rows
+    (2, 9, 7, 6, 3, 3, 3, 1, 1),      # at most four output channels: the direct kernels, ragged channel split
+    (3, 8, 9, 9, 2, 3, 3, 1, 2),      # the same with stride 2
+    (2, 8, 8, 8, 4, 5, 5, 2, 1),      # four channels, 5x5: direct forward, tiled weight gradients
+    (2, 3, 6, 6, 16, 3, 3, 1, 1),     # input gradients of a 3-channel image: the direct forward kernel with flipped weights
 ]
 
 
