@@ -49,6 +49,11 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_event_record": (I, [P]),
     "jzhip_stream_wait_event": (I, [P]),
     "jzhip_event_synchronize": (I, [P]),
+    "jzhip_graph_begin": (I, []),
+    "jzhip_graph_end": (I, [C.POINTER(P)]),
+    "jzhip_graph_recording": (I, []),
+    "jzhip_graph_launch": (I, [P]),
+    "jzhip_graph_destroy": (I, [P]),
     "jzhip_host_alloc": (I, [P, Z]),
     "jzhip_host_free": (I, [P]),
     "jzhip_memcpy_h2d_async": (I, [P, P, Z]),
@@ -121,6 +126,8 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_adam_update": (I, [P, P, P, Z, F, F, F, F, I]),
     "jzhip_adamw_step": (I, [P, P, P, P, Z, F, F, F, F, F, I]),
     "jzhip_adamw_step_multi": (I, [C.POINTER(AdamTensor), I]),
+    "jzhip_adamw_step_multi_counted": (I, [C.POINTER(AdamTensor), I, P]),
+    "jzhip_counter_add": (I, [P, I]),
     "jzhip_im2col": (I, [P, P] + [I] * 12),
     "jzhip_col2im": (I, [P, P] + [I] * 12),
     "jzhip_conv_forward_reshape_bias": (I, [P, P, P, I, I, I]),

@@ -23,6 +23,7 @@
 #define JZ_HIPFUSED_HPP
 
 #include <initializer_list>
+#include <vector>
 #include <typeinfo>
 
 #include "jzhip.h"
@@ -52,6 +53,17 @@ struct AdamItem {
     Matrix<ROCMfloat>* g;
     adam_state<ROCMfloat>* st;
 };
+// What a recording in progress (RocmStepGraph below) needs from the optimiser launches it
+// records: the device counter of replays their step numbers are offset by, and the list
+// of optimiser states whose host-side step count a replay has to advance.
+struct GraphRecording {
+    int* replays_device = nullptr;
+    std::vector<adam_state<ROCMfloat>*> states;
+};
+inline GraphRecording*& current_recording() {
+    static GraphRecording* r = nullptr;
+    return r;
+}
 inline void fused_update(std::initializer_list<AdamItem> items) {
     bool all_plain = items.size() <= 16;
     for (const AdamItem& it : items) {
@@ -60,6 +72,12 @@ inline void fused_update(std::initializer_list<AdamItem> items) {
                     !it.st->v.get_transpose() && it.g->num_row() * it.g->num_col() == n &&
                     it.st->m.num_row() * it.st->m.num_col() == n && it.st->v.num_row() * it.st->v.num_col() == n &&
                     it.g->num_row() == it.w->num_row();
+    }
+    GraphRecording* rec = jzhip_graph_recording() ? current_recording() : nullptr;
+    if (jzhip_graph_recording() && (!rec || !all_plain)) {
+        std::cerr << "juzhen rocm: an optimiser step on transposed views, or outside a RocmStepGraph, cannot be recorded"
+                  << std::endl;
+        ERROR_OUT;
     }
     if (!all_plain) {
         for (const AdamItem& it : items) *it.w -= adam_update(std::move(*it.g), *it.st);
@@ -75,9 +93,90 @@ inline void fused_update(std::initializer_list<AdamItem> items) {
         t[n].iteration = it.st->iteration;
         ++n;
     }
+    if (rec) {
+        // recorded: step number = iteration now + replays so far, formed on the device; the host-side
+        // counts are advanced by RocmStepGraph::replay()
+        must(jzhip_adamw_step_multi_counted(t, n, rec->replays_device), "adamw_step_multi_counted");
+        for (const AdamItem& it : items) rec->states.push_back(it.st);
+        return;
+    }
     must(jzhip_adamw_step_multi(t, n), "adamw_step_multi");
     for (const AdamItem& it : items) it.st->iteration++;
 }
+
+}  // namespace rocm_detail
+
+// A training step recorded once and replayed as one HIP graph launch, for models whose step
+// is a few hundred small kernels and therefore bound by launch cost (no counterpart in the
+// reference, which launches every kernel from the host each step).
+//
+//     RocmStepGraph graph;
+//     graph.begin();                       // calls below are recorded, not run
+//     forward(net, X); ... backprop(net, X);
+//     graph.end();
+//     for (...) graph.replay();            // each replay is the next optimiser step
+//
+// The recorded step works on the buffers it was recorded with (inputs, layer values,
+// temporaries from the pool), so the batch is whatever X holds at replay time and results
+// are read from the same matrices after any replay.  While recording: no host reads of
+// device data (item(), to_host()), no host-to-device construction, no random draws (a
+// replay would repeat them), and parameter updates only through the layers' backward().
+// Run at least one ordinary step first so that the pool already holds every buffer size.
+class RocmStepGraph {
+    void* exec = nullptr;
+    float* counter = nullptr;   // one int in device memory: replays so far
+    rocm_detail::GraphRecording rec;
+    // every buffer created while recording (layer values, temporaries): the replays write
+    // them, so they stay out of the pool until the graph is destroyed
+    std::vector<std::shared_ptr<ROCMfloat[]>> pinned;
+
+   public:
+    RocmStepGraph() = default;
+    RocmStepGraph(const RocmStepGraph&) = delete;
+    RocmStepGraph& operator=(const RocmStepGraph&) = delete;
+    ~RocmStepGraph() {
+        if (exec) jzhip_graph_destroy(exec);   // waits for replays in flight
+        if (counter) jzhip_free(counter);
+        pinned.clear();                        // the buffers return to the pool
+    }
+    void begin() {
+        using namespace rocm_detail;
+        if (exec || current_recording()) {
+            std::cerr << "juzhen rocm: RocmStepGraph::begin() on a graph that is recorded or recording" << std::endl;
+            ERROR_OUT;
+        }
+        must(jzhip_malloc(&counter, 1), "malloc");
+        must(jzhip_fill(counter, 1, 0.0f), "fill");   // all-zero bits: the int 0
+        rec.replays_device = reinterpret_cast<int*>(counter);
+        rec.states.clear();
+        must(jzhip_graph_begin(), "graph_begin");
+        (void)JzRocmFused::take_recording_pins();   // start from an empty list
+        current_recording() = &rec;
+    }
+    void end() {
+        using namespace rocm_detail;
+        if (current_recording() != &rec) {
+            std::cerr << "juzhen rocm: RocmStepGraph::end() without begin()" << std::endl;
+            ERROR_OUT;
+        }
+        // the last recorded launch: every replay advances the optimiser step
+        must(jzhip_counter_add(rec.replays_device, 1), "counter_add");
+        current_recording() = nullptr;
+        must(jzhip_graph_end(&exec), "graph_end");
+        pinned = JzRocmFused::take_recording_pins();
+    }
+    void replay() {
+        using namespace rocm_detail;
+        if (!exec) {
+            std::cerr << "juzhen rocm: RocmStepGraph::replay() before end()" << std::endl;
+            ERROR_OUT;
+        }
+        must(jzhip_graph_launch(exec), "graph_launch");
+        for (adam_state<ROCMfloat>* st : rec.states) st->iteration++;
+    }
+};
+
+namespace rocm_detail {
 
 // weights * input + bias * ones(1, n) (+ ReLU) in one launch: the chain every
 // dense layer's eval() and grad() issues as a product, a rank-1 product, an

@@ -90,9 +90,23 @@ MR::Matrix(const char* name, size_t numrow, size_t numcol, int trans,
            std::shared_ptr<ROCMfloat[]> elements)
     : numcol(numcol), numrow(numrow), transpose(trans != 0), name(name), elements(std::move(elements)) {}
 
+// Buffers created while a step is being recorded (jzhip_graph_begin) are written by every
+// replay of the graph, so they must not go back to the pool while the graph lives: each gets
+// one more owner here, which RocmStepGraph takes over when the recording ends.
+static std::vector<std::shared_ptr<ROCMfloat[]>>& recording_pins() {
+    static std::vector<std::shared_ptr<ROCMfloat[]>> pins;
+    return pins;
+}
+std::vector<std::shared_ptr<ROCMfloat[]>> JzRocmFused::take_recording_pins() {
+    std::vector<std::shared_ptr<ROCMfloat[]>> out;
+    out.swap(recording_pins());
+    return out;
+}
+
 MR::Matrix(const char* name, size_t numrow, size_t numcol, int trans)
     : numcol(numcol), numrow(numrow), transpose(trans != 0), name(name) {
     elements.reset(Memory<ROCMfloat>::allocate(numrow * numcol), pool_release);
+    if (jzhip_graph_recording()) recording_pins().push_back(elements);
 }
 
 MR::Matrix(const Matrix<float>& M)

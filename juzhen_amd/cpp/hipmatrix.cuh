@@ -193,17 +193,26 @@ struct JzRocmFused {
     static size_t phys_cols(const Matrix<ROCMfloat>& M) { return M.numcol; }
     // Materialise the logical transpose of M as a plain (flag 0) matrix.
     static Matrix<ROCMfloat> materialise(const Matrix<ROCMfloat>& M);
+    // The buffers created since jzhip_graph_begin (each with one extra owner): whoever takes
+    // them keeps them out of the pool for as long as the recorded graph may be replayed.
+    static std::vector<std::shared_ptr<ROCMfloat[]>> take_recording_pins();
 };
 
 // adam_update (ml/util.cuh:166-256) as one fused kernel with the arithmetic of
 // the CPU loop (ml/util.cuh:223-245).  adam_state is only forward-declared
 // here, so the body is a template that is instantiated at the end of the
 // including translation unit, where ml/util.cuh has completed the type.
+extern "C" int jzhip_graph_recording(void);
 extern "C" int jzhip_adam_update(float* g, float* m, float* v, size_t count, float alpha, float beta1,
                                  float beta2, float eps, int iteration);
 
 template <class State>
 Matrix<ROCMfloat> jz_rocm_adam_update(Matrix<ROCMfloat>&& g, State& st) {
+    if (jzhip_graph_recording()) {
+        // the step count is a by-value argument of this launch: a replay would repeat step `iteration`
+        LOG_ERROR("adam_update cannot be recorded into a graph: update parameters through a layer's backward()");
+        ERROR_OUT;
+    }
     if (!g.get_transpose() && !st.m.get_transpose() && !st.v.get_transpose()) {
         const int rc = jzhip_adam_update(JzRocmFused::ptr(g), JzRocmFused::ptr(st.m), JzRocmFused::ptr(st.v),
                                          g.num_row() * g.num_col(), st.alpha, st.beta1, st.beta2, st.eps,

@@ -141,13 +141,29 @@ struct AdamMulti {
     unsigned first_block[kMultiMax + 1];
     AdamConst c[kMultiMax];
     int vec[kMultiMax];
+    int base_iteration[kMultiMax];
     int count;
 };
 
-__global__ __launch_bounds__(kBlock) void adam_multi_kernel(AdamMulti p) {
+// COUNTED: the step number of a tensor is its `iteration` plus a counter read from device
+// memory, and the two bias corrections (ml/util.cuh:226-227) are formed here, in double as
+// on the host; with it a recorded launch can be replayed for successive steps.
+template <bool COUNTED>
+__global__ __launch_bounds__(kBlock) void adam_multi_kernel(AdamMulti p, const int* __restrict__ replays) {
     int t = 0;
     while (t + 1 < p.count && blockIdx.x >= p.first_block[t + 1]) ++t;
-    const AdamConst c = p.c[t];
+    AdamConst c = p.c[t];
+    if constexpr (COUNTED) {
+        __shared__ float corr[2];
+        if (threadIdx.x == 0) {
+            const double it = static_cast<double>(p.base_iteration[t] + *replays);
+            corr[0] = static_cast<float>(1.0 / (1.0 - pow(static_cast<double>(c.beta1), it)));
+            corr[1] = static_cast<float>(1.0 / (1.0 - pow(static_cast<double>(c.beta2), it)));
+        }
+        __syncthreads();
+        c.r1 = corr[0];
+        c.r2 = corr[1];
+    }
     float* w = p.w[t];
     const float* g = p.g[t];
     float* m = p.m[t];
@@ -193,22 +209,23 @@ __global__ __launch_bounds__(kBlock) void adam_multi_kernel(AdamMulti p) {
 
 using namespace jz;
 
-JZ_API int jzhip_adamw_step_multi(const jzhip_adam_tensor* tensors, int n_tensors) {
+namespace {
+int adam_multi(const jzhip_adam_tensor* tensors, int n_tensors, const int* replays) {
     if (n_tensors < 0 || (n_tensors > 0 && !tensors)) return -1;
     for (int i = 0; i < n_tensors; ++i) {
         const jzhip_adam_tensor& t = tensors[i];
         if (t.count && (!t.w || !t.g || !t.m || !t.v)) return -1;
         if (t.iteration < 1) return -1;
     }
-    hipStream_t s = stream();
+    hipStream_t s = jz::stream();
     for (int at = 0; at < n_tensors;) {
-        AdamMulti p;
+        jz::AdamMulti p;
         p.count = 0;
         unsigned blocks = 0;
-        for (; at < n_tensors && p.count < kMultiMax; ++at) {
+        for (; at < n_tensors && p.count < jz::kMultiMax; ++at) {
             const jzhip_adam_tensor& t = tensors[at];
             if (t.count == 0) continue;
-            const size_t nb = (t.count + kMultiPerBlock - 1) / kMultiPerBlock;
+            const size_t nb = (t.count + jz::kMultiPerBlock - 1) / jz::kMultiPerBlock;
             if (nb > 0x7fffffffull - blocks) {   // a tensor this large goes alone
                 if (p.count > 0) break;
             }
@@ -216,18 +233,40 @@ JZ_API int jzhip_adamw_step_multi(const jzhip_adam_tensor* tensors, int n_tensor
             p.w[k] = t.w; p.g[k] = t.g; p.m[k] = t.m; p.v[k] = t.v;
             p.n[k] = t.count;
             p.first_block[k] = blocks;
-            p.c[k] = make_const(t.alpha, t.beta1, t.beta2, t.eps, t.weight_decay, t.iteration);
-            p.vec[k] = aligned16(t.w) && aligned16(t.g) && aligned16(t.m) && aligned16(t.v);
+            p.c[k] = jz::make_const(t.alpha, t.beta1, t.beta2, t.eps, t.weight_decay, t.iteration);
+            p.base_iteration[k] = t.iteration;
+            p.vec[k] = jz::aligned16(t.w) && jz::aligned16(t.g) && jz::aligned16(t.m) && jz::aligned16(t.v);
             if (nb > 0x7fffffffull) return -1;
             blocks += static_cast<unsigned>(nb);
         }
         if (p.count == 0) continue;
         p.first_block[p.count] = blocks;
-        adam_multi_kernel<<<blocks, kBlock, 0, s>>>(p);
-        const int rc = launch_rc();
+        if (replays) jz::adam_multi_kernel<true><<<blocks, jz::kBlock, 0, s>>>(p, replays);
+        else jz::adam_multi_kernel<false><<<blocks, jz::kBlock, 0, s>>>(p, nullptr);
+        const int rc = jz::launch_rc();
         if (rc) return rc;
     }
     return 0;
+}
+
+__global__ void counter_add_kernel(int* counter, int delta) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) *counter += delta;
+}
+}  // namespace
+
+JZ_API int jzhip_adamw_step_multi(const jzhip_adam_tensor* tensors, int n_tensors) {
+    return adam_multi(tensors, n_tensors, nullptr);
+}
+
+JZ_API int jzhip_adamw_step_multi_counted(const jzhip_adam_tensor* tensors, int n_tensors, const int* replays_device) {
+    if (!replays_device) return -1;
+    return adam_multi(tensors, n_tensors, replays_device);
+}
+
+JZ_API int jzhip_counter_add(int* counter_device, int delta) {
+    if (!counter_device) return -1;
+    counter_add_kernel<<<1, 64, 0, jz::stream()>>>(counter_device, delta);
+    return jz::launch_rc();
 }
 
 JZ_API int jzhip_adam_update(float* g, float* m, float* v, size_t count, float alpha, float beta1,

@@ -207,7 +207,76 @@ JZ_API int jzhip_memcpy_d2h_async(void* dst_host, const void* src_device, size_t
     return jz::rc_of(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, jz::stream()));
 }
 
+// ── recording a sequence of calls and replaying it as one graph launch ───────
+namespace {
+std::mutex g_graph_mutex;
+hipStream_t g_record_stream = nullptr;   // created on first use, lives until the process ends
+hipStream_t g_stream_before = nullptr;   // the current stream when recording began
+std::atomic<int> g_recording{0};
+}  // namespace
+
+JZ_API int jzhip_graph_begin(void) {
+    std::lock_guard<std::mutex> lock(g_graph_mutex);
+    if (g_recording.load(std::memory_order_acquire)) return -1;
+    if (!g_record_stream) {
+        // a blocking stream of default priority: it keeps the implicit ordering with the null stream
+        int rc = jz::rc_of(hipStreamCreateWithFlags(&g_record_stream, hipStreamDefault));
+        if (rc) return rc;
+    }
+    g_stream_before = jz::stream();
+    int rc = jz::rc_of(hipStreamSynchronize(g_stream_before));
+    if (rc) return rc;
+    jz::g_stream.store(g_record_stream, std::memory_order_relaxed);
+    // the recording stream's workspace must exist before recording starts
+    if (!jz::workspace()) {
+        jz::g_stream.store(g_stream_before, std::memory_order_relaxed);
+        return -2;
+    }
+    rc = jz::rc_of(hipStreamBeginCapture(g_record_stream, hipStreamCaptureModeRelaxed));
+    if (rc) {
+        jz::g_stream.store(g_stream_before, std::memory_order_relaxed);
+        return rc;
+    }
+    g_recording.store(1, std::memory_order_release);
+    return 0;
+}
+
+JZ_API int jzhip_graph_end(void** out_graph) {
+    std::lock_guard<std::mutex> lock(g_graph_mutex);
+    if (!g_recording.load(std::memory_order_acquire)) return -1;
+    hipGraph_t graph = nullptr;
+    int rc = jz::rc_of(hipStreamEndCapture(g_record_stream, &graph));
+    g_recording.store(0, std::memory_order_release);
+    jz::g_stream.store(g_stream_before, std::memory_order_relaxed);
+    if (rc) return rc;
+    if (!out_graph) {
+        (void)hipGraphDestroy(graph);
+        return -1;
+    }
+    hipGraphExec_t exec = nullptr;
+    rc = jz::rc_of(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    (void)hipGraphDestroy(graph);
+    if (rc) return rc;
+    *out_graph = exec;
+    return 0;
+}
+
+JZ_API int jzhip_graph_recording(void) { return g_recording.load(std::memory_order_acquire); }
+
+JZ_API int jzhip_graph_launch(void* graph) {
+    if (!graph || g_recording.load(std::memory_order_acquire)) return -1;
+    // on the current stream, the null stream included
+    return jz::rc_of(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), jz::stream()));
+}
+
+JZ_API int jzhip_graph_destroy(void* graph) {
+    if (!graph) return 0;
+    if (g_record_stream) (void)hipStreamSynchronize(g_record_stream);
+    return jz::rc_of(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+}
+
 JZ_API int jzhip_set_stream(void* hip_stream) {
+    if (g_recording.load(std::memory_order_acquire)) return -1;   // the recording owns the current stream
     jz::g_stream.store(static_cast<hipStream_t>(hip_stream), std::memory_order_relaxed);
     return 0;
 }

@@ -10,6 +10,8 @@
 // Selected through the environment (the library owns main(), cpp/launcher.cu):
 //   JZ_CONFIG = c1 | c2 | c3 | c5  JZ_STEPS = training steps     JZ_OUT = dump dir
 //   JZ_SCALE  = full | small      (small shrinks batch/width for quick runs)
+//   JZ_GRAPH  = 1                 (ROCm build, c2 and c3: record the step once, replay it as a HIP graph)
+//   JZ_STREAM = 1                 (ROCm build: run on a created stream instead of the null stream)
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -144,6 +146,37 @@ int run_c2(const std::string& out, bool small, int steps) {
     std::vector<Matrix<D>> loss_dev;
     loss_dev.reserve(steps);
     double t0 = 0;
+#ifdef ROCM_HIP
+    if (env("JZ_GRAPH", "0") == "1") {
+        // three ordinary steps (they also fill the pool with every buffer size), then the step
+        // is recorded once and replayed: one graph launch per step instead of ~60 kernel launches
+        RocmStepGraph graph;
+        LossLayer<D> loss(nb, Y);
+        Matrix<D> loss_now("loss_now", 1, 1);   // backprop overwrites the loss layer's value
+        const bool every = env("JZ_GRAPH_LOSSES", "1") == "1";
+        auto one_step = [&] {
+            forward(net, X);
+            loss.eval(L2.value());
+            copy(loss_now, loss.value());
+            net.push_front(&loss);
+            backprop(net, X);
+            net.pop_front();
+        };
+        for (int it = 0; it < steps; ++it) {
+            if (it == 3) {
+                sync_device(loss_dev);
+                graph.begin();
+                one_step();
+                graph.end();
+                t0 = now_ms();
+            }
+            if (it < 3) one_step(); else graph.replay();
+            // a copy on the device, ordered after the replay (JZ_GRAPH_LOSSES=0: only the last one)
+            if (every || it == steps - 1) loss_dev.push_back(loss_now);
+            else loss_dev.push_back(Matrix<D>("skipped", 1, 1));
+        }
+    } else
+#endif
     for (int it = 0; it < steps; ++it) {
         if (it == 3) { sync_device(loss_dev); t0 = now_ms(); }
         forward(net, X);
@@ -191,6 +224,30 @@ int run_c3(const std::string& out, bool small, int steps) {
     std::vector<Matrix<D>> loss_dev;
     loss_dev.reserve(steps);
     double t0 = 0;
+#ifdef ROCM_HIP
+    if (env("JZ_GRAPH", "0") == "1") {
+        RocmStepGraph graph;
+        LogisticLayer<D> loss(nb, Y);
+        auto one_step = [&] {
+            forward(net, X);
+            loss.eval(fc.value());
+            net.push_front(&loss);
+            backprop(net, X);
+            net.pop_front();
+        };
+        for (int it = 0; it < steps; ++it) {
+            if (it == 2) {
+                sync_device(loss_dev);
+                graph.begin();
+                one_step();
+                graph.end();
+                t0 = now_ms();
+            }
+            if (it < 2) one_step(); else graph.replay();
+            loss_dev.push_back(loss.value());
+        }
+    } else
+#endif
     for (int it = 0; it < steps; ++it) {
         if (it == 2) { sync_device(loss_dev); t0 = now_ms(); }
         forward(net, X);
@@ -365,6 +422,12 @@ int compute() {
     const bool small = env("JZ_SCALE", "full") == "small";
     const int steps = std::atoi(env("JZ_STEPS", "100").c_str());
     std::printf("RESULT backend %s\n", kBackend);
+#ifdef ROCM_HIP
+    if (env("JZ_STREAM", "0") == "1") {   // everything on a stream of its own instead of the null stream
+        void* s = nullptr;
+        if (jzhip_stream_create(&s) != 0 || jzhip_set_stream(s) != 0) return 1;
+    }
+#endif
     if (cfg == "c1") return run_c1(out, small);
     if (cfg == "c2") return run_c2(out, small, steps);
     if (cfg == "c3") return run_c3(out, small, steps);

@@ -113,3 +113,34 @@ def test_c5_rectified_flow_unet_training(gpu, tmp_path, scale, steps):
     assert worst <= 1e-3
     for name in ("c5_head_W", "c5_e1a_W", "c5_up2_W"):
         assert rel(load(tmp_path, name, "rocm"), load(tmp_path, name, "cpu")) <= 2e-3
+
+
+@pytest.mark.parametrize("config,names", [("c2", ("c2_losses", "c2_W0", "c2_W2")),
+                                          ("c3", ("c3_losses", "c3_conv1_W", "c3_fc_b"))])
+@pytest.mark.parametrize("scale", ["small", "full"])
+def test_recorded_step_replays_like_the_eager_step(gpu, tmp_path, config, names, scale):
+    """RocmStepGraph: the MLP / CNN step recorded once and replayed as a HIP graph, with an
+    eager device copy of the loss between the replays.  Every replay's loss and the final
+    parameters must equal those of the ordinary step-by-step run (the optimiser's step number
+    comes from a device counter in the recorded form; its bias corrections are formed on the
+    device in double as on the host, hence the 1e-6)."""
+    exe = need_ref_binary(BIN / "configs_rocm")
+    steps = 24
+    outs = {}
+    for mode in ("0", "1"):
+        d = tmp_path / f"graph{mode}"
+        d.mkdir()
+        env = dict(os.environ, JZ_CONFIG=config, JZ_SCALE=scale, JZ_STEPS=str(steps), JZ_OUT=str(d), JZ_GRAPH=mode)
+        print(f"running configs_rocm {config} {scale} JZ_GRAPH={mode}", flush=True)
+        r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=600, env=env)
+        assert r.returncode == 0, (r.stdout + r.stderr)[-3000:]
+        outs[mode] = d
+    for name in names:
+        eager, graph = load(outs["0"], name, "rocm"), load(outs["1"], name, "rocm")
+        assert eager.shape == graph.shape and eager.size > 0
+        assert np.all(np.isfinite(graph))
+        err = float(np.max(np.abs(graph - eager)) / max(float(np.max(np.abs(eager))), 1e-30))
+        print(name, scale, f"{err:.1e}")
+        assert err <= 1e-6, (name, err)
+    losses = load(outs["1"], names[0], "rocm")
+    assert losses.size == steps and losses[-1] < losses[0]
