@@ -490,6 +490,37 @@ def test_gemv(gpu, oracle_lib, m, n, trans):
     assert rel_err(to_host(dy), ref) <= TOL_GEMM
 
 
+@pytest.mark.parametrize("m,n,trans,incx,incy", [
+    (2048, 300, 1, 1, 1),      # long columns, A^T x: four columns per workgroup, rows split over its waves
+    (2052, 7, 1, 1, 3),        # the same with a ragged last float4 step and a strided y
+    (4096, 512, 0, 1, 1),      # A x through the thin-product kernel with one vector
+    (4096, 512, 0, 2, 2),      # strided x and y on that path
+    (256, 4096, 1, 1, 1),      # short columns, A^T x: the thin dot form, four columns per wavefront
+    (512, 1030, 1, 3, 1),      # strided x on the dot form
+    (1024, 1, 1, 1, 1), (1, 1024, 0, 1, 1),
+])
+def test_gemv_float4_forms(gpu, oracle_lib, m, n, trans, incx, incy):
+    """Shapes with lda % 4 == 0 and aligned operands, which take the vector kernels (the
+    cases of test_gemv have lda = m + 2 and stay on the scalar ones)."""
+    r = rng(m + 3 * n + trans)
+    lda = m
+    A = r.normal(0, 1, lda * n).astype(np.float32)
+    lx, ly = (m, n) if trans else (n, m)
+    x = r.normal(0, 1, lx * incx).astype(np.float32)
+    y0 = r.normal(0, 1, ly * incy).astype(np.float32)
+    for alpha, beta in ((0.5, 2.0), (1.0, 0.0)):
+        ref = y0.copy()
+        oracle_lib.jzo_gemv(trans, m, n, alpha, hptr(A), lda, hptr(x), incx, beta, hptr(ref), incy)
+        dy = to_dev(y0)
+        gpu.gemv(dp(A), dp(x), dptr(dy), m, n, trans, lda, incx, incy, alpha, beta)
+        got = to_host(dy)
+        assert rel_err(got, ref) <= TOL_GEMM
+        if incy > 1:   # the gaps of a strided y are untouched
+            mask = np.ones(ly * incy, bool)
+            mask[::incy] = False
+            assert np.array_equal(got[mask], y0[mask])
+
+
 @pytest.mark.parametrize("ta,tb", [(1, 0), (0, 1), (0, 0)])
 def test_gemm_strided_batched(gpu, oracle_lib, ta, tb):
     """Attention-shaped batches: per (head, sequence) S x S scores from d_h x S slices."""
