@@ -126,12 +126,53 @@ __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
     }
 }
 
+// No operand is transposed relative to the output (a row block of a vstack, a slice, an
+// addition of two sub-blocks): nothing has to be turned, so a wavefront takes 256
+// consecutive rows of one column (1 KB runs on every operand instead of the 256 B runs of
+// the 64 x 64 tile) and a workgroup 256 rows x 16 columns.
+constexpr int kStripRows = 256, kStripCols = 16;
+template <int OP>
+__global__ __launch_bounds__(kBlock) void ew2d_strip_kernel(float* out, size_t ldo, const float* a, size_t lda,
+                                                            const float* b, size_t ldb, size_t R, size_t C,
+                                                            unsigned strips_r, float s1, float s2) {
+    const unsigned sr = blockIdx.x % strips_r, sc = blockIdx.x / strips_r;
+    const size_t r = static_cast<size_t>(sr) * kStripRows + 4 * (threadIdx.x % kWave);
+    if (r >= R) return;
+    const size_t c0 = static_cast<size_t>(sc) * kStripCols + threadIdx.x / kWave;
+#pragma unroll
+    for (int k = 0; k < kStripCols; k += kBlock / kWave) {
+        const size_t c = c0 + k;
+        if (c < C) {
+            const float4 va = *reinterpret_cast<const float4*>(a + c * lda + r);
+            float4 res = va;
+            if constexpr (OP != kOpCopy) {
+                const float4 vb = *reinterpret_cast<const float4*>(b + c * ldb + r);
+                if constexpr (OP == kOpAxpby) {
+                    res.x = s1 * va.x + s2 * vb.x; res.y = s1 * va.y + s2 * vb.y;
+                    res.z = s1 * va.z + s2 * vb.z; res.w = s1 * va.w + s2 * vb.w;
+                } else {
+                    res.x = va.x * vb.x; res.y = va.y * vb.y; res.z = va.z * vb.z; res.w = va.w * vb.w;
+                }
+            }
+            *reinterpret_cast<float4*>(out + c * ldo + r) = res;
+        }
+    }
+}
+
 template <int OP>
 int launch2d(float* out, size_t ldo, const float* a, size_t lda, int rel_a, const float* b,
              size_t ldb, int rel_b, size_t R, size_t C, float s1, float s2) {
     if (R == 0 || C == 0) return 0;
     const bool vec = R % 4 == 0 && C % 4 == 0 && ldo % 4 == 0 && lda % 4 == 0 && aligned16(out) && aligned16(a) &&
                      (OP == kOpCopy || (ldb % 4 == 0 && aligned16(b)));
+    if (vec && !rel_a && (OP == kOpCopy || !rel_b) && R >= 128) {
+        const size_t sr = (R + kStripRows - 1) / kStripRows, sc = (C + kStripCols - 1) / kStripCols;
+        if (sr * sc <= 0x7fffffffull) {
+            ew2d_strip_kernel<OP><<<static_cast<unsigned>(sr * sc), kBlock, 0, stream()>>>(
+                out, ldo, a, lda, b, ldb, R, C, static_cast<unsigned>(sr), s1, s2);
+            return launch_rc();
+        }
+    }
     if (vec) {
         const size_t tr = (R + kTileV - 1) / kTileV, tc = (C + kTileV - 1) / kTileV;
         if (tr * tc > 0x7fffffffull) return -1;
