@@ -254,18 +254,21 @@ __device__ __forceinline__ bool rowgrid_item(const RowGrid& rg, int& x, int& y, 
     return true;
 }
 
-// One workgroup = one row ph of the patch grid, one sample n, one chunk of 256
-// consecutive k.  The image rows that chunk touches (its channels x kH rows,
-// zero-filled where the window hangs over the border) are staged in LDS; then
-// every wave writes whole 1 KB pieces of patch columns: lane l owns k = k0+4l..k0+4l+3
-// for all pw, so its four LDS offsets are computed once.
+// One workgroup = a band of `band` rows of the patch grid, one sample n, one chunk of 256
+// consecutive k.  The image rows that chunk touches over the band (its channels x
+// (band-1)*stride + kH rows, zero-filled where the window hangs over the border) are
+// staged in LDS once; then every wave writes whole 1 KB pieces of patch columns: lane l
+// owns k = k0+4l..k0+4l+3 for all positions, so its four LDS offsets are computed once.
+// (With one patch row per workgroup every image row was staged kH times over: 203 MB
+// fetched for a 67 MB input at 3x3; a band of four rows stages it 1.5 times: 145 -> 140 us
+// for the 671 MB of patches of 128 x 128 x 32 x 32, which the write side bounds.)
 template <int NSUB>
 __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __restrict__ img,
                                                              float* __restrict__ col, PatchGeom g,
-                                                             int WT, FastDiv dWT, FastDiv dkH) {
-    extern __shared__ float tile[];   // [channels of the chunk][kH][WT]
+                                                             int WT, FastDiv dWT, int band, int nr, FastDiv dnr) {
+    extern __shared__ float tile[];   // [channels of the chunk][nr][WT]
     const int KK = g.kH * g.kW;
-    // (plain dispatch order, chunks of one patch row spread over the XCDs: the
+    // (plain dispatch order, chunks of one band spread over the XCDs: the
     // kernel is write-dominated and this order measured faster than the
     // XCD-grouped one the scatter kernel uses)
     // one 256-wide piece per workgroup; with NSUB = 2 the last workgroup also takes
@@ -273,11 +276,11 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
     const int k0 = blockIdx.x * kPatchChunk;
     const int k1 = (NSUB == 2 && blockIdx.x == gridDim.x - 1) ? g.K
                                                                 : ((k0 + kPatchChunk) < g.K ? (k0 + kPatchChunk) : g.K);
-    const int ph = blockIdx.y, n = blockIdx.z;
+    const int ph0 = blockIdx.y * band, n = blockIdx.z;
     const int c_lo = fdiv(static_cast<uint32_t>(k0), g.dKK);
     const int c_hi = fdiv(static_cast<uint32_t>(k1 - 1), g.dKK);
-    const int rows = (c_hi - c_lo + 1) * g.kH;
-    const int h0 = ph * g.stride_h - g.pad_h;
+    const int rows = (c_hi - c_lo + 1) * nr;
+    const int h0 = ph0 * g.stride_h - g.pad_h;
     const float* src = img + static_cast<size_t>(n) * (g.C * g.H * g.W) + static_cast<size_t>(c_lo) * g.H * g.W;
     // (eight independent loads in flight per thread, then their LDS stores)
     constexpr int kBatch = 8;
@@ -290,9 +293,9 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
             if (idx < rows * WT) {
                 const uint32_t r = fdiv(static_cast<uint32_t>(idx), dWT);
                 const int w = idx - static_cast<int>(r) * WT;
-                const uint32_t chl = fdiv(r, dkH);
-                const int kh = static_cast<int>(r - chl * g.kH);
-                const int ih = h0 + kh, iw = w - g.pad_w;
+                const uint32_t chl = fdiv(r, dnr);
+                const int rr = static_cast<int>(r - chl * nr);
+                const int ih = h0 + rr, iw = w - g.pad_w;
                 if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
                     v[b] = src[(static_cast<size_t>(chl) * g.H + ih) * g.W + iw];
             }
@@ -319,14 +322,19 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
                 const uint32_t rem = k - ch * KK;
                 const uint32_t kh = fdiv(rem, g.dkW);
                 const uint32_t kw = rem - kh * g.kW;
-                off[u][j] = static_cast<int>(((ch - c_lo) * g.kH + kh) * WT + kw);
+                off[u][j] = static_cast<int>(((ch - c_lo) * nr + kh) * WT + kw);
             }
         }
     }
-    float* dst = col + (static_cast<size_t>(n) * g.P + static_cast<size_t>(ph) * g.Wp) * g.K + k0 + 4 * lane;
-    for (int pw = wave; pw < g.Wp; pw += kBlock / kWave) {
-        const int w = pw * g.stride_w;
-        float* d = dst + static_cast<size_t>(pw) * g.K;
+    // the band's positions (row p of the band, column pw) dealt to the waves in turn
+    const int band_rows = (ph0 + band) <= g.Hp ? band : g.Hp - ph0;
+    float* dst = col + (static_cast<size_t>(n) * g.P + static_cast<size_t>(ph0) * g.Wp) * g.K + k0 + 4 * lane;
+    const int positions = band_rows * g.Wp;
+    int p = 0, pw = wave;
+    while (pw >= g.Wp) { pw -= g.Wp; ++p; }
+    for (int pos = wave; pos < positions; pos += kBlock / kWave) {
+        const int w = p * g.stride_h * WT + pw * g.stride_w;
+        float* d = dst + static_cast<size_t>(pos) * g.K;
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             if (off[u][0] >= 0) {
@@ -335,6 +343,8 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
                 *reinterpret_cast<float4*>(d + u * kPatchChunk) = v;
             }
         }
+        pw += kBlock / kWave;
+        while (pw >= g.Wp) { pw -= g.Wp; ++p; }
     }
 }
 
@@ -490,12 +500,24 @@ int gather_patches(const float* img, float* col, const PatchGeom& g) {
         const int pieces = (g.K + kPatchChunk - 1) / kPatchChunk;
         const bool fold = pieces >= 2 && g.K - (pieces - 1) * kPatchChunk <= kPatchChunk / 4;
         const int nch_max = (fold ? kPatchChunk + kPatchChunk / 4 : kPatchChunk) / (g.kH * g.kW) + 2;
-        const size_t lds = static_cast<size_t>(nch_max) * g.kH * WT * sizeof(float);
+        // rows of the patch grid per workgroup: as many (up to four) as keep the staged rows
+        // under 48 KB and leave 16 workgroups per CU to hide the staging phase (with fewer the
+        // saved re-reads cost more in idle time: 30 us against 24 us at 128 x 64 x 32 x 32, stride 2)
+        int band = 4;
+        auto staged_rows = [&](int bd) { return (bd - 1) * g.stride_h + g.kH; };
+        auto lds_bytes = [&](int bd) { return static_cast<size_t>(nch_max) * staged_rows(bd) * WT * sizeof(float); };
+        auto groups = [&](int bd) {
+            return static_cast<size_t>(fold ? pieces - 1 : pieces) * ((g.Hp + bd - 1) / bd) * g.N;
+        };
+        while (band > 1 && (lds_bytes(band) > 48 * 1024 || band > g.Hp || groups(band) < 4096)) band /= 2;
+        const size_t lds = lds_bytes(band);
+        const int bands = (g.Hp + band - 1) / band;
         if (lds <= 48 * 1024) {
-            dim3 grid(fold ? pieces - 1 : pieces, g.Hp, g.N);
-            const FastDiv dWT = make_fastdiv(WT), dkH = make_fastdiv(g.kH);
-            if (fold) im2col_rows_kernel<2><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, dkH);
-            else im2col_rows_kernel<1><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, dkH);
+            dim3 grid(fold ? pieces - 1 : pieces, bands, g.N);
+            const int nr = staged_rows(band);
+            const FastDiv dWT = make_fastdiv(WT), dnr = make_fastdiv(nr);
+            if (fold) im2col_rows_kernel<2><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
+            else im2col_rows_kernel<1><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
             return launch_rc();
         }
     }
