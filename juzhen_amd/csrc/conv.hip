@@ -482,6 +482,181 @@ __global__ __launch_bounds__(kBlock) void col2im_rows_kernel(const float* __rest
     }
 }
 
+// The streamed form of the kernel above for the fixed-geometry cases: one workgroup = CC
+// channels of one sample over `seg` image rows, walking down the patch rows that feed them.
+// A ring of TH + 1 patch rows lives in LDS (TH = the patch rows one image row collects
+// from).  The first four waves only load: kStreamDepth patch rows are in flight in their
+// registers and the oldest enters the ring slot nothing reads; the other four waves sum and
+// write the image rows that the newest staged patch row completes.  One barrier per patch
+// row joins the two.  (Loads and image stores in one instruction stream share the memory
+// counter, and with stores of unknown count between a load and its use the compiler waits
+// for everything outstanding: the prefetch then hides nothing.)  Every patch row is fetched
+// once per segment, in runs of CC*KH*KW floats; the strip form fetches kH - 1 halo rows for
+// every R image rows, 1.5 times the patch matrix at 3x3 with R = 4.
+constexpr int kStreamLoads = 4;   // float4 loads per loading thread per patch row
+constexpr int kStreamDepth = 2;   // patch rows in flight ahead of the ring
+constexpr int kStreamBlock = 2 * kBlock;
+constexpr int kStreamOutputs = 4; // (channel, column) pairs per summing thread
+template <int S, int KH, int KW>
+__global__ __launch_bounds__(kStreamBlock, 8) void col2im_stream_kernel(const float* __restrict__ col,
+                                                                        float* __restrict__ img,
+                                                                        const float* __restrict__ bias,
+                                                                        PatchGeom g, int CC, int seg, int pitch,
+                                                                        FastDiv dL4, RowGrid rg) {
+    static_assert(KH >= S && KW >= S, "every image row must be reached by some patch row");
+    constexpr int TH = (KH + S - 1) / S, TW = (KW + S - 1) / S, RING = TH + 1, KK = KH * KW;
+    extern __shared__ float tile[];   // [RING][Wp][pitch], then the bias of the CC channels
+    int bx, by, n;
+    if (!rowgrid_item(rg, bx, by, n)) return;
+    const int c0 = bx * CC;
+    const int r0 = by * seg;
+    const int r1 = (r0 + seg < g.H ? r0 + seg : g.H) - 1;   // last image row of the segment
+    // patch rows with ph*S - pad + kh inside [r0, r1]
+    int lo = r0 + g.pad_h - (KH - 1);
+    lo = lo <= 0 ? 0 : (lo + S - 1) / S;
+    int hi = (r1 + g.pad_h) / S;
+    if (hi > g.Hp - 1) hi = g.Hp - 1;
+    const int slot = g.Wp * pitch;
+    float* bias_l = tile + RING * slot;
+
+    if (threadIdx.x < kBlock) {
+        // ── loading waves ──
+        const int L4 = CC * KK / 4;          // float4 per patch column of this chunk
+        const int count = g.Wp * L4;         // float4 per patch row (<= kStreamLoads * kBlock)
+        const float* base = col + static_cast<size_t>(n) * g.P * g.K + static_cast<size_t>(c0) * KK;
+        const size_t row_step = static_cast<size_t>(g.Wp) * g.K;
+        // Every thread issues all its loads on every patch row (those past the end of the
+        // row re-read its first float4), so no branch depends on the lane.
+        int src[kStreamLoads], dst[kStreamLoads];
+#pragma unroll
+        for (int b = 0; b < kStreamLoads; ++b) {
+            const int idx = threadIdx.x + b * kBlock;
+            src[b] = 0;
+            dst[b] = -1;
+            if (idx < count) {
+                const int cidx = static_cast<int>(fdiv(static_cast<uint32_t>(idx), dL4));
+                const int kk = (idx - cidx * L4) * 4;
+                src[b] = cidx * g.K + kk;     // < K*P*N < 2^31
+                dst[b] = cidx * pitch + kk;
+            }
+        }
+        if (hi < lo) {
+            __syncthreads();
+            return;
+        }
+        float4 v[kStreamDepth][kStreamLoads];
+        auto fetch = [&](int ph, float4 (&r)[kStreamLoads]) {
+            const float* rowp = base + static_cast<size_t>(ph) * row_step;
+#pragma unroll
+            for (int b = 0; b < kStreamLoads; ++b) r[b] = *reinterpret_cast<const float4*>(rowp + src[b]);
+        };
+        auto stash = [&](int ph, const float4 (&r)[kStreamLoads]) {
+            float* sl = tile + (ph % RING) * slot;
+#pragma unroll
+            for (int b = 0; b < kStreamLoads; ++b)
+                if (dst[b] >= 0) {
+                    float* d = sl + dst[b];
+                    d[0] = r[b].x; d[1] = r[b].y; d[2] = r[b].z; d[3] = r[b].w;
+                }
+        };
+        // Register set u holds patch row lo + u (+ a multiple of the depth); a set is refilled
+        // as soon as its row is in the ring.  Rows past the last one are clamped to it and the
+        // loop body has no branch around a load, so the compiler knows how many younger loads
+        // are outstanding when a set enters the ring and waits for that set only.  (The
+        // clamped rows land in slots nothing reads any more.)
+        auto clamped = [&](int ph) { return ph < hi ? ph : hi; };
+#pragma unroll
+        for (int u = 0; u < kStreamDepth; ++u) fetch(clamped(lo + u), v[u]);
+        stash(lo, v[0]);
+        fetch(clamped(lo + kStreamDepth), v[0]);
+        __syncthreads();
+        for (int ph0 = lo; ph0 <= hi; ph0 += kStreamDepth) {
+#pragma unroll
+            for (int u = 0; u < kStreamDepth; ++u) {
+                const int ph = ph0 + u;   // the row the other waves are working from
+                stash(ph + 1, v[(u + 1) % kStreamDepth]);
+                fetch(clamped(ph + 1 + kStreamDepth), v[(u + 1) % kStreamDepth]);
+                if (ph <= hi) __syncthreads();
+            }
+        }
+        return;
+    }
+
+    // ── summing waves ──
+    // A thread owns up to kStreamOutputs (channel, column) pairs for the whole walk: what
+    // depends on them (bias, which kw reach the column, LDS and image offsets) is worked out
+    // once, and a step is the taps' LDS reads, the adds in the CPU's order (kh, kw descending)
+    // and one store per pair; what depends on the image row is the same for the whole wave.
+    const int tid = threadIdx.x - kBlock;
+    if (tid < CC) bias_l[tid] = bias ? bias[c0 + tid] : 0.0f;
+    const int per_row = CC * g.W;     // <= kStreamOutputs * kBlock
+    int woff[kStreamOutputs], ioff[kStreamOutputs];
+    unsigned taps[kStreamOutputs];    // bit b: tap kw1 - b*S exists and its patch column is inside
+    float init[kStreamOutputs];
+#pragma unroll
+    for (int j = 0; j < kStreamOutputs; ++j) {
+        const int idx = tid + j * kBlock;
+        woff[j] = 0; ioff[j] = -1; taps[j] = 0; init[j] = 0.0f;
+        if (idx < per_row) {
+            const int cl = static_cast<int>(fdiv(static_cast<uint32_t>(idx), g.dW));
+            const int iw = idx - cl * g.W;
+            const int wq = iw + g.pad_w;
+            const int kw1 = (KW - 1) - ((KW - 1 - wq % S) + S) % S;   // largest kw that reaches this column
+            const int pw1 = (wq - kw1) / S;                           // exact
+#pragma unroll
+            for (int b = 0; b < TW; ++b) {
+                const int kw = kw1 - b * S, pw = pw1 + b;
+                if (kw >= 0 && pw >= 0 && pw < g.Wp) taps[j] |= 1u << b;
+            }
+            woff[j] = cl * KK + kw1 + pw1 * pitch;
+            ioff[j] = (c0 + cl) * g.H * g.W + iw;   // < C*H*W*N < 2^31
+        }
+    }
+    __syncthreads();   // first patch row and the bias are in LDS
+#pragma unroll
+    for (int j = 0; j < kStreamOutputs; ++j)
+        if (ioff[j] >= 0) init[j] = bias_l[(ioff[j] / (g.H * g.W)) - c0];
+    float* out = img + static_cast<size_t>(n) * (g.C * g.H * g.W);
+    // image rows e0..e1, every patch row they collect from staged (or none existing)
+    auto emit = [&](int e0, int e1) {
+        for (int ih = e0; ih <= e1; ++ih) {
+            const int hq = ih + g.pad_h;
+            const int kh1 = (KH - 1) - ((KH - 1 - hq % S) + S) % S;   // largest kh that reaches this row; may be negative
+            const int ph1 = (hq - kh1) / S;                           // exact
+#pragma unroll
+            for (int j = 0; j < kStreamOutputs; ++j) {
+                if (j * kBlock < per_row) {
+                    float val = init[j];
+#pragma unroll
+                    for (int a = 0; a < TH; ++a) {
+                        const int kh = kh1 - a * S, ph = ph1 + a;
+                        if (kh >= 0 && ph >= 0 && ph < g.Hp) {
+                            const float* row = tile + (ph % RING) * slot + kh * KW + woff[j];
+#pragma unroll
+                            for (int b = 0; b < TW; ++b)
+                                if (taps[j] >> b & 1u) val += row[b * (pitch - S)];
+                        }
+                    }
+                    if (ioff[j] >= 0) out[ioff[j] + ih * g.W] = val;
+                }
+            }
+        }
+    };
+    if (hi < lo) {     // no patch row reaches this segment
+        emit(r0, r1);
+        return;
+    }
+    for (int ph = lo; ph <= hi; ++ph) {
+        // the image rows whose last patch row is ph
+        int e0 = ph * S - g.pad_h;
+        int e1 = ph == hi ? r1 : e0 + S - 1;
+        if (e0 < r0) e0 = r0;
+        if (e1 > r1) e1 = r1;
+        emit(e0, e1);
+        __syncthreads();
+    }
+}
+
 bool geom_ok(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int stride_h, int stride_w,
              int Hp, int Wp, int N) {
     return C > 0 && H > 0 && W > 0 && kH > 0 && kW > 0 && pad_h >= 0 && pad_w >= 0 && stride_h > 0 &&
@@ -534,6 +709,42 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
     const size_t total = static_cast<size_t>(g.C) * g.H * g.W * g.N;
     if (total >= (size_t(1) << 31)) return -1;
     if (static_cast<size_t>(g.K) * g.P * g.N >= (size_t(1) << 31)) return -1;
+    // streamed form: fixed geometry, float4 runs, one patch row of the chunk within
+    // kStreamLoads loads per thread and the ring within 40 KB (four workgroups per CU)
+    {
+        const int KK = g.kH * g.kW;
+        const int S = g.stride_h == g.stride_w ? g.stride_h : 0;
+        const int form = (S == 1 && g.kH == 3 && g.kW == 3) ? 1 : (S == 2 && g.kH == 3 && g.kW == 3) ? 2
+                       : (S == 2 && g.kH == 4 && g.kW == 4) ? 3 : (S == 1 && g.kH == 5 && g.kW == 5) ? 4 : 0;
+        const int ring = form ? (g.kH + S - 1) / S + 1 : 0;
+        auto fits = [&](int cc) {
+            return g.C % cc == 0 && (cc * KK) % 4 == 0 && g.Wp * (cc * KK / 4) <= kStreamLoads * kBlock &&
+                   cc * g.W <= kStreamOutputs * kBlock &&
+                   static_cast<size_t>(ring) * g.Wp * ((cc * KK) | 1) * sizeof(float) <= 40 * 1024;
+        };
+        int CC = 16;
+        while (CC > 1 && !fits(CC)) CC /= 2;
+        if (form && fits(CC) && g.K % 4 == 0 && aligned16(col)) {
+            // whole images per workgroup unless that leaves fewer than 2048 workgroups:
+            // then segments of rows, each paying kH - 1 halo patch rows
+            int seg = g.H;
+            auto groups = [&](int sg) { return static_cast<size_t>(g.C / CC) * ((g.H + sg - 1) / sg) * g.N; };
+            while (seg > 8 && groups(seg) < 2048) seg = (seg + 1) / 2;
+            const RowGrid rg = make_rowgrid(g.C / CC, (g.H + seg - 1) / seg, g.N);
+            const int pitch = (CC * KK) | 1;
+            const size_t lds = (static_cast<size_t>(ring) * g.Wp * pitch + CC) * sizeof(float);
+            const FastDiv dL4 = make_fastdiv(CC * KK / 4);
+#define JZ_COL2IM_STREAM(S_, KH_, KW_)                                                                       \
+    col2im_stream_kernel<S_, KH_, KW_><<<rg.blocks(), kStreamBlock, lds, stream()>>>(col, img, bias, g, CC, seg,  \
+                                                                               pitch, dL4, rg)
+            if (form == 1) JZ_COL2IM_STREAM(1, 3, 3);
+            else if (form == 2) JZ_COL2IM_STREAM(2, 3, 3);
+            else if (form == 3) JZ_COL2IM_STREAM(2, 4, 4);
+            else JZ_COL2IM_STREAM(1, 5, 5);
+#undef JZ_COL2IM_STREAM
+            return launch_rc();
+        }
+    }
     if (g.W <= 1024) {
         // channels and image rows per workgroup: as many as keep the staged strip
         // under 40 KB (four workgroups per CU), preferring a channel-chunk count

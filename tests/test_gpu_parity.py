@@ -804,6 +804,13 @@ CONV_CASES = [
     (2, 20, 9, 10, 5, 5, 2, 2),
     (1, 16, 8, 8, 2, 2, 0, 1),
     (2, 256, 8, 8, 3, 3, 1, 1),
+    # the streamed scatter: no padding, more padding than the kernel needs, 5x5, 4x4 stride 2, ragged row segments
+    (2, 8, 9, 7, 3, 3, 0, 1),
+    (2, 4, 6, 6, 3, 3, 2, 1),
+    (2, 8, 12, 12, 5, 5, 2, 1),
+    (2, 4, 10, 10, 4, 4, 0, 2),
+    (2, 8, 11, 11, 3, 3, 0, 2),
+    (1, 16, 37, 20, 3, 3, 1, 1),
 ]
 
 
