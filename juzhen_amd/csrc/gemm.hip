@@ -232,13 +232,24 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kerne
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const int cbase = n0 + (wn * TN + j) * 32 + 4 * h;
+                // with beta != 0 the sixteen old values of the tile are requested together
+                // (one load, one wait and one store per element made every element a round trip)
+                float old[16];
+                if (beta != 0.0f) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int col = cbase + 8 * (v / 4) + (v % 4);
+                        old[v] = 0.0f;
+                        if (FAST || (row < M && col < N)) old[v] = C[static_cast<size_t>(col) * ldc + row];
+                    }
+                }
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int col = cbase + 8 * (v / 4) + (v % 4);
                     if (FAST || (row < M && col < N)) {
                         float* dst = C + static_cast<size_t>(col) * ldc + row;
                         float r = alpha * acc[i][j][v];
-                        if (beta != 0.0f) r += beta * *dst;
+                        if (beta != 0.0f) r += beta * old[v];
                         *dst = r;
                     }
                 }
