@@ -190,6 +190,14 @@ int jzhip_clamp(float* out, const float* in, size_t count, float lo, float hi);
 /* out = d_relu(pre) * up in one pass: the product every backward() forms as
  * hadmd(d_relu(Matrix(val)), upstream) (ml/layer.hpp:100,1672-1674,3189). */
 int jzhip_drelu_mul(float* out, const float* pre, const float* up, size_t count);
+/* The squared-error head (LossLayer, ml/layer.hpp:204-227) in one launch each:
+ * out_device[0] = scale * sum((target - pred)^2) over `count` elements, which eval()
+ * forms as sum(sum(square(output - input), 0), 1) / nb, and
+ * out = ((pred - target) * 2) * inv_nb, which grad() forms as 2.0 * (input - output) / nb
+ * (every step rounded as the separate operations round; out may equal pred). Flat
+ * buffers: both operands stored the same way. */
+int jzhip_mse_loss(float* out_device, const float* target, const float* pred, size_t count, float scale);
+int jzhip_mse_grad(float* out, const float* pred, const float* target, size_t count, float inv_nb);
 /* GELU (exact erf form) and its derivative times an upstream gradient. No
  * reference counterpart (the reference FFN is ReLU, ml/layer.hpp:3018); used
  * by the character-LM configuration. */

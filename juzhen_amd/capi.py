@@ -84,6 +84,8 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_sqrt": (I, [P, P, Z]),
     "jzhip_clamp": (I, [P, P, Z, F, F]),
     "jzhip_drelu_mul": (I, [P, P, P, Z]),
+    "jzhip_mse_loss": (I, [P, P, P, Z, F]),
+    "jzhip_mse_grad": (I, [P, P, P, Z, F]),
     "jzhip_gelu": (I, [P, P, Z]),
     "jzhip_dgelu_mul": (I, [P, P, P, Z]),
     "jzhip_axpby2d": (I, [P, I, I, P, I, I, P, I, I, I, I, F, F]),

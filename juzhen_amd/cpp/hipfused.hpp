@@ -257,6 +257,39 @@ inline Matrix<ROCMfloat> Layer<ROCMfloat>::backward(const Matrix<ROCMfloat>& inp
     return W().T() * t;
 }
 
+// ── squared-error head (ml/layer.hpp:204-227) ────────────────────────────────
+// eval() is five matrix operations and seven launches in the generic form, grad() three;
+// with both operands stored the same way each is one launch over the flat buffers, every
+// element rounded as the separate operations round it.
+template <>
+inline void LossLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+    using namespace rocm_detail;
+    if (input.num_row() != output.num_row() || input.num_col() != output.num_col() ||
+        input.get_transpose() != output.get_transpose()) {
+        Layer<ROCMfloat>::val = sum(sum(square(output - input), 0), 1) / Layer<ROCMfloat>::nb;
+        return;
+    }
+    Matrix<ROCMfloat> v = JzRocmFused::make("loss", 1, 1, 0);
+    must(jzhip_mse_loss(p(v), p(output), p(input), input.num_row() * input.num_col(),
+                        (float)(1.0 / Layer<ROCMfloat>::nb)),
+         "mse_loss");
+    Layer<ROCMfloat>::val = std::move(v);
+}
+template <>
+inline Matrix<ROCMfloat> LossLayer<ROCMfloat>::grad(const Matrix<ROCMfloat>& input) const {
+    using namespace rocm_detail;
+    // (a difference is returned untransposed, cpp/core.hpp:414-449: transposed operands keep
+    // the generic form, which turns them)
+    if (input.num_row() != output.num_row() || input.num_col() != output.num_col() ||
+        input.get_transpose() || output.get_transpose())
+        return 2.0 * (input - output) / Layer<ROCMfloat>::nb;
+    Matrix<ROCMfloat> g = JzRocmFused::make("loss_grad", input.num_row(), input.num_col(), 0);
+    must(jzhip_mse_grad(p(g), p(input), p(output), input.num_row() * input.num_col(),
+                        (float)(1.0 / Layer<ROCMfloat>::nb)),
+         "mse_grad");
+    return g;
+}
+
 // ── LayerNorm ────────────────────────────────────────────────────────────────
 
 template <>

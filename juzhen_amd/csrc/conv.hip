@@ -724,7 +724,11 @@ int scatter_patches(const float* col, float* img, const float* bias, const Patch
         };
         int CC = 16;
         while (CC > 1 && !fits(CC)) CC /= 2;
-        if (form && fits(CC) && g.K % 4 == 0 && aligned16(col)) {
+        // (below 64 MB of patches the strip form is as fast alone and its 256-thread
+        // workgroups start sooner behind another kernel: a 29 MB layer ran 3.5 us
+        // slower inside a training step with the streamed form)
+        const bool large = static_cast<size_t>(g.K) * g.P * g.N * sizeof(float) >= (size_t(64) << 20);
+        if (form && large && fits(CC) && g.K % 4 == 0 && aligned16(col)) {
             // whole images per workgroup unless that leaves fewer than 2048 workgroups:
             // then segments of rows, each paying kH - 1 halo patch rows
             int seg = g.H;

@@ -75,6 +75,10 @@ struct AxpbyF {  // cpp/core.hpp:414-449: s1*a + s2*b
     float s1, s2;
     __device__ float operator()(float a, float b) const { return s1 * a + s2 * b; }
 };
+struct MseGradF {  // ml/layer.hpp:214-216: 2.0 * (input - output) / nb, each step rounded
+    float inv_nb;
+    __device__ float operator()(float pred, float target) const { return ((pred - target) * 2.0f) * inv_nb; }
+};
 struct HadamardF {  // cpp/matrix.hpp:428-474
     __device__ float operator()(float a, float b) const { return a * b; }
 };
@@ -226,6 +230,9 @@ JZ_API int jzhip_sqrt(float* out, const float* in, size_t count) {
 }
 JZ_API int jzhip_clamp(float* out, const float* in, size_t count, float lo, float hi) {
     return launch_ew<1>(ClampF{lo, hi}, out, in, nullptr, count);
+}
+JZ_API int jzhip_mse_grad(float* out, const float* pred, const float* target, size_t count, float inv_nb) {
+    return launch_ew<2>(MseGradF{inv_nb}, out, pred, target, count);
 }
 JZ_API int jzhip_drelu_mul(float* out, const float* pre, const float* up, size_t count) {
     return launch_ew<2>(DReluMulF{}, out, pre, up, count);

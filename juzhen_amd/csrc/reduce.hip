@@ -179,11 +179,16 @@ __global__ __launch_bounds__(kBlock) void sum_rows_short_kernel(float* part, con
     }
     red[t] = acc0 + acc1;
     __syncthreads();
-    if (t < numrow) {
-        float s = 0.f;
-        for (int k = t; k < active; k += numrow) s += red[k];
-        part[static_cast<size_t>(blockIdx.x) * numrow + t] = s;
+    // threads of equal row are numrow apart: halve the number of groups of numrow threads
+    // until one is left (with one row a single thread adding 256 values in turn took 9 of
+    // the kernel's 11 us)
+    for (int groups = active / numrow; groups > 1;) {
+        const int half = (groups + 1) / 2;
+        if (t < (groups - half) * numrow) red[t] += red[t + half * numrow];
+        __syncthreads();
+        groups = half;
     }
+    if (t < numrow) part[static_cast<size_t>(blockIdx.x) * numrow + t] = red[t];
 }
 
 // ── flat sum of squares (norm) ───────────────────────────────────────────
@@ -220,6 +225,39 @@ __global__ __launch_bounds__(kBlock) void sqrt_sum_kernel(float* out, const floa
     for (int i = threadIdx.x; i < n; i += kBlock) acc += part[i];
     const float s = block_allreduce<kBlock / kWave>(acc, SumOp{}, red, 0.f);
     if (threadIdx.x == 0) out[0] = sqrtf(s);
+}
+
+// ── mean squared error value: scale * sum((target - pred)^2) ─────────────
+// (LossLayer::eval, ml/layer.hpp:223-226: difference, square, two sums and a scaling as five
+// matrix operations; here the differences and squares round the same way and the sums run
+// over the flat buffer.)  A single workgroup writes the scaled result itself.
+__global__ __launch_bounds__(kBlock) void sqdiff_partial_kernel(float* part, const float* __restrict__ target,
+                                                                const float* __restrict__ pred, size_t n,
+                                                                float scale) {
+    __shared__ float red[kBlock / kWave];
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    float acc0 = 0.f, acc1 = 0.f;
+    size_t i = tid;
+    for (; i + stride < n; i += 2 * stride) {
+        const float d0 = target[i] - pred[i], d1 = target[i + stride] - pred[i + stride];
+        acc0 += d0 * d0;
+        acc1 += d1 * d1;
+    }
+    if (i < n) {
+        const float d0 = target[i] - pred[i];
+        acc0 += d0 * d0;
+    }
+    const float s = block_allreduce<kBlock / kWave>(acc0 + acc1, SumOp{}, red, 0.f);
+    if (threadIdx.x == 0) part[blockIdx.x] = gridDim.x == 1 ? s * scale : s;
+}
+
+__global__ __launch_bounds__(kBlock) void scaled_sum_kernel(float* out, const float* part, int n, float scale) {
+    __shared__ float red[kBlock / kWave];
+    float acc = 0.f;
+    for (int i = threadIdx.x; i < n; i += kBlock) acc += part[i];
+    const float s = block_allreduce<kBlock / kWave>(acc, SumOp{}, red, 0.f);
+    if (threadIdx.x == 0) out[0] = s * scale;
 }
 
 // ── column max / argmax: one wavefront per column ────────────────────────
@@ -403,6 +441,24 @@ JZ_API int jzhip_nrm2(float* out_device, const float* x, size_t count) {
     hipStream_t s = stream();
     sumsq_partial_kernel<<<grid, kBlock, 0, s>>>(part, x, count, aligned16(x) ? 1 : 0);
     sqrt_sum_kernel<<<1, kBlock, 0, s>>>(out_device, part, static_cast<int>(grid));
+    return launch_rc();
+}
+
+JZ_API int jzhip_mse_loss(float* out_device, const float* target, const float* pred, size_t count, float scale) {
+    if (!out_device) return -1;
+    if (count == 0) return jzhip_fill(out_device, 1, 0.f);
+    if (!target || !pred) return -1;
+    hipStream_t s = stream();
+    if (count <= static_cast<size_t>(kBlock) * 32) {
+        sqdiff_partial_kernel<<<1, kBlock, 0, s>>>(out_device, target, pred, count, scale);
+        return launch_rc();
+    }
+    float* part = workspace();
+    if (!part) return -2;
+    const unsigned grid = grid_for(count, static_cast<size_t>(kBlock) * 2, 4);
+    sqdiff_partial_kernel<<<grid, kBlock, 0, s>>>(part, target, pred, count, scale);
+    if (grid > 1) scaled_sum_kernel<<<1, kBlock, 0, s>>>(out_device, part, static_cast<int>(grid), scale);
+    else return jzhip_copy(out_device, part, 1);
     return launch_rc();
 }
 

@@ -194,7 +194,7 @@ def test_slice_and_stack(gpu, oracle_lib, ts, td):
 
 
 # ── reductions ───────────────────────────────────────────────────────────
-SHAPES_RED = [(1, 1), (1, 1000), (1000, 1), (3, 8192), (10, 128), (64, 64), (256, 4096), (257, 33),
+SHAPES_RED = [(1, 1), (1, 1000), (1000, 1), (3, 8192), (10, 128), (64, 64), (7, 300), (33, 100), (1, 4096), (256, 4096), (257, 33),
               (512, 16384), (1024, 1024), (100000, 3), (1 << 20, 1)]
 
 
@@ -241,6 +241,28 @@ def test_nrm2(gpu, oracle_lib, n):
     band = max(TOL_RED, n * 6e-8) * exact
     assert abs(oracle_lib.jzo_norm(hptr(x), n) - exact) <= band
     assert abs(to_host(out)[0] - oracle_lib.jzo_norm(hptr(x), n)) <= band
+
+
+@pytest.mark.parametrize("n,nb", [(1, 1), (4096, 4096), (3 * 1000, 1000), (8192 + 5, 7), (3072 * 128, 128)])
+def test_mse_loss_and_grad(gpu, n, nb):
+    """The squared-error head in one launch each (ml/layer.hpp:214-226): the gradient rounds
+    as 2.0 * (input - output) / nb does through the matrix operators (cpp/operators.hpp:236-264:
+    `/ nb` is a multiplication by float(1.0 / nb)), so it is compared bit for bit; the value is a
+    sum and gets the reduction tolerance."""
+    r = rng(n + nb)
+    pred = r.normal(0, 1, n).astype(np.float32)
+    target = r.normal(0, 1, n).astype(np.float32)
+    inv = np.float32(1.0 / nb)
+    g = dev_empty(n)
+    gpu.mse_grad(dptr(g), dp(pred), dp(target), n, float(inv))
+    assert np.array_equal(to_host(g), ((pred - target) * np.float32(2.0)) * inv)
+    out = dev_empty(1)
+    gpu.mse_loss(dptr(out), dp(target), dp(pred), n, float(inv))
+    d = (target - pred).astype(np.float32)
+    exact = float(np.sum((d * d).astype(np.float32).astype(np.float64))) / nb
+    assert abs(to_host(out)[0] - exact) <= TOL_RED * max(exact, 1e-30)
+    gpu.mse_loss(dptr(out), dp(target), dp(pred), 0, 1.0)
+    assert to_host(out)[0] == 0.0
 
 
 @pytest.mark.parametrize("numrow,numcol", [(1, 5), (10, 128), (256, 16384), (1000, 7), (65, 65)])
@@ -804,13 +826,24 @@ CONV_CASES = [
     (2, 20, 9, 10, 5, 5, 2, 2),
     (1, 16, 8, 8, 2, 2, 0, 1),
     (2, 256, 8, 8, 3, 3, 1, 1),
-    # the streamed scatter: no padding, more padding than the kernel needs, 5x5, 4x4 stride 2, ragged row segments
     (2, 8, 9, 7, 3, 3, 0, 1),
     (2, 4, 6, 6, 3, 3, 2, 1),
     (2, 8, 12, 12, 5, 5, 2, 1),
     (2, 4, 10, 10, 4, 4, 0, 2),
     (2, 8, 11, 11, 3, 3, 0, 2),
     (1, 16, 37, 20, 3, 3, 1, 1),
+    # 64 MB of patches and more, where the scatter walks down the patch rows with a ring in LDS:
+    # no padding, more padding than the kernel needs, 5x5, 4x4 stride 2, whole images per
+    # workgroup (many samples) and ragged row segments (few samples of tall images)
+    (7000, 8, 9, 7, 3, 3, 0, 1),
+    (7400, 4, 6, 6, 3, 3, 2, 1),
+    (600, 8, 12, 12, 5, 5, 2, 1),
+    (16500, 4, 10, 10, 4, 4, 0, 2),
+    (9400, 8, 11, 11, 3, 3, 0, 2),
+    (160, 16, 37, 20, 3, 3, 1, 1),
+    (5, 64, 151, 48, 3, 3, 1, 1),
+    (18, 64, 101, 64, 3, 3, 1, 2),
+    (32, 64, 32, 32, 3, 3, 1, 1),
 ]
 
 
@@ -876,6 +909,9 @@ CT_CASES = [
     (2, 64, 16, 16, 4, 4, 1, 2),
     (2, 128, 8, 8, 4, 4, 1, 2),
     (3, 12, 7, 5, 3, 3, 1, 2),
+    # 64 MB of patches and more (the streamed scatter): whole images and row segments
+    (64, 64, 16, 16, 4, 4, 1, 2),
+    (26, 32, 40, 32, 4, 4, 1, 2),
 ]
 
 
