@@ -381,6 +381,12 @@ int jzhip_attn_softmax_bwd(float* dS, const float* A, const float* dA, int S,
  * one-hot matrix. */
 int jzhip_softmax_xent(float* loss_out, float* dlogits, const float* logits,
                        const int32_t* labels, int K, int N, int ld);
+/* The same against a K x N matrix of targets (leading dimension ld, as the logits), which is
+ * how LogisticLayer holds them: loss_out[0] = -inv_nb * sum_n (sum_k x*y - lse_n)
+ * (ml/layer.hpp:272-283) and dlogits = -(y - softmax) * inv_nb (ml/layer.hpp:252-262).
+ * Either output may be NULL. */
+int jzhip_softmax_xent_dense(float* loss_out, float* dlogits, const float* logits, const float* target,
+                             int K, int N, int ld, float inv_nb);
 
 /* Multi-head self-attention core over the layouts TransformerLayer keeps
  * (ml/layer.hpp:2843-2848): Q, K, V, H are (d_k, S*B) column-major with head hh

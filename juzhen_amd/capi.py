@@ -116,6 +116,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_attn_softmax": (I, [P, P, I, I, F, I, I]),
     "jzhip_attn_softmax_bwd": (I, [P, P, P, I, I, F, I]),
     "jzhip_softmax_xent": (I, [P, P, P, P, I, I, I]),
+    "jzhip_softmax_xent_dense": (I, [P, P, P, P, I, I, I, F]),
     "jzhip_attention_fwd_ld": (I, [P, I, P, P, P, P, I, I, I, I, I, I]),
     "jzhip_attention_bwd_ld": (I, [P, P, P, I, P, P, I, P, P, P, I, P, I, I, I, I, I]),
     "jzhip_attention_fwd": (I, [P, P, P, P, P, I, I, I, I, I]),

@@ -290,6 +290,42 @@ inline Matrix<ROCMfloat> LossLayer<ROCMfloat>::grad(const Matrix<ROCMfloat>& inp
     return g;
 }
 
+// ── softmax cross-entropy head (ml/layer.hpp:232-284) ────────────────────────
+// eval() and grad() are each a dozen matrix operations in the generic form (a functor
+// reduction for the column maxima, two rank-1 products, exp, sums, log, a Hadamard product);
+// here each is one pass over the logits with one wavefront per sample, plus the mean.
+// Operands whose transpose flag is set are turned first, so the kernel sees K x N buffers.
+namespace rocm_detail {
+inline Matrix<ROCMfloat> xent_head(const Matrix<ROCMfloat>& input, const Matrix<ROCMfloat>& target, size_t nb,
+                                   bool want_grad) {
+    if (input.num_row() != target.num_row() || input.num_col() != target.num_col())
+        throw std::invalid_argument("Matrix dimensions are not compatible");
+    Matrix<ROCMfloat> turned_x = JzRocmFused::make("x", 0, 0, 0), turned_y = JzRocmFused::make("y", 0, 0, 0);
+    if (input.get_transpose()) turned_x = JzRocmFused::materialise(input);
+    if (target.get_transpose()) turned_y = JzRocmFused::materialise(target);
+    const Matrix<ROCMfloat>& x = input.get_transpose() ? turned_x : input;
+    const Matrix<ROCMfloat>& y = target.get_transpose() ? turned_y : target;
+    const size_t K = x.num_row(), N = x.num_col();
+    Matrix<ROCMfloat> out = want_grad ? JzRocmFused::make("xent_grad", K, N, 0) : JzRocmFused::make("xent", 1, 1, 0);
+    if (K == 0 || N == 0) {
+        out.zeros();
+        return out;
+    }
+    must(jzhip_softmax_xent_dense(want_grad ? nullptr : p(out), want_grad ? p(out) : nullptr, p(x), p(y), (int)K,
+                                  (int)N, (int)K, (float)(1.0 / nb)),
+         "softmax_xent_dense");
+    return out;
+}
+}  // namespace rocm_detail
+template <>
+inline void LogisticLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input) {
+    Layer<ROCMfloat>::val = rocm_detail::xent_head(input, output, Layer<ROCMfloat>::nb, false);
+}
+template <>
+inline Matrix<ROCMfloat> LogisticLayer<ROCMfloat>::grad(const Matrix<ROCMfloat>& input) const {
+    return rocm_detail::xent_head(input, output, Layer<ROCMfloat>::nb, true);
+}
+
 // ── LayerNorm ────────────────────────────────────────────────────────────────
 
 template <>

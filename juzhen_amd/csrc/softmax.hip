@@ -499,23 +499,29 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_rows_kernel(float* dS, con
 
 // ── softmax cross-entropy against integer labels ─────────────────────────
 // One wavefront per sample column.  per_sample[n] = x[label] - lse.
-template <int NV>
+// DENSE: the targets are a K x N matrix (leading dimension ld) instead of labels, as
+// LogisticLayer holds them: per_sample[n] = sum_k x*y - lse (ml/layer.hpp:281), and the
+// gradient subtracts y itself.
+template <int NV, bool DENSE>
 __global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, float* dlogits,
                                                            const float* logits,
-                                                           const int32_t* labels, int K, int N,
-                                                           size_t ld, float inv_n) {
+                                                           const int32_t* labels, const float* target,
+                                                           int K, int N, size_t ld, float inv_n) {
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
     const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
     for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
         const float* p = logits + col * ld;
-        const int label = labels[col];
+        int label = 0;
+        if constexpr (!DENSE) label = labels[col];
         float x[NV];
+        float y[DENSE ? NV : 1];
         float m = -1e30f;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int r = lane + v * kWave;
             x[v] = r < K ? p[r] : -INFINITY;
+            if constexpr (DENSE) y[v] = r < K ? target[col * ld + r] : 0.f;
             if (r < K) m = m > x[v] ? m : x[v];
         }
         m = wave_max(m);
@@ -526,7 +532,11 @@ __global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, fl
             const int r = lane + v * kWave;
             e[v] = r < K ? exp_neg(x[v] - m) : 0.f;
             s += e[v];
-            if (r == label) picked = x[v];
+            if constexpr (DENSE) {
+                if (r < K) picked += x[v] * y[v];
+            } else {
+                if (r == label) picked = x[v];
+            }
         }
         s = wave_sum(s);
         picked = wave_sum(picked);
@@ -539,9 +549,52 @@ __global__ __launch_bounds__(kBlock) void xent_cols_kernel(float* per_sample, fl
             for (int v = 0; v < NV; ++v) {
                 const int r = lane + v * kWave;
                 if (r < K) {
-                    const float y = (r == label) ? 1.0f : 0.0f;
-                    d[r] = -(y - e[v] * invz) * inv_n;
+                    float yv;
+                    if constexpr (DENSE) yv = y[v];
+                    else yv = (r == label) ? 1.0f : 0.0f;
+                    d[r] = -(yv - e[v] * invz) * inv_n;
                 }
+            }
+        }
+    }
+}
+
+// More than 1024 classes: the same with three sweeps over the column (the second and
+// third hit L2) instead of registers.
+template <bool DENSE>
+__global__ __launch_bounds__(kBlock) void xent_cols_long_kernel(float* per_sample, float* dlogits,
+                                                                const float* logits, const int32_t* labels,
+                                                                const float* target, int K, int N, size_t ld,
+                                                                float inv_n) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
+        const float* p = logits + col * ld;
+        const float* t = DENSE ? target + col * ld : nullptr;
+        int label = 0;
+        if constexpr (!DENSE) label = labels[col];
+        float m = -1e30f;
+        for (int r = lane; r < K; r += kWave) m = m > p[r] ? m : p[r];
+        m = wave_max(m);
+        float s = 0.f, picked = 0.f;
+        for (int r = lane; r < K; r += kWave) {
+            const float x = p[r];
+            s += exp_neg(x - m);
+            if constexpr (DENSE) picked += x * t[r];
+            else if (r == label) picked = x;
+        }
+        s = wave_sum(s);
+        picked = wave_sum(picked);
+        if (lane == 0) per_sample[col] = picked - (logf(s) + m);
+        if (dlogits) {
+            const float invz = static_cast<float>(1.0 / static_cast<double>(s));
+            float* d = dlogits + col * ld;
+            for (int r = lane; r < K; r += kWave) {
+                float yv;
+                if constexpr (DENSE) yv = t[r];
+                else yv = (r == label) ? 1.0f : 0.0f;
+                d[r] = -(yv - exp_neg(p[r] - m) * invz) * inv_n;
             }
         }
     }
@@ -593,13 +646,30 @@ struct SoftmaxBwdColsL {
 template <int NV>
 struct XentL {
     static int run(float* per_sample, float* dlogits, const float* logits, const int32_t* labels,
-                   int K, int N, size_t ld) {
+                   const float* target, int K, int N, size_t ld, float inv_n) {
         const unsigned grid = grid_cover(N, kBlock / kWave);
-        xent_cols_kernel<NV><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, labels, K, N,
-                                                            ld, static_cast<float>(1.0 / N));
+        if (target)
+            xent_cols_kernel<NV, true><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, nullptr, target,
+                                                                      K, N, ld, inv_n);
+        else
+            xent_cols_kernel<NV, false><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, labels, nullptr,
+                                                                       K, N, ld, inv_n);
         return launch_rc();
     }
 };
+
+int xent_impl(float* per_sample, float* dlogits, const float* logits, const int32_t* labels, const float* target,
+              int K, int N, size_t ld, float inv_n) {
+    if (K <= 1024) return dispatch_nv<XentL>(K, per_sample, dlogits, logits, labels, target, K, N, ld, inv_n);
+    const unsigned grid = grid_cover(N, kBlock / kWave);
+    if (target)
+        xent_cols_long_kernel<true><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, nullptr, target, K, N,
+                                                                   ld, inv_n);
+    else
+        xent_cols_long_kernel<false><<<grid, kBlock, 0, stream()>>>(per_sample, dlogits, logits, labels, nullptr, K,
+                                                                    N, ld, inv_n);
+    return launch_rc();
+}
 
 int softmax_cols_impl(float* out, const float* in, int numrow, size_t numcol, size_t ld,
                       ScoreXform xf) {
@@ -741,12 +811,24 @@ JZ_API int jzhip_attn_softmax_bwd(float* dS, const float* A, const float* dA, in
 JZ_API int jzhip_softmax_xent(float* loss_out, float* dlogits, const float* logits,
                               const int32_t* labels, int K, int N, int ld) {
     if (K <= 0 || N <= 0 || ld < K || !loss_out || !logits || !labels) return -1;
-    if (K > 1024) return -1;
     if (static_cast<size_t>(N) > kWorkspaceFloats) return -1;
     float* per_sample = workspace();
     if (!per_sample) return -2;
-    int rc = dispatch_nv<XentL>(K, per_sample, dlogits, logits, labels, K, N, static_cast<size_t>(ld));
+    int rc = xent_impl(per_sample, dlogits, logits, labels, nullptr, K, N, static_cast<size_t>(ld),
+                       static_cast<float>(1.0 / N));
     if (rc) return rc;
     neg_mean_kernel<<<1, kMeanBlock, 0, stream()>>>(loss_out, per_sample, N, static_cast<float>(1.0 / N));
+    return launch_rc();
+}
+
+JZ_API int jzhip_softmax_xent_dense(float* loss_out, float* dlogits, const float* logits, const float* target,
+                                    int K, int N, int ld, float inv_nb) {
+    if (K <= 0 || N <= 0 || ld < K || !logits || !target || (!loss_out && !dlogits)) return -1;
+    if (static_cast<size_t>(N) > kWorkspaceFloats) return -1;
+    float* per_sample = workspace();
+    if (!per_sample) return -2;
+    int rc = xent_impl(per_sample, dlogits, logits, nullptr, target, K, N, static_cast<size_t>(ld), inv_nb);
+    if (rc || !loss_out) return rc;
+    neg_mean_kernel<<<1, kMeanBlock, 0, stream()>>>(loss_out, per_sample, N, inv_nb);
     return launch_rc();
 }

@@ -642,7 +642,7 @@ def test_attn_softmax_fwd_bwd(gpu, oracle_lib, S, nblk, causal, kar):
     assert rel_err(to_host(dS), refd) <= TOL_RED
 
 
-@pytest.mark.parametrize("K,N", [(10, 128), (256, 4096), (2, 1), (77, 300)])
+@pytest.mark.parametrize("K,N", [(10, 128), (256, 4096), (2, 1), (77, 300), (1024, 9), (2000, 17)])
 def test_softmax_xent(gpu, oracle_lib, K, N):
     r = rng(K + N)
     x = r.normal(0, 2, K * N).astype(np.float32)
@@ -661,6 +661,40 @@ def test_softmax_xent(gpu, oracle_lib, K, N):
     # x[label] - lse cancels when the label dominates, so the bound is relative
     # to the magnitude of the terms that are subtracted
     assert abs(to_host(dl)[0] - exact) <= TOL_RED * (abs(exact) + np.abs(lse).mean())
+
+
+@pytest.mark.parametrize("K,N,nb", [(10, 128, 128), (1, 5, 5), (256, 1000, 1000), (1000, 33, 33), (1500, 40, 8), (65, 7, 7)])
+def test_softmax_xent_dense_targets(gpu, oracle_lib, K, N, nb):
+    """The head against a matrix of targets (ml/layer.hpp:252-283): with one-hot targets it agrees
+    with the label form (checked against the oracle's), with soft targets with the closed form in
+    float64; more than 1024 classes take the swept kernel; nb need not equal N."""
+    r = rng(K * 3 + N)
+    x = r.normal(0, 2, K * N).astype(np.float32)
+    lab = r.integers(0, K, N).astype(np.int32)
+    onehot = np.zeros((N, K), np.float32)
+    onehot[np.arange(N), lab] = 1.0
+    refd = np.empty_like(x)
+    ref_loss = oracle_lib.jzo_softmax_xent(hptr(refd), hptr(x), hptr(lab), K, N, K)   # scaled by 1/N
+    dl, dd = dev_empty(1), dev_empty(K * N)
+    gpu.softmax_xent_dense(dptr(dl), dptr(dd), dp(x), dp(onehot.reshape(-1)), K, N, K, 1.0 / nb)
+    assert abs(to_host(dl)[0] * nb / N - ref_loss) <= TOL_RED * (abs(ref_loss) + np.abs(x).max())
+    assert rel_err(to_host(dd) * np.float32(nb / N), refd) <= TOL_RED
+    # soft targets: closed form
+    Y = r.random((N, K)); Y /= Y.sum(1, keepdims=True)
+    y32 = Y.astype(np.float32)
+    X = x.reshape(N, K).astype(np.float64)
+    mx = X.max(1, keepdims=True)
+    E = np.exp(X - mx)
+    lse = np.log(E.sum(1)) + mx[:, 0]
+    exact = -((X * y32).sum(1) - lse).sum() / nb
+    grad = -(y32 - E / E.sum(1, keepdims=True)) / nb
+    gpu.softmax_xent_dense(dptr(dl), dptr(dd), dp(x), dp(y32.reshape(-1)), K, N, K, 1.0 / nb)
+    assert abs(to_host(dl)[0] - exact) <= TOL_RED * (abs(exact) + np.abs(lse).mean() * N / nb)
+    assert rel_err(to_host(dd), grad.reshape(-1)) <= TOL_RED
+    # either output alone
+    only = dev_empty(K * N)
+    gpu.softmax_xent_dense(None, dptr(only), dp(x), dp(y32.reshape(-1)), K, N, K, 1.0 / nb)
+    assert np.array_equal(to_host(only), to_host(dd))
 
 
 # ── LayerNorm ────────────────────────────────────────────────────────────
