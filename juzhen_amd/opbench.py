@@ -198,6 +198,15 @@ def bench_reduce(r):
         lab = torch.randint(0, k, (nb,), device="cuda", dtype=torch.int32)
         r.run("reduce", "jzhip_softmax_xent", f"{k}x{nb}", lambda: jz.softmax_xent(P(loss), P(g), P(z), P(lab), k, nb, k),
               bytes_=8 * k * nb + 4 * nb)
+        y = dev(k * nb, 0)
+        r.run("reduce", "jzhip_softmax_xent_dense (value)", f"{k}x{nb}",
+              lambda: jz.softmax_xent_dense(P(loss), None, P(z), P(y), k, nb, k, 1.0 / nb), bytes_=8 * k * nb)
+        r.run("reduce", "jzhip_softmax_xent_dense (gradient)", f"{k}x{nb}",
+              lambda: jz.softmax_xent_dense(None, P(g), P(z), P(y), k, nb, k, 1.0 / nb), bytes_=12 * k * nb)
+    for n in (4096, 1 << 26):
+        a, b, g, loss = dev(n), dev(n), dev(n, 0), dev(1, 0)
+        r.run("reduce", "jzhip_mse_loss", f"{n}", lambda: jz.mse_loss(P(loss), P(a), P(b), n, 1.0 / 128), bytes_=8 * n)
+        r.run("reduce", "jzhip_mse_grad", f"{n}", lambda: jz.mse_grad(P(g), P(a), P(b), n, 1.0 / 128), bytes_=12 * n)
 
 
 def bench_fused(r):
