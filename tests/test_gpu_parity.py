@@ -154,6 +154,29 @@ def test_axpby_hadamard_2d(gpu, oracle_lib, rows, cols, to, ta, tb):
     assert np.array_equal(to_host(do), ref)
 
 
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (8192, 2048 + 64), (1024, 16384 + 128)])
+@pytest.mark.parametrize("to,ta,tb", [(0, 1, 0), (0, 0, 1), (0, 1, 1), (1, 0, 0)])
+def test_transposed_operands_many_full_tiles(gpu, rows, cols, to, ta, tb):
+    """Several thousand full 64 x 64 tiles: the form in which a workgroup walks a sequence of
+    tiles with the next tile's operands in flight.  Checked against numpy's own transposes
+    (s1*a + s2*b and a*b round as two products and a sum / one product in float32)."""
+    r = rng(rows + cols + ta * 2 + tb)
+    A = r.normal(0, 1, (rows, cols)).astype(np.float32)     # logical matrices
+    B = r.normal(0, 1, (rows, cols)).astype(np.float32)
+    phys = lambda M, t: np.ascontiguousarray(M if t else M.T).reshape(-1)   # column-major, or its transpose
+    a, b = phys(A, ta), phys(B, tb)
+    ldo, lda, ldb = (cols if to else rows), (cols if ta else rows), (cols if tb else rows)
+    da, db, do = to_dev(a), to_dev(b), dev_empty(rows * cols)
+    gpu.axpby2d(dptr(do), ldo, to, dptr(da), lda, ta, dptr(db), ldb, tb, rows, cols, 0.5, 2.0)
+    want = np.float32(0.5) * A + np.float32(2.0) * B
+    assert np.array_equal(to_host(do), phys(want, to))
+    gpu.hadamard2d(dptr(do), ldo, to, dptr(da), lda, ta, dptr(db), ldb, tb, rows, cols)
+    assert np.array_equal(to_host(do), phys(A * B, to))
+    if ta != to:
+        gpu.copy2d(dptr(do), ldo, to, 0, 0, dptr(da), lda, ta, 0, 0, rows, cols)
+        assert np.array_equal(to_host(do), phys(A, to))
+
+
 @pytest.mark.parametrize("ts", [0, 1])
 @pytest.mark.parametrize("td", [0, 1])
 def test_slice_and_stack(gpu, oracle_lib, ts, td):
