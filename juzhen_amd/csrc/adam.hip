@@ -33,7 +33,8 @@ __device__ __forceinline__ float adam_one(float gi, float& mi_io, float& vi_io, 
 }
 
 // FUSE_W = false: g <- step.  FUSE_W = true: w <- decay*w - step, g untouched.
-template <bool FUSE_W, bool VEC>
+// NT: non-temporal loads and stores (a launch that streams past the cache).
+template <bool FUSE_W, bool VEC, bool NT>
 __global__ __launch_bounds__(kBlock) void adam_kernel(float* w, float* g, float* m, float* v,
                                                       size_t n, AdamConst c) {
     // one float4 per thread, grid covers the data once (see elementwise.hip)
@@ -42,18 +43,18 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* w, float* g, float*
     if constexpr (VEC) {
         const size_t n4 = n / 4;
         for (size_t i = tid; i < n4; i += stride) {
-            float4 gv = reinterpret_cast<const float4*>(g)[i];
-            float4 mv = reinterpret_cast<float4*>(m)[i];
-            float4 vv = reinterpret_cast<float4*>(v)[i];
+            float4 gv = load4<NT>(g + 4 * i);
+            float4 mv = load4<NT>(m + 4 * i);
+            float4 vv = load4<NT>(v + 4 * i);
             float4 st;
             st.x = adam_one(gv.x, mv.x, vv.x, c);
             st.y = adam_one(gv.y, mv.y, vv.y, c);
             st.z = adam_one(gv.z, mv.z, vv.z, c);
             st.w = adam_one(gv.w, mv.w, vv.w, c);
-            reinterpret_cast<float4*>(m)[i] = mv;
-            reinterpret_cast<float4*>(v)[i] = vv;
+            store4<NT>(m + 4 * i, mv);
+            store4<NT>(v + 4 * i, vv);
             if constexpr (FUSE_W) {
-                float4 wv = reinterpret_cast<float4*>(w)[i];
+                float4 wv = load4<NT>(w + 4 * i);
                 if (c.use_decay) {
                     wv.x *= c.decay; wv.y *= c.decay; wv.z *= c.decay; wv.w *= c.decay;
                 }
@@ -61,9 +62,9 @@ __global__ __launch_bounds__(kBlock) void adam_kernel(float* w, float* g, float*
                 wv.y = 1.0f * wv.y + -1.0f * st.y;
                 wv.z = 1.0f * wv.z + -1.0f * st.z;
                 wv.w = 1.0f * wv.w + -1.0f * st.w;
-                reinterpret_cast<float4*>(w)[i] = wv;
+                store4<NT>(w + 4 * i, wv);
             } else {
-                reinterpret_cast<float4*>(g)[i] = st;
+                store4<NT>(g + 4 * i, st);
             }
         }
         for (size_t j = n4 * 4 + tid; j < n; j += stride) {
@@ -120,10 +121,14 @@ int launch_adam(float* w, float* g, float* m, float* v, size_t n, const AdamCons
     const size_t blocks = (items + kBlock - 1) / kBlock;
     if (blocks > 0x7fffffffull) return -1;
     const unsigned grid = static_cast<unsigned>(blocks);
-    if (vec)
-        adam_kernel<FUSE_W, true><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
+    // (the moments and weights of a 19 M parameter model, 0.5 GB per step, are partly still in
+    // the last-level cache from the step before: 82 us plain, 95 us hinted; at 3.2 GB the hint wins)
+    if (vec && streams_past_cache((FUSE_W ? 7 : 6) * n * sizeof(float) / 2))
+        adam_kernel<FUSE_W, true, true><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
+    else if (vec)
+        adam_kernel<FUSE_W, true, false><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
     else
-        adam_kernel<FUSE_W, false><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
+        adam_kernel<FUSE_W, false, false><<<grid, kBlock, 0, stream()>>>(w, g, m, v, n, c);
     return launch_rc();
 }
 

@@ -53,8 +53,44 @@ inline unsigned grid_cover(size_t work, size_t per_block) {
     return static_cast<unsigned>(need);
 }
 
+// A launch that moves twice what the 256 MB last-level cache holds gains nothing from
+// keeping its data there; its loads and stores then carry the non-temporal hint (a copy of
+// 2 GB: 6.1 -> 6.4 TB/s, of 0.5 GB 5.8 -> 6.4; column sums of 1 GB 5.5 -> 6.3).  Below
+// that size the plain forms stay: what one kernel writes the next one often reads back out
+// of the cache (hinted loads of a 134 MB operand that was resident ran 15 % slower, a
+// 268 MB slice 7-30 % slower).  Kernels that profit from the cache for longer (the
+// optimiser's moments from step to step, a column softmax that holds whole columns in
+// registers) ask with a fraction of their bytes.
+constexpr size_t kStreamingBytes = size_t(512) << 20;
+inline bool streams_past_cache(size_t bytes) { return bytes >= kStreamingBytes; }
+
 // ── wave64 reductions: DPP inside a 16-lane row, bpermute across rows ────
 #ifdef __HIPCC__
+typedef float jz_f4 __attribute__((ext_vector_type(4)));
+template <bool NT>
+__device__ __forceinline__ float4 load4(const float* p) {
+    if constexpr (NT) {
+        const jz_f4 t = __builtin_nontemporal_load(reinterpret_cast<const jz_f4*>(p));
+        return make_float4(t.x, t.y, t.z, t.w);
+    } else {
+        return *reinterpret_cast<const float4*>(p);
+    }
+}
+template <bool NT>
+__device__ __forceinline__ float load1(const float* p) {
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+template <bool NT>
+__device__ __forceinline__ void store4(float* p, const float4& v) {
+    if constexpr (NT) {
+        jz_f4 t;
+        t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w;
+        __builtin_nontemporal_store(t, reinterpret_cast<jz_f4*>(p));
+    } else {
+        *reinterpret_cast<float4*>(p) = v;
+    }
+}
 template <int CTRL>
 __device__ __forceinline__ float dpp_mov(float v) {
     return __builtin_bit_cast(

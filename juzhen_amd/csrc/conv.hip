@@ -262,7 +262,7 @@ __device__ __forceinline__ bool rowgrid_item(const RowGrid& rg, int& x, int& y, 
 // (With one patch row per workgroup every image row was staged kH times over: 203 MB
 // fetched for a 67 MB input at 3x3; a band of four rows stages it 1.5 times: 145 -> 140 us
 // for the 671 MB of patches of 128 x 128 x 32 x 32, which the write side bounds.)
-template <int NSUB>
+template <int NSUB, bool NT>
 __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __restrict__ img,
                                                              float* __restrict__ col, PatchGeom g,
                                                              int WT, FastDiv dWT, int band, int nr, FastDiv dnr) {
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kBlock) void im2col_rows_kernel(const float* __rest
             if (off[u][0] >= 0) {
                 const float4 v = make_float4(tile[off[u][0] + w], tile[off[u][1] + w], tile[off[u][2] + w],
                                              tile[off[u][3] + w]);
-                *reinterpret_cast<float4*>(d + u * kPatchChunk) = v;
+                store4<NT>(d + u * kPatchChunk, v);
             }
         }
         pw += kBlock / kWave;
@@ -548,6 +548,7 @@ __global__ __launch_bounds__(kStreamBlock, 8) void col2im_stream_kernel(const fl
         auto fetch = [&](int ph, float4 (&r)[kStreamLoads]) {
             const float* rowp = base + static_cast<size_t>(ph) * row_step;
 #pragma unroll
+            // (plain loads: with the streaming hint the 604 MB layer ran 160 us instead of 144)
             for (int b = 0; b < kStreamLoads; ++b) r[b] = *reinterpret_cast<const float4*>(rowp + src[b]);
         };
         auto stash = [&](int ph, const float4 (&r)[kStreamLoads]) {
@@ -691,8 +692,11 @@ int gather_patches(const float* img, float* col, const PatchGeom& g) {
             dim3 grid(fold ? pieces - 1 : pieces, bands, g.N);
             const int nr = staged_rows(band);
             const FastDiv dWT = make_fastdiv(WT), dnr = make_fastdiv(nr);
-            if (fold) im2col_rows_kernel<2><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
-            else im2col_rows_kernel<1><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
+            const bool nt = streams_past_cache(total * sizeof(float));   // patches that the cache cannot hold anyway
+            if (fold && nt) im2col_rows_kernel<2, true><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
+            else if (fold) im2col_rows_kernel<2, false><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
+            else if (nt) im2col_rows_kernel<1, true><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
+            else im2col_rows_kernel<1, false><<<grid, kBlock, lds, stream()>>>(img, col, g, WT, dWT, band, nr, dnr);
             return launch_rc();
         }
     }

@@ -112,15 +112,16 @@ __device__ __forceinline__ float4 apply4(const F& f, const float4& a, const floa
 }
 
 // n4 float4 vectors followed by `tail` (<4) scalars; thread i owns vector i.
-template <int NIN, class F>
+// NT: loads and stores with the non-temporal hint (launches that stream past the cache).
+template <int NIN, class F, bool NT>
 __global__ __launch_bounds__(kBlock) void ew_vec_kernel(F f, float* out, const float* a,
                                                         const float* b, size_t n4, int tail) {
     const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (i < n4) {
         float4 va, vb;
-        if constexpr (NIN >= 1) va = reinterpret_cast<const float4*>(a)[i];
-        if constexpr (NIN >= 2) vb = reinterpret_cast<const float4*>(b)[i];
-        reinterpret_cast<float4*>(out)[i] = apply4<NIN>(f, va, vb);
+        if constexpr (NIN >= 1) va = load4<NT>(a + 4 * i);
+        if constexpr (NIN >= 2) vb = load4<NT>(b + 4 * i);
+        store4<NT>(out + 4 * i, apply4<NIN>(f, va, vb));
     }
     if (blockIdx.x == 0 && static_cast<int>(threadIdx.x) < tail) {
         const size_t j = n4 * 4 + threadIdx.x;
@@ -157,7 +158,10 @@ int launch_ew(F f, float* out, const float* a, const float* b, size_t n) {
         const int tail = static_cast<int>(n % 4);
         const size_t blocks = n4 ? (n4 + kBlock - 1) / kBlock : 1;
         if (blocks > 0x7fffffffull) return -1;
-        ew_vec_kernel<NIN, F><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(f, out, a, b, n4, tail);
+        if (NIN >= 1 && streams_past_cache((NIN + 1) * n * sizeof(float)))   // (a fill is as fast without the hint)
+            ew_vec_kernel<NIN, F, true><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(f, out, a, b, n4, tail);
+        else
+            ew_vec_kernel<NIN, F, false><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(f, out, a, b, n4, tail);
     } else {
         const unsigned grid = grid_for(n, kBlock);
         ew_scalar_kernel<NIN, F><<<grid, kBlock, 0, s>>>(f, out, a, b, n);

@@ -402,6 +402,7 @@ __global__ __launch_bounds__(kBlock) void rank1_vec_kernel(float* C, const float
 }
 
 // y(rows x cols) += b[i]
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void add_bias_kernel(float* y, const float* b, int rows,
                                                           size_t total4) {
     // rows % 4 == 0: a float4 never straddles a column
@@ -409,10 +410,10 @@ __global__ __launch_bounds__(kBlock) void add_bias_kernel(float* y, const float*
     const unsigned rows4 = rows / 4;
     for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < total4; i += stride) {
         const unsigned r4 = static_cast<unsigned>(i % rows4);
-        float4 v = reinterpret_cast<float4*>(y)[i];
+        float4 v = load4<NT>(y + 4 * i);
         const float4 bb = reinterpret_cast<const float4*>(b)[r4];
         v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
-        reinterpret_cast<float4*>(y)[i] = v;
+        store4<NT>(y + 4 * i, v);
     }
 }
 __global__ __launch_bounds__(kBlock) void add_bias_scalar_kernel(float* y, const float* b, int rows,
@@ -844,7 +845,10 @@ JZ_API int jzhip_add_bias(float* y, const float* b, int rows, int cols) {
     if (rows <= 0 || cols <= 0 || !y || !b) return -1;
     const size_t total = static_cast<size_t>(rows) * cols;
     if (rows % 4 == 0 && aligned16(y) && aligned16(b)) {
-        add_bias_kernel<<<grid_cover(total / 4, kBlock), kBlock, 0, stream()>>>(y, b, rows, total / 4);
+        if (streams_past_cache(2 * total * sizeof(float)))
+            add_bias_kernel<true><<<grid_cover(total / 4, kBlock), kBlock, 0, stream()>>>(y, b, rows, total / 4);
+        else
+            add_bias_kernel<false><<<grid_cover(total / 4, kBlock), kBlock, 0, stream()>>>(y, b, rows, total / 4);
     } else {
         add_bias_scalar_kernel<<<grid_for(total, kBlock, 8), kBlock, 0, stream()>>>(y, b, rows, total);
     }

@@ -140,7 +140,7 @@ __device__ __forceinline__ int wave_sum_many(float (&v)[NV], int lane) {
 
 // k contiguous in X: a wavefront takes kThinRows<TT> rows, its lanes stride over k
 // in float4 steps against V staged in LDS (each LDS read serves all the rows).
-template <int TT>
+template <int TT, bool NT>
 __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restrict__ X, size_t xs_l,
                                                           const float* __restrict__ V, size_t vs_t, size_t vs_k,
                                                           float* C, size_t cs_l, size_t cs_t, int L, int K, int T,
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restric
 #pragma unroll
             for (int u = 0; u < R; ++u) {
                 const size_t l = l0 + u < static_cast<size_t>(L) ? l0 + u : L - 1;   // clamped, dropped at the store
-                x[u] = reinterpret_cast<const float4*>(X + l * xs_l)[k4];
+                x[u] = load4<NT>(X + l * xs_l + 4 * static_cast<size_t>(k4));
             }
 #pragma unroll
             for (int t = 0; t < TT; ++t) {
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restric
 // column), the block's waves split the k of a chunk eight at a time, and the
 // chunk's slice of V sits in LDS as [t][chunk_len], zero-filled past the end
 // of K, read as broadcast float4.  Partial sums go to part[chunk][t*L + l].
-template <int TT>
+template <int TT, bool NT>
 __global__ __launch_bounds__(kBlock) void thin_axpy_partial_kernel(const float* __restrict__ X, size_t xs_k,
                                                                    const float* __restrict__ V, size_t vs_t,
                                                                    size_t vs_k, float* part, int L, int K, int T,
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void thin_axpy_partial_kernel(const float* 
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int c = kk + u < len ? kk + u : len - 1;   // clamped; its V entry is zero
-            x[u] = *reinterpret_cast<const float4*>(xp + static_cast<size_t>(c) * xs_k);
+            x[u] = load4<NT>(xp + static_cast<size_t>(c) * xs_k);
         }
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
@@ -309,11 +309,17 @@ struct ThinArgs {
 template <int TT>
 int thin_launch(const ThinArgs& a) {
     hipStream_t s = stream();
+    // the big operand is read once: past the cache size with the streaming hint
+    const bool nt = streams_past_cache(static_cast<size_t>(a.L) * a.K * sizeof(float));
     if (a.xs_k == 1) {
         const size_t groups = (static_cast<size_t>(a.L) + kThinRows<TT> - 1) / kThinRows<TT>;
         const unsigned grid = grid_for(groups, kBlock / kWave, 8);
-        thin_dot_kernel<TT><<<grid, kBlock, static_cast<size_t>(TT) * a.K * sizeof(float), s>>>(
-            a.X, a.xs_l, a.V, a.vs_t, a.vs_k, a.C, a.cs_l, a.cs_t, a.L, a.K, a.T, a.alpha, a.beta);
+        if (nt)
+            thin_dot_kernel<TT, true><<<grid, kBlock, static_cast<size_t>(TT) * a.K * sizeof(float), s>>>(
+                a.X, a.xs_l, a.V, a.vs_t, a.vs_k, a.C, a.cs_l, a.cs_t, a.L, a.K, a.T, a.alpha, a.beta);
+        else
+            thin_dot_kernel<TT, false><<<grid, kBlock, static_cast<size_t>(TT) * a.K * sizeof(float), s>>>(
+                a.X, a.xs_l, a.V, a.vs_t, a.vs_k, a.C, a.cs_l, a.cs_t, a.L, a.K, a.T, a.alpha, a.beta);
         return launch_rc();
     }
     const int row_blocks = (a.L / 4 + kWave - 1) / kWave;
@@ -327,8 +333,14 @@ int thin_launch(const ThinArgs& a) {
     if (outs * chunks > kWorkspaceFloats) return -1;            // thin_ok() rules this out
     float* part = workspace();
     if (!part) return -2;
-    thin_axpy_partial_kernel<TT><<<dim3(row_blocks, chunks), kBlock, static_cast<size_t>(TT) * chunk_len * sizeof(float),
-                                   s>>>(a.X, a.xs_k, a.V, a.vs_t, a.vs_k, part, a.L, a.K, a.T, chunk_len);
+    if (nt)
+        thin_axpy_partial_kernel<TT, true><<<dim3(row_blocks, chunks), kBlock,
+                                             static_cast<size_t>(TT) * chunk_len * sizeof(float), s>>>(
+            a.X, a.xs_k, a.V, a.vs_t, a.vs_k, part, a.L, a.K, a.T, chunk_len);
+    else
+        thin_axpy_partial_kernel<TT, false><<<dim3(row_blocks, chunks), kBlock,
+                                              static_cast<size_t>(TT) * chunk_len * sizeof(float), s>>>(
+            a.X, a.xs_k, a.V, a.vs_t, a.vs_k, part, a.L, a.K, a.T, chunk_len);
     gemv_n_combine_kernel<<<static_cast<unsigned>((outs + kWave - 1) / kWave), kGemvCombineBlock, 0, s>>>(
         a.C, part, static_cast<int>(outs), chunks, a.L, a.cs_l, a.cs_t, a.alpha, a.beta);
     return launch_rc();
@@ -363,6 +375,7 @@ namespace {
 // aligned A and x, incx == 1): a workgroup takes four columns, its four waves a quarter
 // of the rows each, eight float4 loads of A in flight per lane; x comes through the caches.
 constexpr int kGemvTCols = 4;
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void gemv_t_split_kernel(const float* __restrict__ A,
                                                               const float* __restrict__ x, float* y, int m,
                                                               int n, size_t lda, size_t incy, float alpha,
@@ -371,11 +384,11 @@ __global__ __launch_bounds__(kBlock) void gemv_t_split_kernel(const float* __res
     __shared__ float red[NW][kGemvTCols];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const size_t j0 = static_cast<size_t>(blockIdx.x) * kGemvTCols;
-    const float4* col[kGemvTCols];
+    const float* col[kGemvTCols];
 #pragma unroll
     for (int c = 0; c < kGemvTCols; ++c) {
         const size_t j = j0 + c < static_cast<size_t>(n) ? j0 + c : n - 1;   // clamped, dropped at the store
-        col[c] = reinterpret_cast<const float4*>(A + j * lda);
+        col[c] = A + j * lda;
     }
     const float4* x4 = reinterpret_cast<const float4*>(x);
     const int m4 = m / 4;
@@ -386,7 +399,7 @@ __global__ __launch_bounds__(kBlock) void gemv_t_split_kernel(const float* __res
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int c = 0; c < kGemvTCols; ++c) a[u][c] = col[c][i + u * kBlock];
+            for (int c = 0; c < kGemvTCols; ++c) a[u][c] = load4<NT>(col[c] + 4 * static_cast<size_t>(i + u * kBlock));
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const float4 xv = x4[i + u * kBlock];
@@ -399,7 +412,7 @@ __global__ __launch_bounds__(kBlock) void gemv_t_split_kernel(const float* __res
         const float4 xv = x4[i];
 #pragma unroll
         for (int c = 0; c < kGemvTCols; ++c) {
-            const float4 av = col[c][i];
+            const float4 av = load4<NT>(col[c] + 4 * static_cast<size_t>(i));
             acc[c] += av.x * xv.x + av.y * xv.y + av.z * xv.z + av.w * xv.w;
         }
     }
@@ -428,7 +441,10 @@ int gemv_impl(const float* A, const float* x, float* y, int m, int n, bool trans
                              : ThinArgs{A, 1, lda, x, 0, incx, y, incy, 0, m, n, 1, alpha, beta};
     if (trans && incx == 1 && m >= 1024 && m % 4 == 0 && lda % 4 == 0 && aligned16(A) && aligned16(x)) {
         const unsigned grid = static_cast<unsigned>((static_cast<size_t>(n) + kGemvTCols - 1) / kGemvTCols);
-        gemv_t_split_kernel<<<grid, kBlock, 0, stream()>>>(A, x, y, m, n, lda, incy, alpha, beta);
+        if (streams_past_cache(static_cast<size_t>(m) * n * sizeof(float)))
+            gemv_t_split_kernel<true><<<grid, kBlock, 0, stream()>>>(A, x, y, m, n, lda, incy, alpha, beta);
+        else
+            gemv_t_split_kernel<false><<<grid, kBlock, 0, stream()>>>(A, x, y, m, n, lda, incy, alpha, beta);
         return launch_rc();
     }
     if (thin_ok(t)) return thin_impl(t);

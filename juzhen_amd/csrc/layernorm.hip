@@ -16,7 +16,8 @@ namespace {
 constexpr float kLnEps = 1e-5f;
 
 // NV float4 per lane: dim <= 256*NV, dim % 4 == 0, 16-byte aligned columns.
-template <int NV>
+// NT: the streaming hint on the column data (launches past the cache size).
+template <int NV, bool NT>
 __global__ __launch_bounds__(kBlock) void ln_fwd_vec_kernel(float* y, float* xhat, float* inv_std,
                                                             const float* x, const float* gamma,
                                                             const float* beta, int dim, int N) {
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_vec_kernel(float* y, float* xha
         for (int v = 0; v < NV; ++v) {
             const int r = (lane + v * kWave) * 4;
             if (r < dim) {
-                xv[v] = *reinterpret_cast<const float4*>(x + base + r);
+                xv[v] = load4<NT>(x + base + r);
                 s += (xv[v].x + xv[v].y) + (xv[v].z + xv[v].w);
             }
         }
@@ -67,8 +68,8 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_vec_kernel(float* y, float* xha
                 h.x = xv[v].x * inv; h.y = xv[v].y * inv; h.z = xv[v].z * inv; h.w = xv[v].w * inv;
                 o.x = g[v].x * h.x + b[v].x; o.y = g[v].y * h.y + b[v].y;
                 o.z = g[v].z * h.z + b[v].z; o.w = g[v].w * h.w + b[v].w;
-                *reinterpret_cast<float4*>(xhat + base + r) = h;
-                *reinterpret_cast<float4*>(y + base + r) = o;
+                store4<NT>(xhat + base + r, h);
+                store4<NT>(y + base + r, o);
             }
         }
     }
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic_kernel(float* y, float*
 // JVP = false: dx = P(gamma .* dy) (+ res), the backward pass.  JVP = true:
 // out = gamma .* P(dy), the tangent through the same standardisation operator
 // P(v) = inv .* (v - mean(v) - xhat .* mean(xhat .* v)) (ml/layer.hpp:2690-2702).
-template <int NV, bool JVP>
+template <int NV, bool JVP, bool NT>
 __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const float* dy,
                                                             const float* gamma, const float* xhat,
                                                             const float* inv_std, const float* res,
@@ -130,8 +131,8 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
         for (int v = 0; v < NV; ++v) {
             const int r = (lane + v * kWave) * 4;
             if (r < dim) {
-                d[v] = *reinterpret_cast<const float4*>(dy + base + r);
-                h[v] = *reinterpret_cast<const float4*>(xhat + base + r);
+                d[v] = load4<NT>(dy + base + r);
+                h[v] = load4<NT>(xhat + base + r);
                 if constexpr (!JVP) { d[v].x *= g[v].x; d[v].y *= g[v].y; d[v].z *= g[v].z; d[v].w *= g[v].w; }
                 s1 += (d[v].x + d[v].y) + (d[v].z + d[v].w);
                 s2 += (d[v].x * h[v].x + d[v].y * h[v].y) + (d[v].z * h[v].z + d[v].w * h[v].w);
@@ -151,10 +152,10 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_vec_kernel(float* dx, const flo
                 o.w = inv * (d[v].w - m1 - h[v].w * m2);
                 if constexpr (JVP) { o.x *= g[v].x; o.y *= g[v].y; o.z *= g[v].z; o.w *= g[v].w; }
                 if (res) {  // dx = LN'(dy) + res, rounded like a separate add
-                    const float4 rr = *reinterpret_cast<const float4*>(res + base + r);
+                    const float4 rr = load4<NT>(res + base + r);
                     o.x += rr.x; o.y += rr.y; o.z += rr.z; o.w += rr.w;
                 }
-                *reinterpret_cast<float4*>(dx + base + r) = o;
+                store4<NT>(dx + base + r, o);
             }
         }
     }
@@ -232,6 +233,7 @@ __global__ __launch_bounds__(kBlock) void ln_param_partial_kernel(float* part, c
 // float4 form (dim % 4 == 0, aligned operands): a lane owns four rows, a wave
 // 256 rows; each wave walks its columns four at a time, so eight 16-byte loads
 // are in flight per lane.
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void ln_param_partial_vec_kernel(float* part, const float* dy,
                                                                       const float* xhat, int dim, int N,
                                                                       int chunk_len) {
@@ -253,8 +255,8 @@ __global__ __launch_bounds__(kBlock) void ln_param_partial_vec_kernel(float* par
                 const int cc = c + u * NW;
                 if (cc < c_end) {
                     const size_t i = static_cast<size_t>(cc) * dim + row;
-                    d[u] = *reinterpret_cast<const float4*>(dy + i);
-                    h[u] = *reinterpret_cast<const float4*>(xhat + i);
+                    d[u] = load4<NT>(dy + i);
+                    h[u] = load4<NT>(xhat + i);
                 } else {
                     d[u] = make_float4(0.f, 0.f, 0.f, 0.f);
                     h[u] = d[u];
@@ -329,12 +331,16 @@ JZ_API int jzhip_layernorm_fwd(float* y, float* xhat, float* inv_std, const floa
                      aligned16(xhat) && aligned16(gamma) && aligned16(beta);
     const unsigned grid = grid_cover(N, kBlock / kWave);
     hipStream_t s = stream();
-    if (vec && dim <= 256)
-        ln_fwd_vec_kernel<1><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
-    else if (vec && dim <= 512)
-        ln_fwd_vec_kernel<2><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
-    else if (vec)
-        ln_fwd_vec_kernel<4><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
+    const bool nt = streams_past_cache(3 * static_cast<size_t>(dim) * N * sizeof(float));
+#define JZ_LN_FWD(NV_)                                                                                        \
+    do {                                                                                                      \
+        if (nt) ln_fwd_vec_kernel<NV_, true><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);   \
+        else ln_fwd_vec_kernel<NV_, false><<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);     \
+    } while (0)
+    if (vec && dim <= 256) JZ_LN_FWD(1);
+    else if (vec && dim <= 512) JZ_LN_FWD(2);
+    else if (vec) JZ_LN_FWD(4);
+#undef JZ_LN_FWD
     else
         ln_fwd_generic_kernel<<<grid, kBlock, 0, s>>>(y, xhat, inv_std, x, gamma, beta, dim, N);
     return launch_rc();
@@ -349,12 +355,16 @@ int launch_ln_bwd(float* dx, const float* dy, const float* gamma, const float* x
                      aligned16(xhat) && aligned16(gamma) && (!res || aligned16(res));
     const unsigned grid = grid_cover(N, kBlock / kWave);
     hipStream_t s = stream();
-    if (vec && dim <= 256)
-        ln_bwd_vec_kernel<1, JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
-    else if (vec && dim <= 512)
-        ln_bwd_vec_kernel<2, JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
-    else if (vec)
-        ln_bwd_vec_kernel<4, JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+    const bool nt = streams_past_cache((res ? 4 : 3) * static_cast<size_t>(dim) * N * sizeof(float));
+#define JZ_LN_BWD(NV_)                                                                                             \
+    do {                                                                                                           \
+        if (nt) ln_bwd_vec_kernel<NV_, JVP, true><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);  \
+        else ln_bwd_vec_kernel<NV_, JVP, false><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);    \
+    } while (0)
+    if (vec && dim <= 256) JZ_LN_BWD(1);
+    else if (vec && dim <= 512) JZ_LN_BWD(2);
+    else if (vec) JZ_LN_BWD(4);
+#undef JZ_LN_BWD
     else
         ln_bwd_generic_kernel<JVP><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, dim, N);
     return launch_rc();
@@ -396,7 +406,10 @@ JZ_API int jzhip_layernorm_param_grads(float* dgamma, float* dbeta, const float*
     hipStream_t s = stream();
     dim3 grid(row_blocks, chunks);
     if (vec) {
-        ln_param_partial_vec_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
+        if (streams_past_cache(2 * static_cast<size_t>(dim) * N * sizeof(float)))
+            ln_param_partial_vec_kernel<true><<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
+        else
+            ln_param_partial_vec_kernel<false><<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
     } else {
         ln_param_partial_kernel<<<grid, kBlock, 0, s>>>(part, dy, xhat, dim, N, chunk_len);
     }

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kTile* kRowsPerPass) void ew2d_kernel(
 // leading dimensions are multiples of 4: 64x64 tiles, every global access a
 // float4, relatively transposed operands turned in LDS (pitch 65).
 constexpr int kTileV = 64;
-template <int OP>
+template <int OP, bool NT>
 __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
     float* out, size_t ldo, const float* a, size_t lda, int rel_a, const float* b, size_t ldb,
     int rel_b, size_t R, size_t C, unsigned tiles_r, float s1, float s2) {
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
         for (int k = 0; k < kTileV; k += 16) {
             const size_t r = r0 + l + k, c = c0 + 4 * q;
             if (r < R && c < C) {
-                const float4 v = *reinterpret_cast<const float4*>(x + r * ldx + c);
+                const float4 v = load4<NT>(x + r * ldx + c);
                 float* d = &t[l + k][4 * q];
                 d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
             }
@@ -108,12 +108,12 @@ __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
         if (r < R && c < C) {
             float4 va;
             if (rel_a) va = make_float4(ta[4 * q][cl], ta[4 * q + 1][cl], ta[4 * q + 2][cl], ta[4 * q + 3][cl]);
-            else va = *reinterpret_cast<const float4*>(a + c * lda + r);
+            else va = load4<NT>(a + c * lda + r);
             float4 res = va;
             if constexpr (OP != kOpCopy) {
                 float4 vb;
                 if (rel_b) vb = make_float4(tb[4 * q][cl], tb[4 * q + 1][cl], tb[4 * q + 2][cl], tb[4 * q + 3][cl]);
-                else vb = *reinterpret_cast<const float4*>(b + c * ldb + r);
+                else vb = load4<NT>(b + c * ldb + r);
                 if constexpr (OP == kOpAxpby) {
                     res.x = s1 * va.x + s2 * vb.x; res.y = s1 * va.y + s2 * vb.y;
                     res.z = s1 * va.z + s2 * vb.z; res.w = s1 * va.w + s2 * vb.w;
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
                     res.x = va.x * vb.x; res.y = va.y * vb.y; res.z = va.z * vb.z; res.w = va.w * vb.w;
                 }
             }
-            *reinterpret_cast<float4*>(out + c * ldo + r) = res;
+            store4<NT>(out + c * ldo + r, res);
         }
     }
 }
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void ew2d_vec_kernel(
 // consecutive rows of one column (1 KB runs on every operand instead of the 256 B runs of
 // the 64 x 64 tile) and a workgroup 256 rows x 16 columns.
 constexpr int kStripRows = 256, kStripCols = 16;
-template <int OP>
+template <int OP, bool NT>
 __global__ __launch_bounds__(kBlock) void ew2d_strip_kernel(float* out, size_t ldo, const float* a, size_t lda,
                                                             const float* b, size_t ldb, size_t R, size_t C,
                                                             unsigned strips_r, float s1, float s2) {
@@ -143,10 +143,10 @@ __global__ __launch_bounds__(kBlock) void ew2d_strip_kernel(float* out, size_t l
     for (int k = 0; k < kStripCols; k += kBlock / kWave) {
         const size_t c = c0 + k;
         if (c < C) {
-            const float4 va = *reinterpret_cast<const float4*>(a + c * lda + r);
+            const float4 va = load4<NT>(a + c * lda + r);
             float4 res = va;
             if constexpr (OP != kOpCopy) {
-                const float4 vb = *reinterpret_cast<const float4*>(b + c * ldb + r);
+                const float4 vb = load4<NT>(b + c * ldb + r);
                 if constexpr (OP == kOpAxpby) {
                     res.x = s1 * va.x + s2 * vb.x; res.y = s1 * va.y + s2 * vb.y;
                     res.z = s1 * va.z + s2 * vb.z; res.w = s1 * va.w + s2 * vb.w;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(kBlock) void ew2d_strip_kernel(float* out, size_t l
                     res.x = va.x * vb.x; res.y = va.y * vb.y; res.z = va.z * vb.z; res.w = va.w * vb.w;
                 }
             }
-            *reinterpret_cast<float4*>(out + c * ldo + r) = res;
+            store4<NT>(out + c * ldo + r, res);
         }
     }
 }
@@ -165,19 +165,28 @@ int launch2d(float* out, size_t ldo, const float* a, size_t lda, int rel_a, cons
     if (R == 0 || C == 0) return 0;
     const bool vec = R % 4 == 0 && C % 4 == 0 && ldo % 4 == 0 && lda % 4 == 0 && aligned16(out) && aligned16(a) &&
                      (OP == kOpCopy || (ldb % 4 == 0 && aligned16(b)));
+    const bool past_cache = streams_past_cache((OP == kOpCopy ? 2 : 3) * R * C * sizeof(float));
     if (vec && !rel_a && (OP == kOpCopy || !rel_b) && R >= 128) {
         const size_t sr = (R + kStripRows - 1) / kStripRows, sc = (C + kStripCols - 1) / kStripCols;
         if (sr * sc <= 0x7fffffffull) {
-            ew2d_strip_kernel<OP><<<static_cast<unsigned>(sr * sc), kBlock, 0, stream()>>>(
-                out, ldo, a, lda, b, ldb, R, C, static_cast<unsigned>(sr), s1, s2);
+            if (past_cache)
+                ew2d_strip_kernel<OP, true><<<static_cast<unsigned>(sr * sc), kBlock, 0, stream()>>>(
+                    out, ldo, a, lda, b, ldb, R, C, static_cast<unsigned>(sr), s1, s2);
+            else
+                ew2d_strip_kernel<OP, false><<<static_cast<unsigned>(sr * sc), kBlock, 0, stream()>>>(
+                    out, ldo, a, lda, b, ldb, R, C, static_cast<unsigned>(sr), s1, s2);
             return launch_rc();
         }
     }
     if (vec) {
         const size_t tr = (R + kTileV - 1) / kTileV, tc = (C + kTileV - 1) / kTileV;
         if (tr * tc > 0x7fffffffull) return -1;
-        ew2d_vec_kernel<OP><<<static_cast<unsigned>(tr * tc), kBlock, 0, stream()>>>(
-            out, ldo, a, lda, rel_a, b, ldb, rel_b, R, C, static_cast<unsigned>(tr), s1, s2);
+        if (past_cache)
+            ew2d_vec_kernel<OP, true><<<static_cast<unsigned>(tr * tc), kBlock, 0, stream()>>>(
+                out, ldo, a, lda, rel_a, b, ldb, rel_b, R, C, static_cast<unsigned>(tr), s1, s2);
+        else
+            ew2d_vec_kernel<OP, false><<<static_cast<unsigned>(tr * tc), kBlock, 0, stream()>>>(
+                out, ldo, a, lda, rel_a, b, ldb, rel_b, R, C, static_cast<unsigned>(tr), s1, s2);
         return launch_rc();
     }
     const size_t tiles_r = (R + kTile - 1) / kTile;

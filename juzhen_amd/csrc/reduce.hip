@@ -16,7 +16,7 @@ namespace {
 // One wavefront per (column, row-chunk).  VEC=4 uses float4 loads and needs
 // ld % 4 == 0, a 16-byte aligned base and chunk boundaries that are multiples
 // of 4.
-template <int VEC>
+template <int VEC, bool NT = false>
 __global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const float* a, int numrow,
                                                           int numcol, size_t ld, int chunks,
                                                           int chunk_len) {
@@ -38,10 +38,10 @@ __global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const floa
             // four float4 loads in flight per lane (4 KB per wave), then two
             float acc2 = 0.f, acc3 = 0.f;
             for (; r + 3 * kWave * 4 < v_end; r += 4 * kWave * 4) {
-                const float4 x = *reinterpret_cast<const float4*>(p + r);
-                const float4 y = *reinterpret_cast<const float4*>(p + r + kWave * 4);
-                const float4 z = *reinterpret_cast<const float4*>(p + r + 2 * kWave * 4);
-                const float4 w = *reinterpret_cast<const float4*>(p + r + 3 * kWave * 4);
+                const float4 x = load4<NT>(p + r);
+                const float4 y = load4<NT>(p + r + kWave * 4);
+                const float4 z = load4<NT>(p + r + 2 * kWave * 4);
+                const float4 w = load4<NT>(p + r + 3 * kWave * 4);
                 acc0 += (x.x + x.y) + (x.z + x.w);
                 acc1 += (y.x + y.y) + (y.z + y.w);
                 acc2 += (z.x + z.y) + (z.z + z.w);
@@ -50,13 +50,13 @@ __global__ __launch_bounds__(kBlock) void sum_cols_kernel(float* out, const floa
             acc0 += acc2;
             acc1 += acc3;
             for (; r + kWave * 4 < v_end; r += 2 * kWave * 4) {
-                const float4 x = *reinterpret_cast<const float4*>(p + r);
-                const float4 y = *reinterpret_cast<const float4*>(p + r + kWave * 4);
+                const float4 x = load4<NT>(p + r);
+                const float4 y = load4<NT>(p + r + kWave * 4);
                 acc0 += (x.x + x.y) + (x.z + x.w);
                 acc1 += (y.x + y.y) + (y.z + y.w);
             }
             for (; r < v_end; r += kWave * 4) {
-                const float4 x = *reinterpret_cast<const float4*>(p + r);
+                const float4 x = load4<NT>(p + r);
                 acc0 += (x.x + x.y) + (x.z + x.w);
             }
             for (int t = v_end + lane; t < r_end; t += kWave) acc1 += p[t];
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kCombineBlock) void combine_partials_kernel(float* 
 // Lanes run along rows (the contiguous dimension); the four waves of a block
 // take interleaved columns of the block's column chunk and are combined
 // through LDS.  VEC rows per lane.
-template <int VEC>
+template <int VEC, bool NT = false>
 __global__ __launch_bounds__(kBlock) void sum_rows_kernel(float* out, const float* a, int numrow,
                                                           int numcol, size_t ld, int chunk_len) {
     constexpr int NW = kBlock / kWave;
@@ -128,14 +128,14 @@ __global__ __launch_bounds__(kBlock) void sum_rows_kernel(float* out, const floa
             // numrow % 4 == 0 is guaranteed by the launcher
             int c = c_begin + wave;
             for (; c + NW < c_end; c += 2 * NW) {
-                const float4 x = *reinterpret_cast<const float4*>(a + static_cast<size_t>(c) * ld + row);
+                const float4 x = load4<NT>(a + static_cast<size_t>(c) * ld + row);
                 const float4 y =
-                    *reinterpret_cast<const float4*>(a + static_cast<size_t>(c + NW) * ld + row);
+                    load4<NT>(a + static_cast<size_t>(c + NW) * ld + row);
                 acc[0] += x.x; acc[1] += x.y; acc[2] += x.z; acc[3] += x.w;
                 acc[0] += y.x; acc[1] += y.y; acc[2] += y.z; acc[3] += y.w;
             }
             for (; c < c_end; c += NW) {
-                const float4 x = *reinterpret_cast<const float4*>(a + static_cast<size_t>(c) * ld + row);
+                const float4 x = load4<NT>(a + static_cast<size_t>(c) * ld + row);
                 acc[0] += x.x; acc[1] += x.y; acc[2] += x.z; acc[3] += x.w;
             }
         } else {
@@ -192,6 +192,7 @@ __global__ __launch_bounds__(kBlock) void sum_rows_short_kernel(float* part, con
 }
 
 // ── flat sum of squares (norm) ───────────────────────────────────────────
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(float* part, const float* x, size_t n,
                                                                int vec_ok) {
     __shared__ float red[kBlock / kWave];
@@ -203,12 +204,12 @@ __global__ __launch_bounds__(kBlock) void sumsq_partial_kernel(float* part, cons
         const float4* x4 = reinterpret_cast<const float4*>(x);
         size_t i = tid;
         for (; i + stride < n4; i += 2 * stride) {
-            const float4 p = x4[i], q = x4[i + stride];
+            const float4 p = load4<NT>(x + 4 * i), q = load4<NT>(x + 4 * (i + stride));
             acc0 += (p.x * p.x + p.y * p.y) + (p.z * p.z + p.w * p.w);
             acc1 += (q.x * q.x + q.y * q.y) + (q.z * q.z + q.w * q.w);
         }
         if (i < n4) {
-            const float4 p = x4[i];
+            const float4 p = load4<NT>(x + 4 * i);
             acc0 += (p.x * p.x + p.y * p.y) + (p.z * p.z + p.w * p.w);
         }
         for (size_t j = n4 * 4 + tid; j < n; j += stride) acc1 += x[j] * x[j];
@@ -231,6 +232,7 @@ __global__ __launch_bounds__(kBlock) void sqrt_sum_kernel(float* out, const floa
 // (LossLayer::eval, ml/layer.hpp:223-226: difference, square, two sums and a scaling as five
 // matrix operations; here the differences and squares round the same way and the sums run
 // over the flat buffer.)  A single workgroup writes the scaled result itself.
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void sqdiff_partial_kernel(float* part, const float* __restrict__ target,
                                                                 const float* __restrict__ pred, size_t n,
                                                                 float scale) {
@@ -240,7 +242,8 @@ __global__ __launch_bounds__(kBlock) void sqdiff_partial_kernel(float* part, con
     float acc0 = 0.f, acc1 = 0.f;
     size_t i = tid;
     for (; i + stride < n; i += 2 * stride) {
-        const float d0 = target[i] - pred[i], d1 = target[i + stride] - pred[i + stride];
+        const float d0 = load1<NT>(target + i) - load1<NT>(pred + i);
+        const float d1 = load1<NT>(target + i + stride) - load1<NT>(pred + i + stride);
         acc0 += d0 * d0;
         acc1 += d1 * d1;
     }
@@ -261,7 +264,7 @@ __global__ __launch_bounds__(kBlock) void scaled_sum_kernel(float* out, const fl
 }
 
 // ── column max / argmax: one wavefront per column ────────────────────────
-template <bool ARG>
+template <bool ARG, bool NT>
 __global__ __launch_bounds__(kBlock) void max_cols_kernel(float* out_val, int32_t* out_idx,
                                                           const float* a, int numrow, int numcol,
                                                           size_t ld) {
@@ -283,7 +286,7 @@ __global__ __launch_bounds__(kBlock) void max_cols_kernel(float* out_val, int32_
         for (; r + 7 * kWave < numrow; r += 8 * kWave) {
             float v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = p[r + u * kWave];
+            for (int u = 0; u < 8; ++u) v[u] = load1<NT>(p + r + u * kWave);
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 if (best < v[u]) {
@@ -352,7 +355,9 @@ JZ_API int jzhip_sum_cols(float* out, const float* a, int numrow, int numcol, in
     const size_t items = static_cast<size_t>(numcol) * chunks;
     const unsigned grid = grid_cover(items, kBlock / kWave);
     hipStream_t s = stream();
-    if (vec)
+    if (vec && streams_past_cache(static_cast<size_t>(numrow) * numcol * sizeof(float)))
+        sum_cols_kernel<4, true><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
+    else if (vec)
         sum_cols_kernel<4><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
     else
         sum_cols_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunks, chunk_len);
@@ -412,7 +417,9 @@ int sum_rows_impl(float* out, const float* a, int numrow, int numcol, int ld, si
         if (!dst) return -2;
     }
     dim3 grid(row_blocks, chunks);
-    if (vec)
+    if (vec && streams_past_cache(static_cast<size_t>(numrow) * numcol * sizeof(float)))
+        sum_rows_kernel<4, true><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
+    else if (vec)
         sum_rows_kernel<4><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
     else
         sum_rows_kernel<1><<<grid, kBlock, 0, s>>>(dst, a, numrow, numcol, ld, chunk_len);
@@ -439,7 +446,10 @@ JZ_API int jzhip_nrm2(float* out_device, const float* x, size_t count) {
     if (!part) return -2;
     const unsigned grid = grid_for(count / 4 + 1, static_cast<size_t>(kBlock) * 2, 4);
     hipStream_t s = stream();
-    sumsq_partial_kernel<<<grid, kBlock, 0, s>>>(part, x, count, aligned16(x) ? 1 : 0);
+    if (streams_past_cache(count * sizeof(float)))
+        sumsq_partial_kernel<true><<<grid, kBlock, 0, s>>>(part, x, count, aligned16(x) ? 1 : 0);
+    else
+        sumsq_partial_kernel<false><<<grid, kBlock, 0, s>>>(part, x, count, aligned16(x) ? 1 : 0);
     sqrt_sum_kernel<<<1, kBlock, 0, s>>>(out_device, part, static_cast<int>(grid));
     return launch_rc();
 }
@@ -450,13 +460,16 @@ JZ_API int jzhip_mse_loss(float* out_device, const float* target, const float* p
     if (!target || !pred) return -1;
     hipStream_t s = stream();
     if (count <= static_cast<size_t>(kBlock) * 32) {
-        sqdiff_partial_kernel<<<1, kBlock, 0, s>>>(out_device, target, pred, count, scale);
+        sqdiff_partial_kernel<false><<<1, kBlock, 0, s>>>(out_device, target, pred, count, scale);
         return launch_rc();
     }
     float* part = workspace();
     if (!part) return -2;
     const unsigned grid = grid_for(count, static_cast<size_t>(kBlock) * 2, 4);
-    sqdiff_partial_kernel<<<grid, kBlock, 0, s>>>(part, target, pred, count, scale);
+    if (streams_past_cache(2 * count * sizeof(float)))
+        sqdiff_partial_kernel<true><<<grid, kBlock, 0, s>>>(part, target, pred, count, scale);
+    else
+        sqdiff_partial_kernel<false><<<grid, kBlock, 0, s>>>(part, target, pred, count, scale);
     if (grid > 1) scaled_sum_kernel<<<1, kBlock, 0, s>>>(out_device, part, static_cast<int>(grid), scale);
     else return jzhip_copy(out_device, part, 1);
     return launch_rc();
@@ -465,14 +478,20 @@ JZ_API int jzhip_mse_loss(float* out_device, const float* target, const float* p
 JZ_API int jzhip_max_cols(float* out, const float* a, int numrow, int numcol, int ld) {
     if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
     const unsigned grid = grid_cover(numcol, kBlock / kWave);
-    max_cols_kernel<false><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
+    if (streams_past_cache(static_cast<size_t>(numrow) * numcol * sizeof(float)))
+        max_cols_kernel<false, true><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
+    else
+        max_cols_kernel<false, false><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
     return launch_rc();
 }
 
 JZ_API int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numcol, int ld) {
     if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
     const unsigned grid = grid_cover(numcol, kBlock / kWave);
-    max_cols_kernel<true><<<grid, kBlock, 0, stream()>>>(nullptr, out, a, numrow, numcol, ld);
+    if (streams_past_cache(static_cast<size_t>(numrow) * numcol * sizeof(float)))
+        max_cols_kernel<true, true><<<grid, kBlock, 0, stream()>>>(nullptr, out, a, numrow, numcol, ld);
+    else
+        max_cols_kernel<true, false><<<grid, kBlock, 0, stream()>>>(nullptr, out, a, numrow, numcol, ld);
     return launch_rc();
 }
 
