@@ -256,6 +256,7 @@ inline Matrix<ROCMfloat> adam_update(Matrix<ROCMfloat>&& g, adam_state<ROCMfloat
 // on overwriting its input while it selects minima).
 
 namespace jzrocm {
+constexpr size_t kStreamingBytes = size_t(512) << 20;   // launches from this size on stream past the caches
 constexpr int kThreads = 256;
 inline hipStream_t stream() { return static_cast<hipStream_t>(jzhip_get_stream()); }
 inline unsigned grid_cover(size_t items) {
@@ -265,21 +266,26 @@ inline unsigned grid_cover(size_t items) {
     return static_cast<unsigned>(need);
 }
 
-template <class Function>
+// NT: loads and stores with the non-temporal hint, for launches that move more than the
+// last-level cache can hold (a map over 2^28 floats: 6.1 -> 6.5 TB/s).
+template <bool NT, class Function>
 __global__ __launch_bounds__(kThreads) void elemwise_kernel(Function func, float* dst,
                                                             const float* src, size_t n, int vec) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
     const size_t stride = static_cast<size_t>(gridDim.x) * kThreads;
     const size_t tid = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (vec) {
         const size_t n4 = n / 4;
         for (size_t i = tid; i < n4; i += stride) {
-            const float4 x = reinterpret_cast<const float4*>(src)[i];
-            float4 y;
+            f4 x, y;
+            if constexpr (NT) x = __builtin_nontemporal_load(reinterpret_cast<const f4*>(src) + i);
+            else x = reinterpret_cast<const f4*>(src)[i];
             y.x = func(x.x);
             y.y = func(x.y);
             y.z = func(x.z);
             y.w = func(x.w);
-            reinterpret_cast<float4*>(dst)[i] = y;
+            if constexpr (NT) __builtin_nontemporal_store(y, reinterpret_cast<f4*>(dst) + i);
+            else reinterpret_cast<f4*>(dst)[i] = y;
         }
         for (size_t j = n4 * 4 + tid; j < n; j += stride) dst[j] = func(src[j]);
     } else {
@@ -379,8 +385,12 @@ Matrix<ROCMfloat> elemwise(Function func, const Matrix<ROCMfloat>& M) {
     Matrix<ROCMfloat> result("resM", M.numrow, M.numcol, M.transpose);
     const size_t n = M.count();
     const int vec = ((reinterpret_cast<uintptr_t>(M.dev()) | reinterpret_cast<uintptr_t>(result.dev())) & 15) == 0;
-    jzrocm::elemwise_kernel<<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
-        func, result.dev(), M.dev(), n, vec);
+    if (n * 2 * sizeof(float) >= jzrocm::kStreamingBytes)
+        jzrocm::elemwise_kernel<true><<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+            func, result.dev(), M.dev(), n, vec);
+    else
+        jzrocm::elemwise_kernel<false><<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+            func, result.dev(), M.dev(), n, vec);
     return result;
 }
 
@@ -388,8 +398,12 @@ template <class Function>
 Matrix<ROCMfloat> elemwise(Function func, Matrix<ROCMfloat>&& M) {
     const size_t n = M.count();
     const int vec = (reinterpret_cast<uintptr_t>(M.dev()) & 15) == 0;
-    jzrocm::elemwise_kernel<<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
-        func, M.dev(), M.dev(), n, vec);
+    if (n * sizeof(float) >= jzrocm::kStreamingBytes)   // in place: one buffer
+        jzrocm::elemwise_kernel<true><<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+            func, M.dev(), M.dev(), n, vec);
+    else
+        jzrocm::elemwise_kernel<false><<<jzrocm::grid_cover(vec ? n / 4 + 1 : n), jzrocm::kThreads, 0, jzrocm::stream()>>>(
+            func, M.dev(), M.dev(), n, vec);
     return std::move(M);
 }
 

@@ -82,6 +82,11 @@ __device__ __forceinline__ float load1(const float* p) {
     else return *p;
 }
 template <bool NT>
+__device__ __forceinline__ void store1(float* p, float v) {
+    if constexpr (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+template <bool NT>
 __device__ __forceinline__ void store4(float* p, const float4& v) {
     if constexpr (NT) {
         jz_f4 t;

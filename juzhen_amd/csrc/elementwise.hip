@@ -158,7 +158,10 @@ int launch_ew(F f, float* out, const float* a, const float* b, size_t n) {
         const int tail = static_cast<int>(n % 4);
         const size_t blocks = n4 ? (n4 + kBlock - 1) / kBlock : 1;
         if (blocks > 0x7fffffffull) return -1;
-        if (NIN >= 1 && streams_past_cache((NIN + 1) * n * sizeof(float)))   // (a fill is as fast without the hint)
+        // distinct buffers of the launch (an in-place form keeps its one buffer in the cache
+        // for twice as long); a fill is as fast without the hint
+        const int buffers = 1 + (NIN >= 1 && a != out) + (NIN >= 2 && b != out && b != a);
+        if (NIN >= 1 && streams_past_cache(buffers * n * sizeof(float)))
             ew_vec_kernel<NIN, F, true><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(f, out, a, b, n4, tail);
         else
             ew_vec_kernel<NIN, F, false><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(f, out, a, b, n4, tail);

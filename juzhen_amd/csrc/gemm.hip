@@ -845,7 +845,7 @@ JZ_API int jzhip_add_bias(float* y, const float* b, int rows, int cols) {
     if (rows <= 0 || cols <= 0 || !y || !b) return -1;
     const size_t total = static_cast<size_t>(rows) * cols;
     if (rows % 4 == 0 && aligned16(y) && aligned16(b)) {
-        if (streams_past_cache(2 * total * sizeof(float)))
+        if (streams_past_cache(total * sizeof(float)))   // in place: one buffer
             add_bias_kernel<true><<<grid_cover(total / 4, kBlock), kBlock, 0, stream()>>>(y, b, rows, total / 4);
         else
             add_bias_kernel<false><<<grid_cover(total / 4, kBlock), kBlock, 0, stream()>>>(y, b, rows, total / 4);

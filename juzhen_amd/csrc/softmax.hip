@@ -274,6 +274,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(float* out, co
 // part layout: [chunk][2][numrow]; rowstat layout: [2][numrow].
 constexpr int kRowUnroll = 8;
 
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* part, const float* in,
                                                                       int numrow, int numcol,
                                                                       size_t ld, int chunk_len) {
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_partial_kernel(float* par
 #pragma unroll
             for (int u = 0; u < kRowUnroll; ++u) {
                 const int cc = c + u * CP;
-                t[u] = cc < c1 ? in[static_cast<size_t>(cc) * ld + row] : -1e30f;
+                t[u] = cc < c1 ? load1<NT>(in + static_cast<size_t>(cc) * ld + row) : -1e30f;
                 tm = tm > t[u] ? tm : t[u];
             }
             const float mn = m > tm ? m : tm;
@@ -366,6 +367,7 @@ __global__ __launch_bounds__(kFoldThreads) void softmax_rows_fold_kernel(float* 
     }
 }
 
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, const float* in,
                                                                     const float* rowstat, int numrow,
                                                                     int numcol, size_t ld,
@@ -382,12 +384,12 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, 
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int cc = c + u * CP;
-            t[u] = cc < c1 ? in[static_cast<size_t>(cc) * ld + row] : 0.f;
+            t[u] = cc < c1 ? load1<NT>(in + static_cast<size_t>(cc) * ld + row) : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int cc = c + u * CP;
-            if (cc < c1) out[static_cast<size_t>(cc) * ld + row] = exp_neg(t[u] - M) * inv;
+            if (cc < c1) store1<NT>(out + static_cast<size_t>(cc) * ld + row, exp_neg(t[u] - M) * inv);
         }
     }
 }
@@ -746,9 +748,12 @@ int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_
             if (!part) return -2;
             float* rowstat = part + static_cast<size_t>(chunks) * numrow * 2;
             dim3 grid(row_blocks, chunks);
-            softmax_rows_partial_kernel<<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
+            const bool nt = streams_past_cache(static_cast<size_t>(numrow) * numcol * sizeof(float));
+            if (nt) softmax_rows_partial_kernel<true><<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
+            else softmax_rows_partial_kernel<false><<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
             softmax_rows_fold_kernel<<<row_blocks, kFoldThreads, 0, s>>>(rowstat, part, numrow, chunks);
-            softmax_rows_apply_kernel<<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
+            if (nt) softmax_rows_apply_kernel<true><<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
+            else softmax_rows_apply_kernel<false><<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
             return launch_rc();
         }
     }
