@@ -63,7 +63,11 @@ def test_argument_validation_without_gpu():
     assert lib.jzhip_im2col(None, None, 1, 4, 4, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
     assert lib.jzhip_layernorm_fwd(None, None, None, None, None, None, 8, 8) == -1
     assert lib.jzhip_adam_update(None, None, None, 4, 1e-3, 0.9, 0.999, 1e-8, 1) == -1
-    assert lib.jzhip_fill(None, 0, 1.0) == 0          # empty input is a no-op
+    assert lib.jzhip_softmax_xent_dense(None, None, None, None, 4, 4, 4, 0.25) == -1
+    assert lib.jzhip_mse_loss(None, None, None, 4, 1.0) == -1
+    assert lib.jzhip_mse_grad(None, None, None, 4, 1.0) == -1
+    assert lib.jzhip_mse_grad(None, None, None, 0, 1.0) == 0   # empty input is a no-op
+    assert lib.jzhip_fill(None, 0, 1.0) == 0
     assert lib.jzhip_error_string(-1).decode().startswith("jzhip")
     assert lib.jzhip_version() >= 100
 
