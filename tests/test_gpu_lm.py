@@ -148,7 +148,7 @@ def torch_twin(cfg, params, tokens, steps, lr, wd):
             x = R + p("W2") @ torch.nn.functional.gelu(f1) + p("b2")
         logits = P["embed"].T @ x                                       # (V, N)
         loss = torch.nn.functional.cross_entropy(logits.T, tgt)
-        losses.append(float(loss))
+        losses.append(float(loss.detach()))
         opt.zero_grad()
         loss.backward()
         if not first_grads:
