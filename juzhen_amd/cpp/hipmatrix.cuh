@@ -256,7 +256,7 @@ inline Matrix<ROCMfloat> adam_update(Matrix<ROCMfloat>&& g, adam_state<ROCMfloat
 // on overwriting its input while it selects minima).
 
 namespace jzrocm {
-constexpr size_t kStreamingBytes = size_t(512) << 20;   // launches from this size on stream past the caches
+constexpr size_t kStreamingBytes = size_t(384) << 20;   // launches from this size on stream past the caches
 constexpr int kThreads = 256;
 inline hipStream_t stream() { return static_cast<hipStream_t>(jzhip_get_stream()); }
 inline unsigned grid_cover(size_t items) {

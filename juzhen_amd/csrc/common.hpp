@@ -53,15 +53,16 @@ inline unsigned grid_cover(size_t work, size_t per_block) {
     return static_cast<unsigned>(need);
 }
 
-// A launch that moves twice what the 256 MB last-level cache holds gains nothing from
+// A launch that moves one and a half times what the 256 MB last-level cache holds gains nothing from
 // keeping its data there; its loads and stores then carry the non-temporal hint (a copy of
 // 2 GB: 6.1 -> 6.4 TB/s, of 0.5 GB 5.8 -> 6.4; column sums of 1 GB 5.5 -> 6.3).  Below
 // that size the plain forms stay: what one kernel writes the next one often reads back out
 // of the cache (hinted loads of a 134 MB operand that was resident ran 15 % slower, a
-// 268 MB slice 7-30 % slower).  Kernels that profit from the cache for longer (the
+// 268 MB slice 7-30 % slower; a product of two 134 MB operands into a third, 403 MB in all, is the
+// smallest launch measured that gains: 5.5 -> 6.3 TB/s).  Kernels that profit from the cache for longer (the
 // optimiser's moments from step to step, a column softmax that holds whole columns in
 // registers) ask with a fraction of their bytes.
-constexpr size_t kStreamingBytes = size_t(512) << 20;
+constexpr size_t kStreamingBytes = size_t(384) << 20;
 inline bool streams_past_cache(size_t bytes) { return bytes >= kStreamingBytes; }
 
 // ── wave64 reductions: DPP inside a 16-lane row, bpermute across rows ────

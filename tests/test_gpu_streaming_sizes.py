@@ -1,4 +1,4 @@
-"""The bandwidth-bound kernels at launch sizes of 512 MB and more, where their loads and
+"""The bandwidth-bound kernels at launch sizes of 512 MB and more (the threshold is 384 MB), where their loads and
 stores carry the non-temporal hint (a separate template instance of every kernel).
 
 A hinted launch must produce what the plain launch produces.  Elementwise forms are run
