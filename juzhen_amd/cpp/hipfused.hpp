@@ -409,6 +409,27 @@ inline Matrix<ROCMfloat> fused_product(const Matrix<ROCMfloat>& W, bool transpos
     return out;
 }
 // LayerNorm::backward followed by `+ residual` (ml/layer.hpp:3309, 3371) as one pass over dy
+// The three projections of a block can share a launch when their weights are stored alike
+// (plain column-major, equal shapes) and the input is plain too.
+inline bool qkv_as_one_launch(const Matrix<ROCMfloat>& Wq, const Matrix<ROCMfloat>& Wk, const Matrix<ROCMfloat>& Wv,
+                              const Matrix<ROCMfloat>& x) {
+    auto same = [&](const Matrix<ROCMfloat>& W) {
+        return !W.get_transpose() && W.num_row() == Wq.num_row() && W.num_col() == Wq.num_col();
+    };
+    return same(Wq) && same(Wk) && same(Wv) && !x.get_transpose() && x.num_row() == Wq.num_col() &&
+           Wq.num_row() > 0 && Wq.num_col() > 0 && x.num_col() > 0;
+}
+// a, b, c (equal shapes, plain) copied back to back into one buffer
+inline Matrix<ROCMfloat> stacked_blocks(const char* name, const Matrix<ROCMfloat>& a, const Matrix<ROCMfloat>& b,
+                                        const Matrix<ROCMfloat>& c) {
+    const size_t n = a.num_row() * a.num_col();
+    Matrix<ROCMfloat> out = JzRocmFused::make(name, a.num_row(), 3 * a.num_col(), 0);
+    must(jzhip_copy(p(out), p(a), n), "copy");
+    must(jzhip_copy(p(out) + n, p(b), n), "copy");
+    must(jzhip_copy(p(out) + 2 * n, p(c), n), "copy");
+    return out;
+}
+
 inline Matrix<ROCMfloat> ln_backward_plus(LayerNorm<ROCMfloat>& ln, Matrix<ROCMfloat>&& dy,
                                           const Matrix<ROCMfloat>& residual, bool update) {
     if (dy.get_transpose() || residual.get_transpose()) return ln.backward(std::move(dy), update) + residual;
@@ -440,9 +461,24 @@ inline void TransformerLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input_in)
     const int N = seq_len * batchN;
     // pre-norm attention
     cached_x1 = ln1.forward(input);
-    cached_Q = Wq * cached_x1;
-    cached_K = Wk * cached_x1;
-    cached_V = Wv * cached_x1;
+    if (qkv_as_one_launch(Wq, Wk, Wv, cached_x1)) {
+        // Q, K, V = Wq x1, Wk x1, Wv x1 as one strided-batched launch: the weights copied into
+        // three consecutive blocks, the results three consecutive blocks of one buffer (three
+        // products of 512 tiles each fill half the chip; together they run as one and a half rounds)
+        const size_t wsz = (size_t)d_k * d_model, qsz = (size_t)d_k * N;
+        MD wblk = stacked_blocks("wqkv", Wq, Wk, Wv);
+        MD qkv = JzRocmFused::make("qkv", d_k, 3 * (size_t)N, 0);
+        must(jzhip_gemm_strided_batched(p(wblk), p(cached_x1), p(qkv), d_k, N, d_model, 0, 0, d_k, d_model, d_k,
+                                        (long long)wsz, 0, (long long)qsz, 3, 1.0f, 0.0f),
+             "gemm_strided_batched");
+        cached_Q = JzRocmFused::block("tq", qkv, 0, d_k, N);
+        cached_K = JzRocmFused::block("tk", qkv, qsz, d_k, N);
+        cached_V = JzRocmFused::block("tv", qkv, 2 * qsz, d_k, N);
+    } else {
+        cached_Q = Wq * cached_x1;
+        cached_K = Wk * cached_x1;
+        cached_V = Wv * cached_x1;
+    }
     must(jzhip_attention_fwd(p(cached_H), p(cached_A), p(cached_Q), p(cached_K), p(cached_V), d_k, num_heads,
                              seq_len, batchN, causal ? 1 : 0),
          "attention_fwd");
@@ -480,14 +516,30 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
     MD dH = Wo.T() * dR;
 
     // attention core, all heads and sequences at once
-    MD dQ("dQ", d_k, N), dK("dK", d_k, N), dV("dV", d_k, N);
+    // (three blocks of one buffer, so that the weight gradients below can be one batched launch)
+    MD dqkv = JzRocmFused::make("dqkv", d_k, 3 * (size_t)N, 0);
+    const size_t qsz = (size_t)d_k * N, wsz = (size_t)d_k * d_model;
+    MD dQ = JzRocmFused::block("dQ", dqkv, 0, d_k, N), dK = JzRocmFused::block("dK", dqkv, qsz, d_k, N),
+       dV = JzRocmFused::block("dV", dqkv, 2 * qsz, d_k, N);
     must(jzhip_attention_bwd(p(dQ), p(dK), p(dV), p(attn_dS_scratch), p(dH), p(cached_Q), p(cached_K),
                              p(cached_V), p(cached_A), d_k, num_heads, seq_len, batchN),
          "attention_bwd");
 
-    MD dWq = dQ * cached_x1.T();
-    MD dWk = dK * cached_x1.T();
-    MD dWv = dV * cached_x1.T();
+    MD dWq = JzRocmFused::make("dWq", 0, 0, 0), dWk = JzRocmFused::make("dWk", 0, 0, 0), dWv = JzRocmFused::make("dWv", 0, 0, 0);
+    if (qkv_as_one_launch(Wq, Wk, Wv, cached_x1)) {
+        // dW_i = dX_i x1^T for the three projections: one batched launch, K split over the tokens
+        MD dw = JzRocmFused::make("dwqkv", d_k, 3 * (size_t)d_model, 0);
+        must(jzhip_gemm_strided_batched(p(dqkv), p(cached_x1), p(dw), d_k, d_model, N, 0, 1, d_k, d_model, d_k,
+                                        (long long)qsz, 0, (long long)wsz, 3, 1.0f, 0.0f),
+             "gemm_strided_batched");
+        dWq = JzRocmFused::block("dWq", dw, 0, d_k, d_model);
+        dWk = JzRocmFused::block("dWk", dw, wsz, d_k, d_model);
+        dWv = JzRocmFused::block("dWv", dw, 2 * wsz, d_k, d_model);
+    } else {
+        dWq = dQ * cached_x1.T();
+        dWk = dK * cached_x1.T();
+        dWv = dV * cached_x1.T();
+    }
     // dx1 = Wq^T dQ + Wk^T dK + Wv^T dV: the second and third products add into the first
     MD dx1 = Wq.T() * dQ;
     auto add_product = [&](const MD& W, const MD& g) {

@@ -189,6 +189,12 @@ struct JzRocmFused {
     static Matrix<ROCMfloat> make(const char* name, size_t r, size_t c, int trans) {
         return Matrix<ROCMfloat>(name, r, c, trans);
     }
+    // A dense r x c matrix that starts `offset` floats into M's buffer and keeps that buffer alive
+    // (several matrices laid out back to back for one strided-batched launch).
+    static Matrix<ROCMfloat> block(const char* name, const Matrix<ROCMfloat>& M, size_t offset, size_t r, size_t c) {
+        std::shared_ptr<ROCMfloat[]> alias(M.elements, M.elements.get() + offset);
+        return Matrix<ROCMfloat>(name, r, c, 0, alias);
+    }
     static size_t phys_rows(const Matrix<ROCMfloat>& M) { return M.numrow; }
     static size_t phys_cols(const Matrix<ROCMfloat>& M) { return M.numcol; }
     // Materialise the logical transpose of M as a plain (flag 0) matrix.

@@ -531,7 +531,10 @@ int launch_tile(const GemmArgs& g) {
     int splits = 1;
     const long long tiles = static_cast<long long>(tiles_m) * tiles_n * g.batch * g.batch2;
     const long long cus = num_cus();
-    if (g.batch * g.batch2 == 1 && tiles * 2 <= cus && g.K >= 256 && !g.ep.any) {
+    // (also for a handful of batched problems: the three weight gradients of a block's
+    // Q, K, V projections as one launch; each problem keeps its own run of partials)
+    const int nb = g.batch * g.batch2;
+    if (nb <= 8 && tiles * 2 <= cus && g.K >= 256 && !g.ep.any) {
         splits = static_cast<int>((cus * 2 + tiles - 1) / tiles);
         // The K chunk is the fastest-varying part of the workgroup id and
         // workgroups are dealt round-robin to 8 XCDs: with a count that divides 8
@@ -561,7 +564,7 @@ int launch_tile(const GemmArgs& g) {
         // gradients) is still cut, down to four steps, because a handful of
         // workgroups walking it alone only wait for their loads
         const int max_by_k = g.K >= 1024 ? g.K / 256 : g.K / 64;
-        const size_t per = static_cast<size_t>(g.M) * g.N;
+        const size_t per = static_cast<size_t>(g.M) * g.N * nb;
         while (splits > 1 && (splits > max_by_k || per * splits > kWorkspaceFloats))
             splits = splits > 8 ? splits - 8 : splits / 2;
         if (splits < 2) splits = 1;
@@ -571,6 +574,7 @@ int launch_tile(const GemmArgs& g) {
     size_t ldc = g.ldc;
     float alpha = g.alpha, beta = g.beta;
     long long split_stride = 0;
+    long long sC = g.sC, sC2 = g.sC2;
     if (splits > 1) {
         k_chunk = ((g.K + splits - 1) / splits + BK - 1) / BK * BK;
         splits = (g.K + k_chunk - 1) / k_chunk;
@@ -580,6 +584,8 @@ int launch_tile(const GemmArgs& g) {
         alpha = 1.0f;
         beta = 0.0f;
         split_stride = static_cast<long long>(g.M) * g.N;
+        sC = split_stride * splits;      // partials laid out [problem][chunk][M x N]
+        sC2 = sC * g.batch;
     }
     const bool fast = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && (g.lda % 4 == 0) &&
                       (g.ldb % 4 == 0) && aligned16(g.A) && aligned16(g.B) && (g.sA % 4 == 0) &&
@@ -603,8 +609,8 @@ int launch_tile(const GemmArgs& g) {
     }
 #define JZ_LAUNCH_GEMM(FASTV, EPIV)                                                                         \
     gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, FASTV, EPIV><<<grid, kBlock, 0, s>>>(                        \
-        g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, g.sC, g.batch, g.sA2, g.sB2, \
-        g.sC2, tiles_m, tiles_n, k_chunk, split_stride, g.ep)
+        g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, sC, g.batch, g.sA2, g.sB2, \
+        sC2, tiles_m, tiles_n, k_chunk, split_stride, g.ep)
     if (g.ep.any) {
         if (fast) JZ_LAUNCH_GEMM(true, true); else JZ_LAUNCH_GEMM(false, true);
     } else {
@@ -616,7 +622,13 @@ int launch_tile(const GemmArgs& g) {
         std::lock_guard<std::mutex> lock(prof.mu);
         prof.recs.push_back(rec);
     }
-    if (splits > 1) launch_splitk_reduce(g.C, out, g.M, g.N, g.ldc, splits, g.alpha, g.beta);
+    if (splits > 1) {
+        for (int b = 0; b < nb; ++b) {
+            const int b_in = b % g.batch, b_out = b / g.batch;
+            launch_splitk_reduce(g.C + b_in * g.sC + b_out * g.sC2, out + b * sC, g.M, g.N, g.ldc, splits, g.alpha,
+                                 g.beta);
+        }
+    }
     return launch_rc();
 }
 
@@ -655,7 +667,7 @@ int launch_shape(const GemmArgs& g) {
     // 2304 x 128 x 32768 as 18 tiles x 24 chunks)
     const long long t128 = tiles(128, 128);
     const long long chunks_wanted = (2 * cus + t128 - 1) / t128;
-    const bool splittable = g.batch * g.batch2 == 1 && g.K >= 2048 && !g.ep.any &&
+    const bool splittable = g.batch * g.batch2 <= 8 && g.K >= 2048 && !g.ep.any &&
                             (t128 * 8 >= cus || g.K >= 600 * chunks_wanted);
     if (t128 < cus && !splittable) return launch_tile<2, 2, 1, 1, TA, TB>(g);  // 64 x 64
     return launch_tile<2, 2, 2, 2, TA, TB>(g);                  // 128 x 128

@@ -592,6 +592,24 @@ def test_gemm_strided_batched(gpu, oracle_lib, ta, tb):
     assert rel_err(to_host(dC), out) <= TOL_GEMM
 
 
+@pytest.mark.parametrize("m,n,k,batch,beta", [(128, 96, 8192, 3, 0.0), (64, 64, 4096, 5, 0.5), (192, 128, 16384, 3, 0.0)])
+def test_gemm_batched_problems_with_a_long_contraction(gpu, m, n, k, batch, beta):
+    """A few batched problems whose outputs cannot fill the chip and whose contraction is long
+    (the weight gradients of three projections sharing their input): K is split over workgroups
+    for every problem, each with its own run of partial sums.  B is shared (stride 0), as there.
+    Checked against float64 products; alpha and beta apply once, in the reduction."""
+    r = rng(m + n + k)
+    A = r.normal(0, 1, (batch, k, m)).astype(np.float32)      # column-major m x k per problem
+    B = r.normal(0, 1, (k, n)).astype(np.float32)             # column-major n x k, used transposed
+    C0 = r.normal(0, 1, (batch, n, m)).astype(np.float32)     # column-major m x n per problem
+    dA, dB, dC = to_dev(A.reshape(-1)), to_dev(B.reshape(-1)), to_dev(C0.reshape(-1))
+    gpu.gemm_strided_batched(dptr(dA), dptr(dB), dptr(dC), m, n, k, 0, 1, m, n, m, m * k, 0, m * n, batch, 0.75, beta)
+    got = to_host(dC).reshape(batch, n, m)
+    for b in range(batch):
+        want = 0.75 * (B.astype(np.float64).T @ A[b].astype(np.float64)) + beta * C0[b]
+        assert np.max(np.abs(got[b] - want)) <= TOL_GEMM * np.sqrt(k)
+
+
 def test_add_bias(gpu):
     r = rng(3)
     for rows, cols in ((512, 100), (10, 33), (1, 7)):
