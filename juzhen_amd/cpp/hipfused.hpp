@@ -515,40 +515,52 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
     MD dbo = sum(dR, 1);
     MD dH = Wo.T() * dR;
 
-    // attention core, all heads and sequences at once
-    // (three blocks of one buffer, so that the weight gradients below can be one batched launch)
-    MD dqkv = JzRocmFused::make("dqkv", d_k, 3 * (size_t)N, 0);
-    const size_t qsz = (size_t)d_k * N, wsz = (size_t)d_k * d_model;
-    MD dQ = JzRocmFused::block("dQ", dqkv, 0, d_k, N), dK = JzRocmFused::block("dK", dqkv, qsz, d_k, N),
-       dV = JzRocmFused::block("dV", dqkv, 2 * qsz, d_k, N);
-    must(jzhip_attention_bwd(p(dQ), p(dK), p(dV), p(attn_dS_scratch), p(dH), p(cached_Q), p(cached_K),
-                             p(cached_V), p(cached_A), d_k, num_heads, seq_len, batchN),
-         "attention_bwd");
-
+    // attention core, all heads and sequences at once, then the three projections
+    const size_t wsz = (size_t)d_k * d_model;
     MD dWq = JzRocmFused::make("dWq", 0, 0, 0), dWk = JzRocmFused::make("dWk", 0, 0, 0), dWv = JzRocmFused::make("dWv", 0, 0, 0);
+    MD dx1 = JzRocmFused::make("dx1", 0, 0, 0);
     if (qkv_as_one_launch(Wq, Wk, Wv, cached_x1)) {
+        // dQ, dK, dV as the row blocks of one (3 d_k x N) matrix.  The core is told when the forward
+        // pass was causal: the probabilities above the diagonal are exact zeros and those key tiles
+        // are skipped.
+        MD dqkv = JzRocmFused::make("dqkv", 3 * (size_t)d_k, N, 0);
+        must(jzhip_attention_bwd_ld(p(dqkv), p(dqkv) + d_k, p(dqkv) + 2 * (size_t)d_k, 3 * d_k, p(attn_dS_scratch), p(dH),
+                                    d_k, p(cached_Q), p(cached_K), p(cached_V), d_k, p(cached_A), d_k, num_heads,
+                                    seq_len, batchN, causal ? 1 : 0),
+             "attention_bwd");
         // dW_i = dX_i x1^T for the three projections: one batched launch, K split over the tokens
         MD dw = JzRocmFused::make("dwqkv", d_k, 3 * (size_t)d_model, 0);
-        must(jzhip_gemm_strided_batched(p(dqkv), p(cached_x1), p(dw), d_k, d_model, N, 0, 1, d_k, d_model, d_k,
-                                        (long long)qsz, 0, (long long)wsz, 3, 1.0f, 0.0f),
+        must(jzhip_gemm_strided_batched(p(dqkv), p(cached_x1), p(dw), d_k, d_model, N, 0, 1, 3 * d_k, d_model, d_k,
+                                        (long long)d_k, 0, (long long)wsz, 3, 1.0f, 0.0f),
              "gemm_strided_batched");
         dWq = JzRocmFused::block("dWq", dw, 0, d_k, d_model);
         dWk = JzRocmFused::block("dWk", dw, wsz, d_k, d_model);
         dWv = JzRocmFused::block("dWv", dw, 2 * wsz, d_k, d_model);
+        // dx1 = Wq^T dQ + Wk^T dK + Wv^T dV = [Wq; Wk; Wv]^T [dQ; dK; dV]: one product over 3 d_k
+        MD wrows = JzRocmFused::make("wqkv_rows", 3 * (size_t)d_k, d_model, 0);
+        const MD* ws[3] = {&Wq, &Wk, &Wv};
+        for (int i = 0; i < 3; ++i)
+            must(jzhip_stack_copy_rows(p(wrows), 3 * (size_t)d_k, (size_t)i * d_k, p(*ws[i]), d_k, d_model, 0), "stack_copy_rows");
+        dx1 = JzRocmFused::make("dx1", d_model, N, 0);
+        must(jzhip_gemm(p(wrows), p(dqkv), p(dx1), d_model, N, 3 * d_k, 1, 0, 3 * d_k, 3 * d_k, d_model, 1.0f, 0.0f), "gemm");
     } else {
+        MD dQ("dQ", d_k, N), dK("dK", d_k, N), dV("dV", d_k, N);
+        must(jzhip_attention_bwd(p(dQ), p(dK), p(dV), p(attn_dS_scratch), p(dH), p(cached_Q), p(cached_K),
+                                 p(cached_V), p(cached_A), d_k, num_heads, seq_len, batchN),
+             "attention_bwd");
         dWq = dQ * cached_x1.T();
         dWk = dK * cached_x1.T();
         dWv = dV * cached_x1.T();
+        // dx1 = Wq^T dQ + Wk^T dK + Wv^T dV: the second and third products add into the first
+        dx1 = Wq.T() * dQ;
+        auto add_product = [&](const MD& W, const MD& g) {
+            must(jzhip_gemm(p(W), p(g), p(dx1), d_model, N, d_k, W.get_transpose() ? 0 : 1, 0, (int)JzRocmFused::phys_rows(W),
+                            d_k, d_model, 1.0f, 1.0f),
+                 "gemm");
+        };
+        add_product(Wk, dK);
+        add_product(Wv, dV);
     }
-    // dx1 = Wq^T dQ + Wk^T dK + Wv^T dV: the second and third products add into the first
-    MD dx1 = Wq.T() * dQ;
-    auto add_product = [&](const MD& W, const MD& g) {
-        must(jzhip_gemm(p(W), p(g), p(dx1), d_model, N, d_k, W.get_transpose() ? 0 : 1, 0, (int)JzRocmFused::phys_rows(W),
-                        d_k, d_model, 1.0f, 1.0f),
-             "gemm");
-    };
-    add_product(Wk, dK);
-    add_product(Wv, dV);
     MD dx = ln_backward_plus(ln1, std::move(dx1), dR, this->need_update);
 
     if (this->need_update) {
