@@ -71,7 +71,7 @@ struct Epilogue {
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST, bool EPI>
-__global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kernel(
+__global__ __launch_bounds__(kBlock, EPI ? 4 : FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
@@ -144,28 +144,36 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kerne
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    floatx4 ra[LA::kPasses], rb[LB::kPasses];  // next stage in flight, global -> registers
+    // Stages in flight, global -> registers.  The plain kernel keeps two register sets, so
+    // the loads of stage t+2 leave at the top of stage t, a whole stage before the set is
+    // written to LDS; the kernel with the fused tail, held to 128 registers, has one set and
+    // loads stage t+2 once the stores of stage t+1 have emptied it.
+    constexpr int NSET = EPI ? 1 : JZ_GEMM_SETS;
+    floatx4 ra[NSET][LA::kPasses], rb[NSET][LB::kPasses];
     unsigned offa[LA::kPasses], offb[LB::kPasses];
     if constexpr (FAST) {
         LA::offsets(offa, static_cast<unsigned>(lda));
         LB::offsets(offb, static_cast<unsigned>(ldb));
     }
-    auto load_stage = [&](int k0) {
+    auto load_stage = [&](auto set_c, int k0) {
+        constexpr int S = decltype(set_c)::value;
         if constexpr (FAST) {
-            LA::load_fast(ra, LA::origin(A, lda, m0, k0), offa);
-            LB::load_fast(rb, LB::origin(B, ldb, n0, k0), offb);
+            LA::load_fast(ra[S], LA::origin(A, lda, m0, k0), offa);
+            LB::load_fast(rb[S], LB::origin(B, ldb, n0, k0), offb);
         } else {
-            LA::load_checked(ra, A, lda, m0, k0, M, k_hi);
-            LB::load_checked(rb, B, ldb, n0, k0, N, k_hi);
+            LA::load_checked(ra[S], A, lda, m0, k0, M, k_hi);
+            LB::load_checked(rb[S], B, ldb, n0, k0, N, k_hi);
         }
     };
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, NSET - 1>;
 
     const int nk = (k_hi - k_lo + BK - 1) / BK;
-    load_stage(k_lo);
-    LA::store(ra, As[0]);
-    LB::store(rb, Bs[0]);
+    load_stage(Set0{}, k_lo);
+    LA::store(ra[0], As[0]);
+    LB::store(rb[0], Bs[0]);
     __syncthreads();
-    if (nk > 1) load_stage(k_lo + BK);   // stage 1 waits in registers
+    if (nk > 1) load_stage(Set1{}, k_lo + BK);   // stage 1 waits in registers
 
     // Software pipeline of one K stage (KS MFMA steps of k = 2):
     //  * the operand fragments of step kk+1 are read from LDS before the MFMAs of
@@ -198,29 +206,64 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : JZ_GEMM_OCC) void gemm_mfma_kerne
                                                                  acc[i][j], 0, 0, 0);
     };
 
-    int cur = 0;
-    read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
-    for (int kt = 0; kt < nk; ++kt) {
-        const bool more = kt + 1 < nk;
+    // One stage.  LD names the register set that takes stage kt+2, ST the set that holds
+    // stage kt+1.  With two sets nothing inside a stage is conditional and the stages of a
+    // pair follow each other without a branch: the last two stages are separate instances
+    // (FETCH and KEEP say whether stage kt+2 is loaded and stage kt+1 written to LDS).  A
+    // branch around the loads or the stores turns the waits for the staging registers into
+    // waits for every load in flight, and a branch between the stages of a pair lets the
+    // loads sink into the second one, next to their use.
+    auto stage = [&](auto ld_c, auto st_c, auto fetch_c, auto keep_c, int kt, int cur) {
+        constexpr int ST = decltype(st_c)::value;
+        constexpr bool FETCH = decltype(fetch_c)::value, KEEP = decltype(keep_c)::value;
+        const bool more = NSET == 2 ? KEEP : kt + 1 < nk;
         const float* as = As[cur] + a_off;
         const float* bs = Bs[cur] + b_off;
+        if constexpr (NSET == 2 && FETCH) load_stage(ld_c, k_lo + (kt + 2) * BK);
 #pragma unroll
         for (int kk = 0; kk < KS - 1; ++kk) {
             read_frags((kk + 1) & 1, as, bs, kk + 1);
             if (more) {
-                if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
-                else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
+                if (kk < LA::kPasses) LA::store_pass(ra[ST], As[cur ^ 1], kk);
+                else if (kk < kStorePasses) LB::store_pass(rb[ST], Bs[cur ^ 1], kk - LA::kPasses);
             }
-            if (kk == kStorePasses && kt + 2 < nk) load_stage(k_lo + (kt + 2) * BK);
+            if constexpr (NSET == 1) {
+                if (kk == kStorePasses && kt + 2 < nk) load_stage(ld_c, k_lo + (kt + 2) * BK);
+            }
             __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs they do not feed
             mfma_step(kk & 1);
             __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
-        cur ^= 1;
-        if (more) read_frags(0, As[cur] + a_off, Bs[cur] + b_off, 0);
+        if (NSET == 1 || more) __syncthreads();
+        if (more) read_frags(0, As[cur ^ 1] + a_off, Bs[cur ^ 1] + b_off, 0);
         __builtin_amdgcn_sched_barrier(0);
         mfma_step((KS - 1) & 1);
+    };
+    using Yes = std::true_type;
+    using No = std::false_type;
+    read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
+    if constexpr (NSET == 2) {
+        int kt = 0;
+        for (; kt + 3 < nk; kt += 2) {      // stages kt+2 and kt+3 exist
+            stage(Set0{}, Set1{}, Yes{}, Yes{}, kt, 0);
+            stage(Set1{}, Set0{}, Yes{}, Yes{}, kt + 1, 1);
+        }
+        if (kt + 3 == nk) {                  // three stages left
+            stage(Set0{}, Set1{}, Yes{}, Yes{}, kt, 0);
+            stage(Set1{}, Set0{}, No{}, Yes{}, kt + 1, 1);
+            stage(Set0{}, Set1{}, No{}, No{}, kt + 2, 0);
+        } else if (kt + 2 == nk) {
+            stage(Set0{}, Set1{}, No{}, Yes{}, kt, 0);
+            stage(Set1{}, Set0{}, No{}, No{}, kt + 1, 1);
+        } else {
+            stage(Set0{}, Set1{}, No{}, No{}, kt, 0);
+        }
+    } else {
+        int cur = 0;
+        for (int kt = 0; kt < nk; ++kt) {
+            stage(Set0{}, Set0{}, Yes{}, Yes{}, kt, cur);
+            cur ^= 1;
+        }
     }
 
     // Epilogue.  Register v of lane (h, l32) holds C(row, col) with

@@ -15,7 +15,10 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 #ifndef JZ_GEMM_OCC
-#define JZ_GEMM_OCC 2
+#define JZ_GEMM_OCC 3
+#endif
+#ifndef JZ_GEMM_SETS
+#define JZ_GEMM_SETS 2
 #endif
 #ifndef JZ_GEMM_BK
 #define JZ_GEMM_BK 16

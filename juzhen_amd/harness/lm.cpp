@@ -91,7 +91,11 @@ struct Model {
     // Weight, bias and LayerNorm-parameter gradients are leaves of the backward
     // graph: with `overlap` they go to a second stream and fill the gaps the
     // gradient chain leaves (tile prologues and tails, bandwidth-bound kernels).
-    bool overlap = true;
+    // Off by default: since the tiled products keep two stages of loads in flight
+    // they leave little to fill, and two of them sharing the CUs measured 2 % slower
+    // per step than one after the other (with the earlier single-stage products the
+    // second stream gained 2 %).
+    bool overlap = false;
     void* side = nullptr;
     static constexpr int kEvents = 8, kDone = 4;
     void* ev[kEvents] = {};
