@@ -71,7 +71,7 @@ struct Epilogue {
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST, bool EPI>
-__global__ __launch_bounds__(kBlock, EPI ? 4 : FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kernel(
+__global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
@@ -144,11 +144,11 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : FAST ? JZ_GEMM_OCC : 2) void gemm
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // Stages in flight, global -> registers.  The plain kernel keeps two register sets, so
-    // the loads of stage t+2 leave at the top of stage t, a whole stage before the set is
-    // written to LDS; the kernel with the fused tail, held to 128 registers, has one set and
-    // loads stage t+2 once the stores of stage t+1 have emptied it.
-    constexpr int NSET = EPI ? 1 : JZ_GEMM_SETS;
+    // Stages in flight, global -> registers.  With two register sets the loads of stage
+    // t+2 leave at the top of stage t, a whole stage before the set is written to LDS
+    // (4096^3: 129 -> 135-144 TFLOP/s; with the fused tail 130 -> 142); with one set they
+    // leave once the stores of stage t+1 have emptied it, half a stage before.
+    constexpr int NSET = JZ_GEMM_SETS;
     floatx4 ra[NSET][LA::kPasses], rb[NSET][LB::kPasses];
     unsigned offa[LA::kPasses], offb[LB::kPasses];
     if constexpr (FAST) {
@@ -169,11 +169,24 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : FAST ? JZ_GEMM_OCC : 2) void gemm
     using Set1 = std::integral_constant<int, NSET - 1>;
 
     const int nk = (k_hi - k_lo + BK - 1) / BK;
+    // With two register sets the stages run in pairs (even stage: LDS buffer 0, loads
+    // into set 0; odd stage: buffer 1, set 1).  An odd stage count starts one stage
+    // late in that cycle: stage 0 then sits in buffer 1 and stage 1 in set 0, and the
+    // second half of a pair runs once before the loop.
+    const int odd = NSET == 2 ? (nk & 1) : 0;
+    const int k_last = k_lo + (nk - 1) * BK;
     load_stage(Set0{}, k_lo);
-    LA::store(ra[0], As[0]);
-    LB::store(rb[0], Bs[0]);
+    LA::store(ra[0], As[odd]);
+    LB::store(rb[0], Bs[odd]);
     __syncthreads();
-    if (nk > 1) load_stage(Set1{}, k_lo + BK);   // stage 1 waits in registers
+    if constexpr (NSET == 2) {
+        // stage 1 waits in registers (a single stage is fetched again and dropped)
+        const int k1 = nk > 1 ? k_lo + BK : k_lo;
+        if (odd) load_stage(Set0{}, k1);
+        else load_stage(Set1{}, k1);
+    } else {
+        if (nk > 1) load_stage(Set0{}, k_lo + BK);
+    }
 
     // Software pipeline of one K stage (KS MFMA steps of k = 2):
     //  * the operand fragments of step kk+1 are read from LDS before the MFMAs of
@@ -207,19 +220,22 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : FAST ? JZ_GEMM_OCC : 2) void gemm
     };
 
     // One stage.  LD names the register set that takes stage kt+2, ST the set that holds
-    // stage kt+1.  With two sets nothing inside a stage is conditional and the stages of a
-    // pair follow each other without a branch: the last two stages are separate instances
-    // (FETCH and KEEP say whether stage kt+2 is loaded and stage kt+1 written to LDS).  A
-    // branch around the loads or the stores turns the waits for the staging registers into
-    // waits for every load in flight, and a branch between the stages of a pair lets the
-    // loads sink into the second one, next to their use.
-    auto stage = [&](auto ld_c, auto st_c, auto fetch_c, auto keep_c, int kt, int cur) {
+    // stage kt+1.  With two sets nothing inside a stage is conditional and the loop body
+    // is one pair of stages without a branch between them: past the end the last stage
+    // is fetched again and written to the LDS buffer that nobody reads any more.  A
+    // branch around the loads or the stores turns the waits for the staging registers
+    // into waits for every load in flight, a branch between the stages of a pair lets
+    // the loads sink into the second one, next to their use, and separate copies of
+    // the last stages made the accumulators spill there.
+    auto stage = [&](auto ld_c, auto st_c, int kt, int cur) {
         constexpr int ST = decltype(st_c)::value;
-        constexpr bool FETCH = decltype(fetch_c)::value, KEEP = decltype(keep_c)::value;
-        const bool more = NSET == 2 ? KEEP : kt + 1 < nk;
+        const bool more = NSET == 2 || kt + 1 < nk;
         const float* as = As[cur] + a_off;
         const float* bs = Bs[cur] + b_off;
-        if constexpr (NSET == 2 && FETCH) load_stage(ld_c, k_lo + (kt + 2) * BK);
+        if constexpr (NSET == 2) {
+            const int k2 = k_lo + (kt + 2) * BK;
+            load_stage(ld_c, k2 < k_last ? k2 : k_last);
+        }
 #pragma unroll
         for (int kk = 0; kk < KS - 1; ++kk) {
             read_frags((kk + 1) & 1, as, bs, kk + 1);
@@ -234,34 +250,22 @@ __global__ __launch_bounds__(kBlock, EPI ? 4 : FAST ? JZ_GEMM_OCC : 2) void gemm
             mfma_step(kk & 1);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (NSET == 1 || more) __syncthreads();
+        __syncthreads();
         if (more) read_frags(0, As[cur ^ 1] + a_off, Bs[cur ^ 1] + b_off, 0);
         __builtin_amdgcn_sched_barrier(0);
         mfma_step((KS - 1) & 1);
     };
-    using Yes = std::true_type;
-    using No = std::false_type;
-    read_frags(0, As[0] + a_off, Bs[0] + b_off, 0);
+    read_frags(0, As[odd] + a_off, Bs[odd] + b_off, 0);
     if constexpr (NSET == 2) {
-        int kt = 0;
-        for (; kt + 3 < nk; kt += 2) {      // stages kt+2 and kt+3 exist
-            stage(Set0{}, Set1{}, Yes{}, Yes{}, kt, 0);
-            stage(Set1{}, Set0{}, Yes{}, Yes{}, kt + 1, 1);
-        }
-        if (kt + 3 == nk) {                  // three stages left
-            stage(Set0{}, Set1{}, Yes{}, Yes{}, kt, 0);
-            stage(Set1{}, Set0{}, No{}, Yes{}, kt + 1, 1);
-            stage(Set0{}, Set1{}, No{}, No{}, kt + 2, 0);
-        } else if (kt + 2 == nk) {
-            stage(Set0{}, Set1{}, No{}, Yes{}, kt, 0);
-            stage(Set1{}, Set0{}, No{}, No{}, kt + 1, 1);
-        } else {
-            stage(Set0{}, Set1{}, No{}, No{}, kt, 0);
+        if (odd) stage(Set1{}, Set0{}, 0, 1);
+        for (int kt = odd; kt < nk; kt += 2) {
+            stage(Set0{}, Set1{}, kt, 0);
+            stage(Set1{}, Set0{}, kt + 1, 1);
         }
     } else {
         int cur = 0;
         for (int kt = 0; kt < nk; ++kt) {
-            stage(Set0{}, Set0{}, Yes{}, Yes{}, kt, cur);
+            stage(Set0{}, Set0{}, kt, cur);
             cur ^= 1;
         }
     }
