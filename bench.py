@@ -87,11 +87,11 @@ class HipEvents:
 # what the same counters read for a plain 256 MiB copy (FETCH_SIZE x1.9998,
 # WRITE_SIZE x1.0000); the counter tables are kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_mfma_kernel<2, 2, 2, 2, false, true, true, false>": 203.9e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, true>": 240.2e6,
+    "gemm_mfma_kernel<2, 2, 2, 2, false, true, true, false>": 209.6e6,
+    "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, true>": 244.5e6,
     "gemm_mfma_kernel<2, 2, 2, 2, true, false, true, false>": 140.8e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, true, false, true, true>": 392.7e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, false>": 177.8e6,
+    "gemm_mfma_kernel<2, 2, 2, 2, true, false, true, true>": 399.9e6,
+    "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, false>": 183.2e6,
     "gemm_mfma_kernel<2, 2, 1, 1, false, true, true, false>": 71.4e6,
 }
 

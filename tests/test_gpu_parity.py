@@ -492,6 +492,61 @@ def test_gemm_fused_epilogue(gpu, m, n, k, ta, tb, act):
     assert rel_err(got, v.T.reshape(-1)) <= TOL_GEMM
 
 
+# Products with more full 128 x 128 tiles than workgroups fit on the chip at once (768), so
+# that tiles start while others are half way and the XCD-wise tile order wraps unevenly
+# (7 x 111 tiles).  A tile's arithmetic does not depend on when or where it runs, so the
+# result must equal, bit for bit, the same product computed in column blocks of at most
+# half that many tiles.  k = 32 is the shortest contraction with two K stages.
+@pytest.mark.parametrize("m,n,k", [(1536, 16384, 512), (896, 14208, 32), (2048, 8320, 64)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_gemm_more_tiles_than_workgroups(gpu, m, n, k, ta, tb, fused):
+    import torch
+    assert (m // 128) * (n // 128) > 768 and (k // 16) % 2 == 0
+    g = torch.Generator(device="cuda")
+    g.manual_seed(m + n + k + 2 * ta + tb)
+    lda, ldb = (k if ta else m), (n if tb else k)
+    A = torch.randn(lda * (m if ta else k), generator=g, device="cuda") / math.sqrt(k)
+    B = torch.randn(ldb * (k if tb else n), generator=g, device="cuda")
+    bias = torch.randn(m, generator=g, device="cuda")
+    res = torch.randn(m * n, generator=g, device="cuda")
+    old = torch.randn(m * n, generator=g, device="cuda")
+    whole, pieces = old.clone(), old.clone()
+    aux_w, aux_p = torch.zeros(m * n, device="cuda"), torch.zeros(m * n, device="cuda")
+    beta = 0.0 if fused else 0.5
+
+    def run(C_, aux_, col0, cols):
+        # columns [col0, col0 + cols) of op(B) and C
+        b_off = col0 if tb else col0 * ldb
+        pb = C.c_void_p(B.data_ptr() + 4 * b_off)
+        pc = C.c_void_p(C_.data_ptr() + 4 * col0 * m)
+        if fused:
+            gpu.gemm_fused(dptr(A), pb, pc, m, cols, k, ta, tb, lda, ldb, m, 1.0, beta, dptr(bias), 2,
+                           C.c_void_p(aux_.data_ptr() + 4 * col0 * m), m,
+                           C.c_void_p(res.data_ptr() + 4 * col0 * m), m)
+        else:
+            gpu.gemm(dptr(A), pb, pc, m, cols, k, ta, tb, lda, ldb, m, 1.0, beta)
+
+    run(whole, aux_w, 0, n)
+    step = 128 * (768 // (m // 128) // 2)          # at most half the tiles that would be walked
+    for col0 in range(0, n, step):
+        run(pieces, aux_p, col0, min(step, n - col0))
+    torch.cuda.synchronize()
+    assert torch.equal(whole, pieces)
+    assert torch.equal(aux_w, aux_p)
+    # and against float64 on the device
+    Am = A.double().view(-1, lda).T
+    Bm = B.double().view(-1, ldb).T
+    v = (Am.T if ta else Am) @ (Bm.T if tb else Bm)            # m x n
+    if fused:
+        v = v + bias.double()[:, None]
+        assert rel_err(to_host(aux_w), to_host(v.T.reshape(-1))) <= TOL_GEMM
+        v = 0.5 * v * (1 + torch.erf(v / math.sqrt(2))) + res.double().view(n, m).T
+    else:
+        v = v + beta * old.double().view(n, m).T
+    assert rel_err(to_host(whole), to_host(v.T.reshape(-1))) <= TOL_GEMM
+
+
 def test_gemm_fused_rejects_bad_arguments(gpu):
     from juzhen_amd import capi
     lib = capi.load()
