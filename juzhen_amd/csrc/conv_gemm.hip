@@ -318,16 +318,20 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
                 if (kk < LA::kPasses) LA::store_pass(ra, As[cur ^ 1], kk);
                 else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
             }
-            // pass p of the patch operand is requested one step after its registers went to LDS
-            if (kt + 2 < nk) {
+            // pass p of the patch operand is requested one step after its registers went to LDS.
+            // The requests are unconditional (past the end the last stage is fetched again and
+            // dropped): inside a branch they made the wait of the staging store that follows
+            // them a wait for all loads in flight, these fresh ones included.
+            {
+                const int k2 = (kt + 2 < nk ? kt + 2 : nk - 1) * BK;
                 if constexpr (TAB) {
-                    if (kk == 0) stage_taps_tab((kt + 2) * BK);
+                    if (kk == 0) stage_taps_tab(k2);
                     if (kk >= 1 && kk - 1 < LA::kPasses) load_a_tab(kk - 1);
                 } else {
-                    if (kk == 1) stage_taps((kt + 2) * BK);
+                    if (kk == 1) stage_taps(k2);
                     if (kk >= 1 && kk - 1 < LA::kPasses) load_a(kk - 1);
                 }
-                if (kk == kStorePasses) load_b((kt + 2) * BK);
+                if (kk == kStorePasses) load_b(k2);
             }
             __builtin_amdgcn_sched_barrier(0);
             mfma_step(kk & 1);
@@ -342,6 +346,16 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
 
     // store: register v of lane (h, l32) is (row l32, column 8*(v/4) + 4*h + v%4) of a 32x32 tile
     const long long CoP = static_cast<long long>(g.Cout) * g.P;
+    // the bias values of the wave's output channels, requested together (one load and one
+    // wait per stored element made the store loop a chain of round trips)
+    float bv[TN][16];
+#pragma unroll
+    for (int jn = 0; jn < TN; ++jn)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int co = n0 + (wn * TN + jn) * 32 + 4 * h + 8 * (v / 4) + (v % 4);
+            bv[jn][v] = (bias && co < g.Cout) ? bias[co] : 0.0f;
+        }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const long long j = m0 + (wm * TM + i) * 32 + l32;
@@ -357,7 +371,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
                 const int co = cbase + 8 * (v / 4) + (v % 4);
                 if (co < g.Cout) {
                     float r = acc[i][jn][v];
-                    if (bias) r += bias[co];
+                    if (bias) r += bv[jn][v];
                     if (relu) r = r > 0.0f ? r : 0.0f;
                     dst[static_cast<long long>(co) * g.P] = r;
                 }
@@ -562,6 +576,8 @@ __global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restr
                     else if (kk < kStorePasses) LB::store_pass(rb, Bs[cur ^ 1], kk - LA::kPasses);
                 }
                 // pass p of an operand is requested one step after its registers went to LDS
+                // (stage_sites moves the site along from the stage before, so a stage cannot
+                // be requested twice: these requests stay behind the test for a further stage)
                 if (kt + 2 < nk) {
                     if (kk == 1) stage_sites(j_lo + static_cast<long long>(kt + 2) * BK);
                     if (kk >= 1 && kk - 1 < LA::kPasses) load_a(kk - 1);
