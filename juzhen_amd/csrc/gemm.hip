@@ -197,7 +197,9 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
     //    to the other LDS buffer one float4-pass per MFMA step instead of in a
     //    burst before the barrier, so fragment reads of the other workgroups on
     //    the CU never queue behind a block of stores;
-    //  * the global loads of stage t+2 are issued once those registers are free.
+    //  * the global loads of stage t+2 are issued at the top of stage t into the
+    //    register set that stage t's data left one stage earlier (with a single
+    //    set: once the stores of stage t+1 have emptied it).
     constexpr int KS = BK / 2;  // MFMA steps per stage
     static_assert(KS % 2 == 0, "fragment double buffer assumes an even step count");
     constexpr int kStorePasses = LA::kPasses + LB::kPasses;
