@@ -85,7 +85,7 @@ class HipEvents:
 # HBM bytes per launch of the tiled-GEMM instances of this workload, averaged over
 # their dispatches: rocprofv3 FETCH_SIZE and WRITE_SIZE runs of this script scaled by
 # what the same counters read for a plain 256 MiB copy (FETCH_SIZE x1.9998,
-# WRITE_SIZE x1.0000); the counter tables are kept under profiles/.
+# WRITE_SIZE x0.9998); the counter tables are kept under profiles/.
 MEASURED_TRAFFIC_BYTES = {
     "gemm_mfma_kernel<2, 2, 2, 2, false, true, true, false>": 209.6e6,
     "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, true>": 244.5e6,
