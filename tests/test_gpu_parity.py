@@ -321,7 +321,10 @@ def naive_gemm64(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, Cm, ldc):
 
 GEMM_SHAPES = [(1, 1, 1), (2, 2, 2), (3, 5, 7), (1, 40, 33), (40, 1, 33), (17, 19, 1), (64, 64, 64),
                (128, 128, 16), (129, 127, 17), (33, 300, 9), (300, 33, 70), (256, 512, 128),
-               (32, 1000, 288), (10, 128, 1254), (65, 250, 130)]
+               (32, 1000, 288), (10, 128, 1254), (65, 250, 130),
+               # full tiles with two, three and five K stages of 16: the stage loop runs in
+               # pairs, and an odd count starts half a pair in
+               (256, 256, 32), (128, 384, 48), (256, 128, 80)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
