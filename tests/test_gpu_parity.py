@@ -433,8 +433,10 @@ def test_gemm_thin_products_at_the_output_convolution_size(gpu):
 
 # (10, 128, 2560): the split-K form; (5, 300, 64): thin; (40, 50, 1): rank-1; (300, 1, 70): matrix-vector --
 # the fused entry point keeps those forms and runs the tail as separate kernels
+# (128, 256, 48) and (256, 256, 16): full tiles with an odd number of K stages (three, one)
 @pytest.mark.parametrize("m,n,k", [(3, 5, 7), (64, 64, 64), (129, 127, 17), (256, 512, 128), (128, 1024, 96),
-                                   (10, 128, 2560), (5, 300, 64), (40, 50, 1), (300, 1, 70)])
+                                   (10, 128, 2560), (5, 300, 64), (40, 50, 1), (300, 1, 70),
+                                   (128, 256, 48), (256, 256, 16)])
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1)])
 @pytest.mark.parametrize("act", [0, 1, 2, 3, 4])
 def test_gemm_fused_epilogue(gpu, m, n, k, ta, tb, act):
