@@ -324,7 +324,9 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 2), (3, 5, 7), (1, 40, 33), (40, 1, 33), (17, 1
                (32, 1000, 288), (10, 128, 1254), (65, 250, 130),
                # full tiles with two, three and five K stages of 16: the stage loop runs in
                # pairs, and an odd count starts half a pair in
-               (256, 256, 32), (128, 384, 48), (256, 128, 80)]
+               (256, 256, 32), (128, 384, 48), (256, 128, 80),
+               # four tiles and a contraction cut into 8 chunks of five stages each
+               (256, 256, 640)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
