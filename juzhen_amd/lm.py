@@ -81,8 +81,8 @@ class CharLM:
             self.set_overlap(overlap)
 
     def set_overlap(self, on):
-        """Weight-gradient work of the backward pass on a second stream (the default)
-        or everything on one stream in program order."""
+        """Weight-gradient work of the backward pass on a second stream, or everything
+        on one stream in program order (the default)."""
         self.lib.jzlm_set_overlap(self.h, int(bool(on)))
 
     def _check(self, what, rc):
