@@ -148,7 +148,10 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
     // t+2 leave at the top of stage t, a whole stage before the set is written to LDS
     // (4096^3: 129 -> 135-144 TFLOP/s; with the fused tail 130 -> 142); with one set they
     // leave once the stores of stage t+1 have emptied it, half a stage before.
-    constexpr int NSET = JZ_GEMM_SETS;
+    // The bounds-checked loaders of ragged shapes keep one set: their address arithmetic
+    // makes the two stages fetched past the end cost more than the earlier start gains
+    // (32 x 256 tiles of a 64 x 25088 x 288 product: 20.4 us with one set, 24.2 with two).
+    constexpr int NSET = FAST ? JZ_GEMM_SETS : 1;
     floatx4 ra[NSET][LA::kPasses], rb[NSET][LB::kPasses];
     unsigned offa[LA::kPasses], offb[LB::kPasses];
     if constexpr (FAST) {
