@@ -91,3 +91,21 @@ def test_product_code_never_reaches_into_the_oracle():
         elif re.search(r'#include\s*[<"][^>"]*(oracle|jz_oracle|ref_shim)', text) or "jzo_" in text or "jzref_" in text:
             bad.append(str(p))
     assert not bad, bad
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: `--gpus N` with N above 1, or a launch under a
+    multi-rank launcher, exits with status 2 and says why, before anything touches
+    a GPU."""
+    import os
+    import subprocess
+    import sys
+    env = {k: v for k, v in os.environ.items() if k not in ("WORLD_SIZE", "RANK", "LOCAL_RANK")}
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       env=env, timeout=300)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py")], capture_output=True, text=True,
+                       env={**env, "WORLD_SIZE": "2"}, timeout=300)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr
