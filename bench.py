@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: transformer train-step tokens/s on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--two-stream] [--no-cpu-baseline] [--no-dropin]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--two-stream] [--no-cpu-baseline] [--no-dropin] [--no-legs]
 
 Workload (the character-level transformer configuration): language model over
 vocab 256 byte tokens drawn from Zipf(s=1.1), context 256, batch 64 (16 384 tokens per step), 6
@@ -26,7 +26,9 @@ reference's own CPU path (oracle/_ref, OpenBLAS build when available) on a
 bounded sample of the same workload.  `dropin_api` is the same model written on
 the reference's layer classes and run through the drop-in Matrix<ROCMfloat> API
 (a prebuilt program started after the timed region; `--no-dropin` skips it, as
-the profiler commands do).
+the profiler commands do).  `gemm_4096`, `streaming`, `c1_ops` and `configs` are
+the other legs of the metric and the other benchmark configurations
+(juzhen_amd/benchlegs.py), measured after the timed region; `--no-legs` skips them.
 """
 from __future__ import annotations
 
@@ -82,18 +84,27 @@ class HipEvents:
         assert self.hip.hipDeviceSynchronize() == 0
 
 
-# HBM bytes per launch of the tiled-GEMM instances of this workload, averaged over
-# their dispatches: rocprofv3 FETCH_SIZE and WRITE_SIZE runs of this script scaled by
-# what the same counters read for a plain 256 MiB copy (FETCH_SIZE x1.9998,
-# WRITE_SIZE x0.9998); the counter tables are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    "gemm_mfma_kernel<2, 2, 2, 2, false, true, true, false>": 209.6e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, true>": 244.5e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, true, false, true, false>": 140.8e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, true, false, true, true>": 399.9e6,
-    "gemm_mfma_kernel<2, 2, 2, 2, false, false, true, false>": 183.2e6,
-    "gemm_mfma_kernel<2, 2, 1, 1, false, true, true, false>": 71.4e6,
-}
+TRAFFIC_PROFILE = ROOT / "profiles" / "train_step_c4_hbm_traffic.txt"
+
+
+def measured_traffic_bytes(kernel, path=TRAFFIC_PROFILE):
+    """HBM bytes per launch of `kernel`, averaged over its dispatches in the counter runs of
+    this script: the row of that kernel in the committed summary (rocprofv3 FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the same counter reads for a plain 256 MiB copy; columns
+    `kernel  dispatches  fetch KiB  write KiB  total MiB`).  A kernel the summary does not
+    hold raises: a renamed or re-tuned kernel must not report another kernel's bytes."""
+    import re
+    row = re.compile(r"^(?P<name>\S.*?)\s+(?P<n>\d+)\s+(?P<f>[\d.]+)\s+(?P<w>[\d.]+)\s+(?P<t>[\d.]+)\s*$")
+    names = []
+    for line in Path(path).read_text().splitlines():
+        m = row.match(line)
+        if not m:
+            continue
+        names.append(m["name"])
+        # the summary truncates long names; the names compared are those of this library's kernels
+        if m["name"] == kernel or (len(m["name"]) >= 60 and kernel.startswith(m["name"])):
+            return (float(m["f"]) + float(m["w"])) * 1024.0
+    raise KeyError(f"{path.name} holds no row for kernel {kernel!r} (rows: {names}); regenerate the counter summary")
 
 
 def cpu_baseline(seconds_budget=40.0):
@@ -168,12 +179,34 @@ def cpu_baseline(seconds_budget=40.0):
     }
 
 
+def cpu_configs(rows):
+    """CPU baseline of the other configurations: oracle/_ref/bin/configs_cpu, the reference's
+    Matrix<float> build (OpenBLAS for products, one core elsewhere) of the program whose
+    Matrix<ROCMfloat> build produced `rows`, run after it on the same box for a few steps."""
+    import tempfile
+    from juzhen_amd import benchlegs
+    exe = ROOT / "oracle" / "_ref" / "bin" / "configs_cpu"
+    if not exe.exists():
+        return
+    with tempfile.TemporaryDirectory() as tmp:
+        for cfg, (_, steps, key) in benchlegs.CONFIG_RUNS.items():
+            val, wall = benchlegs.run_config_program(exe, cfg, steps, key, tmp)
+            rows[cfg].update({"cpu_ms": val, "cpu_steps": steps, "cpu_wall_s": wall})
+            if val and rows[cfg].get("gpu_ms"):
+                rows[cfg]["speedup"] = round(val / rows[cfg]["gpu_ms"], 1)
+    rows["cpu"] = ("reference Matrix<float> build of the same program (oracle/_ref/bin/configs_cpu), OpenBLAS with "
+                   f"{os.environ.get('OMP_NUM_THREADS', os.cpu_count())} threads for products, one core elsewhere")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-legs", action="store_true",
+                    help="skip the other legs of the metric (4096^3 GEMM, streaming kernels at 1 GiB, the "
+                         "expression-chain ops and the MLP / CNN / UNet configurations), which run after the timed region")
     ap.add_argument("--no-dropin", action="store_true",
                     help="skip the run of the same model on the reference's layer classes (dropin_api key)")
     ap.add_argument("--two-stream", action="store_true",
@@ -268,7 +301,8 @@ def main():
     roofline = {
         "bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(dom["kernel"]),
+        "traffic": round(measured_traffic_bytes(dom["kernel"])),
+        "traffic_source": "profiles/train_step_c4_hbm_traffic.txt (rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this script)",
         "kernel": dom["kernel"], "launches_per_step": dom["launches"] // prof_steps,
         "avg_launch_us": round(dom["total_ms"] * 1e3 / dom["launches"], 2),
         "flops_per_launch": round(dom["flops"] / dom["launches"], 1),
@@ -294,7 +328,7 @@ def main():
     # what a user of Matrix<ROCMfloat> gets without the harness.  A prebuilt program; run
     # after the timed region, reported beside the headline number, never part of it.
     dropin = None
-    dropin_bin = Path(__file__).resolve().parent / "oracle" / "_ref" / "bin" / "lm_dropin_rocm"
+    dropin_bin = ROOT / "juzhen_amd" / "bin" / "lm_dropin_rocm"
     if not args.no_dropin and dropin_bin.exists():
         try:
             import re
@@ -306,9 +340,24 @@ def main():
                       "steps": int(kv["steps"]), "warmup": int(kv["warmup"]),
                       "model": "LinearLayer + 6 x TransformerLayer<ROCMfloat> + LinearLayer + LogisticLayer "
                                "(ml/layer.hpp), d_model 512, 8 heads, FFN 2048 ReLU, context 256, batch 64, Adam",
-                      "program": "oracle/_ref/bin/lm_dropin_rocm (juzhen_amd/harness/lm_dropin.cu)"}
+                      "program": "juzhen_amd/bin/lm_dropin_rocm (juzhen_amd/harness/lm_dropin.cu)"}
         except Exception as exc:
             dropin = {"tokens_per_s": None, "error": str(exc)}
+
+    param_count = int(model.param_count)
+    model.close()
+    # The other legs of the metric (GEMM TFLOP/s and elementwise GB/s against their rooflines) and the
+    # other benchmark configurations, measured in this run after the timed region; with the CPU
+    # baseline enabled, the reference's CPU build of the same configurations program is timed beside them.
+    legs = None
+    if not args.no_legs:
+        try:
+            from juzhen_amd import benchlegs
+            legs = benchlegs.run_all()
+            if not args.no_cpu_baseline:
+                cpu_configs(legs["configs"])
+        except Exception as exc:
+            legs = {"error": f"{type(exc).__name__}: {exc}"}
 
     out = {
         "metric": "transformer train-step tokens/s", "value": round(value, 1), "unit": "tokens/s",
@@ -320,7 +369,7 @@ def main():
                    "backward_streams": 2 if args.two_stream and not args.serial else 1,
                    "batch_upload": "every step (host ids -> device inside the timed region)" if fresh
                                    else "once, before the timed region",
-                   "parameters": int(model.param_count), "loss_first": round(first_loss, 4),
+                   "parameters": param_count, "loss_first": round(first_loss, 4),
                    "loss_last": round(last_loss, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 3)},
         "roofline": roofline,
         "cpu_baseline": cpu,
@@ -328,7 +377,8 @@ def main():
     }
     if cpu and cpu.get("value"):
         out["speedup_vs_cpu_baseline"] = round(value / cpu["value"], 1)
-    model.close()
+    if legs:
+        out.update(legs)
     print(json.dumps(out))
 
 

@@ -106,6 +106,16 @@ int jzhip_event_synchronize(void* event);
  * while recording (it is allocated at once, not replayed).  `jzhip_graph_launch`
  * enqueues one replay on the current stream (the null stream included) and
  * returns without waiting.  `jzhip_graph_recording` is 1 between begin and end.
+ * `jzhip_graph_destroy` waits for every stream the graph was replayed on, then
+ * destroys it (-1 while another recording is in progress): after it returns the
+ * caller may free the buffers the recording used.  Every recording bakes the
+ * record stream's one workspace (split-K partials, reduction partials, flipped
+ * convolution weights) into its nodes: replays of recorded graphs must therefore
+ * be serialised with each other and with eager calls made while recording, i.e.
+ * launched on one stream or ordered with events; two graphs replayed on two
+ * streams at once race on that workspace.  The record stream is a blocking
+ * stream, so work that other code puts on the legacy null stream while a
+ * recording is open invalidates the recording (`jzhip_graph_end` then fails).
  * What it buys on MI355X: the MLP step of ~60 kernels 0.196 -> 0.186 ms, the CNN
  * step 0.341 -> 0.334 ms; such steps are bound by the device's dispatch of short
  * dependent kernels, which a graph does not remove, not by host launch cost. */
@@ -291,6 +301,11 @@ int jzhip_max_cols(float* out, const float* a, int numrow, int numcol, int ld);
  * first-maximum rule of std::max_element (ml/util.cuh:104-110,
  * examples/demo_transformer.cu:350-357). Bit-exact. */
 int jzhip_argmax_cols(int32_t* out, const float* a, int numrow, int numcol, int ld);
+/* predict_one_hot (ml/util.cuh:258-279: reduce<F> column maximum, rank-1 product,
+ * subtraction, elemwise<F> threshold) as one launch: out (numrow x numcol, dense) holds
+ * 1 where (double)(a - max of its column) > -1e-5, else 0; bit-identical to the chain,
+ * ties and NaNs included.  out must not alias a. */
+int jzhip_predict_one_hot(float* out, const float* a, int numrow, int numcol, int ld);
 
 /* ── GEMM family ─────────────────────────────────────────────────────── */
 
@@ -561,6 +576,17 @@ int jzhip_conv2d_backward_data(const float* t, const float* weights, float* dx, 
                                int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
                                int pad_w, int stride_h, int stride_w, int H_out, int W_out,
                                int N);
+/* No reference counterpart.  0 when the entry point above named by `which` (0 forward,
+ * 1 backward_weights, 2 backward_data) accepts this geometry, -1 when it would refuse it:
+ * a dimension that is not positive, an index product beyond the kernels' 32-bit
+ * arithmetic (C*H*W of an image >= 2^30, K = C_in*kH*kW >= 2^24), a patch grid larger
+ * than (H_in + 2*pad - kH)/stride + 1, and for backward_data a stride other than 1,
+ * pad > k - 1, H_in != H_out + kH - 1 - 2*pad or more than 16 Mi weights (they are
+ * flipped into the workspace).  Nothing is launched.  Callers that have a patch-matrix
+ * route to fall back to (ConvLayer, convtransLayer) pick their route with it. */
+int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out, int kH, int kW,
+                       int pad_h, int pad_w, int stride_h, int stride_w, int H_out,
+                       int W_out, int N);
 
 #ifdef __cplusplus
 }

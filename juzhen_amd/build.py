@@ -83,11 +83,14 @@ def build(force: bool = False, jobs: int = 6) -> Path:
 # reference tree.  It never copies reference sources: it builds a directory of
 # symlinks ("overlay") in which those three names point at our files and every
 # other name points into the reference tree, compiles the reference's own
-# ROCm test programs in that overlay against libjzhip.so, and writes the
-# binaries (which contain compiled reference code) to oracle/_ref/bin/.
+# ROCm test programs in that overlay against libjzhip.so, and writes those
+# binaries (the reference's own tests: checkers) to oracle/_ref/bin/.  The
+# programs of juzhen_amd/harness/*.cu, this package's own sources written
+# against the Matrix<ROCMfloat> API, go to juzhen_amd/bin/.
 REFERENCE_ROOT = Path(os.environ.get("JUZHEN_REFERENCE", "/root/reference"))
 OVERLAY = OBJ / "overlay"
 REF_BIN = ROOT / "oracle" / "_ref" / "bin"
+BIN = PKG / "bin"
 HOST_SRC = PKG / "cpp"
 OURS = {"hipmatrix.cuh", "hipmatrix.cpp", "hipkernels.cpp"}
 # a writable PROJECT_DIR that exists on any box (tests that dump files use it)
@@ -182,10 +185,11 @@ def build_host(force: bool = False, jobs: int = 6):
     """Compile the Matrix<ROCMfloat> mirror and the reference's ROCm programs.
     Returns the list of binaries, or [] when the reference tree is absent."""
     if not REFERENCE_ROOT.exists():
-        return sorted(REF_BIN.glob("*")) if REF_BIN.exists() else []
+        return [*(sorted(REF_BIN.glob("*")) if REF_BIN.exists() else []), *(sorted(BIN.glob("*")) if BIN.exists() else [])]
     build()
     ov = make_overlay()
     REF_BIN.mkdir(parents=True, exist_ok=True)
+    BIN.mkdir(parents=True, exist_ok=True)
     hostobj = OBJ / "host"
     hostobj.mkdir(parents=True, exist_ok=True)
     ours = [HOST_SRC / n for n in sorted(OURS)] + list(HOST_SRC.glob("*.hpp"))
@@ -226,11 +230,8 @@ def build_host(force: bool = False, jobs: int = 6):
     tpl_obj = hostobj / "templates_bench_rocm.o"
     if force or _stale(tpl_obj, [tpl_src, *ours, ROOT / "include" / "jzhip.h"]):
         _hipcc([*HOST_FLAGS, f"-I{ov / 'tests'}", "-c", str(tpl_src), "-o", str(tpl_obj)], "compile templates_bench.cu")
-    REFERENCE_PROGRAMS_ALL = list(zip(REFERENCE_PROGRAMS, prog_objs)) + [("harness/configs_rocm.cu", cfg_obj),
-                                                                         ("harness/templates_bench_rocm.cu", tpl_obj),
-                                                                         ("harness/jvp_check_rocm.cu", jvp_obj),
-                                                                         ("harness/semantics_rocm.cu", sem_obj),
-                                                                         ("harness/lm_dropin_rocm.cu", dro_obj)]
+    harness_programs = [("configs_rocm", cfg_obj), ("templates_bench_rocm", tpl_obj), ("jvp_check_rocm", jvp_obj),
+                        ("semantics_rocm", sem_obj), ("lm_dropin_rocm", dro_obj)]
     cpu_bin = REF_BIN / "configs_cpu"
     if force or _stale(cpu_bin, [cfg_src]):
         blas = sorted(Path("/usr/local/lib").glob("python3*/dist-packages/scipy.libs/libscipy_openblas*.so"))
@@ -248,13 +249,19 @@ def build_host(force: bool = False, jobs: int = 6):
         if r.returncode != 0:
             raise RuntimeError(f"configs.cu (cpu) failed:\n{r.stderr[-4000:]}")
     bins = [cpu_bin]
-    for rel, obj in REFERENCE_PROGRAMS_ALL:
-        out = REF_BIN / Path(rel).stem
+    links = [(REF_BIN / Path(rel).stem, obj, "$ORIGIN/../../../juzhen_amd/lib") for rel, obj in zip(REFERENCE_PROGRAMS, prog_objs)]
+    links += [(BIN / name, obj, "$ORIGIN/../lib") for name, obj in harness_programs]
+    for out, obj, rpath in links:
         if force or _stale(out, [obj, *lib_objs, LIB]):
             _hipcc(["--offload-arch=gfx950", "-o", str(out), str(obj), *map(str, lib_objs),
-                    f"-L{LIB.parent}", "-ljzhip", "-Wl,-rpath,$ORIGIN/../../../juzhen_amd/lib"],
+                    f"-L{LIB.parent}", "-ljzhip", f"-Wl,-rpath,{rpath}"],
                    f"link {out.name}")
         bins.append(out)
+    # earlier builds wrote the harness programs beside the reference's tests
+    for name, _ in harness_programs:
+        stale = REF_BIN / name
+        if stale.exists():
+            stale.unlink()
     return bins
 
 

@@ -103,6 +103,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_nrm2": (I, [P, P, Z]),
     "jzhip_max_cols": (I, [P, P, I, I, I]),
     "jzhip_argmax_cols": (I, [P, P, I, I, I]),
+    "jzhip_predict_one_hot": (I, [P, P, I, I, I]),
     "jzhip_gemm": (I, [P, P, P, I, I, I, I, I, I, I, I, F, F]),
     "jzhip_gemm_nn": (I, [P, P, P, I, I, I, F, F]),
     "jzhip_gemv": (I, [P, P, P, I, I, I, I, I, I, F, F]),
@@ -141,6 +142,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_conv2d_forward": (I, [P, P, P, P] + [I] * 14),
     "jzhip_conv2d_backward_weights": (I, [P, P, P] + [I] * 13),
     "jzhip_conv2d_backward_data": (I, [P, P, P] + [I] * 13),
+    "jzhip_conv2d_check": (I, [I] * 14),
 }
 
 

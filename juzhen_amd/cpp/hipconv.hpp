@@ -96,6 +96,14 @@ class ConvLayer : public Layer<ROCMfloat> {
         // input gradients: stride 1 only; needs channels on both sides and a grid of 16 x 16 or more
         dx_implicit = stride == 1 && pad <= kH - 1 && pad <= kW - 1 && C_in >= 32 && (long long)H_in * W_in >= 256 &&
                       (long long)H_in * W_in * N >= 16384;
+        // shapes beyond what the implicit entry points accept keep the patch-matrix route
+        auto accepted = [&](int which) {
+            return jzhip_conv2d_check(which, C_in, H_in, W_in, C_out, kH, kW, pad, pad, stride, stride, H_out, W_out,
+                                      N) == 0;
+        };
+        fwd_implicit = fwd_implicit && accepted(0);
+        dw_implicit = dw_implicit && accepted(1);
+        dx_implicit = dx_implicit && accepted(2);
     }
 
     void eval(const Matrix<D>& input) override { conv_into(this->val, input, ptr(this->bias), use_relu); }
@@ -189,6 +197,9 @@ class convtransLayer : public Layer<ROCMfloat> {
     int H_out, W_out;
     int batchN;
     bool use_relu = true;
+    // backward() as two implicit products; false for shapes those entry points refuse,
+    // which keep the gather + product route
+    bool bwd_implicit = true;
 
     static float* ptr(const Matrix<D>& m) { return JzRocmFused::ptr(m); }
     static void must(int rc, const char* what) { rocm_detail::must(rc, what); }
@@ -224,6 +235,11 @@ class convtransLayer : public Layer<ROCMfloat> {
         this->val = Matrix<D>("convtrans_out", (size_t)C_out * H_out * W_out, N);
         this->adamW = adam_state<D>(0.0001, wcount, 1);
         this->adamb = adam_state<D>(0.0001, C_out, 1);
+        // the two products of backward() seen as a convolution over the upstream gradient
+        bwd_implicit = jzhip_conv2d_check(0, C_out, H_out, W_out, C_in, kH, kW, pad, pad, stride, stride, H_in, W_in,
+                                          N) == 0 &&
+                       jzhip_conv2d_check(1, C_out, H_out, W_out, C_in, kH, kW, pad, pad, stride, stride, H_in, W_in,
+                                          N) == 0;
     }
 
     void eval(const Matrix<D>& input) override {
@@ -248,16 +264,34 @@ class convtransLayer : public Layer<ROCMfloat> {
         if (use_relu)
             must(jzhip_drelu_mul(ptr(t), ptr(this->val), ptr(t), (size_t)C_out * P_out * batchN), "drelu_mul");
 
-        // weight gradients in the stored (rows, C_in) layout
+        // weight gradients in the stored (rows, C_in) layout, and input gradients with the
+        // weights as they were in the forward pass
         Matrix<D> dW("deconv_dW", (size_t)rows * C_in, 1);
-        must(jzhip_conv2d_backward_weights(ptr(t), ptr(input), ptr(dW), C_out, H_out, W_out, C_in, kH, kW, pad_h, pad_w,
-                                           stride_h, stride_w, H_in, W_in, batchN),
-             "conv2d_backward_weights");
-        // input gradients with the weights as they were in the forward pass
         Matrix<D> dx("deconv_dx", (size_t)C_in * P_in, batchN);
-        must(jzhip_conv2d_forward(ptr(t), ptr(this->weights), nullptr, ptr(dx), C_out, H_out, W_out, C_in, kH, kW, pad_h,
-                                  pad_w, stride_h, stride_w, H_in, W_in, batchN, 0),
-             "conv2d_forward");
+        if (bwd_implicit) {
+            must(jzhip_conv2d_backward_weights(ptr(t), ptr(input), ptr(dW), C_out, H_out, W_out, C_in, kH, kW, pad_h,
+                                               pad_w, stride_h, stride_w, H_in, W_in, batchN),
+                 "conv2d_backward_weights");
+            must(jzhip_conv2d_forward(ptr(t), ptr(this->weights), nullptr, ptr(dx), C_out, H_out, W_out, C_in, kH, kW,
+                                      pad_h, pad_w, stride_h, stride_w, H_in, W_in, batchN, 0),
+                 "conv2d_forward");
+        } else {
+            // the sequence of ml/layer.hpp:1826-1852: tp = gather(t), x2d = pack(input),
+            // dW = tp x2d^T, dx = unpack(W^T tp)
+            const size_t cols = (size_t)P_in * batchN;
+            Matrix<D> tp("deconv_tp", rows, cols);
+            must(jzhip_convtrans_gather(ptr(t), ptr(tp), C_out, H_out, W_out, H_in, W_in, kH, kW, pad_h, pad_w, stride_h,
+                                        stride_w, batchN),
+                 "convtrans gather");
+            Matrix<D> x2d("deconv_x2d", C_in, cols);
+            must(jzhip_convtrans_reshape(ptr(input), ptr(x2d), C_in, P_in, batchN, 0), "convtrans reshape");
+            must(jzhip_gemm(ptr(tp), ptr(x2d), ptr(dW), rows, C_in, (int)cols, 0, 1, rows, C_in, rows, 1.0f, 0.0f), "gemm");
+            Matrix<D> dx2d("deconv_dx2d", C_in, cols);
+            must(jzhip_gemm(ptr(this->weights), ptr(tp), ptr(dx2d), C_in, (int)cols, rows, 1, 0, rows, rows, C_in, 1.0f,
+                            0.0f),
+                 "gemm");
+            must(jzhip_convtrans_reshape(ptr(dx2d), ptr(dx), C_in, P_in, batchN, 1), "convtrans reshape");
+        }
         // bias gradients: t read as a (P_out, C_out*N) matrix, column sums, then the N images
         Matrix<D> db("deconv_db", C_out, 1);
         {

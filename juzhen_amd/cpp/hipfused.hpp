@@ -135,7 +135,7 @@ class RocmStepGraph {
     RocmStepGraph(const RocmStepGraph&) = delete;
     RocmStepGraph& operator=(const RocmStepGraph&) = delete;
     ~RocmStepGraph() {
-        if (exec) jzhip_graph_destroy(exec);   // waits for replays in flight
+        if (exec) jzhip_graph_destroy(exec);   // waits for the streams the replays were launched on
         if (counter) jzhip_free(counter);
         pinned.clear();                        // the buffers return to the pool
     }

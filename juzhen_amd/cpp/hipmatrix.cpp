@@ -461,6 +461,28 @@ MR col_softmax(const MR& M) {
     return JzRocmFused::materialise(tmp);
 }
 
+}  // namespace Juzhen
+
+// 1 where an entry is within 1e-5 of its logical column's maximum, else 0; a plain
+// rows x cols matrix, as the generic chain of ml/util.cuh:258-279 returns
+MR predict_one_hot(const MR& input) {
+    MR out = JzRocmFused::make("one_hot_pred", input.num_row(), input.num_col(), 0);
+    if (input.num_row() == 0 || input.num_col() == 0) return out;
+    if (!input.get_transpose()) {
+        const int pr = as_int(JzRocmFused::phys_rows(input)), pc = as_int(JzRocmFused::phys_cols(input));
+        ok(jzhip_predict_one_hot(JzRocmFused::ptr(out), JzRocmFused::ptr(input), pr, pc, pr), "predict_one_hot");
+        return out;
+    }
+    // logical columns are strided in a transposed view: lay them out contiguously first
+    MR plain = JzRocmFused::materialise(input);
+    ok(jzhip_predict_one_hot(JzRocmFused::ptr(out), JzRocmFused::ptr(plain), as_int(input.num_row()),
+                             as_int(input.num_col()), as_int(input.num_row())),
+       "predict_one_hot");
+    return out;
+}
+
+namespace Juzhen {
+
 // row_softmax(M) = col_softmax(M.T()).T()  (ml/layer.hpp:2364-2367): the result
 // is always a transposed view of a plain (cols x rows) buffer, like the CPU's.
 MR row_softmax(const MR& M) {

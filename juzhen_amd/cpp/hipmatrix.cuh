@@ -9,7 +9,8 @@
 // Additions over the reference header, all ROCm-only and found by ordinary
 // overload resolution (a non-template overload beats the generic template, the
 // mechanism the reference uses for its Metal backend, ml/layer.hpp:2333-2339):
-// fused col_softmax/row_softmax, adam_update, relu/d_relu and predict_one_hot.
+// fused col_softmax/row_softmax, relu/d_relu and predict_one_hot here, adam_update and the
+// layer classes in hipfused_util.hpp / hipfused.hpp.
 #ifndef HIPMATRIX_CUH
 #define HIPMATRIX_CUH
 
@@ -179,6 +180,9 @@ namespace Juzhen {
 Matrix<ROCMfloat> col_softmax(const Matrix<ROCMfloat>& M);
 Matrix<ROCMfloat> row_softmax(const Matrix<ROCMfloat>& M);
 }  // namespace Juzhen
+// predict_one_hot (ml/util.cuh:258-279): column maximum and threshold in one launch
+// instead of reduce<F>, a rank-1 product, a subtraction and elemwise<F>.
+Matrix<ROCMfloat> predict_one_hot(const Matrix<ROCMfloat>& input);
 
 // Internal access point for the fused paths.
 struct JzRocmFused {

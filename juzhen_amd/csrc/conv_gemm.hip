@@ -770,7 +770,23 @@ bool dims_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
     // every index product must stay inside the 32-bit arithmetic the kernels use per image
     const long long chw = static_cast<long long>(C_in) * H_in * W_in, cop = static_cast<long long>(C_out) * H_out * W_out;
     const long long j = static_cast<long long>(H_out) * W_out * N, k = static_cast<long long>(C_in) * kH * kW;
-    return chw < (1ll << 30) && cop < (1ll << 30) && j < (1ll << 31) && k < (1ll << 24);
+    if (!(chw < (1ll << 30) && cop < (1ll << 30) && j < (1ll << 31) && k < (1ll << 24))) return false;
+    // the patch grid must be the one the geometry implies (or smaller): out, t and dx are sized
+    // from it by the caller, and a larger grid would be written past their end
+    const long long span_h = static_cast<long long>(H_in) + 2ll * pad_h - kH, span_w = static_cast<long long>(W_in) + 2ll * pad_w - kW;
+    if (span_h < 0 || span_w < 0) return false;
+    return H_out <= span_h / sh + 1 && W_out <= span_w / sw + 1;
+}
+
+// What jzhip_conv2d_backward_data needs beyond dims_ok: stride 1, the padding of a "full"
+// correlation non-negative, the input grid exactly the one a stride-1 layer maps to the
+// output grid, and the flipped weights small enough for the workspace.
+bool data_grad_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int sh, int sw,
+                  int H_out, int W_out) {
+    if (sh != 1 || sw != 1) return false;
+    if (pad_h > kH - 1 || pad_w > kW - 1) return false;
+    if (H_in != H_out + kH - 1 - 2 * pad_h || W_in != W_out + kW - 1 - 2 * pad_w) return false;
+    return static_cast<size_t>(C_out) * kH * kW * C_in <= kWorkspaceFloats;
 }
 
 int launch_fwd(const float* in, const float* Wt, const float* bias, float* out, const ConvGeom& g, int relu) {
@@ -906,10 +922,8 @@ JZ_API int jzhip_conv2d_backward_data(const float* t, const float* weights, floa
                                       int H_out, int W_out, int N) {
     if (!t || !weights || !dx) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
-    if (stride_h != 1 || stride_w != 1) return -1;
-    if (pad_h > kH - 1 || pad_w > kW - 1) return -1;
+    if (!data_grad_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out)) return -1;
     const size_t wcount = static_cast<size_t>(C_out) * kH * kW * C_in;
-    if (wcount > kWorkspaceFloats) return -1;
     float* flipped = workspace();
     if (!flipped) return -2;
     hipStream_t s = stream();
@@ -918,4 +932,13 @@ JZ_API int jzhip_conv2d_backward_data(const float* t, const float* weights, floa
     // flipped taps and padding k-1-pad lands on the H_in x W_in grid
     const ConvGeom g = make_geom(C_out, H_out, W_out, kH, kW, kH - 1 - pad_h, kW - 1 - pad_w, 1, 1, H_in, W_in, N, C_in);
     return launch_fwd(t, flipped, nullptr, dx, g, 0);
+}
+
+JZ_API int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w,
+                              int stride_h, int stride_w, int H_out, int W_out, int N) {
+    if (which < 0 || which > 2) return -1;
+    if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    if (which == 2 && !data_grad_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out))
+        return -1;
+    return 0;
 }

@@ -321,6 +321,40 @@ __global__ __launch_bounds__(kBlock) void max_cols_kernel(float* out_val, int32_
     }
 }
 
+// predict_one_hot (ml/util.cuh:258-279) in one launch: the column's maximum as the
+// generic chain's functor finds it (strictly-greater updates from the lowest value, so
+// NaNs never become the maximum), then x - max > -1e-5 evaluated in double, as the
+// chain's element-wise functor does after its float subtraction.  A wave per column;
+// the second sweep over the column is served by the cache.
+__global__ __launch_bounds__(kBlock) void one_hot_max_cols_kernel(float* out, const float* a, int numrow,
+                                                                  int numcol, size_t ld) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * (kBlock / kWave);
+    for (size_t col = wave0; col < static_cast<size_t>(numcol); col += nwaves) {
+        const float* p = a + col * ld;
+        float* q = out + col * static_cast<size_t>(numrow);
+        float best = -INFINITY;
+        int r = lane;
+        for (; r + 7 * kWave < numrow; r += 8 * kWave) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = p[r + u * kWave];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) best = v[u] > best ? v[u] : best;
+        }
+        for (; r < numrow; r += kWave) {
+            const float v = p[r];
+            best = v > best ? v : best;
+        }
+        const float m = wave_max(best);
+        for (r = lane; r < numrow; r += kWave) {
+            const float d = p[r] - m;
+            q[r] = static_cast<double>(d) > -1e-5 ? 1.0f : 0.0f;
+        }
+    }
+}
+
 int pick_chunks(size_t independent, size_t length, size_t min_len) {
     // enough (independent x chunks) work items to give every SIMD a few waves
     const size_t want = static_cast<size_t>(num_cus()) * 16;
@@ -482,6 +516,13 @@ JZ_API int jzhip_max_cols(float* out, const float* a, int numrow, int numcol, in
         max_cols_kernel<false, true><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
     else
         max_cols_kernel<false, false><<<grid, kBlock, 0, stream()>>>(out, nullptr, a, numrow, numcol, ld);
+    return launch_rc();
+}
+
+JZ_API int jzhip_predict_one_hot(float* out, const float* a, int numrow, int numcol, int ld) {
+    if (numrow <= 0 || numcol <= 0 || ld < numrow || !out || !a) return -1;
+    const unsigned grid = grid_cover(numcol, kBlock / kWave);
+    one_hot_max_cols_kernel<<<grid, kBlock, 0, stream()>>>(out, a, numrow, numcol, ld);
     return launch_rc();
 }
 

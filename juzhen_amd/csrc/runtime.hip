@@ -5,8 +5,11 @@
 
 #include <cstdint>
 
+#include <algorithm>
 #include <atomic>
 #include <mutex>
+#include <unordered_map>
+#include <vector>
 
 namespace jz {
 
@@ -213,6 +216,10 @@ std::mutex g_graph_mutex;
 hipStream_t g_record_stream = nullptr;   // created on first use, lives until the process ends
 hipStream_t g_stream_before = nullptr;   // the current stream when recording began
 std::atomic<int> g_recording{0};
+// the streams every recorded graph has been replayed on since it was made: a
+// replay runs on the current stream of its launch, never on the record stream,
+// and destroying the executable graph must wait for those
+std::unordered_map<void*, std::vector<hipStream_t>> g_replay_streams;
 }  // namespace
 
 JZ_API int jzhip_graph_begin(void) {
@@ -266,13 +273,37 @@ JZ_API int jzhip_graph_recording(void) { return g_recording.load(std::memory_ord
 JZ_API int jzhip_graph_launch(void* graph) {
     if (!graph || g_recording.load(std::memory_order_acquire)) return -1;
     // on the current stream, the null stream included
-    return jz::rc_of(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), jz::stream()));
+    const hipStream_t s = jz::stream();
+    {
+        std::lock_guard<std::mutex> lock(g_graph_mutex);
+        std::vector<hipStream_t>& used = g_replay_streams[graph];
+        if (std::find(used.begin(), used.end(), s) == used.end()) used.push_back(s);
+    }
+    return jz::rc_of(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), s));
 }
 
 JZ_API int jzhip_graph_destroy(void* graph) {
     if (!graph) return 0;
-    if (g_record_stream) (void)hipStreamSynchronize(g_record_stream);
-    return jz::rc_of(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+    if (g_recording.load(std::memory_order_acquire)) return -1;   // a wait would break the recording
+    // Replays may still be running on the streams they were launched on; their
+    // kernels read the executable graph's argument storage and the buffers the
+    // caller frees next, so wait for every such stream before the graph goes.
+    std::vector<hipStream_t> used;
+    {
+        std::lock_guard<std::mutex> lock(g_graph_mutex);
+        auto it = g_replay_streams.find(graph);
+        if (it != g_replay_streams.end()) {
+            used.swap(it->second);
+            g_replay_streams.erase(it);
+        }
+    }
+    int rc = 0;
+    for (hipStream_t s : used) {
+        const int r = jz::rc_of(hipStreamSynchronize(s));
+        if (r && !rc) rc = r;
+    }
+    const int rc2 = jz::rc_of(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+    return rc ? rc : rc2;
 }
 
 JZ_API int jzhip_set_stream(void* hip_stream) {
@@ -297,7 +328,25 @@ JZ_API int jzhip_stream_create(void** out_stream) {
 JZ_API int jzhip_stream_destroy(void* hip_stream) {
     if (!hip_stream) return 0;
     if (jz::stream() == static_cast<hipStream_t>(hip_stream)) jzhip_set_stream(nullptr);
-    const int rc = jz::release_workspace(static_cast<hipStream_t>(hip_stream));
+    int rc = jz::release_workspace(static_cast<hipStream_t>(hip_stream));
+    // replays launched on this stream must be over before its handle goes stale
+    // in the per-graph lists jzhip_graph_destroy walks
+    bool listed = false;
+    {
+        std::lock_guard<std::mutex> lock(g_graph_mutex);
+        for (auto& kv : g_replay_streams) {
+            auto& v = kv.second;
+            auto it = std::find(v.begin(), v.end(), static_cast<hipStream_t>(hip_stream));
+            if (it != v.end()) {
+                v.erase(it);
+                listed = true;
+            }
+        }
+    }
+    if (listed) {
+        const int r = jz::rc_of(hipStreamSynchronize(static_cast<hipStream_t>(hip_stream)));
+        if (r && !rc) rc = r;
+    }
     const int rc2 = jz::rc_of(hipStreamDestroy(static_cast<hipStream_t>(hip_stream)));
     return rc ? rc : rc2;
 }

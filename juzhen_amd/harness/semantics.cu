@@ -267,6 +267,10 @@ void battery(std::vector<Rec>& out, int r, int c, const std::string& tag) {
     out.push_back(rec(N("col_softmax(At)"), col_softmax(A.T()), 1e-4));
     out.push_back(rec(N("row_softmax(At)"), row_softmax(A.T()), 1e-4));
     out.push_back(rec(N("row_softmax(A)"), row_softmax(A), 1e-4));
+    // predict_one_hot (ml/util.cuh:258-279): plain result, every entry tied with its column's
+    // maximum gets a 1 (the quarter-integer inputs tie often)
+    out.push_back(rec(N("predict_one_hot(A)"), predict_one_hot(A)));
+    out.push_back(rec(N("predict_one_hot(At)"), predict_one_hot(A.T())));
     // copies keep the flag, T() aliases, to_host carries flag and physical dims
     {
         Matrix<D> X = deep(A.T());

@@ -109,3 +109,23 @@ def test_bench_refuses_more_than_one_gpu():
                        env={**env, "WORLD_SIZE": "2"}, timeout=300)
     assert r.returncode == 2
     assert "one GPU" in r.stderr
+
+
+def test_roofline_traffic_comes_from_the_committed_counter_summary():
+    """bench.py reads the HBM bytes per launch of its dominant kernel from the rocprofv3
+    summary under profiles/ instead of carrying constants: every tiled-GEMM row parses,
+    the bytes are fetch + write KiB of the row, and a kernel the summary does not hold
+    raises instead of reporting nothing."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", ROOT / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    text = bench.TRAFFIC_PROFILE.read_text()
+    rows = [l for l in text.splitlines() if l.startswith("gemm_mfma_kernel<")]
+    assert len(rows) >= 4
+    for l in rows:
+        name = l[:l.index(">") + 1]
+        f, w = (float(x) for x in l.split()[-3:-1])
+        assert bench.measured_traffic_bytes(name) == (f + w) * 1024.0
+    with pytest.raises(KeyError):
+        bench.measured_traffic_bytes("gemm_mfma_kernel<9, 9, 9, 9, false, false, false, false>")

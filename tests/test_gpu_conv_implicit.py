@@ -57,6 +57,11 @@ SMALL = [
     (3, 8, 9, 9, 2, 3, 3, 1, 2),      # the same with stride 2
     (2, 8, 8, 8, 4, 5, 5, 2, 1),      # four channels, 5x5: direct forward, tiled weight gradients
     (2, 3, 6, 6, 16, 3, 3, 1, 1),     # input gradients of a 3-channel image: the direct forward kernel with flipped weights
+    # kernels of more than 32 taps and patch rows beyond the tap table (K > 3072) take the loaders that
+    # decode every element's index, here with three and more K stages
+    (2, 3, 12, 12, 8, 7, 7, 3, 1),    # 7x7 stem, K = 147
+    (2, 3, 12, 12, 8, 7, 7, 3, 2),    # the same with stride 2
+    (1, 344, 4, 4, 8, 3, 3, 1, 1),    # K = 3096
 ]
 
 
@@ -190,3 +195,15 @@ def test_rejects_bad_arguments(gpu):
     assert lib.jzhip_conv2d_forward(None, dptr(d), None, dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1, 0) == -1
     assert lib.jzhip_conv2d_forward(dptr(d), dptr(d), None, dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 0, 1, 4, 4, 1, 0) == -1
     assert lib.jzhip_conv2d_backward_weights(dptr(d), dptr(d), None, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    # a patch grid larger than the geometry implies: (4 + 2 - 3)/1 + 1 = 4, not 5
+    assert lib.jzhip_conv2d_forward(dptr(d), dptr(d), None, dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 5, 4, 1, 0) == -1
+    assert lib.jzhip_conv2d_backward_weights(dptr(d), dptr(d), dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 5, 1) == -1
+    # input gradients need H_in == H_out + kH - 1 - 2*pad: a 3x3 grid under a 4x4 input with pad 1 is not that
+    assert lib.jzhip_conv2d_backward_data(dptr(d), dptr(d), dptr(d), 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 3, 3, 1) == -1
+    # the same answers from the query that launches nothing
+    assert lib.jzhip_conv2d_check(0, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == 0
+    assert lib.jzhip_conv2d_check(0, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 5, 4, 1) == -1
+    assert lib.jzhip_conv2d_check(2, 1, 4, 4, 1, 3, 3, 1, 1, 2, 2, 2, 2, 1) == -1      # stride 2
+    assert lib.jzhip_conv2d_check(2, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1   # 18.9 Mi weights
+    assert lib.jzhip_conv2d_check(1, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == 0
+    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1

@@ -9,6 +9,8 @@
     are not pinned by it; they are checked against an independent float64
     PyTorch autograd model on the CPU (closed-form definitions only).
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -133,15 +135,12 @@ def torch_twin(cfg, params, tokens, steps, lr, wd):
         for l in range(L):
             p = lambda n: P[f"block{l}.{n}"]
             x1 = ln(x, p("ln1_gamma"), p("ln1_beta"))
-            q, k, v = p("Wq") @ x1, p("Wk") @ x1, p("Wv") @ x1
-            H = torch.zeros_like(q)
-            for hh in range(heads):
-                for b in range(B):
-                    rs, cs = slice(hh * dh, (hh + 1) * dh), slice(b * S, (b + 1) * S)
-                    s = (q[rs, cs].T @ k[rs, cs]) / np.sqrt(dh)
-                    s = s.masked_fill(mask, -1e9)
-                    a = torch.softmax(s, dim=1)
-                    H[rs, cs] = v[rs, cs] @ a.T
+            # head hh owns rows [hh*dh, (hh+1)*dh), sequence b columns [b*S, (b+1)*S): all
+            # (head, sequence) blocks at once as (heads, dh, B, S) views
+            q, k, v = (t.reshape(heads, dh, B, S) for t in (p("Wq") @ x1, p("Wk") @ x1, p("Wv") @ x1))
+            s = torch.einsum("hdbq,hdbk->hbqk", q, k) / np.sqrt(dh)
+            a = torch.softmax(s.masked_fill(mask, -1e9), dim=3)
+            H = torch.einsum("hdbk,hbqk->hdbq", v, a).reshape(d, B * S)
             R = x + p("Wo") @ H + p("bo")
             x2 = ln(R, p("ln2_gamma"), p("ln2_beta"))
             f1 = p("W1") @ x2 + p("b1")
@@ -185,6 +184,113 @@ def test_gelu_tied_adamw_against_float64_autograd(gpu):
         a, b = m.get(n), final[n]
         assert np.linalg.norm(a - b) <= 2e-3 * np.linalg.norm(b), n
     m.close()
+
+
+def test_headline_variant_at_full_width_against_float64_autograd(gpu):
+    """The benchmark's own variant (exact-erf GELU, tied embeddings, AdamW with the decay
+    group) at the benchmark's width, depth, context and batch (d 512, 8 heads, ff 2048,
+    6 blocks, 256 x 64 tokens) beside the float64 autograd statement of the same model:
+    the loss and the gradients of the token table, the position table and one FFN weight
+    before any update, then the losses of two optimiser steps, all within 1e-3."""
+    import torch
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 256, 512, 8, 2048, 6, 256, 64
+    lr, wd = 3e-4, 0.01
+    rng = np.random.default_rng(31)
+    m = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=True, adamw=True, lr=lr, weight_decay=wd)
+    m.init_random(8)
+    for n in m.names:                      # live biases and gains
+        r, c = m.shape(n)
+        if c == 1:
+            m.set(n, m.get(n) + rng.normal(0, 0.05, (r, 1)).astype(np.float32))
+    params = {n: m.get(n).astype(np.float64) for n in m.names}
+    tokens = make_tokens(rng, V, B, S)
+    m.set_batch(tokens)
+    m.forward()
+    m.backward(update=False)
+    loss0 = m.loss()
+    grads = {n: m.get(n, which=1) for n in ("embed", "pos", "block0.W1", f"block{L - 1}.Wq", "block2.ln1_gamma")}
+    got = []
+    for _ in range(2):
+        m.step()
+        got.append(m.loss())
+    m.close()
+    print("float64 twin of the full-size model: two steps on the CPU ...", flush=True)
+    want, _, first = torch_twin((V, d, heads, ff, L, S, B), params, tokens, 2, lr, wd)
+    print(f"headline variant, full size: float64 losses {want}, ours {[loss0] + got[1:]}")
+    assert abs(loss0 - want[0]) <= 1e-3 * abs(want[0])
+    assert abs(got[0] - want[0]) <= 1e-3 * abs(want[0])
+    assert abs(got[1] - want[1]) <= 1e-3 * abs(want[1])
+    for n, g in grads.items():
+        rel = np.linalg.norm(g - first[n]) / np.linalg.norm(first[n])
+        print(f"  gradient of {n}: rel err {rel:.2e}")
+        assert rel <= 1e-3, (n, rel)
+
+
+def test_full_size_properties_of_the_headline_variant(gpu):
+    """Size-independent properties at the benchmark's full size: every parameter stays
+    finite over 20 steps and the loss falls; the gradient of the tied token table is the
+    sum of the head product's gradient and the lookup's gradient, which an untied model on
+    the same weights (head = table transposed, zero biases) yields separately."""
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 256, 512, 8, 2048, 6, 256, 64
+    rng = np.random.default_rng(77)
+    tokens = make_tokens(rng, V, B, S)
+    tied = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=True, adamw=True, lr=3e-4, weight_decay=0.01)
+    tied.init_random(9)
+    tied.set_batch(tokens)
+    tied.forward()
+    tied.backward(update=False)
+    g_tied = tied.get("embed", which=1)
+    untied = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=False, adamw=True, lr=3e-4, weight_decay=0.01)
+    for n in untied.names:
+        if n == "head":
+            untied.set(n, tied.get("embed").T)
+        elif n in ("embed_bias", "head_bias"):
+            r, c = untied.shape(n)
+            untied.set(n, np.zeros((r, c), np.float32))
+        else:
+            untied.set(n, tied.get(n))
+    untied.set_batch(tokens)
+    untied.forward()
+    untied.backward(update=False)
+    assert abs(untied.loss() - tied.loss()) <= 1e-6 * abs(tied.loss())
+    parts = untied.get("embed", which=1).astype(np.float64) + untied.get("head", which=1).astype(np.float64).T
+    rel = np.linalg.norm(g_tied - parts) / np.linalg.norm(parts)
+    print(f"tied-table gradient against lookup part + head part: rel err {rel:.2e}")
+    assert rel <= 1e-5
+    untied.close()
+    first = None
+    for i in range(20):
+        tied.step()
+        if i == 0:
+            first = tied.loss()
+    last = tied.loss()
+    assert np.isfinite(last) and last < first
+    for n in tied.names:
+        assert np.isfinite(tied.get(n)).all(), n
+        assert np.isfinite(tied.get(n, which=1)).all(), n
+    tied.close()
+
+
+def test_zero_gradient_adamw_step_is_the_decay_alone(gpu):
+    """With zero gradients and zero moments the update term is exactly 0, so a step of the
+    fused AdamW leaves w * (1 - lr*wd), the factor formed in fp32 as the kernel forms it,
+    bit for bit, on as many elements as the headline model has parameters; with wd = 0 the
+    weights do not move at all."""
+    import torch
+    n = 19_000_000 + 3
+    lr, wd = 3e-4, 0.01
+    w0 = torch.randn(n, device="cuda")
+    for decay in (wd, 0.0):
+        w, g, mm, vv = w0.clone(), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+        gpu.adamw_step(C.c_void_p(w.data_ptr()), C.c_void_p(g.data_ptr()), C.c_void_p(mm.data_ptr()),
+                       C.c_void_p(vv.data_ptr()), n, lr, 0.9, 0.999, 1e-8, decay, 1)
+        gpu.synchronize()
+        factor = np.float32(1.0) - np.float32(lr) * np.float32(decay)
+        want = w0.cpu().numpy() * factor if decay else w0.cpu().numpy()
+        assert np.array_equal(w.cpu().numpy(), want)
+        assert not mm.any() and not vv.any()
 
 
 def test_gradients_against_float64_autograd(gpu):

@@ -3,7 +3,9 @@ backend (juzhen_amd/cpp/hipmatrix.cuh, hipmatrix.cpp, hipkernels.cpp swapped
 into an overlay of the reference tree) and run on the GPU.  The binaries are
 built in the container by `python -m juzhen_amd.build --host` into
 oracle/_ref/bin/ and travel with the working tree; each must exit 0
-(the reference's ctest convention, CMakeLists.txt:320-400; 77 = skip)."""
+(the reference's ctest convention, CMakeLists.txt:320-400; 77 = skip).
+The programs of juzhen_amd/harness/ (this package's own sources on the
+Matrix<ROCMfloat> API) are built by the same step into juzhen_amd/bin/."""
 import json
 import os
 import struct
@@ -18,6 +20,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = Path(__file__).resolve().parent.parent
 BIN = ROOT / "oracle" / "_ref" / "bin"
+HARNESS_BIN = ROOT / "juzhen_amd" / "bin"
 PROJECT_DIR = Path("/tmp/jz_project")   # the PROJECT_DIR the programs were compiled with
 
 PROGRAMS = ["testRocmDeviceProof", "testRocmOpsSmoke", "testRocmCpuParity", "testbasic", "testStackOps",
@@ -56,7 +59,7 @@ def test_mirror_transpose_and_ownership_semantics(gpu, project_dir):
     shape-mismatch exceptions, Matrix<ROCMfloat> against Matrix<float> in one
     program, bit for bit (tests/testbasic.cu and tests/testStackOps.cu hold no
     ROCMfloat section, so a ROCm build of those two runs the CPU type only)."""
-    exe = need_ref_binary(BIN / "semantics_rocm")
+    exe = need_ref_binary(HARNESS_BIN / "semantics_rocm")
     r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300, cwd=str(project_dir))
     lines = [l for l in (r.stdout + r.stderr).splitlines() if not l.startswith("profiler:")]
     print("\n".join(lines[-30:]))
@@ -70,7 +73,7 @@ def test_forward_mode_tangents(gpu, project_dir):
     weights (1e-3; 1e-4 for the dense stack and LayerNorm), adjoint consistency with
     backprop on the device (1e-4) and central differences (5e-2, the criteria of
     tests/testJVP.cu:60-95, which itself skips on ROCm)."""
-    exe = need_ref_binary(BIN / "jvp_check_rocm")
+    exe = need_ref_binary(HARNESS_BIN / "jvp_check_rocm")
     r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300, cwd=str(project_dir))
     lines = [l for l in (r.stdout + r.stderr).splitlines() if l.startswith(("ok", "FAIL", "PASSED"))]
     print("\n".join(lines))

@@ -61,8 +61,9 @@ def hp(a):
 
 
 def need_ref_binary(exe):
-    """Programs built from the reference tree live under oracle/_ref (never
-    committed).  A missing one is a failure wherever a reference build was
+    """Programs built from the reference tree live under oracle/_ref, the
+    programs of juzhen_amd/harness (compiled against the reference's headers)
+    under juzhen_amd/bin (neither is committed).  A missing one is a failure wherever a reference build was
     possible or has happened (the tree is mounted, or oracle/_ref exists), and
     a skip only in a checkout that never saw the reference."""
     import os
