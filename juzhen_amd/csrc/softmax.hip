@@ -384,7 +384,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, 
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int cc = c + u * CP;
-            t[u] = cc < c1 ? load1<NT>(in + static_cast<size_t>(cc) * ld + row) : 0.f;
+            t[u] = cc < c1 ? in[static_cast<size_t>(cc) * ld + row] : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
@@ -394,48 +394,145 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_apply_kernel(float* out, 
     }
 }
 
-// Rows of up to 2048 columns held in registers by a 1024-thread block: 16 row
-// lanes x 64 column phases, NV columns per thread.  One read and one write per
-// element with numrow/16 workgroups (the 64-row form above leaves most of the
-// chip idle on a 1024 x 1024 matrix).
-constexpr int kWideThreads = 1024, kWideRows = 16, kWidePhases = kWideThreads / kWideRows;
-template <int NV>
-__global__ __launch_bounds__(kWideThreads) void softmax_rows_wide_kernel(float* out, const float* in,
-                                                                         int numrow, int numcol,
-                                                                         size_t ld) {
-    __shared__ float red[kWidePhases][kWideRows + 1];
-    const int rl = threadIdx.x % kWideRows, cp = threadIdx.x / kWideRows;
-    const int row = blockIdx.x * kWideRows + rl;
+// Whole rows in the registers of one workgroup, any split of its threads into RL row lanes
+// (consecutive rows: the coalesced direction) and THREADS/RL column phases; a thread holds
+// the NV columns cp, cp + CP, ... of its row.  One read and one write per element.  Column
+// phases that share a wave are combined by lane exchanges, the waves through LDS.
+// The split is picked per shape by softmax_rows_single_read below.  What decides it, as
+// measured on MI355X: the loads a thread has in flight (16 columns per thread: 6 us at
+// 1024 x 1024, 32: 8-9 us, 64: 17-20 us, whatever the run length), then the bytes a wave
+// reads contiguously per column (16-byte runs: 10.8 us), then the workgroup count.
+template <int THREADS, int RL, int NV>
+__global__ __launch_bounds__(THREADS) void softmax_rows_tile_kernel(float* out, const float* in, int numrow,
+                                                                    int numcol, size_t ld) {
+    constexpr int CP = THREADS / RL;          // column phases
+    constexpr int NW = THREADS / kWave;       // waves
+    constexpr int PPW = RL >= kWave ? 1 : kWave / RL;   // column phases inside one wave
+    constexpr int RPW = RL >= kWave ? kWave : RL;       // distinct rows inside one wave
+    constexpr int WPR = RL >= kWave ? RL / kWave : 1;   // waves side by side along the rows
+    static_assert(THREADS % kWave == 0 && (RL % kWave == 0 || kWave % RL == 0), "shape");
+    __shared__ float red[NW][RPW];
+    const int rl = threadIdx.x % RL, cp = threadIdx.x / RL;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lr = lane % RPW;                // row slot inside the wave
+    const int wr = wave % WPR;                // which row group of the workgroup this wave sits in
+    const int row = blockIdx.x * RL + rl;
     const bool live = row < numrow;
+    const float* p = in + row;
     float x[NV];
     float m = -1e30f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int c = cp + v * kWidePhases;
-        x[v] = (live && c < numcol) ? in[static_cast<size_t>(c) * ld + row] : -1e30f;
+        const int c = cp + v * CP;
+        x[v] = (live && c < numcol) ? p[static_cast<size_t>(c) * ld] : -1e30f;
         m = m > x[v] ? m : x[v];
     }
-    red[cp][rl] = m;
-    __syncthreads();
-    for (int k = 0; k < kWidePhases; ++k) m = m > red[k][rl] ? m : red[k][rl];
-    __syncthreads();
+    auto combine = [&](float val, auto op) {
+#pragma unroll
+        for (int off = RPW; off < kWave; off <<= 1) val = op(val, __shfl_xor(val, off, kWave));
+        if constexpr (NW > WPR) {
+            __syncthreads();                  // red may still be read from the previous round
+            if (lane < RPW) red[wave][lr] = val;
+            __syncthreads();
+            val = red[wr][lr];
+#pragma unroll
+            for (int w = WPR; w < NW; w += WPR) val = op(val, red[wr + w][lr]);
+        }
+        return val;
+    };
+    m = combine(m, MaxOp{});
     float s = 0.f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int c = cp + v * kWidePhases;
+        const int c = cp + v * CP;
         x[v] = (live && c < numcol) ? exp_neg(x[v] - m) : 0.f;
         s += x[v];
     }
-    red[cp][rl] = s;
-    __syncthreads();
-    s = 0.f;
-    for (int k = 0; k < kWidePhases; ++k) s += red[k][rl];
+    s = combine(s, SumOp{});
     const float inv = 1.0f / (s + 1e-12f);
     if (live) {
+        float* q = out + row;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int c = cp + v * kWidePhases;
-            if (c < numcol) out[static_cast<size_t>(c) * ld + row] = x[v] * inv;
+            const int c = cp + v * CP;
+            if (c < numcol) q[static_cast<size_t>(c) * ld] = x[v] * inv;
+        }
+    }
+}
+
+// The same with four consecutive rows per thread (one float4 per column): a quarter of the
+// load and store instructions for the same bytes, and RL4 row lanes cover 4*RL4 rows, so a
+// wave reads 16*RL4 contiguous bytes of each column.  Needs numrow % 4 == 0, ld % 4 == 0
+// and 16-byte aligned pointers.
+template <int THREADS, int RL4, int NV>
+__global__ __launch_bounds__(THREADS) void softmax_rows_tile4_kernel(float* out, const float* in, int numrow,
+                                                                     int numcol, size_t ld) {
+    constexpr int CP = THREADS / RL4;
+    constexpr int NW = THREADS / kWave;
+    constexpr int RPW = RL4 >= kWave ? kWave : RL4;     // distinct row lanes inside one wave
+    constexpr int WPR = RL4 >= kWave ? RL4 / kWave : 1;
+    static_assert(THREADS % kWave == 0 && (RL4 % kWave == 0 || kWave % RL4 == 0), "shape");
+    __shared__ float4 red[NW][RPW];
+    const int rl = threadIdx.x % RL4, cp = threadIdx.x / RL4;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lr = lane % RPW, wr = wave % WPR;
+    const int row = (blockIdx.x * RL4 + rl) * 4;
+    const bool live = row < numrow;
+    const float* p = in + row;
+    float4 x[NV];
+    float4 m = make_float4(-1e30f, -1e30f, -1e30f, -1e30f);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = cp + v * CP;
+        if (live && c < numcol) x[v] = *reinterpret_cast<const float4*>(p + static_cast<size_t>(c) * ld);
+        else x[v] = make_float4(-1e30f, -1e30f, -1e30f, -1e30f);
+        m.x = m.x > x[v].x ? m.x : x[v].x; m.y = m.y > x[v].y ? m.y : x[v].y;
+        m.z = m.z > x[v].z ? m.z : x[v].z; m.w = m.w > x[v].w ? m.w : x[v].w;
+    }
+    auto combine = [&](float4 val, auto op) {
+#pragma unroll
+        for (int off = RPW; off < kWave; off <<= 1) {
+            val.x = op(val.x, __shfl_xor(val.x, off, kWave)); val.y = op(val.y, __shfl_xor(val.y, off, kWave));
+            val.z = op(val.z, __shfl_xor(val.z, off, kWave)); val.w = op(val.w, __shfl_xor(val.w, off, kWave));
+        }
+        if constexpr (NW > WPR) {
+            __syncthreads();
+            if (lane < RPW) red[wave][lr] = val;
+            __syncthreads();
+            val = red[wr][lr];
+#pragma unroll
+            for (int w = WPR; w < NW; w += WPR) {
+                const float4 o = red[wr + w][lr];
+                val.x = op(val.x, o.x); val.y = op(val.y, o.y); val.z = op(val.z, o.z); val.w = op(val.w, o.w);
+            }
+        }
+        return val;
+    };
+    m = combine(m, MaxOp{});
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = cp + v * CP;
+        if (live && c < numcol) {
+            x[v].x = exp_neg(x[v].x - m.x); x[v].y = exp_neg(x[v].y - m.y);
+            x[v].z = exp_neg(x[v].z - m.z); x[v].w = exp_neg(x[v].w - m.w);
+        } else {
+            x[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        s.x += x[v].x; s.y += x[v].y; s.z += x[v].z; s.w += x[v].w;
+    }
+    s = combine(s, SumOp{});
+    const float4 inv = make_float4(1.0f / (s.x + 1e-12f), 1.0f / (s.y + 1e-12f), 1.0f / (s.z + 1e-12f),
+                                   1.0f / (s.w + 1e-12f));
+    if (live) {
+        float* q = out + row;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int c = cp + v * CP;
+            if (c < numcol) {
+                x[v].x *= inv.x; x[v].y *= inv.y; x[v].z *= inv.z; x[v].w *= inv.w;
+                *reinterpret_cast<float4*>(q + static_cast<size_t>(c) * ld) = x[v];
+            }
         }
     }
 }
@@ -700,13 +797,53 @@ int softmax_cols_impl(float* out, const float* in, int numrow, size_t numcol, si
     return launch_rc();
 }
 
+// Rows of at most 2048 columns: one read and one write per element, the split of the
+// workgroup chosen from the shapes measured (us on MI355X in brackets).
+int softmax_rows_single_read(float* out, const float* in, int numrow, int numcol, size_t ld, hipStream_t s) {
+#define JZ_ROWS_TILE(T, RL, NV)                                                                              \
+    do {                                                                                                     \
+        softmax_rows_tile_kernel<T, RL, NV><<<(numrow + RL - 1) / RL, T, 0, s>>>(out, in, numrow, numcol, ld); \
+        return launch_rc();                                                                                  \
+    } while (0)
+#define JZ_ROWS_TILE4(T, RL4, NV)                                                                                      \
+    do {                                                                                                               \
+        softmax_rows_tile4_kernel<T, RL4, NV><<<(numrow / 4 + RL4 - 1) / RL4, T, 0, s>>>(out, in, numrow, numcol, ld); \
+        return launch_rc();                                                                                            \
+    } while (0)
+    const bool f4 = numrow % 4 == 0 && ld % 4 == 0 && aligned16(in) && aligned16(out);
+    if (numcol <= 256) {
+        if (f4 && numrow >= 16384) JZ_ROWS_TILE4(256, 16, 16);   // 131072 x 256: 41 us, 6.5 TB/s (64 scalar row lanes: 94)
+        if (f4) JZ_ROWS_TILE4(256, 8, 8);                        // 16384 x 128: 5.4 us
+        JZ_ROWS_TILE(1024, 64, 16);                              // 131072 x 256: 44 us
+    }
+    if (numcol <= 512) {
+        if (f4 && numrow >= 4096) JZ_ROWS_TILE4(512, 8, 8);      // 16384 x 512: 14.3 us (scalar 16 x 64 split: 22)
+        if (numrow >= 4096) JZ_ROWS_TILE(1024, 64, 32);          // 16384 x 512: 15.2 us
+        JZ_ROWS_TILE(512, 8, 8);                                 // 512 x 512: 3.9 us, 1024 x 512: 4.1 us
+    }
+    if (numcol <= 1024) {
+        if (f4 && numrow >= 4096) JZ_ROWS_TILE4(1024, 8, 8);     // 4096 x 1024: 11.2 us, 65536 x 1024: 142 us
+        if (numrow >= 4096) JZ_ROWS_TILE(1024, 32, 32);          // 4096 x 1024: 11.3 us
+        if (numrow >= 2048) JZ_ROWS_TILE(1024, 16, 16);          // 2048 x 1024: 6.7 us
+        JZ_ROWS_TILE(512, 8, 16);                                // 1024 x 1024: 5.8 us (column form: 5.7)
+    }
+    if (f4 && numrow >= 8192) JZ_ROWS_TILE4(512, 8, 32);         // 16384 x 2048: 57 us (16 x 64 split: 80), 65536 x 2048: 292 (411)
+    if (f4) JZ_ROWS_TILE4(512, 4, 16);                           // 2048 x 2048: 15.1 us
+    if (numrow >= 8192) JZ_ROWS_TILE(1024, 32, 64);              // 16384 x 2048: 68 us
+    JZ_ROWS_TILE(1024, 16, 32);                                  // 2048 x 2048: 15.0 us
+#undef JZ_ROWS_TILE
+#undef JZ_ROWS_TILE4
+}
+
 int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_t ld, int batch,
                       size_t batch_stride, ScoreXform xf) {
     if (batch > 65535) return -1;
     hipStream_t s = stream();
     const int row_blocks = (numrow + kWave - 1) / kWave;
+    if (batch == 1 && !xf.S && numcol <= 2048 && numrow >= 256)
+        return softmax_rows_single_read(out, in, numrow, numcol, ld, s);
     if (numcol <= 256) {
-        // whole row in registers
+        // whole row in registers (batches of score blocks, short matrices)
         dim3 grid(row_blocks, batch);
         if (numcol <= 16)
             softmax_rows_reg_kernel<4><<<grid, kBlock, 0, s>>>(out, in, numrow, numcol, ld, batch_stride, xf);
@@ -719,17 +856,6 @@ int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_
         return launch_rc();
     }
     if (batch == 1 && !xf.S) {
-        if (numcol <= 2048 && numrow >= 512) {
-            // medium rows: registers of a 1024-thread block, numrow/16 workgroups
-            const unsigned grid = (numrow + kWideRows - 1) / kWideRows;
-            if (numcol <= 512)
-                softmax_rows_wide_kernel<8><<<grid, kWideThreads, 0, s>>>(out, in, numrow, numcol, ld);
-            else if (numcol <= 1024)
-                softmax_rows_wide_kernel<16><<<grid, kWideThreads, 0, s>>>(out, in, numrow, numcol, ld);
-            else
-                softmax_rows_wide_kernel<32><<<grid, kWideThreads, 0, s>>>(out, in, numrow, numcol, ld);
-            return launch_rc();
-        }
         // long rows: two passes with the columns split over grid.y so that
         // row_blocks x chunks fills the chip.  (Measured and dropped: four rows per lane with
         // float4 loads, 672 against 680 us at 16384 x 16384 and slower below; walking the
@@ -748,11 +874,16 @@ int softmax_rows_impl(float* out, const float* in, int numrow, int numcol, size_
             if (!part) return -2;
             float* rowstat = part + static_cast<size_t>(chunks) * numrow * 2;
             dim3 grid(row_blocks, chunks);
-            const bool nt = streams_past_cache(static_cast<size_t>(numrow) * numcol * sizeof(float));
-            if (nt) softmax_rows_partial_kernel<true><<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
-            else softmax_rows_partial_kernel<false><<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
+            // Loads stay plain in both passes (what the first pass leaves in the memory-side
+            // cache serves part of the second); the result is written with the streaming hint
+            // from 192 MB up, where it would only push the input out of that cache.  Measured,
+            // plain / hinted loads and stores / hinted stores only: 16384 x 4096 175 / 164 / 131 us,
+            // 8192 x 8192 180 / 167 / 134, 16384 x 16384 673 / 624 / 603; 2048 x 16384 (134 MB)
+            // 70 / 82 / 72, so smaller matrices keep plain stores.
+            const bool nt_out = static_cast<size_t>(numrow) * numcol * sizeof(float) >= (size_t(192) << 20);
+            softmax_rows_partial_kernel<false><<<grid, kBlock, 0, s>>>(part, in, numrow, numcol, ld, chunk_len);
             softmax_rows_fold_kernel<<<row_blocks, kFoldThreads, 0, s>>>(rowstat, part, numrow, chunks);
-            if (nt) softmax_rows_apply_kernel<true><<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
+            if (nt_out) softmax_rows_apply_kernel<true><<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
             else softmax_rows_apply_kernel<false><<<grid, kBlock, 0, s>>>(out, in, rowstat, numrow, numcol, ld, chunk_len);
             return launch_rc();
         }

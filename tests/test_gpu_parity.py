@@ -719,6 +719,28 @@ def test_softmax_cols_rows(gpu, oracle_lib, rows, cols):
     assert np.allclose(got.reshape(cols, rows).sum(axis=0), 1.0, atol=1e-5)
 
 
+@pytest.mark.parametrize("rows,cols,pad", [
+    # rows of at most 2048 columns are held in the registers of one workgroup; the split of the
+    # workgroup depends on the column count, the height and whether float4 access applies
+    # (rows and leading dimension multiples of 4): one case per branch, ragged edges included
+    (16384, 200, 0), (260, 100, 0), (301, 250, 3), (16388, 256, 4),
+    (4096, 400, 0), (4099, 300, 1), (300, 500, 0), (4100, 512, 8),
+    (4096, 1000, 0), (4097, 1024, 0), (2049, 700, 2), (1024, 1024, 0), (257, 900, 0),
+    (8192, 2048, 0), (2048, 1500, 4), (8193, 1100, 0), (1001, 2047, 0), (8200, 1025, 0)])
+def test_softmax_rows_single_read_forms(gpu, oracle_lib, rows, cols, pad):
+    ld = rows + pad
+    x = rng(rows + 3 * cols + pad).normal(0, 3, ld * cols).astype(np.float32)
+    ref = x.copy()                                   # the padding rows must come back untouched
+    oracle_lib.jzo_softmax_rows(hptr(ref), hptr(x), rows, cols, ld)
+    out = to_dev(x)
+    gpu.softmax_rows(dptr(out), dptr(out), rows, cols, ld)   # in place, as row_softmax of a view does
+    got = to_host(out).reshape(cols, ld)
+    ref = ref.reshape(cols, ld)
+    assert rel_err(got[:, :rows], ref[:, :rows]) <= TOL_RED
+    assert np.array_equal(got[:, rows:], x.reshape(cols, ld)[:, rows:])
+    assert np.allclose(got[:, :rows].sum(axis=0), 1.0, atol=1e-5)
+
+
 @pytest.mark.parametrize("S,nblk", [(8, 3), (64, 4), (100, 2), (256, 6)])
 @pytest.mark.parametrize("causal", [0, 1])
 @pytest.mark.parametrize("kar", [0, 1])
