@@ -441,6 +441,32 @@ int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv,
                            const float* Q, const float* K, const float* V,
                            int ld_qkv, const float* A, int d_k, int heads, int S,
                            int B, int causal);
+/* No reference counterpart (the reference caches four S x S x batch x heads buffers per
+ * block, ml/layer.hpp:2843-2848): the same attention core without any S x S matrix in
+ * memory.  `jzhip_attention_flash_fwd` computes H as jzhip_attention_fwd_ld does and keeps,
+ * instead of the probabilities A, two floats per query: stats, 2*S*heads*B floats, holds
+ * for block hh*B + b the S row maxima of the scaled, masked scores followed by the S
+ * values 1/(sum + 1e-12).  `jzhip_attention_flash_bwd` recomputes the probabilities tile
+ * by tile from Q, K and stats, forms the score gradients in registers and writes dQ, dK
+ * and dV from one kernel; it also needs H, the forward output (the row term of the
+ * softmax derivative is sum_d dH .* H).  Every element is summed in a fixed order, so
+ * results are reproducible bit for bit; against the materialising pair above they agree
+ * to rounding (1e-6 relative).  Shapes: head width 32 or 64, S a multiple of 32 up to 256,
+ * leading dimensions multiples of 4 and 16-byte aligned pointers; causal is 0 or 1.
+ * `jzhip_attention_flash_supported` says whether a shape qualifies (1) or not (0); the two
+ * calls return -1 for shapes that do not, and callers then use the pair above.  The first
+ * backward call for a given (S, causal) uploads a 268-byte visiting order with a blocking
+ * copy, so make that call outside a graph recording.  At S 256, 8 heads of 64, batch 64
+ * the six blocks of the character model keep 1.6 MB of stats instead of 1.6 GB of
+ * probabilities, and the shared 268 MB score-gradient scratch is not needed. */
+int jzhip_attention_flash_supported(int d_k, int heads, int S, int B);
+int jzhip_attention_flash_fwd(float* H, int ld_h, float* stats, const float* Q, const float* K,
+                              const float* V, int ld_qkv, int d_k, int heads, int S, int B,
+                              int causal);
+int jzhip_attention_flash_bwd(float* dQ, float* dK, float* dV, int ld_dqkv, const float* dH,
+                              int ld_dh, const float* Q, const float* K, const float* V,
+                              int ld_qkv, const float* H, int ld_h, const float* stats, int d_k,
+                              int heads, int S, int B, int causal);
 
 /* ── LayerNorm ───────────────────────────────────────────────────────── */
 

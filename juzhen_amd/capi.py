@@ -120,6 +120,9 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_softmax_xent_dense": (I, [P, P, P, P, I, I, I, F]),
     "jzhip_attention_fwd_ld": (I, [P, I, P, P, P, P, I, I, I, I, I, I]),
     "jzhip_attention_bwd_ld": (I, [P, P, P, I, P, P, I, P, P, P, I, P, I, I, I, I, I]),
+    "jzhip_attention_flash_supported": (I, [I, I, I, I]),
+    "jzhip_attention_flash_fwd": (I, [P, I, P, P, P, P, I, I, I, I, I, I]),
+    "jzhip_attention_flash_bwd": (I, [P, P, P, I, P, I, P, P, P, I, P, I, P, I, I, I, I, I]),
     "jzhip_attention_fwd": (I, [P, P, P, P, P, I, I, I, I, I]),
     "jzhip_attention_bwd": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I]),
     "jzhip_layernorm_fwd": (I, [P, P, P, P, P, P, I, I]),
@@ -186,7 +189,7 @@ class _Checked:
         name = "jzhip_" + short
         fn = getattr(load(), name)
         res = SIGNATURES[name][0]
-        if res is not I or short in ("runtime_available", "version", "num_compute_units"):
+        if res is not I or short in ("runtime_available", "version", "num_compute_units", "attention_flash_supported"):
             return fn
 
         def call(*args):

@@ -66,7 +66,7 @@ template <int DH> constexpr int kLD1 = DH == 64 ? kMaxKeys + 1 : kMaxKeys + 2;
 // step s of the second product contracts exactly the keys held in register s.
 template <int DH, bool BWD, int NQ>
 __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, float* __restrict__ Ablk,
-                                           float* __restrict__ dSblk, const float (&xf)[DH / 4],
+                                           float* __restrict__ dSblk, float* __restrict__ stat, const float (&xf)[DH / 4],
                                            const float* t1, const float* t2, int S, int nkt, int g,
                                            int l16, int kq, float scale, int causal) {
     constexpr int HD4 = DH / 4;       // contraction steps of the first product
@@ -144,14 +144,30 @@ __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, 
         sum += __shfl_xor(sum, 16);
         sum += __shfl_xor(sum, 32);
         const float inv = 1.0f / (sum + 1e-12f);
+        if (stat) {
+            // the probabilities are not kept: the backward pass recomputes them from the
+            // query's maximum and reciprocal sum (S maxima, then S reciprocals per block)
+            if (kq == 0) {
+                stat[q] = m;
+                stat[S + q] = inv;
+            }
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if (t < nkt) {
+            for (int t = 0; t < NT; ++t) {
+                if (t < nkt) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float pv = sc[t][v] * inv;
-                    sc[t][v] = pv;
-                    (Ablk + static_cast<size_t>(16 * t + v) * S)[lane_off] = pv;
+                    for (int v = 0; v < 4; ++v) sc[t][v] *= inv;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                if (t < nkt) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float pv = sc[t][v] * inv;
+                        sc[t][v] = pv;
+                        (Ablk + static_cast<size_t>(16 * t + v) * S)[lane_off] = pv;
+                    }
                 }
             }
         }
@@ -204,7 +220,7 @@ __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, 
     }
     // key tiles past the causal range hold exact zeros (causal == 2: the caller
     // states that they already do, from an earlier call on the same buffer)
-    if (causal != 2)
+    if (causal != 2 && (BWD || !stat))
         for (int t = nkt; t < S / 16; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) ((BWD ? dSblk : Ablk) + static_cast<size_t>(16 * t + v) * S)[lane_off] = 0.0f;
@@ -249,7 +265,7 @@ __device__ __forceinline__ void attn_group(float* __restrict__ out, int ld_out, 
 template <int DH, bool BWD>
 __global__ __launch_bounds__(kAttnThreads) void attn_core_kernel(
     float* __restrict__ Out, int ld_out, float* __restrict__ Aio, float* __restrict__ dS_out,
-    const float* __restrict__ X1, int ld_x1, const float* __restrict__ M1, const float* __restrict__ M2,
+    float* __restrict__ stats, const float* __restrict__ X1, int ld_x1, const float* __restrict__ M1, const float* __restrict__ M2,
     int ld_m, int heads, int S, int B, float scale, int causal) {
     constexpr int HD4 = DH / 4;
     constexpr int LD2 = DH + 4;
@@ -268,8 +284,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_core_kernel(
     const float* x1 = X1 + col0 * ld_x1 + hh * DH;
     float* out = Out + col0 * ld_out + hh * DH;
     const size_t blk_off = static_cast<size_t>(blk) * S * S;
-    float* Ablk = Aio + blk_off;
+    float* Ablk = Aio ? Aio + blk_off : nullptr;
     float* dSblk = BWD ? dS_out + blk_off : nullptr;
+    float* stat = (!BWD && stats) ? stats + static_cast<size_t>(blk) * 2 * S : nullptr;
 
     // the four waves of a SIMD (w, w+4, w+8, w+12) take query groups s, 7-s,
     // 8+s, 15-s: with the causal triangle every SIMD gets the same work
@@ -326,10 +343,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_core_kernel(
     if (mine) {
         const int nkt = causal ? g + 1 : GQ;          // key tiles that are not entirely masked
         switch ((nkt + 3) / 4) {
-        case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
-        case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
-        case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
-        default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        case 1: attn_group<DH, BWD, 1>(out, ld_out, Ablk, dSblk, stat, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        case 2: attn_group<DH, BWD, 2>(out, ld_out, Ablk, dSblk, stat, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        case 3: attn_group<DH, BWD, 3>(out, ld_out, Ablk, dSblk, stat, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
+        default: attn_group<DH, BWD, 4>(out, ld_out, Ablk, dSblk, stat, xf, t1, t2, S, nkt, g, l16, kq, scale, causal); break;
         }
     }
 }
@@ -352,8 +369,8 @@ bool attn_core_ok(int d_h, int S, int heads, int B, const void* p0, const void* 
 }
 
 template <int DH, bool BWD>
-int launch_attn_core(float* Out, int ld_out, float* Aio, float* dS, const float* X1, int ld_x1, const float* M1,
-                     const float* M2, int ld_m, int heads, int S, int B, float scale, int causal) {
+int launch_attn_core(float* Out, int ld_out, float* Aio, float* dS, float* stats, const float* X1, int ld_x1,
+                     const float* M1, const float* M2, int ld_m, int heads, int S, int B, float scale, int causal) {
     const size_t lds = attn_core_lds_bytes(DH, S);
     static std::once_flag once;   // per instantiation
     static int configure_rc = 0;
@@ -362,8 +379,8 @@ int launch_attn_core(float* Out, int ld_out, float* Aio, float* dS, const float*
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     });
     if (configure_rc) return configure_rc;
-    attn_core_kernel<DH, BWD><<<heads * B, kAttnThreads, lds, stream()>>>(Out, ld_out, Aio, dS, X1, ld_x1, M1, M2, ld_m,
-                                                                   heads, S, B, scale, causal);
+    attn_core_kernel<DH, BWD><<<heads * B, kAttnThreads, lds, stream()>>>(Out, ld_out, Aio, dS, stats, X1, ld_x1, M1, M2,
+                                                                   ld_m, heads, S, B, scale, causal);
     return launch_rc();
 }
 
@@ -383,9 +400,9 @@ JZ_API int jzhip_attention_fwd_ld(float* H, int ld_h, float* A, const float* Q, 
     const float scale = 1.0f / sqrtf(static_cast<float>(d_h));
     if (jz::attn_core_ok(d_h, S, heads, B, H, Q, K, V, ld_h, ld_qkv, ld_qkv)) {
         if (d_h == 64)
-            return jz::launch_attn_core<64, false>(H, ld_h, A, nullptr, Q, ld_qkv, K, V, ld_qkv, heads, S, B, scale,
-                                                   causal);
-        return jz::launch_attn_core<32, false>(H, ld_h, A, nullptr, Q, ld_qkv, K, V, ld_qkv, heads, S, B, scale,
+            return jz::launch_attn_core<64, false>(H, ld_h, A, nullptr, nullptr, Q, ld_qkv, K, V, ld_qkv, heads, S, B,
+                                                   scale, causal);
+        return jz::launch_attn_core<32, false>(H, ld_h, A, nullptr, nullptr, Q, ld_qkv, K, V, ld_qkv, heads, S, B, scale,
                                                causal);
     }
     // scores[q, k] = <Q_i[:, q], K_i[:, k]>
@@ -426,10 +443,10 @@ JZ_API int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv, 
     if (jz::attn_core_ok(d_h, S, heads, B, dQ, dH, K, V, ld_dqkv, ld_dh, ld_qkv)) {
         // dA, dS and dQ in one launch; with causal set the key tiles above the
         // diagonal (exact zeros in A) are skipped
-        rc = d_h == 64 ? jz::launch_attn_core<64, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, dH, ld_dh, V,
-                                                        K, ld_qkv, heads, S, B, scale, causal)
-                       : jz::launch_attn_core<32, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, dH, ld_dh, V,
-                                                        K, ld_qkv, heads, S, B, scale, causal);
+        rc = d_h == 64 ? jz::launch_attn_core<64, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, nullptr, dH,
+                                                        ld_dh, V, K, ld_qkv, heads, S, B, scale, causal)
+                       : jz::launch_attn_core<32, true>(dQ, ld_dqkv, const_cast<float*>(A), dA_scratch, nullptr, dH,
+                                                        ld_dh, V, K, ld_qkv, heads, S, B, scale, causal);
         if (rc) return rc;
         // dK_i = Q_i * dS_i
         return jz::gemm_batched2(Q, dA_scratch, dK, d_h, S, S, false, false, ld_qkv, S, ld_dqkv, seq, blk, seq_d, B,
@@ -455,4 +472,19 @@ JZ_API int jzhip_attention_bwd(float* dQ, float* dK, float* dV, float* dA_scratc
                                const float* Q, const float* K, const float* V, const float* A,
                                int d_k, int heads, int S, int B) {
     return jzhip_attention_bwd_ld(dQ, dK, dV, d_k, dA_scratch, dH, d_k, Q, K, V, d_k, A, d_k, heads, S, B, 0);
+}
+
+JZ_API int jzhip_attention_flash_fwd(float* H, int ld_h, float* stats, const float* Q, const float* K, const float* V,
+                                     int ld_qkv, int d_k, int heads, int S, int B, int causal) {
+    if (!H || !stats || !Q || !K || !V) return -1;
+    if (!jzhip_attention_flash_supported(d_k, heads, S, B)) return -1;
+    if (ld_h < d_k || ld_qkv < d_k || causal < 0 || causal > 1) return -1;
+    const int d_h = d_k / heads;
+    if (!jz::attn_core_ok(d_h, S, heads, B, H, Q, K, V, ld_h, ld_qkv, ld_qkv)) return -1;
+    const float scale = 1.0f / sqrtf(static_cast<float>(d_h));
+    if (d_h == 64)
+        return jz::launch_attn_core<64, false>(H, ld_h, nullptr, nullptr, stats, Q, ld_qkv, K, V, ld_qkv, heads, S, B,
+                                               scale, causal);
+    return jz::launch_attn_core<32, false>(H, ld_h, nullptr, nullptr, stats, Q, ld_qkv, K, V, ld_qkv, heads, S, B, scale,
+                                           causal);
 }
