@@ -345,6 +345,7 @@ def main():
             dropin = {"tokens_per_s": None, "error": str(exc)}
 
     param_count = int(model.param_count)
+    flash_attention = model.flash_attention
     model.close()
     # The other legs of the metric (GEMM TFLOP/s and elementwise GB/s against their rooflines) and the
     # other benchmark configurations, measured in this run after the timed region; with the CPU
@@ -369,6 +370,8 @@ def main():
                    "backward_streams": 2 if args.two_stream and not args.serial else 1,
                    "batch_upload": "every step (host ids -> device inside the timed region)" if fresh
                                    else "once, before the timed region",
+                   "attention": "no S x S matrix kept (jzhip_attention_flash_fwd/_bwd)" if flash_attention
+                                else "probabilities materialised (jzhip_attention_fwd_ld/_bwd_ld)",
                    "parameters": param_count, "loss_first": round(first_loss, 4),
                    "loss_last": round(last_loss, 4), "gpu_ms_per_step": round(gpu_ms / args.steps, 3)},
         "roofline": roofline,

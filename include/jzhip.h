@@ -460,6 +460,15 @@ int jzhip_attention_bwd_ld(float* dQ, float* dK, float* dV, int ld_dqkv,
  * the six blocks of the character model keep 1.6 MB of stats instead of 1.6 GB of
  * probabilities, and the shared 268 MB score-gradient scratch is not needed. */
 int jzhip_attention_flash_supported(int d_k, int heads, int S, int B);
+/* Host only, no GPU needed: the order in which jzhip_attention_flash_bwd visits the
+ * (query tile, key tile) cells of one S x S block (tiles of 16).  The kernel runs S/32
+ * waves; in step j wave o works on cells[2*(j*S/32 + o)] (query tile) and
+ * cells[2*(j*S/32 + o) + 1] (key tile).  Returns the number of steps (S/16 + 1 with the
+ * causal mask, 2*S/16 without) or -1 (bad arguments, capacity below 2*steps*S/32 ints).
+ * What makes the result reproducible bit for bit: the waves of one step are on distinct
+ * query tiles, every cell is visited exactly once, and a wave finishes one key tile
+ * before it starts its other one. */
+int jzhip_attention_flash_order(int S, int causal, int* cells, int capacity);
 int jzhip_attention_flash_fwd(float* H, int ld_h, float* stats, const float* Q, const float* K,
                               const float* V, int ld_qkv, int d_k, int heads, int S, int B,
                               int causal);

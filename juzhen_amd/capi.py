@@ -121,6 +121,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_attention_fwd_ld": (I, [P, I, P, P, P, P, I, I, I, I, I, I]),
     "jzhip_attention_bwd_ld": (I, [P, P, P, I, P, P, I, P, P, P, I, P, I, I, I, I, I]),
     "jzhip_attention_flash_supported": (I, [I, I, I, I]),
+    "jzhip_attention_flash_order": (I, [I, I, P, I]),
     "jzhip_attention_flash_fwd": (I, [P, I, P, P, P, P, I, I, I, I, I, I]),
     "jzhip_attention_flash_bwd": (I, [P, P, P, I, P, I, P, P, P, I, P, I, P, I, I, I, I, I]),
     "jzhip_attention_fwd": (I, [P, P, P, P, P, I, I, I, I, I]),
@@ -189,7 +190,8 @@ class _Checked:
         name = "jzhip_" + short
         fn = getattr(load(), name)
         res = SIGNATURES[name][0]
-        if res is not I or short in ("runtime_available", "version", "num_compute_units", "attention_flash_supported"):
+        if res is not I or short in ("runtime_available", "version", "num_compute_units", "attention_flash_supported",
+                                    "attention_flash_order"):
             return fn
 
         def call(*args):

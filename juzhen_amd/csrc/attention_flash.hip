@@ -47,12 +47,19 @@ constexpr int kMaxOwners = kMaxTiles / 2;
 constexpr int kMaxSteps = 2 * kMaxTiles;   // without a mask every wave visits 2 * S/16 cells
 
 // row[j][o]: query tile of wave o's cell in step j.  Steps [0, first[o]) of wave o
-// belong to key tile o, the others to key tile tiles-1-o.
+// belong to key tile o, the others to key tile tiles-1-o.  packed[o] holds wave o's
+// column of row[][] as 4-bit fields, step j in bits 4*(j%16) of word j/16: two scalar
+// loads give a wave its whole visiting order.
+// Everything the kernel reads is a 4-byte or 8-byte field at an aligned offset: the
+// compiler folds a wave-uniform byte index into the base of a scalar load, and scalar
+// loads drop the two low address bits (a byte-sized `first` made waves 1, 2, 3 of
+// every four read another wave's order).
 struct FlashSchedule {
-    uint8_t row[kMaxSteps][kMaxOwners];
-    uint8_t first[kMaxOwners];
+    uint64_t packed[kMaxOwners][2];
+    int32_t first[kMaxOwners];
     int32_t steps;
     int32_t tiles;
+    uint8_t row[kMaxSteps][kMaxOwners];   // host side only: the table the packed form is made from
 };
 
 // Cells (query tile t, key tile k), t >= k under the causal mask.  Every wave walks
@@ -134,13 +141,16 @@ bool build_schedule(int tiles, bool causal, FlashSchedule* s) {
         for (int h = 0; h < 2; ++h) {
             const int k = q.key_tile(o, h);
             q.left[o][h] = causal ? static_cast<uint16_t>(all & ~((1u << k) - 1u)) : all;
-            if (h == 0) s->first[o] = static_cast<uint8_t>(__builtin_popcount(q.left[o][0]));
+            if (h == 0) s->first[o] = __builtin_popcount(q.left[o][0]);
         }
-    return q.step(0);
+    if (!q.step(0)) return false;
+    for (int o = 0; o < q.owners; ++o)
+        for (int j = 0; j < q.steps; ++j) s->packed[o][j / 16] |= static_cast<uint64_t>(s->row[j][o]) << (4 * (j % 16));
+    return true;
 }
 
 // One table per (S/32, causal) in device memory, built and uploaded on first use
-// and kept until the process ends (4.5 KB in all).
+// and kept until the process ends (6.5 KB in all).
 constexpr int kScheduleSlots = kMaxOwners * 2;
 struct ScheduleStore {
     std::mutex mutex;
@@ -221,7 +231,61 @@ __global__ __launch_bounds__(512) void attn_flash_bwd_kernel(
     const int l16 = lane & 15, kq = lane >> 4;
     const int tiles = S / 16;
 
-    // ── prologue: clear the dQ accumulator, fetch the row statistics, form D ──
+
+    float* stage_q = stage_all + static_cast<size_t>(o) * 2 * 16 * LDP;   // [16 queries][LDP]
+    float* stage_dh = stage_q + 16 * LDP;
+    float* patch = patch_all + static_cast<size_t>(o) * FlashLds<DH>::kPatch;
+
+    // fragments of a 16-token tile as the operand whose free index is the token: lane (l16, kq)
+    // holds d = HD4*kq .. HD4*kq + HD4-1 of token 16*tile + l16 (one contiguous run)
+    auto load_rows = [&](const float* base, int ld, int tile, float (&f)[HD4]) {
+        const float* src = base + static_cast<size_t>(16 * tile + l16) * ld + HD4 * kq;
+#pragma unroll
+        for (int i = 0; i < HD4 / 4; ++i) {
+            const floatx4 t4 = *reinterpret_cast<const floatx4*>(src + 4 * i);
+            f[4 * i] = t4.x; f[4 * i + 1] = t4.y; f[4 * i + 2] = t4.z; f[4 * i + 3] = t4.w;
+        }
+    };
+
+    // K, V of a key tile as B operands of S^T and dA^T (kb, vb) and K as the A operand of the dQ
+    // product (ka: d = 16u + l16, key 4kq + s).  Both key tiles of the wave are fetched before the
+    // loop: a fetch in the step where a wave changes tiles would hold every wave at that step's
+    // barrier, and the eight waves change at eight different steps.
+    auto load_key_tile = [&](int kt, float (&kb)[HD4], float (&vb)[HD4], float (&ka)[NDT][4]) {
+        load_rows(k_blk, ld_qkv, kt, kb);
+        load_rows(v_blk, ld_qkv, kt, vb);
+#pragma unroll
+        for (int u = 0; u < NDT; ++u)
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                ka[u][s] = k_blk[static_cast<size_t>(16 * kt + 4 * kq + s) * ld_qkv + 16 * u + l16];
+    };
+    // register v of accumulator tile u is d = 16u + 4kq + v of key 16*kt + l16
+    auto store_key_tile = [&](int kt, const floatx4 (&dv_acc)[NDT], const floatx4 (&dk_acc)[NDT]) {
+        float* pv = dv_blk + static_cast<size_t>(16 * kt + l16) * ld_d + 4 * kq;
+        float* pk = dk_blk + static_cast<size_t>(16 * kt + l16) * ld_d + 4 * kq;
+#pragma unroll
+        for (int u = 0; u < NDT; ++u) {
+            *reinterpret_cast<floatx4*>(pv + 16 * u) = dv_acc[u];
+            *reinterpret_cast<floatx4*>(pk + 16 * u) = dk_acc[u];
+        }
+    };
+    float kb0[HD4], vb0[HD4], ka0[NDT][4], kb1[HD4], vb1[HD4], ka1[NDT][4];
+    load_key_tile(o, kb0, vb0, ka0);
+    load_key_tile(tiles - 1 - o, kb1, vb1, ka1);
+
+    const int steps = sched->steps;
+    const int first = sched->first[o];
+    const uint64_t order_lo = sched->packed[o][0], order_hi = sched->packed[o][1];
+    auto row_of = [&](int j) { return static_cast<int>(((j < 16 ? order_lo : order_hi) >> (4 * (j & 15))) & 15u); };
+    float qf[HD4], hf[HD4];          // the step's query tile: Q and dH, token-major fragments
+    int t = row_of(0);
+    load_rows(q_blk, ld_qkv, t, qf);
+    load_rows(dh_blk, ld_dh, t, hf);
+
+    // ── prologue: clear the dQ accumulator, fetch the row statistics, form D.  It comes after the
+    // requests for the key tiles and the first query tile, so that all of the block's first
+    // reads are in flight together instead of one latency after another ──
     for (int i = tid; i < S * LDP / 4; i += blockDim.x)
         reinterpret_cast<floatx4*>(dq_acc)[i] = floatx4{0.f, 0.f, 0.f, 0.f};
     {
@@ -245,65 +309,11 @@ __global__ __launch_bounds__(512) void attn_flash_bwd_kernel(
     }
     __syncthreads();
 
-    float* stage_q = stage_all + static_cast<size_t>(o) * 2 * 16 * LDP;   // [16 queries][LDP]
-    float* stage_dh = stage_q + 16 * LDP;
-    float* patch = patch_all + static_cast<size_t>(o) * FlashLds<DH>::kPatch;
-
-    // fragments of a 16-token tile as the operand whose free index is the token: lane (l16, kq)
-    // holds d = HD4*kq .. HD4*kq + HD4-1 of token 16*tile + l16 (one contiguous run)
-    auto load_rows = [&](const float* base, int ld, int tile, float (&f)[HD4]) {
-        const float* src = base + static_cast<size_t>(16 * tile + l16) * ld + HD4 * kq;
-#pragma unroll
-        for (int i = 0; i < HD4 / 4; ++i) {
-            const floatx4 t4 = *reinterpret_cast<const floatx4*>(src + 4 * i);
-            f[4 * i] = t4.x; f[4 * i + 1] = t4.y; f[4 * i + 2] = t4.z; f[4 * i + 3] = t4.w;
-        }
-    };
-
-    float kb[HD4], vb[HD4];          // key tile's K, V: B operands of S^T and dA^T
-    float ka[NDT][4];                // key tile's K as the A operand of the dQ product: d = 16u + l16, key 4kq + s
-    floatx4 dv_acc[NDT], dk_acc[NDT];
-    int kt = o;                      // current key tile
-    auto load_key_tile = [&]() {
-        load_rows(k_blk, ld_qkv, kt, kb);
-        load_rows(v_blk, ld_qkv, kt, vb);
-#pragma unroll
-        for (int u = 0; u < NDT; ++u)
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                ka[u][s] = k_blk[static_cast<size_t>(16 * kt + 4 * kq + s) * ld_qkv + 16 * u + l16];
-#pragma unroll
-        for (int u = 0; u < NDT; ++u) {
-            dv_acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-            dk_acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
-        }
-    };
-    // register v of accumulator tile u is d = 16u + 4kq + v of key 16*kt + l16
-    auto store_key_tile = [&]() {
-        float* pv = dv_blk + static_cast<size_t>(16 * kt + l16) * ld_d + 4 * kq;
-        float* pk = dk_blk + static_cast<size_t>(16 * kt + l16) * ld_d + 4 * kq;
-#pragma unroll
-        for (int u = 0; u < NDT; ++u) {
-            *reinterpret_cast<floatx4*>(pv + 16 * u) = dv_acc[u];
-            *reinterpret_cast<floatx4*>(pk + 16 * u) = dk_acc[u];
-        }
-    };
-    load_key_tile();
-
-    const int steps = sched->steps;
-    const int first = sched->first[o];
-    float qf[HD4], hf[HD4];          // the step's query tile: Q and dH, token-major fragments
-    int t = sched->row[0][o];
-    load_rows(q_blk, ld_qkv, t, qf);
-    load_rows(dh_blk, ld_dh, t, hf);
-
-    for (int j = 0; j < steps; ++j) {
-        if (j == first) {            // second key tile of this wave
-            store_key_tile();
-            kt = tiles - 1 - o;
-            load_key_tile();
-        }
-        // the wave's copy of the query tile, [query][d]
+    // one cell: query tile t against key tile kt
+    auto cell = [&](int j, int kt, const float (&kb)[HD4], const float (&vb)[HD4], const float (&ka)[NDT][4],
+                    floatx4 (&dv_acc)[NDT], floatx4 (&dk_acc)[NDT]) {
+        // the wave's copy of the query tile, [query][d]; the tile's slice of the dQ accumulator
+        // (nobody else touches query tile t in this step) is requested now and used last
         {
             float* dq_ = stage_q + l16 * LDP + HD4 * kq;
             float* dh_ = stage_dh + l16 * LDP + HD4 * kq;
@@ -313,6 +323,13 @@ __global__ __launch_bounds__(512) void attn_flash_bwd_kernel(
                 *reinterpret_cast<floatx4*>(dh_ + 4 * i) = floatx4{hf[4 * i], hf[4 * i + 1], hf[4 * i + 2], hf[4 * i + 3]};
             }
         }
+        float* acc = dq_acc + static_cast<size_t>(16 * t + l16) * LDP + 4 * kq;
+        floatx4 cur[NDT];
+#pragma unroll
+        for (int u = 0; u < NDT; ++u) cur[u] = *reinterpret_cast<floatx4*>(acc + 16 * u);
+        const floatx4 m4 = *reinterpret_cast<const floatx4*>(st_m + 16 * t + 4 * kq);
+        const floatx4 i4 = *reinterpret_cast<const floatx4*>(st_inv + 16 * t + 4 * kq);
+        const floatx4 d4 = *reinterpret_cast<const floatx4*>(st_D + 16 * t + 4 * kq);
         // S^T and dA^T: rows = queries of tile t, columns = keys of tile kt
         floatx4 sc = {0.f, 0.f, 0.f, 0.f}, da = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -321,14 +338,11 @@ __global__ __launch_bounds__(512) void attn_flash_bwd_kernel(
             da = __builtin_amdgcn_mfma_f32_16x16x4f32(hf[kk], vb[kk], da, 0, 0, 0);
         }
         // the next step's query tile leaves now: its registers are free
-        const int t_next = j + 1 < steps ? sched->row[j + 1][o] : t;
+        const int t_next = j + 1 < steps ? row_of(j + 1) : t;
         load_rows(q_blk, ld_qkv, t_next, qf);
         load_rows(dh_blk, ld_dh, t_next, hf);
 
         // P^T and dS^T: register v is query 16t + 4kq + v, the lane's key is 16kt + l16
-        const floatx4 m4 = *reinterpret_cast<const floatx4*>(st_m + 16 * t + 4 * kq);
-        const floatx4 i4 = *reinterpret_cast<const floatx4*>(st_inv + 16 * t + 4 * kq);
-        const floatx4 d4 = *reinterpret_cast<const floatx4*>(st_D + 16 * t + 4 * kq);
         floatx4 p, ds;
         const int key = 16 * kt + l16;
 #pragma unroll
@@ -339,30 +353,49 @@ __global__ __launch_bounds__(512) void attn_flash_bwd_kernel(
             p[v] = pv;
             ds[v] = (pv * (da[v] - d4[v])) * scale;
         }
-        // dS^T into the patch as [query][key] for the dQ product
+        // dS^T into the patch as [query][key], read back as the B operand of the dQ product
+        // (query l16, key 4kq + s); the wave's LDS accesses run in program order
 #pragma unroll
         for (int v = 0; v < 4; ++v) patch[(4 * kq + v) * 20 + l16] = ds[v];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const floatx4 dst = *reinterpret_cast<const floatx4*>(patch + l16 * 20 + 4 * kq);
 
-        // dV += dH P^T, dK += Q dS^T: A operand d = 16u + l16, query 4kq + s from the wave's copy
+        // dV += dH P^T, dK += Q dS^T: A operand d = 16u + l16, query 4kq + s from the wave's copy;
+        // the fragments of step s + 1 are requested before the MFMAs of step s are issued
+        float av[NDT], ak[NDT], avn[NDT], akn[NDT];
+        const float* rq = stage_q + (4 * kq) * LDP + l16;
+        const float* rh = stage_dh + (4 * kq) * LDP + l16;
+#pragma unroll
+        for (int u = 0; u < NDT; ++u) {
+            av[u] = rh[16 * u];
+            ak[u] = rq[16 * u];
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            float av[NDT], ak[NDT];
+            if (s + 1 < 4) {
 #pragma unroll
-            for (int u = 0; u < NDT; ++u) {
-                av[u] = stage_dh[(4 * kq + s) * LDP + 16 * u + l16];
-                ak[u] = stage_q[(4 * kq + s) * LDP + 16 * u + l16];
+                for (int u = 0; u < NDT; ++u) {
+                    avn[u] = rh[(s + 1) * LDP + 16 * u];
+                    akn[u] = rq[(s + 1) * LDP + 16 * u];
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < NDT; ++u) {
                 dv_acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], p[s], dv_acc[u], 0, 0, 0);
                 dk_acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(ak[u], ds[s], dk_acc[u], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < NDT; ++u) {
+                av[u] = avn[u];
+                ak[u] = akn[u];
+            }
         }
-        // dQ contribution of this cell: B operand query l16, key 4kq + s
-        const floatx4 dst = *reinterpret_cast<const floatx4*>(patch + l16 * 20 + 4 * kq);
+        // dQ contribution of this cell, added to the accumulator slice read above:
+        // register v of tile u is d = 16u + 4kq + v of query 16t + l16
         floatx4 dqc[NDT];
 #pragma unroll
         for (int u = 0; u < NDT; ++u) dqc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -370,21 +403,27 @@ __global__ __launch_bounds__(512) void attn_flash_bwd_kernel(
         for (int s = 0; s < 4; ++s)
 #pragma unroll
             for (int u = 0; u < NDT; ++u) dqc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[u][s], dst[s], dqc[u], 0, 0, 0);
-        // register v of tile u is d = 16u + 4kq + v of query 16t + l16: no other wave works on
-        // query tile t in this step
-        {
-            float* acc = dq_acc + static_cast<size_t>(16 * t + l16) * LDP + 4 * kq;
 #pragma unroll
-            for (int u = 0; u < NDT; ++u) {
-                floatx4 cur = *reinterpret_cast<floatx4*>(acc + 16 * u);
-                cur += dqc[u];
-                *reinterpret_cast<floatx4*>(acc + 16 * u) = cur;
-            }
-        }
+        for (int u = 0; u < NDT; ++u) *reinterpret_cast<floatx4*>(acc + 16 * u) = cur[u] + dqc[u];
         t = t_next;
-        __syncthreads();
-    }
-    store_key_tile();
+        __syncthreads();   // the next step's cells touch other query tiles of the accumulator
+    };
+
+    floatx4 dv_acc[NDT], dk_acc[NDT];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int u = 0; u < NDT; ++u) {
+            dv_acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+            dk_acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    clear_acc();
+    for (int j = 0; j < first; ++j) cell(j, o, kb0, vb0, ka0, dv_acc, dk_acc);
+    store_key_tile(o, dv_acc, dk_acc);
+    clear_acc();
+    for (int j = first; j < steps; ++j) cell(j, tiles - 1 - o, kb1, vb1, ka1, dv_acc, dk_acc);
+    store_key_tile(tiles - 1 - o, dv_acc, dk_acc);
+    __syncthreads();
     // dQ of the block: S columns of DH contiguous floats
     for (int i = tid; i < S * (DH / 4); i += blockDim.x) {
         const int q = i / (DH / 4), c4 = i % (DH / 4);
@@ -420,6 +459,22 @@ bool flash_shape_ok(int d_k, int heads, int S, int B) {
 
 }  // namespace
 }  // namespace jz
+
+JZ_API int jzhip_attention_flash_order(int S, int causal, int* cells, int capacity) {
+    if (S <= 0 || S % 32 != 0 || S > 16 * jz::kMaxTiles || !cells || causal < 0 || causal > 1) return -1;
+    jz::FlashSchedule s;
+    if (!jz::build_schedule(S / 16, causal != 0, &s)) return -1;
+    const int owners = S / 32;
+    if (capacity < 2 * s.steps * owners) return -1;
+    for (int j = 0; j < s.steps; ++j)
+        for (int o = 0; o < owners; ++o) {
+            // decoded the way the kernel decodes it
+            const uint64_t word = j < 16 ? s.packed[o][0] : s.packed[o][1];
+            cells[2 * (j * owners + o)] = static_cast<int>((word >> (4 * (j & 15))) & 15u);
+            cells[2 * (j * owners + o) + 1] = j < s.first[o] ? o : s.tiles - 1 - o;
+        }
+    return s.steps;
+}
 
 JZ_API int jzhip_attention_flash_supported(int d_k, int heads, int S, int B) {
     return jz::flash_shape_ok(d_k, heads, S, B) ? 1 : 0;

@@ -68,6 +68,7 @@ struct Arena {
 struct Block {
     int Wq, Wk, Wv, Wo, bo, W1, b1, W2, b2, g1, be1, g2, be2;           // tensor indices
     float *x1, *xhat1, *inv1, *QKV, *A, *H, *R, *x2, *xhat2, *inv2, *F1, *F1a, *out;  // cached activations
+    float* stats = nullptr;       // per query: score maximum and reciprocal sum (the attention that keeps no S x S matrix)
     bool A_masked_zero = false;   // A's entries above the diagonal already hold the zeros of a first forward call
 };
 
@@ -88,6 +89,10 @@ struct Model {
     float *dx[3] = {}, *dR[2] = {}, *dtmp[2] = {}, *dtmp1[2] = {}, *dQKV[2] = {}, *dF1[2] = {};
     float *dH = nullptr, *dA = nullptr;
     bool dA_masked_zero = false;   // dA's entries above the diagonal already hold the zeros of a first backward call
+    // Attention without the S x S probabilities (jzhip_attention_flash_*): two floats per query are
+    // kept instead of A, and the backward pass needs no score-gradient scratch.  Taken whenever the
+    // shape qualifies; JZLM_MATERIALISE_ATTENTION=1 keeps the buffers of the reference's layout.
+    bool flash = false;
     // Weight, bias and LayerNorm-parameter gradients are leaves of the backward
     // graph: with `overlap` they go to a second stream and fill the gaps the
     // gradient chain leaves (tile prologues and tails, bandwidth-bound kernels).
@@ -187,9 +192,14 @@ void forward(Model& M) {
         gemm(M, M.t[b.Wq].w, false, b.x1, false, b.QKV, 3 * d, N, d);
         // the weights above the diagonal are zeros written by the first call; later
         // calls leave them alone (a third of the kernel's stores)
-        M.ck(jzhip_attention_fwd_ld(b.H, d, b.A, b.QKV, b.QKV + d, b.QKV + 2 * d, 3 * d, d, c.heads, c.seq,
-                                    c.batch, b.A_masked_zero ? 2 : 1));
-        b.A_masked_zero = true;
+        if (M.flash) {
+            M.ck(jzhip_attention_flash_fwd(b.H, d, b.stats, b.QKV, b.QKV + d, b.QKV + 2 * d, 3 * d, d, c.heads, c.seq,
+                                           c.batch, 1));
+        } else {
+            M.ck(jzhip_attention_fwd_ld(b.H, d, b.A, b.QKV, b.QKV + d, b.QKV + 2 * d, 3 * d, d, c.heads, c.seq,
+                                        c.batch, b.A_masked_zero ? 2 : 1));
+            b.A_masked_zero = true;
+        }
         // R = x + (Wo*H + bo)
         gemm_tail(M, M.t[b.Wo].w, false, b.H, b.R, d, N, d, M.t[b.bo].w, 0, nullptr, x);
         M.ck(jzhip_layernorm_fwd(b.x2, b.xhat2, b.inv2, b.R, M.t[b.g2].w, M.t[b.be2].w, d, N));
@@ -316,9 +326,15 @@ void backward(Model& M, bool update) {
         lanes.back();
         gemm(M, M.t[b.Wo].w, true, dR, false, M.dH, d, N, d);
         // attention core, gradients into the stacked (3d x N) buffer
-        M.ck(jzhip_attention_bwd_ld(dQKV, dQKV + d, dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
-                                    b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch, M.dA_masked_zero ? 2 : 1));
-        M.dA_masked_zero = true;   // the score-gradient scratch is shared by all blocks and only ever used here
+        if (M.flash) {
+            M.ck(jzhip_attention_flash_bwd(dQKV, dQKV + d, dQKV + 2 * d, 3 * d, M.dH, d, b.QKV, b.QKV + d, b.QKV + 2 * d,
+                                           3 * d, b.H, d, b.stats, d, c.heads, c.seq, c.batch, 1));
+        } else {
+            M.ck(jzhip_attention_bwd_ld(dQKV, dQKV + d, dQKV + 2 * d, 3 * d, M.dA, M.dH, d, b.QKV, b.QKV + d,
+                                        b.QKV + 2 * d, 3 * d, b.A, d, c.heads, c.seq, c.batch,
+                                        M.dA_masked_zero ? 2 : 1));
+            M.dA_masked_zero = true;   // the score-gradient scratch is shared by all blocks and only ever used here
+        }
         lanes.fork();
         gemm(M, dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
         lanes.back();
@@ -365,6 +381,12 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
     const int N = M->N = c.seq * c.batch;
     const size_t dN = static_cast<size_t>(d) * N, fN = static_cast<size_t>(ff) * N;
     const size_t aN = static_cast<size_t>(S) * S * c.batch * c.heads;
+    {
+        const char* keep = std::getenv("JZLM_MATERIALISE_ATTENTION");
+        // the stacked (3d x N) projection and d-row outputs are 16-byte aligned when d % 4 == 0
+        M->flash = !(keep && std::atoi(keep) != 0) && d % 4 == 0 &&
+                   jzhip_attention_flash_supported(d, c.heads, S, c.batch) == 1;
+    }
 
     M->E = M->add("embed", d, V, kDecay);
     M->P = M->add("pos", d, S, kDecay);
@@ -391,7 +413,9 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
         M->ck(jzhip_fill(M->t[b.g1].w, d, 1.0f));
         M->ck(jzhip_fill(M->t[b.g2].w, d, 1.0f));
         b.x1 = M->alloc(dN); b.xhat1 = M->alloc(dN); b.inv1 = M->alloc(N);
-        b.QKV = M->alloc(3 * dN); b.A = M->alloc(aN); b.H = M->alloc(dN);
+        b.QKV = M->alloc(3 * dN); b.H = M->alloc(dN);
+        if (M->flash) b.stats = M->alloc(2 * static_cast<size_t>(S) * c.batch * c.heads);
+        else b.A = M->alloc(aN);
         b.R = M->alloc(dN); b.x2 = M->alloc(dN); b.xhat2 = M->alloc(dN); b.inv2 = M->alloc(N);
         b.F1 = M->alloc(fN); b.F1a = M->alloc(fN); b.out = M->alloc(dN);
     }
@@ -407,7 +431,8 @@ JZLM_API void* jzlm_create(const jzlm_config* cfg) {
         M->dR[k] = M->alloc(dN); M->dtmp[k] = M->alloc(dN); M->dtmp1[k] = M->alloc(dN);
         M->dQKV[k] = M->alloc(3 * dN); M->dF1[k] = M->alloc(fN);
     }
-    M->dH = M->alloc(dN); M->dA = M->alloc(aN);
+    M->dH = M->alloc(dN);
+    if (!M->flash) M->dA = M->alloc(aN);
     if (M->rc != 0) {
         std::fprintf(stderr, "jzlm_create: device allocation failed (%s)\n", jzhip_error_string(M->rc));
         return M;
@@ -443,6 +468,8 @@ JZLM_API void jzlm_destroy(void* h) {
 // 1: weight-gradient work of the backward pass on a second stream (default);
 // 0: everything on the library's current stream in program order.
 JZLM_API void jzlm_set_overlap(void* h, int on) { static_cast<Model*>(h)->overlap = on != 0; }
+// 1 when the model runs the attention that keeps no S x S matrix, 0 when it keeps the probabilities
+JZLM_API int jzlm_flash_attention(void* h) { return static_cast<Model*>(h)->flash ? 1 : 0; }
 
 JZLM_API int jzlm_status(void* h) { return static_cast<Model*>(h)->rc; }
 JZLM_API int jzlm_num_tensors(void* h) { return static_cast<int>(static_cast<Model*>(h)->t.size()); }

@@ -58,6 +58,8 @@ def load():
         lib.jzlm_set_iteration.argtypes = [C.c_void_p, C.c_int]
         lib.jzlm_set_overlap.argtypes = [C.c_void_p, C.c_int]
         lib.jzlm_set_overlap.restype = None
+        lib.jzlm_flash_attention.restype = C.c_int
+        lib.jzlm_flash_attention.argtypes = [C.c_void_p]
         _lib = lib
     return _lib
 
@@ -84,6 +86,12 @@ class CharLM:
         """Weight-gradient work of the backward pass on a second stream, or everything
         on one stream in program order (the default)."""
         self.lib.jzlm_set_overlap(self.h, int(bool(on)))
+
+    @property
+    def flash_attention(self):
+        """True when the attention core keeps two floats per query instead of the S x S
+        probabilities (head width 32 or 64, context a multiple of 32 up to 256)."""
+        return bool(self.lib.jzlm_flash_attention(self.h))
 
     def _check(self, what, rc):
         if rc != 0:

@@ -129,3 +129,35 @@ def test_roofline_traffic_comes_from_the_committed_counter_summary():
         assert bench.measured_traffic_bytes(name) == (f + w) * 1024.0
     with pytest.raises(KeyError):
         bench.measured_traffic_bytes("gemm_mfma_kernel<9, 9, 9, 9, false, false, false, false>")
+
+
+@pytest.mark.parametrize("S", [32, 64, 96, 128, 160, 192, 224, 256])
+@pytest.mark.parametrize("causal", [0, 1])
+def test_flash_attention_visiting_order(S, causal):
+    """Host logic of the attention backward that keeps no S x S matrix: every cell
+    (query tile, key tile) the mask leaves is visited exactly once, the waves of a step
+    are on distinct query tiles (each element of dQ therefore has one summation order),
+    a wave owns key tiles o and S/16-1-o and finishes the first before the second, and
+    under the causal mask every wave gets the same number of cells."""
+    import numpy as np
+    from juzhen_amd import capi
+    lib = ctypes.CDLL(str(capi.LIB_PATH))
+    tiles, owners = S // 16, S // 32
+    cells = (ctypes.c_int * (2 * 2 * tiles * owners))()
+    steps = lib.jzhip_attention_flash_order(S, causal, cells, len(cells))
+    assert steps == (tiles + 1 if causal else 2 * tiles)
+    c = np.array(cells[:2 * steps * owners]).reshape(steps, owners, 2)
+    seen = np.zeros((tiles, tiles), int)
+    for j in range(steps):
+        assert len(set(c[j, :, 0])) == owners                      # distinct query tiles within a step
+        for o in range(owners):
+            t, k = c[j, o]
+            assert k in (o, tiles - 1 - o) and (not causal or t >= k)
+            seen[t, k] += 1
+    want = np.tril(np.ones((tiles, tiles), int)) if causal else np.ones((tiles, tiles), int)
+    assert np.array_equal(seen, want)
+    for o in range(owners):
+        ks = list(c[:, o, 1])
+        assert ks == sorted(ks, key=lambda k: k != o)               # all of key tile o first
+    assert lib.jzhip_attention_flash_order(S, causal, cells, 3) == -1
+    assert lib.jzhip_attention_flash_order(S + 16, causal, cells, len(cells)) == -1

@@ -293,6 +293,42 @@ def test_zero_gradient_adamw_step_is_the_decay_alone(gpu):
         assert not mm.any() and not vv.any()
 
 
+def test_attention_without_the_score_matrices_trains_like_the_materialising_path(gpu, monkeypatch):
+    """The harness keeps two floats per query instead of the S x S probabilities whenever
+    the shape allows it.  Same model, same batches, both ways (JZLM_MATERIALISE_ATTENTION=1
+    selects the buffers of the reference's layout): the two runs differ only in the order of
+    a few sums, so losses agree to 1e-5 over ten steps and gradients to 1e-5."""
+    from juzhen_amd.lm import CharLM
+    V, d, heads, ff, L, S, B = 64, 128, 4, 256, 3, 96, 5          # head width 32, six key tiles
+    rng = np.random.default_rng(12)
+    tokens = make_tokens(rng, V, B, S)
+    runs = []
+    for keep in ("1", "0"):
+        monkeypatch.setenv("JZLM_MATERIALISE_ATTENTION", keep)
+        m = CharLM(V, d, heads, ff, L, S, B, gelu=True, tied=True, adamw=True, lr=1e-3)
+        assert m.flash_attention == (keep == "0")
+        m.init_random(5)
+        m.set_batch(tokens)
+        m.forward()
+        m.backward(update=False)
+        grads = {n: m.get(n, which=1) for n in ("embed", "block0.Wq", "block2.Wv", "block1.ln1_gamma")}
+        losses = []
+        for _ in range(10):
+            m.step()
+            losses.append(m.loss())
+        runs.append((losses, grads))
+        m.close()
+    (l0, g0), (l1, g1) = runs
+    assert np.allclose(l0, l1, rtol=1e-5)
+    for n in g0:
+        assert np.linalg.norm(g0[n] - g1[n]) <= 1e-5 * np.linalg.norm(g0[n]), n
+    # a shape the kernels do not cover (head width 8) keeps the probabilities
+    monkeypatch.delenv("JZLM_MATERIALISE_ATTENTION")
+    m = CharLM(17, 32, 4, 64, 1, 12, 2)
+    assert not m.flash_attention
+    m.close()
+
+
 def test_gradients_against_float64_autograd(gpu):
     """One backward pass: every parameter gradient against autograd (no optimiser)."""
     from juzhen_amd.lm import CharLM
