@@ -611,8 +611,32 @@ int jzhip_conv2d_backward_data(const float* t, const float* weights, float* dx, 
                                int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
                                int pad_w, int stride_h, int stride_w, int H_out, int W_out,
                                int N);
+/* Transposed convolution without the patch matrix:
+ *   out(co, oy, ox; n) = bias(co) + sum over (ci, ky, kx) with (oy + pad_h - ky) % stride_h == 0 and
+ *                        (ox + pad_w - kx) % stride_w == 0 of
+ *                        x(ci, (oy + pad_h - ky)/stride_h, (ox + pad_w - kx)/stride_w; n) * W((co, ky, kx), ci),
+ * taps outside the input counting as zero, [relu].  x is (C_in*H_in*W_in, N), out
+ * (C_out*H_out*W_out, N), W the (C_out*kH*kW, C_in) column-major matrix convtransLayer stores
+ * (ml/layer.hpp:1728-1766); bias may be NULL.  Replaces RocmConvTransReshape + RocmGemm +
+ * RocmConvTransScatter (+ relu) of convtransLayer::eval (ml/layer.hpp:1770-1790; oracle
+ * :2112-2160).  The stored (K, C_out) weights of a ConvLayer are the same bytes as the
+ * (C_in*kH*kW, C_out) matrix of the transposed layer that maps its output grid back onto its
+ * input grid, so with x = the upstream gradient t, C_in = the layer's C_out, C_out = the
+ * layer's C_in and (H_out, W_out) = the layer's input grid this call is the input gradient of
+ * a strided convolution, RocmGemm(W t2d) + RocmCol2im (ml/layer.hpp:1698-1709).  The output
+ * rows with equal (oy + pad_h) % stride_h share their taps: each of the stride_h*stride_w
+ * residue classes is a stride-1 convolution with the sub-kernel of those taps, run through the
+ * forward kernel in one launch and stored to every stride-th pixel; the weights are regrouped
+ * per class in the workspace first.  Results agree with the scatter / col2im order to
+ * rounding, not bit for bit.  Limits: stride_h*stride_w <= 4, kH >= stride_h, kW >= stride_w,
+ * C_in*kH*kW*C_out <= 16 Mi, H_out at most stride_h - 1 beyond (H_in-1)*stride_h - 2*pad_h + kH
+ * (likewise W_out); -1 otherwise (`jzhip_conv2d_check` with which = 3 asks without launching). */
+int jzhip_conv2d_transposed(const float* x, const float* weights, const float* bias, float* out,
+                            int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h,
+                            int pad_w, int stride_h, int stride_w, int H_out, int W_out, int N,
+                            int relu);
 /* No reference counterpart.  0 when the entry point above named by `which` (0 forward,
- * 1 backward_weights, 2 backward_data) accepts this geometry, -1 when it would refuse it:
+ * 1 backward_weights, 2 backward_data, 3 transposed) accepts this geometry, -1 when it would refuse it:
  * a dimension that is not positive, an index product beyond the kernels' 32-bit
  * arithmetic (C*H*W of an image >= 2^30, K = C_in*kH*kW >= 2^24), a patch grid larger
  * than (H_in + 2*pad - kH)/stride + 1, and for backward_data a stride other than 1,

@@ -147,6 +147,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_conv2d_backward_weights": (I, [P, P, P] + [I] * 13),
     "jzhip_conv2d_backward_data": (I, [P, P, P] + [I] * 13),
     "jzhip_conv2d_check": (I, [I] * 14),
+    "jzhip_conv2d_transposed": (I, [P, P, P, P] + [I] * 14),
 }
 
 

@@ -9,7 +9,8 @@
 // What changes: the reference always writes the patch matrix col(K, P*N) with
 // RocmIm2col, multiplies it and reshapes the result.  Here each of the three
 // products takes the route that is faster for the layer's shape:
-//   * implicit GEMM (jzhip_conv2d_forward / _backward_weights / _backward_data):
+//   * implicit GEMM (jzhip_conv2d_forward / _backward_weights / _backward_data, and
+//     jzhip_conv2d_transposed for the input gradients of a strided layer):
 //     the patch matrix is formed inside the product and never stored; bias,
 //     ReLU and the (C_out*P, N) layout are part of the forward store;
 //   * the patch-matrix route of the reference (im2col, product, reshape or
@@ -34,7 +35,7 @@ class ConvLayer : public Layer<ROCMfloat> {
     int batchN;
     bool use_relu = true;
     // route per product, fixed by the shape (thresholds measured on MI355X)
-    bool fwd_implicit, dw_implicit, dx_implicit;
+    bool fwd_implicit, dw_implicit, dx_implicit, dx_transposed;
 
     static float* ptr(const Matrix<D>& m) { return JzRocmFused::ptr(m); }
     static void must(int rc, const char* what) { rocm_detail::must(rc, what); }
@@ -104,6 +105,11 @@ class ConvLayer : public Layer<ROCMfloat> {
         fwd_implicit = fwd_implicit && accepted(0);
         dw_implicit = dw_implicit && accepted(1);
         dx_implicit = dx_implicit && accepted(2);
+        // input gradients of a strided layer: the transposed convolution of the upstream gradient
+        // with the stored weights; pays when its output channels (C_in) fill a 64-wide tile
+        dx_transposed = stride > 1 && C_in >= 64 && (long long)H_in * W_in * N >= 16384 &&
+                        jzhip_conv2d_check(3, C_out, H_out, W_out, C_in, kH, kW, pad, pad, stride, stride, H_in, W_in,
+                                           N) == 0;
     }
 
     void eval(const Matrix<D>& input) override { conv_into(this->val, input, ptr(this->bias), use_relu); }
@@ -127,7 +133,7 @@ class ConvLayer : public Layer<ROCMfloat> {
         // hadmd(d_relu(val), upstream): val > 0 exactly where the pre-activation was
         if (use_relu) must(jzhip_drelu_mul(ptr(t), ptr(this->val), ptr(t), out_count), "drelu_mul");
 
-        const bool need_t2d = !dw_implicit || !dx_implicit;
+        const bool need_t2d = !dw_implicit || !(dx_implicit || dx_transposed);
         Matrix<D> t2d("conv_t2d", need_t2d ? C_out : 1, need_t2d ? (size_t)P * batchN : 1);
         if (need_t2d) must(jzhip_conv_backward_reshape(ptr(t), ptr(t2d), C_out, P, batchN), "conv reshape");
 
@@ -148,6 +154,10 @@ class ConvLayer : public Layer<ROCMfloat> {
             must(jzhip_conv2d_backward_data(ptr(t), ptr(this->weights), ptr(dx), C_in, H_in, W_in, C_out, kH, kW, pad_h,
                                             pad_w, stride_h, stride_w, H_out, W_out, batchN),
                  "conv2d_backward_data");
+        } else if (dx_transposed) {
+            must(jzhip_conv2d_transposed(ptr(t), ptr(this->weights), nullptr, ptr(dx), C_out, H_out, W_out, C_in, kH, kW,
+                                         pad_h, pad_w, stride_h, stride_w, H_in, W_in, batchN, 0),
+                 "conv2d_transposed");
         } else {
             Matrix<D> dx_col("conv_dx_col", K, (size_t)P * batchN);
             must(jzhip_gemm(ptr(this->weights), ptr(t2d), ptr(dx_col), K, P * batchN, C_out, 0, 0, K, C_out, K, 1.0f, 0.0f),
@@ -179,8 +189,10 @@ class ConvLayer : public Layer<ROCMfloat> {
 // Transposed convolution for the ROCm backend: drop-in for convtransLayer of the
 // `#if defined(ROCM_HIP)` block of ml/layer.hpp (:1728-1870); same constructor, members,
 // layouts (weights the (C_out*kH*kW, C_in) column-major matrix stored as a column) and
-// order of operations.  eval() and jvp() keep the reference's route (pack, product,
-// scatter).  backward() differs: the reference gathers the upstream gradient into
+// order of operations.  eval() and jvp() run jzhip_conv2d_transposed (one stride-1
+// convolution per residue class of the output pixels, bias and ReLU in its store) where it
+// accepts the shape and the reference's route (pack, product, scatter) elsewhere.
+// backward() differs too: the reference gathers the upstream gradient into
 // tp(C_out*kH*kW, P_in*N), which is the patch matrix of a convolution over t seen as a
 // (C_out, H_out, W_out) image on the H_in x W_in patch grid, so
 //   dx = W^T tp       is jzhip_conv2d_forward of t with the stored weights, landing in
@@ -200,22 +212,33 @@ class convtransLayer : public Layer<ROCMfloat> {
     // backward() as two implicit products; false for shapes those entry points refuse,
     // which keep the gather + product route
     bool bwd_implicit = true;
+    // eval() and jvp() without the patch matrix
+    bool fwd_implicit = false;
 
     static float* ptr(const Matrix<D>& m) { return JzRocmFused::ptr(m); }
     static void must(int rc, const char* what) { rocm_detail::must(rc, what); }
 
-    // out(C_out*H_out*W_out, N) = scatter(W x2d) + bias
-    void deconv_into(Matrix<D>& out, const Matrix<D>& x, const Matrix<D>& b) const {
+    // out(C_out*H_out*W_out, N) = scatter(W x2d) + bias (bias_ptr may be null), then relu when asked
+    void deconv_into(Matrix<D>& out, const Matrix<D>& x, const float* bias_ptr, bool relu) const {
         const int P_in = H_in * W_in, rows = C_out * kH * kW;
+        if (fwd_implicit) {
+            must(jzhip_conv2d_transposed(ptr(x), ptr(this->weights), bias_ptr, ptr(out), C_in, H_in, W_in, C_out, kH, kW,
+                                         pad_h, pad_w, stride_h, stride_w, H_out, W_out, batchN, relu ? 1 : 0),
+                 "conv2d_transposed");
+            return;
+        }
+        Matrix<D> zero = bias_ptr ? Matrix<D>("deconv_nobias", 1, 1) : Matrix<D>::zeros(C_out, 1);
+        const float* b = bias_ptr ? bias_ptr : ptr(zero);
         Matrix<D> x2d("deconv_x2d", C_in, (size_t)P_in * batchN);
         must(jzhip_convtrans_reshape(ptr(x), ptr(x2d), C_in, P_in, batchN, 0), "convtrans reshape");
         Matrix<D> patches("deconv_patches", rows, (size_t)P_in * batchN);
         must(jzhip_gemm(ptr(this->weights), ptr(x2d), ptr(patches), rows, P_in * batchN, C_in, 0, 0, rows, C_in, rows,
                         1.0f, 0.0f),
              "gemm");
-        must(jzhip_convtrans_scatter(ptr(patches), ptr(out), ptr(b), C_out, H_out, W_out, H_in, W_in, kH, kW, pad_h, pad_w,
+        must(jzhip_convtrans_scatter(ptr(patches), ptr(out), b, C_out, H_out, W_out, H_in, W_in, kH, kW, pad_h, pad_w,
                                      stride_h, stride_w, batchN),
              "convtrans scatter");
+        if (relu) must(jzhip_relu(ptr(out), ptr(out), (size_t)C_out * H_out * W_out * batchN), "relu");
     }
 
    public:
@@ -240,18 +263,19 @@ class convtransLayer : public Layer<ROCMfloat> {
                                           N) == 0 &&
                        jzhip_conv2d_check(1, C_out, H_out, W_out, C_in, kH, kW, pad, pad, stride, stride, H_in, W_in,
                                           N) == 0;
+        // forward as stride-1 convolutions per residue class: needs channels for a 64-wide tile
+        // and enough output pixels to fill the chip
+        fwd_implicit = C_out >= 32 && (long long)H_out * W_out * N >= 16384 &&
+                       jzhip_conv2d_check(3, C_in, H_in, W_in, C_out, kH, kW, pad, pad, stride, stride, H_out, W_out,
+                                          N) == 0;
     }
 
-    void eval(const Matrix<D>& input) override {
-        deconv_into(this->val, input, this->bias);
-        if (use_relu)
-            must(jzhip_relu(ptr(this->val), ptr(this->val), (size_t)C_out * H_out * W_out * batchN), "relu");
-    }
+    void eval(const Matrix<D>& input) override { deconv_into(this->val, input, ptr(this->bias), use_relu); }
 
     Matrix<D> jvp(const Matrix<D>&, const Matrix<D>& tangent) override {
         const size_t count = (size_t)C_out * H_out * W_out * batchN;
         Matrix<D> out("convtrans_jvp", (size_t)C_out * H_out * W_out, batchN);
-        deconv_into(out, tangent, Matrix<D>::zeros(C_out, 1));
+        deconv_into(out, tangent, nullptr, false);
         if (use_relu) must(jzhip_drelu_mul(ptr(out), ptr(this->val), ptr(out), count), "drelu_mul");
         return out;
     }

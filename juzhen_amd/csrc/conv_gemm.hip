@@ -17,6 +17,9 @@
 #include "common.hpp"
 #include "gemm_tile.hpp"
 
+#include <type_traits>
+#include <utility>
+
 namespace jz {
 void launch_splitk_reduce(float* C, const float* part, int M, int N, size_t ldc, int splits, float alpha,
                           float beta);
@@ -31,6 +34,17 @@ struct ConvGeom {
     int K, P, HW, CHW, khw;
     long long J;          // P * N
     FastDiv dP, dWo, dkhw, dkW;
+    // Where the forward kernel stores patch-grid position (oh, ow): pixel
+    // (oh*out_sh + out_oh0, ow*out_sw + out_ow0) of an out_W-wide image of out_P pixels.
+    // A convolution writes its own grid (1, 1, 0, 0, Wo, P); one residue class of a
+    // transposed convolution writes every out_sh-th row and out_sw-th column.
+    int out_sh, out_sw, out_oh0, out_ow0, out_W, out_P;
+    long long w_off;      // this geometry's weights start w_off floats into the weight buffer
+};
+// The residue classes of a transposed convolution as one launch: blockIdx.y picks the class.
+constexpr int kMaxClasses = 4;
+struct ConvClasses {
+    ConvGeom g[kMaxClasses];
 };
 
 ConvGeom make_geom(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int sh, int sw, int Ho, int Wo, int N,
@@ -48,6 +62,8 @@ ConvGeom make_geom(int C, int H, int W, int kH, int kW, int pad_h, int pad_w, in
     g.dWo = make_fastdiv(Wo);
     g.dkhw = make_fastdiv(g.khw);
     g.dkW = make_fastdiv(kW);
+    g.out_sh = 1; g.out_sw = 1; g.out_oh0 = 0; g.out_ow0 = 0; g.out_W = Wo; g.out_P = g.P;
+    g.w_off = 0;
     return g;
 }
 
@@ -145,12 +161,19 @@ constexpr int kWGM = 2, kWGN = 2, kTM = 2;   // 128 rows per workgroup tile
 // each of a thread's pixels carries a 32-bit mask of the taps that fall inside the image,
 // so an element costs a table read, an AND and an address add instead of two divisions
 // and four comparisons.
-template <int TM, int TN, bool FASTB, bool TAB>
+template <int TM, int TN, bool FASTB, bool TAB, bool MULTI = false>
 __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __restrict__ in, const float* __restrict__ Wt,
                                                              const float* __restrict__ bias, float* __restrict__ out,
-                                                             ConvGeom g, int relu, int tiles_n, unsigned in_bytes) {
+                                                             std::conditional_t<MULTI, ConvClasses, ConvGeom> geo,
+                                                             int relu, int tiles_n, unsigned in_bytes) {
     constexpr int BM = kWGM * TM * 32;
     constexpr int BN = kWGN * TN * 32;
+    // MULTI: blockIdx.y selects one of up to four geometries (their weights lie behind each other)
+    const ConvGeom& g = [&]() -> const ConvGeom& {
+        if constexpr (MULTI) return geo.g[blockIdx.y];
+        else return geo;
+    }();
+    Wt += g.w_off;
     using LA = TileLoader<BM, false, TM>;
     using LB = TileLoader<BN, false, TN>;
     constexpr int LDA_S = LA::LD, LDB_S = LB::LD;
@@ -169,6 +192,9 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
     const int tile_m = pid / tiles_n, tile_n = pid % tiles_n;
     const long long m0 = static_cast<long long>(tile_m) * BM;
     const int n0 = tile_n * BN;
+    if constexpr (MULTI) {
+        if (m0 >= g.J) return;   // the grid is sized for the largest class
+    }
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -345,7 +371,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
     }
 
     // store: register v of lane (h, l32) is (row l32, column 8*(v/4) + 4*h + v%4) of a 32x32 tile
-    const long long CoP = static_cast<long long>(g.Cout) * g.P;
+    const long long CoP = static_cast<long long>(g.Cout) * g.out_P;
     // the bias values of the wave's output channels, requested together (one load and one
     // wait per stored element made the store loop a chain of round trips)
     float bv[TN][16];
@@ -361,7 +387,12 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
         const long long j = m0 + (wm * TM + i) * 32 + l32;
         if (j >= g.J) continue;
         const int n = static_cast<int>(fdiv(static_cast<uint32_t>(j), g.dP));
-        const int p = static_cast<int>(j - static_cast<long long>(n) * g.P);
+        int p = static_cast<int>(j - static_cast<long long>(n) * g.P);
+        if constexpr (MULTI) {
+            const int oh = static_cast<int>(fdiv(static_cast<uint32_t>(p), g.dWo));
+            const int ow = p - oh * g.Wo;
+            p = (oh * g.out_sh + g.out_oh0) * g.out_W + ow * g.out_sw + g.out_ow0;
+        }
         float* dst = out + static_cast<long long>(n) * CoP + p;
 #pragma unroll
         for (int jn = 0; jn < TN; ++jn) {
@@ -373,7 +404,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_kernel(const float* __rest
                     float r = acc[i][jn][v];
                     if (bias) r += bv[jn][v];
                     if (relu) r = r > 0.0f ? r : 0.0f;
-                    dst[static_cast<long long>(co) * g.P] = r;
+                    dst[static_cast<long long>(co) * g.out_P] = r;
                 }
             }
         }
@@ -836,10 +867,170 @@ int launch_fwd(const float* in, const float* Wt, const float* bias, float* out, 
     return launch_rc();
 }
 
+// ── transposed convolution as stride-1 convolutions, one per residue class ───
+// out(co, oy, ox) = bias(co) + sum over (ci, ky, kx) with (oy + pad - ky) divisible by the
+// stride of x(ci, (oy + pad - ky)/s, (ox + pad - kx)/s) * W((co, ky, kx), ci).
+// Output rows with the same residue (oy + pad) mod s use the same taps ky = r, r + s, ...
+// and consecutive input rows: for those rows the sum is a stride-1 convolution of x with
+// the sub-kernel made of these taps (in reversed order), on a patch grid that maps to every
+// s-th output row.  The s_h * s_w classes partition both the output pixels and the taps,
+// so together they do exactly the multiply-adds of the scatter formulation
+// (ml/layer.hpp:1770-1790, 2112-2160) and write every output pixel once.
+struct ClassAxis {
+    int o0;      // first output index of the class
+    int taps;    // sub-kernel extent
+    int r;       // first tap: k = r + s*m
+    int pad;     // padding of the stride-1 sub-convolution (may be negative)
+    int count;   // output indices in the class
+};
+ClassAxis class_axis(int o0, int k, int s, int pad, int out) {
+    ClassAxis a;
+    a.o0 = o0;
+    a.r = (o0 + pad) % s;
+    a.taps = a.r < k ? (k - a.r + s - 1) / s : 0;
+    const int q0 = (o0 + pad) / s;           // input index of tap m = 0 for the class's first output
+    a.pad = (a.taps - 1) - q0;
+    a.count = o0 < out ? (out - o0 + s - 1) / s : 0;
+    return a;
+}
+
+// Wsub of class (cy, cx): (K_sub, C_out) column-major, row (ci, ky2, kx2) holds the tap
+// ky = ry + sh*(ty - 1 - ky2), kx likewise; classes behind each other in (cy, cx) order.
+__global__ __launch_bounds__(kBlock) void convtrans_pack_kernel(float* __restrict__ packed, const float* __restrict__ W,
+                                                                int C_in, int C_out, int kH, int kW, int sh, int sw,
+                                                                int pad_h, int pad_w, long long total) {
+    const long long e = static_cast<long long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total) return;
+    // source element ((co, ky, kx), ci) of the (C_out*kH*kW, C_in) column-major matrix
+    const int rows = C_out * kH * kW;
+    const int ci = static_cast<int>(e / rows);
+    int r = static_cast<int>(e - static_cast<long long>(ci) * rows);
+    const int kx = r % kW;
+    r /= kW;
+    const int ky = r % kH;
+    const int co = r / kH;
+    // the class whose first tap has this residue, and the classes before it
+    long long off = 0;
+    int ty = 0, tx = 0;
+    for (int cy = 0; cy < sh; ++cy)
+        for (int cx = 0; cx < sw; ++cx) {
+            const int ry = (cy + pad_h) % sh, rx = (cx + pad_w) % sw;
+            const int ny = ry < kH ? (kH - ry + sh - 1) / sh : 0, nx = rx < kW ? (kW - rx + sw - 1) / sw : 0;
+            if (ry == ky % sh && rx == kx % sw) {
+                ty = ny;
+                tx = nx;
+                cy = sh;     // leave both loops
+                break;
+            }
+            off += static_cast<long long>(C_in) * ny * nx * C_out;
+        }
+    const int ky2 = ty - 1 - ky / sh, kx2 = tx - 1 - kx / sw;
+    const long long Ksub = static_cast<long long>(C_in) * ty * tx;
+    packed[off + static_cast<long long>(co) * Ksub + (static_cast<long long>(ci) * ty + ky2) * tx + kx2] = W[e];
+}
+
+bool transposed_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int sh, int sw, int H_out,
+                   int W_out, int N) {
+    if (C_in <= 0 || H_in <= 0 || W_in <= 0 || C_out <= 0 || kH <= 0 || kW <= 0 || pad_h < 0 || pad_w < 0 || sh <= 0 ||
+        sw <= 0 || H_out <= 0 || W_out <= 0 || N <= 0)
+        return false;
+    if (sh * sw > kMaxClasses) return false;
+    const long long chw = static_cast<long long>(C_in) * H_in * W_in, cop = static_cast<long long>(C_out) * H_out * W_out;
+    const long long j = static_cast<long long>(H_in + kH) * (W_in + kW) * N, k = static_cast<long long>(C_in) * kH * kW;
+    if (!(chw < (1ll << 30) && cop < (1ll << 30) && j < (1ll << 31) && k < (1ll << 24))) return false;
+    if (static_cast<size_t>(k) * C_out > kWorkspaceFloats) return false;
+    // the output may be the natural extent (H_in-1)*s - 2*pad + kH or up to s-1 rows more (the
+    // input gradient of a strided convolution whose last rows no patch reached from below)
+    const long long nat_h = static_cast<long long>(H_in - 1) * sh - 2ll * pad_h + kH;
+    const long long nat_w = static_cast<long long>(W_in - 1) * sw - 2ll * pad_w + kW;
+    if (!(H_out <= nat_h + sh - 1 && W_out <= nat_w + sw - 1)) return false;
+    return kH >= sh && kW >= sw;   // every residue class needs at least one tap
+}
+
+int launch_transposed(const float* x, const float* W, const float* bias, float* out, int C_in, int H_in, int W_in,
+                      int C_out, int kH, int kW, int pad_h, int pad_w, int sh, int sw, int H_out, int W_out, int N,
+                      int relu) {
+    float* packed = workspace();
+    if (!packed) return -2;
+    hipStream_t s = stream();
+    const long long wcount = static_cast<long long>(C_in) * kH * kW * C_out;
+    convtrans_pack_kernel<<<grid_cover(static_cast<size_t>(wcount), kBlock), kBlock, 0, s>>>(packed, W, C_in, C_out, kH, kW,
+                                                                                         sh, sw, pad_h, pad_w, wcount);
+    ConvClasses cls;
+    int ncls = 0;
+    long long off = 0, max_j = 0;
+    int max_k = 0, max_khw = 0;
+    bool k_aligned = true, k_long = true;
+    for (int cy = 0; cy < sh; ++cy)
+        for (int cx = 0; cx < sw; ++cx) {
+            const ClassAxis ay = class_axis(cy, kH, sh, pad_h, H_out), ax = class_axis(cx, kW, sw, pad_w, W_out);
+            if (ay.taps <= 0 || ax.taps <= 0) return -1;   // kernel extent below the stride: refused by the entry point
+            // a class without output pixels (an output narrower than the stride) keeps its weights' place and runs no tile
+            ConvGeom g = make_geom(C_in, H_in, W_in, ay.taps, ax.taps, ay.pad, ax.pad, 1, 1, ay.count > 0 ? ay.count : 1,
+                                   ax.count > 0 ? ax.count : 1, N, C_out);
+            g.w_off = off;
+            off += static_cast<long long>(C_in) * ay.taps * ax.taps * C_out;
+            if (ay.count <= 0 || ax.count <= 0) g.J = 0;
+            g.out_sh = sh; g.out_sw = sw; g.out_oh0 = cy; g.out_ow0 = cx; g.out_W = W_out; g.out_P = H_out * W_out;
+            cls.g[ncls++] = g;
+            if (g.J > max_j) max_j = g.J;
+            if (g.K > max_k) max_k = g.K;
+            if (g.khw > max_khw) max_khw = g.khw;
+            k_aligned = k_aligned && g.K % BK == 0 && g.w_off % 4 == 0;
+            k_long = k_long && g.K > 2 * BK;
+        }
+    // classes with more taps first: the workgroups of the longest K walks start earliest
+    for (int a = 1; a < ncls; ++a)
+        for (int b = a; b > 0 && cls.g[b].K > cls.g[b - 1].K; --b) std::swap(cls.g[b], cls.g[b - 1]);
+    for (int c = ncls; c < kMaxClasses; ++c) cls.g[c] = cls.g[0];
+    // tile choice as in launch_fwd, over all classes together
+    const long long want = 2ll * num_cus();
+    auto tiles = [&](int bm, int bn) { return ((max_j + bm - 1) / bm) * ((C_out + bn - 1) / bn) * ncls; };
+    int TM = 2, TN = C_out > 64 ? 2 : 1;
+    if (tiles(64 * TM, 64 * TN) < want) TM = 1;
+    if (tiles(64 * TM, 64 * TN) < want) TN = 1;
+    const int BM = 64 * TM, BN = 64 * TN;
+    const int tiles_n = (C_out + BN - 1) / BN;
+    const long long per_class = ((max_j + BM - 1) / BM) * tiles_n;
+    if (per_class > 0x7fffffffll) return -1;
+    const bool fastb = k_aligned && C_out % BN == 0 && aligned16(packed);
+    const size_t tab_bytes = static_cast<size_t>((max_k + BK - 1) / BK * BK) * sizeof(int2);
+    const long long in_bytes = static_cast<long long>(N) * C_in * H_in * W_in * static_cast<long long>(sizeof(float));
+    const bool tab = max_khw <= 32 && tab_bytes <= 24 * 1024 && k_long && in_bytes <= kBufferMaxBytes;
+    const unsigned in_b = tab ? static_cast<unsigned>(in_bytes) : 0u;
+    const dim3 grid(static_cast<unsigned>(per_class), ncls);
+#define JZ_CONVT_T(TMV, TNV, FB)                                                                                   \
+    do {                                                                                                           \
+        if (tab) conv_fwd_kernel<TMV, TNV, FB, true, true><<<grid, kBlock, tab_bytes, s>>>(x, packed, bias, out, cls, relu, tiles_n, in_b); \
+        else conv_fwd_kernel<TMV, TNV, FB, false, true><<<grid, kBlock, 0, s>>>(x, packed, bias, out, cls, relu, tiles_n, in_b);  \
+    } while (0)
+#define JZ_CONVT(TMV, TNV)                   \
+    do {                                     \
+        if (fastb) JZ_CONVT_T(TMV, TNV, true); \
+        else JZ_CONVT_T(TMV, TNV, false);    \
+    } while (0)
+    if (TM == 2 && TN == 2) JZ_CONVT(2, 2);
+    else if (TM == 2) JZ_CONVT(2, 1);
+    else if (TN == 2) JZ_CONVT(1, 2);
+    else JZ_CONVT(1, 1);
+#undef JZ_CONVT_T
+#undef JZ_CONVT
+    return launch_rc();
+}
+
 }  // namespace
 }  // namespace jz
 
 using namespace jz;
+
+JZ_API int jzhip_conv2d_transposed(const float* x, const float* weights, const float* bias, float* out, int C_in,
+                                   int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int stride_h,
+                                   int stride_w, int H_out, int W_out, int N, int relu) {
+    if (!x || !weights || !out) return -1;
+    if (!transposed_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    return launch_transposed(x, weights, bias, out, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w,
+                             H_out, W_out, N, relu ? 1 : 0);
+}
 
 JZ_API int jzhip_conv2d_forward(const float* input, const float* weights, const float* bias, float* out, int C_in,
                                 int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w, int stride_h,
@@ -936,6 +1127,8 @@ JZ_API int jzhip_conv2d_backward_data(const float* t, const float* weights, floa
 
 JZ_API int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out, int kH, int kW, int pad_h, int pad_w,
                               int stride_h, int stride_w, int H_out, int W_out, int N) {
+    if (which == 3)
+        return transposed_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N) ? 0 : -1;
     if (which < 0 || which > 2) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
     if (which == 2 && !data_grad_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out))

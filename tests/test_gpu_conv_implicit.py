@@ -1,5 +1,5 @@
 """Convolution products without the patch matrix (jzhip_conv2d_forward,
-_backward_weights, _backward_data) through the C ABI.
+_backward_weights, _backward_data, _transposed) through the C ABI.
 
 Small cases are compared with the CPU oracle's restatement of the layer's own
 chain (make_im2col + gemm + reshape/bias, ml/layer.hpp:1897-1999 and the ROCm
@@ -206,4 +206,166 @@ def test_rejects_bad_arguments(gpu):
     assert lib.jzhip_conv2d_check(2, 1, 4, 4, 1, 3, 3, 1, 1, 2, 2, 2, 2, 1) == -1      # stride 2
     assert lib.jzhip_conv2d_check(2, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1   # 18.9 Mi weights
     assert lib.jzhip_conv2d_check(1, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == 0
-    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    assert lib.jzhip_conv2d_check(4, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    # transposed: 4x4 -> (4-1)*2 - 2 + 4 = 8; one row more is the input grid of a strided layer, two are not
+    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 8, 8, 1) == 0
+    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 9, 9, 1) == 0
+    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 10, 8, 1) == -1
+    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 1, 1, 0, 0, 2, 2, 7, 7, 1) == -1      # kernel extent below the stride
+    assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 3, 3, 1, 1, 3, 3, 10, 10, 1) == -1    # nine residue classes
+    assert lib.jzhip_conv2d_transposed(dptr(d), dptr(d), None, dptr(d), 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 10, 8, 1, 0) == -1
+    assert lib.jzhip_conv2d_transposed(dptr(d), None, None, dptr(d), 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 8, 8, 1, 0) == -1
+
+
+# ── transposed convolution as stride-1 convolutions per residue class ─────────
+def direct_transposed64(x, w, b, N, Ci, H, W, Co, kH, kW, pad, sh, sw, Ho, Wo):
+    """Scatter formulation in float64: x (N, Ci, H, W); w the (Co*kH*kW, Ci) column-major matrix."""
+    wk = w.astype(np.float64).reshape(Ci, Co, kH, kW)
+    big = np.zeros((N, Co, (H - 1) * sh + kH + sh, (W - 1) * sw + kW + sw))
+    for ky in range(kH):
+        for kx in range(kW):
+            big[:, :, ky:ky + sh * (H - 1) + 1:sh, kx:kx + sw * (W - 1) + 1:sw] += np.einsum(
+                "nchw,co->nohw", x, wk[:, :, ky, kx])
+    out = big[:, :, pad:pad + Ho, pad:pad + Wo].copy()
+    if b is not None:
+        out += b.astype(np.float64)[None, :, None, None]
+    return out
+
+
+TRANSPOSED = [
+    # N, Ci, H, W, Co, kH, kW, pad, stride_h, stride_w
+    (2, 3, 4, 4, 5, 4, 4, 1, 2, 2),      # the UNet's up-sampling geometry
+    (3, 5, 5, 7, 4, 3, 3, 1, 2, 2),      # odd extents, classes with 2x2, 2x1, 1x2 and 1x1 taps
+    (2, 4, 6, 6, 70, 4, 4, 1, 2, 2),     # masked channel tile
+    (1, 6, 5, 5, 130, 2, 2, 0, 2, 2),    # non-overlapping up-sampling, two channel tiles
+    (2, 7, 6, 5, 3, 5, 5, 2, 2, 2),      # 3x3 / 3x2 / 2x3 / 2x2 sub-kernels
+    (2, 5, 7, 7, 6, 3, 3, 1, 1, 1),      # stride 1: a single class, the flipped kernel
+    (3, 2, 6, 6, 4, 3, 3, 0, 1, 1),
+    (2, 40, 4, 4, 8, 4, 4, 1, 2, 2),     # K of a class = 160: the tap-table loaders
+    (2, 48, 5, 5, 64, 4, 4, 1, 2, 2),    # K = 192, full channel tile: the unchecked weight loader
+    (2, 3, 5, 6, 4, 4, 3, 1, 2, 1),      # stride on one axis only
+    (2, 3, 5, 6, 4, 3, 4, 0, 1, 2),
+    (2, 9, 3, 3, 5, 4, 4, 0, 2, 2),      # no padding: output 8x8 from 3x3
+    (1, 2, 1, 1, 3, 4, 4, 1, 2, 2),      # a single input pixel
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSED)
+@pytest.mark.parametrize("relu", [0, 1])
+def test_transposed_small(gpu, oracle_lib, case, relu):
+    """Against the oracle's chain of convtransLayer::eval (ml/layer.hpp:1770-1790): pack the input,
+    one GEMM with the stored weights, scatter + bias; and against the float64 scatter sum."""
+    N, Ci, H, W, Co, kH, kW, pad, sh, sw = case
+    Ho, Wo = (H - 1) * sh - 2 * pad + kH, (W - 1) * sw - 2 * pad + kW
+    R, Pin = Co * kH * kW, H * W
+    r = np.random.default_rng(sum(case) + 7 * relu)
+    x = r.normal(0, 1, N * Ci * H * W).astype(np.float32)
+    w = r.normal(0, 1 / np.sqrt(Ci * kH * kW / (sh * sw)), R * Ci).astype(np.float32)
+    b = r.normal(0, 0.5, Co).astype(np.float32)
+    x2d = np.empty(Ci * Pin * N, np.float32)
+    oracle_lib.jzo_convtrans_reshape(hptr(x), hptr(x2d), Ci, Pin, N, 0)
+    patches = np.zeros(R * Pin * N, np.float32)
+    oracle_lib.jzo_gemm(0, 0, R, Pin * N, Ci, 1.0, hptr(w), R, hptr(x2d), Ci, 0.0, hptr(patches), R)
+    want = np.empty(Co * Ho * Wo * N, np.float32)
+    oracle_lib.jzo_convtrans_scatter(hptr(patches), hptr(want), hptr(b), Co, Ho, Wo, H, W, kH, kW, pad, pad, sh, sw, N)
+    if relu:
+        want = np.maximum(want, 0)
+    got = to_dev(np.full(Co * Ho * Wo * N, np.nan, np.float32))
+    from juzhen_amd import capi
+    lib = capi.load()
+    assert lib.jzhip_conv2d_check(3, Ci, H, W, Co, kH, kW, pad, pad, sh, sw, Ho, Wo, N) == 0
+    gpu.conv2d_transposed(dp(x), dp(w), dp(b), dptr(got), Ci, H, W, Co, kH, kW, pad, pad, sh, sw, Ho, Wo, N, relu)
+    got = to_host(got)
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) <= TOL_GEMM
+    ref = direct_transposed64(x.reshape(N, Ci, H, W).astype(np.float64), w, b, N, Ci, H, W, Co, kH, kW, pad, sh, sw, Ho, Wo)
+    if relu:
+        ref = np.maximum(ref, 0)
+    assert rel_err(got, ref) <= TOL_GEMM
+    if not relu:   # without the bias pointer the sum alone
+        got0 = to_dev(np.full(Co * Ho * Wo * N, np.nan, np.float32))
+        gpu.conv2d_transposed(dp(x), dp(w), None, dptr(got0), Ci, H, W, Co, kH, kW, pad, pad, sh, sw, Ho, Wo, N, 0)
+        assert rel_err(to_host(got0) + np.tile(np.repeat(b, Ho * Wo), N), want) <= TOL_GEMM
+
+
+@pytest.mark.parametrize("case", [c for c in SMALL if c[8] > 1] + [
+    (2, 6, 9, 9, 5, 3, 3, 1, 2),       # (9 + 2 - 3) % 2 == 0: every input row is reached
+    (2, 6, 10, 10, 5, 3, 3, 1, 2),     # the last input row is reached by no patch from below: one row beyond the natural extent
+    (2, 4, 11, 8, 7, 3, 3, 0, 2),
+    (2, 4, 12, 12, 6, 2, 2, 0, 2),
+])
+def test_strided_input_gradients_through_the_transposed_product(gpu, oracle_lib, case):
+    """dx of a strided ConvLayer (ml/layer.hpp:1698-1709: W t2d, then col2im) is the transposed
+    convolution of the upstream gradient with the layer's stored weights read as a
+    (C_in*kH*kW, C_out) matrix."""
+    N, Ci, H, W, Co, kH, kW, pad, stride = case
+    Ho, Wo = dims(H, W, kH, kW, pad, stride)
+    K, P = Ci * kH * kW, Ho * Wo
+    r = np.random.default_rng(sum(case) + 3)
+    w = r.normal(0, 1 / np.sqrt(K), K * Co).astype(np.float32)
+    t = r.normal(0, 1, Co * P * N).astype(np.float32)
+    t2d = np.empty(Co * P * N, np.float32)
+    oracle_lib.jzo_conv_backward_reshape(hptr(t), hptr(t2d), Co, P, N)
+    dcol = np.zeros(K * P * N, np.float32)
+    oracle_lib.jzo_gemm(0, 0, K, P * N, Co, 1.0, hptr(w), K, hptr(t2d), Co, 0.0, hptr(dcol), K)
+    dx = np.empty(Ci * H * W * N, np.float32)
+    oracle_lib.jzo_col2im(hptr(dcol), hptr(dx), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    gdx = to_dev(np.full(Ci * H * W * N, np.nan, np.float32))
+    gpu.conv2d_transposed(dp(t), dp(w), None, dptr(gdx), Co, Ho, Wo, Ci, kH, kW, pad, pad, stride, stride, H, W, N, 0)
+    got = to_host(gdx)
+    assert np.isfinite(got).all()
+    assert rel_err(got, dx) <= TOL_GEMM
+
+
+TRANSPOSED_LAYERS = [
+    # the UNet configuration's up-sampling layers (batch 128): N, Ci, H, W, Co, kH, kW, pad, stride
+    (128, 256, 8, 8, 128, 4, 4, 1, 2), (128, 128, 16, 16, 64, 4, 4, 1, 2),
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSED_LAYERS)
+def test_transposed_layer_sizes_against_the_scatter_route(gpu, case):
+    import torch
+    N, Ci, H, W, Co, kH, kW, pad, s = case
+    Ho, Wo = (H - 1) * s - 2 * pad + kH, (W - 1) * s - 2 * pad + kW
+    R, Pin = Co * kH * kW, H * W
+    g = torch.Generator(device="cuda")
+    g.manual_seed(sum(case))
+    x = torch.randn(N * Ci * Pin, generator=g, device="cuda")
+    w = torch.randn(R * Ci, generator=g, device="cuda") / np.sqrt(Ci * 4)
+    b = torch.randn(Co, generator=g, device="cuda")
+    x2d = torch.empty_like(x)
+    gpu.convtrans_reshape(dptr(x), dptr(x2d), Ci, Pin, N, 0)
+    patches = torch.empty(R * Pin * N, device="cuda")
+    gpu.gemm(dptr(w), dptr(x2d), dptr(patches), R, Pin * N, Ci, 0, 0, R, Ci, R, 1.0, 0.0)
+    want = torch.empty(Co * Ho * Wo * N, device="cuda")
+    gpu.convtrans_scatter(dptr(patches), dptr(want), dptr(b), Co, Ho, Wo, H, W, kH, kW, pad, pad, s, s, N)
+    gpu.relu(dptr(want), dptr(want), want.numel())
+    got = torch.full((Co * Ho * Wo * N,), float("nan"), device="cuda")
+    gpu.conv2d_transposed(dptr(x), dptr(w), dptr(b), dptr(got), Ci, H, W, Co, kH, kW, pad, pad, s, s, Ho, Wo, N, 1)
+    gpu.synchronize()
+    assert bool(torch.isfinite(got).all())
+    assert float((got - want).norm() / want.norm()) <= 1e-5
+
+
+@pytest.mark.parametrize("case", [c for c in LAYERS if c[8] > 1])
+def test_strided_layer_input_gradients_against_the_patch_matrix_route(gpu, case):
+    import torch
+    N, Ci, H, W, Co, kH, kW, pad, stride = case
+    Ho, Wo = dims(H, W, kH, kW, pad, stride)
+    K, P = Ci * kH * kW, Ho * Wo
+    g = torch.Generator(device="cuda")
+    g.manual_seed(sum(case) + 5)
+    w = torch.randn(K * Co, generator=g, device="cuda") / np.sqrt(K)
+    t = torch.randn(Co * P * N, generator=g, device="cuda")
+    t2d = torch.empty_like(t)
+    gpu.conv_backward_reshape(dptr(t), dptr(t2d), Co, P, N)
+    dcol = torch.empty(K * P * N, device="cuda")
+    gpu.gemm(dptr(w), dptr(t2d), dptr(dcol), K, P * N, Co, 0, 0, K, Co, K, 1.0, 0.0)
+    dx = torch.empty(Ci * H * W * N, device="cuda")
+    gpu.col2im(dptr(dcol), dptr(dx), Ci, H, W, kH, kW, pad, pad, stride, stride, Ho, Wo, N)
+    gdx = torch.full((Ci * H * W * N,), float("nan"), device="cuda")
+    gpu.conv2d_transposed(dptr(t), dptr(w), None, dptr(gdx), Co, Ho, Wo, Ci, kH, kW, pad, pad, stride, stride, H, W, N, 0)
+    gpu.synchronize()
+    assert bool(torch.isfinite(gdx).all())
+    assert float((gdx - dx).norm() / dx.norm()) <= 1e-5
