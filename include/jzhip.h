@@ -641,8 +641,12 @@ int jzhip_conv2d_transposed(const float* x, const float* weights, const float* b
  * arithmetic (C*H*W of an image >= 2^30, K = C_in*kH*kW >= 2^24), a patch grid larger
  * than (H_in + 2*pad - kH)/stride + 1, and for backward_data a stride other than 1,
  * pad > k - 1, H_in != H_out + kH - 1 - 2*pad or more than 16 Mi weights (they are
- * flipped into the workspace).  Nothing is launched.  Callers that have a patch-matrix
- * route to fall back to (ConvLayer, convtransLayer) pick their route with it. */
+ * flipped into the workspace).  which = 4 asks whether backward_weights takes its kernel for
+ * 3x3, stride-1, pad-1 layers that stages image strips in LDS (rows of 8, 16, 32 or 64
+ * pixels, a whole number of 64-pixel stages per image and four or more in all, channel
+ * counts in multiples of 32 on both sides, operands 16-byte aligned and under 2 GiB each);
+ * other accepted shapes run the general kernel.  Nothing is launched.  Callers that have a
+ * patch-matrix route to fall back to (ConvLayer, convtransLayer) pick their route with it. */
 int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out, int kH, int kW,
                        int pad_h, int pad_w, int stride_h, int stride_w, int H_out,
                        int W_out, int N);

@@ -103,7 +103,9 @@ class ConvLayer : public Layer<ROCMfloat> {
                                       N) == 0;
         };
         fwd_implicit = fwd_implicit && accepted(0);
-        dw_implicit = dw_implicit && accepted(1);
+        // 3x3 stride-1 layers with channels in multiples of 32: the weight-gradient kernel that
+        // stages image strips in LDS wins at every size it takes
+        dw_implicit = (dw_implicit || accepted(4)) && accepted(1);
         dx_implicit = dx_implicit && accepted(2);
         // input gradients of a strided layer: the transposed convolution of the upstream gradient
         // with the stored weights; pays when its output channels (C_in) fill a 64-wide tile

@@ -17,12 +17,17 @@
 #include "common.hpp"
 #include "gemm_tile.hpp"
 
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
 namespace jz {
 void launch_splitk_reduce(float* C, const float* part, int M, int N, size_t ldc, int splits, float alpha,
                           float beta);
+// conv_dw_strip.hip: 3x3 stride-1 weight gradients from image strips in LDS
+bool conv_dw_strip_ok(const float* x, const float* t, int C, int H, int W, int Cout, int kH, int kW, int pad_h,
+                      int pad_w, int sh, int sw, int Ho, int Wo, int N);
+int launch_conv_dw_strip(const float* x, const float* t, float* dW, int C, int H, int W, int Cout, int N);
 namespace {
 
 struct ConvGeom {
@@ -1070,6 +1075,16 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
             return launch_rc();
         }
     }
+    {
+        // JZHIP_CONV_DW_STRIP=0 keeps the general kernel for every shape (for comparisons)
+        static const bool strip_on = [] {
+            const char* e = std::getenv("JZHIP_CONV_DW_STRIP");
+            return !(e && e[0] == '0');
+        }();
+        if (strip_on && conv_dw_strip_ok(input, t, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out,
+                                         W_out, N))
+            return launch_conv_dw_strip(input, t, dW, C_in, H_in, W_in, C_out, N);
+    }
     const bool wide = C_out > 64;
     const int BN = wide ? 128 : 64;
     const int tiles_n = (C_out + BN - 1) / BN, tiles_m = (g.K + 127) / 128;
@@ -1129,6 +1144,15 @@ JZ_API int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out
                               int stride_h, int stride_w, int H_out, int W_out, int N) {
     if (which == 3)
         return transposed_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N) ? 0 : -1;
+    if (which == 4) {
+        // backward_weights with the strip kernel (operands assumed 16-byte aligned)
+        const float* aligned = reinterpret_cast<const float*>(uintptr_t(256));
+        return dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N) &&
+                       conv_dw_strip_ok(aligned, aligned, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w,
+                                        H_out, W_out, N)
+                   ? 0
+                   : -1;
+    }
     if (which < 0 || which > 2) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
     if (which == 2 && !data_grad_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out))

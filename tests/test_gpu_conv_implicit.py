@@ -206,7 +206,13 @@ def test_rejects_bad_arguments(gpu):
     assert lib.jzhip_conv2d_check(2, 1, 4, 4, 1, 3, 3, 1, 1, 2, 2, 2, 2, 1) == -1      # stride 2
     assert lib.jzhip_conv2d_check(2, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1   # 18.9 Mi weights
     assert lib.jzhip_conv2d_check(1, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == 0
-    assert lib.jzhip_conv2d_check(4, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    assert lib.jzhip_conv2d_check(5, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    # which = 4: weight gradients from image strips
+    assert lib.jzhip_conv2d_check(4, 64, 32, 32, 64, 3, 3, 1, 1, 1, 1, 32, 32, 128) == 0
+    assert lib.jzhip_conv2d_check(4, 64, 32, 32, 48, 3, 3, 1, 1, 1, 1, 32, 32, 128) == -1   # 48 output channels
+    assert lib.jzhip_conv2d_check(4, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1, 28, 28, 128) == -1   # rows of 28 pixels
+    assert lib.jzhip_conv2d_check(4, 64, 32, 32, 64, 3, 3, 1, 1, 2, 2, 16, 16, 128) == -1   # stride 2
+    assert lib.jzhip_conv2d_check(4, 32, 8, 8, 32, 3, 3, 1, 1, 1, 1, 8, 8, 3) == -1         # three stages in all
     # transposed: 4x4 -> (4-1)*2 - 2 + 4 = 8; one row more is the input grid of a strided layer, two are not
     assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 8, 8, 1) == 0
     assert lib.jzhip_conv2d_check(3, 1, 4, 4, 1, 4, 4, 1, 1, 2, 2, 9, 9, 1) == 0
@@ -369,3 +375,47 @@ def test_strided_layer_input_gradients_against_the_patch_matrix_route(gpu, case)
     gpu.synchronize()
     assert bool(torch.isfinite(gdx).all())
     assert float((gdx - dx).norm() / dx.norm()) <= 1e-5
+
+
+# ── weight gradients from image strips (3x3, stride 1, pad 1, channels in multiples of 32) ──
+DW_STRIP = [
+    # N, Ci, H, W, Co: rows of 8, 16, 32 and 64 pixels; chunk counts that are and are not multiples of 8;
+    # a last chunk shorter than the others; several tiles on either side
+    (4, 32, 8, 8, 32), (5, 32, 16, 16, 32), (3, 64, 16, 16, 32), (2, 32, 32, 32, 64), (16, 32, 32, 32, 64),
+    (9, 64, 32, 32, 96), (2, 32, 4, 64, 32), (7, 32, 8, 8, 64), (33, 32, 8, 8, 32), (3, 32, 6, 32, 32),
+]
+
+
+@pytest.mark.parametrize("case", DW_STRIP)
+def test_weight_gradients_from_strips(gpu, oracle_lib, case):
+    """Against the oracle's col * t2d^T of ConvLayer::backward (ml/layer.hpp:1679-1695) and a float64
+    sum over shifted images; the general kernel (JZHIP_CONV_DW_STRIP unset selects the strip form
+    for these shapes) is covered by test_backward_small."""
+    N, Ci, H, W, Co = case
+    K, P = Ci * 9, H * W
+    r = np.random.default_rng(sum(case))
+    x = r.normal(0, 1, N * Ci * P).astype(np.float32)
+    t = r.normal(0, 1, Co * P * N).astype(np.float32)
+    t2d = np.empty(Co * P * N, np.float32)
+    oracle_lib.jzo_conv_backward_reshape(hptr(t), hptr(t2d), Co, P, N)
+    col = np.empty(K * P * N, np.float32)
+    oracle_lib.jzo_im2col(hptr(x), hptr(col), Ci, H, W, 3, 3, 1, 1, 1, 1, H, W, N)
+    dW = np.zeros(K * Co, np.float32)
+    oracle_lib.jzo_gemm(0, 1, K, Co, P * N, 1.0, hptr(col), K, hptr(t2d), Co, 0.0, hptr(dW), K)
+    got = to_dev(np.full(K * Co, np.nan, np.float32))
+    gpu.conv2d_backward_weights(dp(x), dp(t), dptr(got), Ci, H, W, Co, 3, 3, 1, 1, 1, 1, H, W, N)
+    got = to_host(got)
+    assert np.isfinite(got).all()
+    assert rel_err(got, dW) <= TOL_GEMM
+    xp = np.zeros((N, Ci, H + 2, W + 2))
+    xp[:, :, 1:-1, 1:-1] = x.reshape(N, Ci, H, W)
+    t4 = t.reshape(N, Co, H, W).astype(np.float64)
+    ref = np.empty((Co, Ci, 3, 3))
+    for ky in range(3):
+        for kx in range(3):
+            ref[:, :, ky, kx] = np.einsum("nchw,nohw->oc", xp[:, :, ky:ky + H, kx:kx + W], t4)
+    assert rel_err(got, ref.ravel()) <= 1e-5
+    # the same sums on a second call (fixed summation order)
+    again = to_dev(np.full(K * Co, np.nan, np.float32))
+    gpu.conv2d_backward_weights(dp(x), dp(t), dptr(again), Ci, H, W, Co, 3, 3, 1, 1, 1, 1, H, W, N)
+    assert np.array_equal(to_host(again), got)
