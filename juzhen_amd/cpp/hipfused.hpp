@@ -18,10 +18,13 @@
 //   TransformerLayer::add_bias      one broadcast kernel instead of a rank-1 GEMM
 //   TransformerLayer::eval/backward attention for all heads and sequences as
 //                                   batched GEMMs with the mask and softmax
-//                                   (and its backward) on the device
+//                                   (and its backward) on the device; causal
+//                                   blocks of a supported shape keep no S x S
+//                                   matrix at all (two floats per query)
 #ifndef JZ_HIPFUSED_HPP
 #define JZ_HIPFUSED_HPP
 
+#include <cstdlib>
 #include <initializer_list>
 #include <vector>
 #include <typeinfo>
@@ -448,6 +451,21 @@ inline Matrix<ROCMfloat> ln_backward_plus(LayerNorm<ROCMfloat>& ln, Matrix<ROCMf
 }
 }  // namespace rocm_detail
 
+namespace rocm_detail {
+// Causal blocks of a supported shape run the attention pair that keeps no S x S matrix:
+// eval() leaves two floats per query in the head of attn_scores_scratch instead of the
+// probabilities in cached_A, backward() recomputes them tile by tile, and jvp(), which
+// reads cached_A, fills it first.  (Without the mask the materialising pair is the faster
+// one on MI355X and stays.)  JZ_MATERIALISE_ATTENTION=1 keeps the probabilities for every block.
+inline bool attention_without_scores(bool causal, int d_k, int heads, int S, int B) {
+    static const bool forced_off = [] {
+        const char* e = std::getenv("JZ_MATERIALISE_ATTENTION");
+        return e && e[0] == '1';
+    }();
+    return causal && !forced_off && jzhip_attention_flash_supported(d_k, heads, S, B) == 1;
+}
+}  // namespace rocm_detail
+
 // TransformerLayer::eval (ml/layer.hpp:2946-3031) with the same statements in the same
 // order; biases, ReLU and the two residual additions ride in the stores of the products
 // they follow instead of being passes of their own over (d, N) and (d_ff, N) matrices.
@@ -479,9 +497,15 @@ inline void TransformerLayer<ROCMfloat>::eval(const Matrix<ROCMfloat>& input_in)
         cached_K = Wk * cached_x1;
         cached_V = Wv * cached_x1;
     }
-    must(jzhip_attention_fwd(p(cached_H), p(cached_A), p(cached_Q), p(cached_K), p(cached_V), d_k, num_heads,
-                             seq_len, batchN, causal ? 1 : 0),
-         "attention_fwd");
+    if (attention_without_scores(causal, d_k, num_heads, seq_len, batchN)) {
+        must(jzhip_attention_flash_fwd(p(cached_H), d_k, p(attn_scores_scratch), p(cached_Q), p(cached_K), p(cached_V), d_k,
+                                       d_k, num_heads, seq_len, batchN, 1),
+             "attention_flash_fwd");
+    } else {
+        must(jzhip_attention_fwd(p(cached_H), p(cached_A), p(cached_Q), p(cached_K), p(cached_V), d_k, num_heads,
+                                 seq_len, batchN, causal ? 1 : 0),
+             "attention_fwd");
+    }
     // R = input + (Wo H + bo)
     cached_R = fused_product(Wo, false, cached_H, &bo, 0, nullptr, &input);
     // pre-norm feed-forward: F1 = W1 x2 + b1 kept beside relu(F1)
@@ -524,10 +548,17 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
         // pass was causal: the probabilities above the diagonal are exact zeros and those key tiles
         // are skipped.
         MD dqkv = JzRocmFused::make("dqkv", 3 * (size_t)d_k, N, 0);
-        must(jzhip_attention_bwd_ld(p(dqkv), p(dqkv) + d_k, p(dqkv) + 2 * (size_t)d_k, 3 * d_k, p(attn_dS_scratch), p(dH),
-                                    d_k, p(cached_Q), p(cached_K), p(cached_V), d_k, p(cached_A), d_k, num_heads,
-                                    seq_len, batchN, causal ? 1 : 0),
-             "attention_bwd");
+        if (attention_without_scores(causal, d_k, num_heads, seq_len, batchN)) {
+            must(jzhip_attention_flash_bwd(p(dqkv), p(dqkv) + d_k, p(dqkv) + 2 * (size_t)d_k, 3 * d_k, p(dH), d_k, p(cached_Q),
+                                           p(cached_K), p(cached_V), d_k, p(cached_H), d_k, p(attn_scores_scratch), d_k,
+                                           num_heads, seq_len, batchN, 1),
+                 "attention_flash_bwd");
+        } else {
+            must(jzhip_attention_bwd_ld(p(dqkv), p(dqkv) + d_k, p(dqkv) + 2 * (size_t)d_k, 3 * d_k, p(attn_dS_scratch), p(dH),
+                                        d_k, p(cached_Q), p(cached_K), p(cached_V), d_k, p(cached_A), d_k, num_heads,
+                                        seq_len, batchN, causal ? 1 : 0),
+                 "attention_bwd");
+        }
         // dW_i = dX_i x1^T for the three projections: one batched launch, K split over the tokens
         MD dw = JzRocmFused::make("dwqkv", d_k, 3 * (size_t)d_model, 0);
         must(jzhip_gemm_strided_batched(p(dqkv), p(cached_x1), p(dw), d_k, d_model, N, 0, 1, 3 * d_k, d_model, d_k,
@@ -545,9 +576,15 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
         must(jzhip_gemm(p(wrows), p(dqkv), p(dx1), d_model, N, 3 * d_k, 1, 0, 3 * d_k, 3 * d_k, d_model, 1.0f, 0.0f), "gemm");
     } else {
         MD dQ("dQ", d_k, N), dK("dK", d_k, N), dV("dV", d_k, N);
-        must(jzhip_attention_bwd(p(dQ), p(dK), p(dV), p(attn_dS_scratch), p(dH), p(cached_Q), p(cached_K),
-                                 p(cached_V), p(cached_A), d_k, num_heads, seq_len, batchN),
-             "attention_bwd");
+        if (attention_without_scores(causal, d_k, num_heads, seq_len, batchN)) {
+            must(jzhip_attention_flash_bwd(p(dQ), p(dK), p(dV), d_k, p(dH), d_k, p(cached_Q), p(cached_K), p(cached_V), d_k,
+                                           p(cached_H), d_k, p(attn_scores_scratch), d_k, num_heads, seq_len, batchN, 1),
+                 "attention_flash_bwd");
+        } else {
+            must(jzhip_attention_bwd(p(dQ), p(dK), p(dV), p(attn_dS_scratch), p(dH), p(cached_Q), p(cached_K),
+                                     p(cached_V), p(cached_A), d_k, num_heads, seq_len, batchN),
+                 "attention_bwd");
+        }
         dWq = dQ * cached_x1.T();
         dWk = dK * cached_x1.T();
         dWv = dV * cached_x1.T();
@@ -585,6 +622,12 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::jvp(const Matrix<ROCMfloat
     const int N = seq_len * batchN;
     const float scale = 1.0f / sqrtf((float)d_h);
     const MD tangent = plain(tangent_in);
+    if (attention_without_scores(causal, d_k, num_heads, seq_len, batchN)) {
+        // eval() kept no probabilities: form them now (H comes out the same)
+        must(jzhip_attention_fwd(p(cached_H), p(cached_A), p(cached_Q), p(cached_K), p(cached_V), d_k, num_heads, seq_len,
+                                 batchN, 1),
+             "attention_fwd");
+    }
 
     MD dx1 = ln1.jvp(tangent);
     MD dQ = Wq * dx1;

@@ -192,6 +192,18 @@ def bench_reduce(r):
         r.run("reduce", "jzhip_nrm2", s, lambda: jz.nrm2(P(o), P(a), rows * cols), bytes_=4 * rows * cols)
         r.run("reduce", "jzhip_softmax_cols", s, lambda: jz.softmax_cols(P(a), P(a), rows, cols, rows), bytes_=8 * rows * cols)
         r.run("reduce", "jzhip_softmax_rows", s, lambda: jz.softmax_rows(P(a), P(a), rows, cols, rows), bytes_=8 * rows * cols)
+    # row softmax on rows of at most 2048 columns (whole rows in registers, one read)
+    for rows, cols in ((131072, 256), (16384, 512), (16384, 2048), (65536, 2048)):
+        a = dev(rows * cols)
+        r.run("reduce", "jzhip_softmax_rows (single read)", f"{rows}x{cols}",
+              lambda: jz.softmax_rows(P(a), P(a), rows, cols, rows), bytes_=8 * rows * cols)
+        del a
+    a, o = dev(10 * 16384), dev(10 * 16384, 0)
+    r.run("reduce", "jzhip_predict_one_hot", "10x16384", lambda: jz.predict_one_hot(P(o), P(a), 10, 16384, 10), bytes_=8 * 10 * 16384)
+    a, o = dev(1024 * 16384), dev(1024 * 16384, 0)
+    r.run("reduce", "jzhip_predict_one_hot", "1024x16384", lambda: jz.predict_one_hot(P(o), P(a), 1024, 16384, 1024),
+          bytes_=8 * 1024 * 16384)
+    del a, o
     # loss of C3 and C4: softmax cross-entropy over columns
     for k, nb in ((10, 128), (256, 16384)):
         z, g, loss = dev(k * nb), dev(k * nb, 0), dev(1, 0)
@@ -243,6 +255,17 @@ def bench_fused(r):
           lambda: jz.attention_fwd(P(H), P(A), P(Q), P(K), P(V), dk, heads, S, B, 1), flops=fl)
     r.run("fused", "jzhip_attention_bwd", f"S{S} d_k{dk} h{heads} B{B}",
           lambda: jz.attention_bwd(P(dQ), P(dK), P(dV), P(dA), P(H), P(Q), P(K), P(V), P(A), dk, heads, S, B), flops=2 * fl)
+    # the same core without the score matrices: forward keeps (max, 1/sum) per query, backward recomputes
+    stats = dev(2 * S * heads * B, 0)
+    dH = dev(dk * heads * N)
+    for causal in (1, 0):
+        tag = f"S{S} d_k{dk} h{heads} B{B} causal={causal}"
+        r.run("fused", "jzhip_attention_flash_fwd", tag,
+              lambda: jz.attention_flash_fwd(P(H), dk, P(stats), P(Q), P(K), P(V), dk, dk, heads, S, B, causal),
+              flops=fl)
+        r.run("fused", "jzhip_attention_flash_bwd", tag,
+              lambda: jz.attention_flash_bwd(P(dQ), P(dK), P(dV), dk, P(dH), dk, P(Q), P(K), P(V), dk, P(H), dk, P(stats),
+                                             dk, heads, S, B, causal), flops=2 * fl)
     # token embedding and one-hot construction of C4 (vocab 256, d_model 512, 16384 tokens)
     import torch
     Vc, dm = 256, 512
@@ -364,7 +387,31 @@ def bench_conv_implicit(r):
         r.run("conv", "input gradients, patch-matrix route (2 launches)", shape, dx_patch, flops=fl)
         if s == 1:
             r.run("conv", "jzhip_conv2d_backward_data", shape, lambda: jz.conv2d_backward_data(P(t), P(w), P(dx), *dims), flops=fl)
+        else:
+            r.run("conv", "jzhip_conv2d_transposed (input gradients of the strided layer)", shape,
+                  lambda: jz.conv2d_transposed(P(t), P(w), None, P(dx), Co, Ho, Ho, Ci, k, k, pad, pad, s, s, H, H, N, 0), flops=fl)
         del x, w, b, t, col, y2d, out, dW, dx
+        torch.cuda.empty_cache()
+    # the UNet's up-sampling layers: 4x4, stride 2, pad 1
+    for label, N, Ci, H, Co in (("C5 up2", 128, 256, 8, 128), ("C5 up1", 128, 128, 16, 64)):
+        k, pad, s = 4, 1, 2
+        Ho = (H - 1) * s - 2 * pad + k
+        R, Pin = Co * k * k, H * H
+        x, w, b = dev(N * Ci * Pin), dev(R * Ci), dev(Co)
+        x2d, patches, out = dev(N * Ci * Pin, 0), dev(R * Pin * N, 0), dev(Co * Ho * Ho * N, 0)
+        fl = 2.0 * N * Pin * Ci * R
+        shape = f"{label} N{N} {Ci}>{Co} {H}x{H}>{Ho}x{Ho} k4 s2"
+
+        def up_patch():
+            jz.convtrans_reshape(P(x), P(x2d), Ci, Pin, N, 0)
+            jz.gemm(P(w), P(x2d), P(patches), R, Pin * N, Ci, 0, 0, R, Ci, R, 1.0, 0.0)
+            jz.convtrans_scatter(P(patches), P(out), P(b), Co, Ho, Ho, H, H, k, k, pad, pad, s, s, N)
+            jz.relu(P(out), P(out), Co * Ho * Ho * N)
+
+        r.run("conv", "transposed forward, patch-matrix route (4 launches)", shape, up_patch, flops=fl)
+        r.run("conv", "jzhip_conv2d_transposed", shape,
+              lambda: jz.conv2d_transposed(P(x), P(w), P(b), P(out), Ci, H, H, Co, k, k, pad, pad, s, s, Ho, Ho, N, 1), flops=fl)
+        del x, w, b, x2d, patches, out
         torch.cuda.empty_cache()
 
 
