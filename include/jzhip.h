@@ -593,6 +593,9 @@ int jzhip_convtrans_reshape(const float* src, float* dst, int C, int spatial,
  *                                 RocmGemm(col t2d^T): dW in the stored (K, C_out)
  *                                 layout, t the upstream gradient after the
  *                                 activation derivative                       (:1679-1696)
+ * 3x3, stride-1, pad-1 layers whose shape qualifies (jzhip_conv2d_check with which = 4, 5,
+ * 6) run from image strips staged in LDS instead: every pixel is fetched once per stage, the
+ * taps are the same strip at another offset.
  *   jzhip_conv2d_backward_data    replaces RocmGemm(W t2d) + RocmCol2im for stride 1
  *                                 (returns -1 for other strides: those keep the
  *                                 patch-matrix route); the taps of one input
@@ -645,7 +648,12 @@ int jzhip_conv2d_transposed(const float* x, const float* weights, const float* b
  * 3x3, stride-1, pad-1 layers that stages image strips in LDS (rows of 8, 16, 32 or 64
  * pixels, a whole number of 64-pixel stages per image and four or more in all, channel
  * counts in multiples of 32 on both sides, operands 16-byte aligned and under 2 GiB each);
- * other accepted shapes run the general kernel.  Nothing is launched.  Callers that have a
+ * other accepted shapes run the general kernel.  which = 5 and 6 ask the same of forward
+ * and backward_data, whose strip kernel takes 3x3, stride-1, pad-1 layers with rows of 8, 16
+ * or 32 pixels in whole tiles of 8, 8 or 4 rows, the product's input channels in multiples
+ * of 8 and its output channels in multiples of 64 (for backward_data the product's input is
+ * t and its output dx), operands 16-byte aligned and under 2 GiB each; the weights are
+ * regrouped into the workspace by one small launch first.  Nothing is launched.  Callers that have a
  * patch-matrix route to fall back to (ConvLayer, convtransLayer) pick their route with it. */
 int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out, int kH, int kW,
                        int pad_h, int pad_w, int stride_h, int stride_w, int H_out,

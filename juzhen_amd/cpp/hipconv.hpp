@@ -102,11 +102,12 @@ class ConvLayer : public Layer<ROCMfloat> {
             return jzhip_conv2d_check(which, C_in, H_in, W_in, C_out, kH, kW, pad, pad, stride, stride, H_out, W_out,
                                       N) == 0;
         };
-        fwd_implicit = fwd_implicit && accepted(0);
+        // (the forward and input-gradient kernels that stage image strips win wherever they apply)
+        fwd_implicit = (fwd_implicit || accepted(5)) && accepted(0);
         // 3x3 stride-1 layers with channels in multiples of 32: the weight-gradient kernel that
         // stages image strips in LDS wins at every size it takes
         dw_implicit = (dw_implicit || accepted(4)) && accepted(1);
-        dx_implicit = dx_implicit && accepted(2);
+        dx_implicit = (dx_implicit || accepted(6)) && accepted(2);
         // input gradients of a strided layer: the transposed convolution of the upstream gradient
         // with the stored weights; pays when its output channels (C_in) fill a 64-wide tile
         dx_transposed = stride > 1 && C_in >= 64 && (long long)H_in * W_in * N >= 16384 &&

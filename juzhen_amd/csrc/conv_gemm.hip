@@ -28,6 +28,11 @@ void launch_splitk_reduce(float* C, const float* part, int M, int N, size_t ldc,
 bool conv_dw_strip_ok(const float* x, const float* t, int C, int H, int W, int Cout, int kH, int kW, int pad_h,
                       int pad_w, int sh, int sw, int Ho, int Wo, int N);
 int launch_conv_dw_strip(const float* x, const float* t, float* dW, int C, int H, int W, int Cout, int N);
+// conv_fwd_strip.hip: the forward product (and, with flipped weights, the input gradients) of such layers
+bool conv_fwd_strip_ok(const float* x, const float* out, int C, int H, int W, int Cout, int kH, int kW, int pad_h,
+                       int pad_w, int sh, int sw, int Ho, int Wo, int N);
+int launch_conv_fwd_strip(const float* x, const float* weights, const float* bias, float* out, int C, int H, int W,
+                          int Cout, int N, int relu, int flip);
 namespace {
 
 struct ConvGeom {
@@ -825,6 +830,15 @@ bool data_grad_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int p
     return static_cast<size_t>(C_out) * kH * kW * C_in <= kWorkspaceFloats;
 }
 
+// JZHIP_CONV_FWD_STRIP=0 keeps the general forward kernel for every shape (for comparisons)
+bool fwd_strip_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("JZHIP_CONV_FWD_STRIP");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 int launch_fwd(const float* in, const float* Wt, const float* bias, float* out, const ConvGeom& g, int relu) {
     if (g.Cout <= kThinCout && g.C >= 8) {
         const size_t lds = (static_cast<size_t>(g.K) + 3 * kWave) * sizeof(floatx4);
@@ -1042,6 +1056,9 @@ JZ_API int jzhip_conv2d_forward(const float* input, const float* weights, const 
                                 int stride_w, int H_out, int W_out, int N, int relu) {
     if (!input || !weights || !out) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    if (fwd_strip_enabled() &&
+        conv_fwd_strip_ok(input, out, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N))
+        return launch_conv_fwd_strip(input, weights, bias, out, C_in, H_in, W_in, C_out, N, relu ? 1 : 0, 0);
     const ConvGeom g = make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N, C_out);
     return launch_fwd(input, weights, bias, out, g, relu ? 1 : 0);
 }
@@ -1129,6 +1146,10 @@ JZ_API int jzhip_conv2d_backward_data(const float* t, const float* weights, floa
     if (!t || !weights || !dx) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
     if (!data_grad_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out)) return -1;
+    // the product: t (C_out channels on the H_out x W_out grid) against the mirrored taps, padding k-1-pad
+    if (fwd_strip_enabled() && conv_fwd_strip_ok(t, dx, C_out, H_out, W_out, C_in, kH, kW, kH - 1 - pad_h, kW - 1 - pad_w, 1, 1,
+                                                 H_in, W_in, N))
+        return launch_conv_fwd_strip(t, weights, nullptr, dx, C_out, H_out, W_out, C_in, N, 0, 1);
     const size_t wcount = static_cast<size_t>(C_out) * kH * kW * C_in;
     float* flipped = workspace();
     if (!flipped) return -2;
@@ -1150,6 +1171,21 @@ JZ_API int jzhip_conv2d_check(int which, int C_in, int H_in, int W_in, int C_out
         return dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N) &&
                        conv_dw_strip_ok(aligned, aligned, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w,
                                         H_out, W_out, N)
+                   ? 0
+                   : -1;
+    }
+    if (which == 5 || which == 6) {
+        // forward (5) / backward_data (6) with the kernel that stages image strips
+        const float* aligned = reinterpret_cast<const float*>(uintptr_t(256));
+        if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+        if (which == 5)
+            return conv_fwd_strip_ok(aligned, aligned, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out,
+                                     W_out, N)
+                       ? 0
+                       : -1;
+        return data_grad_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out) &&
+                       conv_fwd_strip_ok(aligned, aligned, C_out, H_out, W_out, C_in, kH, kW, kH - 1 - pad_h, kW - 1 - pad_w, 1, 1,
+                                         H_in, W_in, N)
                    ? 0
                    : -1;
     }

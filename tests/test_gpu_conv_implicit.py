@@ -138,6 +138,7 @@ LAYERS = [
     (128, 3, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 128, 3, 3, 1, 2),
     (128, 128, 16, 16, 128, 3, 3, 1, 1), (128, 128, 16, 16, 256, 3, 3, 1, 2), (128, 256, 8, 8, 256, 3, 3, 1, 1),
     (128, 256, 16, 16, 128, 3, 3, 1, 1), (128, 128, 32, 32, 64, 3, 3, 1, 1), (128, 64, 32, 32, 3, 3, 3, 1, 1),
+    (64, 32, 32, 32, 128, 3, 3, 1, 1),   # forward strips with 128-channel tiles (512 pixel tiles x 1)
     # the backward pass of the UNet's 4x4 stride-2 transposed convolutions is a convolution over the
     # upstream gradient: image = (C_out, H_out, W_out), patch grid = (H_in, W_in), "channels out" = C_in
     (128, 128, 16, 16, 256, 4, 4, 1, 2), (128, 64, 32, 32, 128, 4, 4, 1, 2),
@@ -206,7 +207,14 @@ def test_rejects_bad_arguments(gpu):
     assert lib.jzhip_conv2d_check(2, 1, 4, 4, 1, 3, 3, 1, 1, 2, 2, 2, 2, 1) == -1      # stride 2
     assert lib.jzhip_conv2d_check(2, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1   # 18.9 Mi weights
     assert lib.jzhip_conv2d_check(1, 2048, 4, 4, 1024, 3, 3, 1, 1, 1, 1, 4, 4, 1) == 0
-    assert lib.jzhip_conv2d_check(5, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    assert lib.jzhip_conv2d_check(7, 1, 4, 4, 1, 3, 3, 1, 1, 1, 1, 4, 4, 1) == -1
+    # which = 5 / 6: forward and input gradients from image strips
+    assert lib.jzhip_conv2d_check(5, 64, 32, 32, 64, 3, 3, 1, 1, 1, 1, 32, 32, 128) == 0
+    assert lib.jzhip_conv2d_check(5, 64, 32, 32, 32, 3, 3, 1, 1, 1, 1, 32, 32, 128) == -1   # 32 output channels
+    assert lib.jzhip_conv2d_check(5, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1, 32, 32, 128) == -1    # 3 input channels
+    assert lib.jzhip_conv2d_check(6, 64, 32, 32, 8, 3, 3, 1, 1, 1, 1, 32, 32, 128) == 0     # dx: 8 channels in, 64 out
+    assert lib.jzhip_conv2d_check(6, 8, 32, 32, 64, 3, 3, 1, 1, 1, 1, 32, 32, 128) == -1    # dx would have 8 output channels
+    assert lib.jzhip_conv2d_check(5, 64, 6, 32, 64, 3, 3, 1, 1, 1, 1, 6, 32, 128) == -1     # six rows: no whole tiles of four
     # which = 4: weight gradients from image strips
     assert lib.jzhip_conv2d_check(4, 64, 32, 32, 64, 3, 3, 1, 1, 1, 1, 32, 32, 128) == 0
     assert lib.jzhip_conv2d_check(4, 64, 32, 32, 48, 3, 3, 1, 1, 1, 1, 32, 32, 128) == -1   # 48 output channels
@@ -419,3 +427,66 @@ def test_weight_gradients_from_strips(gpu, oracle_lib, case):
     again = to_dev(np.full(K * Co, np.nan, np.float32))
     gpu.conv2d_backward_weights(dp(x), dp(t), dptr(again), Ci, H, W, Co, 3, 3, 1, 1, 1, 1, H, W, N)
     assert np.array_equal(to_host(again), got)
+
+
+# ── forward product and input gradients from image strips (3x3, stride 1, pad 1) ──
+FWD_STRIP = [
+    # N, Ci, H, W, Co: input channels in multiples of 8, output channels in multiples of 64, rows of 32 / 16 / 8
+    # pixels in tiles of 4 / 8 / 8 rows; one and several stages, one and several tiles per image
+    (2, 8, 4, 32, 64), (1, 16, 8, 32, 128), (3, 8, 8, 16, 64), (2, 24, 16, 16, 128), (2, 8, 8, 8, 64),
+    (5, 16, 8, 8, 128), (2, 40, 4, 32, 64), (1, 8, 16, 8, 64),
+]
+
+
+@pytest.mark.parametrize("case", FWD_STRIP)
+@pytest.mark.parametrize("relu", [0, 1])
+def test_forward_from_strips(gpu, oracle_lib, case, relu):
+    N, Ci, H, W, Co = case
+    K, P = Ci * 9, H * W
+    r = np.random.default_rng(sum(case) + relu)
+    x = r.normal(0, 1, N * Ci * P).astype(np.float32)
+    w = r.normal(0, 1 / np.sqrt(K), K * Co).astype(np.float32)
+    b = r.normal(0, 0.5, Co).astype(np.float32)
+    col = np.empty(K * P * N, np.float32)
+    oracle_lib.jzo_im2col(hptr(x), hptr(col), Ci, H, W, 3, 3, 1, 1, 1, 1, H, W, N)
+    y2d = np.zeros(Co * P * N, np.float32)
+    oracle_lib.jzo_gemm(1, 0, Co, P * N, K, 1.0, hptr(w), K, hptr(col), K, 0.0, hptr(y2d), Co)
+    want = np.empty(Co * P * N, np.float32)
+    oracle_lib.jzo_conv_forward_reshape_bias(hptr(y2d), hptr(want), hptr(b), Co, P, N)
+    if relu:
+        want = np.maximum(want, 0)
+    got = to_dev(np.full(Co * P * N, np.nan, np.float32))
+    gpu.conv2d_forward(dp(x), dp(w), dp(b), dptr(got), Ci, H, W, Co, 3, 3, 1, 1, 1, 1, H, W, N, relu)
+    got = to_host(got)
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) <= TOL_GEMM
+    ref = direct_conv64(x.reshape(N, Ci, H, W).astype(np.float64), w, b, N, Ci, H, W, Co, 3, 3, 1, 1, relu)
+    assert rel_err(got, ref) <= 1e-5
+    if not relu:   # without the bias pointer
+        got0 = to_dev(np.full(Co * P * N, np.nan, np.float32))
+        gpu.conv2d_forward(dp(x), dp(w), None, dptr(got0), Ci, H, W, Co, 3, 3, 1, 1, 1, 1, H, W, N, 0)
+        ref0 = direct_conv64(x.reshape(N, Ci, H, W).astype(np.float64), w, None, N, Ci, H, W, Co, 3, 3, 1, 1, 0)
+        assert rel_err(to_host(got0), ref0) <= 1e-5
+
+
+@pytest.mark.parametrize("case", FWD_STRIP)
+def test_input_gradients_from_strips(gpu, oracle_lib, case):
+    """The layer of each case read backwards: Co channels come in as the upstream gradient of a
+    layer with Co input channels... the roles swap, so the layer here has C_in = the case's Co and
+    C_out = the case's Ci (the product's input channels)."""
+    N, Cout_l, H, W, Cin_l = case
+    K, P = Cin_l * 9, H * W
+    r = np.random.default_rng(sum(case) + 11)
+    w = r.normal(0, 1 / np.sqrt(K), K * Cout_l).astype(np.float32)
+    t = r.normal(0, 1, Cout_l * P * N).astype(np.float32)
+    t2d = np.empty(Cout_l * P * N, np.float32)
+    oracle_lib.jzo_conv_backward_reshape(hptr(t), hptr(t2d), Cout_l, P, N)
+    dcol = np.zeros(K * P * N, np.float32)
+    oracle_lib.jzo_gemm(0, 0, K, P * N, Cout_l, 1.0, hptr(w), K, hptr(t2d), Cout_l, 0.0, hptr(dcol), K)
+    dx = np.empty(Cin_l * P * N, np.float32)
+    oracle_lib.jzo_col2im(hptr(dcol), hptr(dx), Cin_l, H, W, 3, 3, 1, 1, 1, 1, H, W, N)
+    gdx = to_dev(np.full(Cin_l * P * N, np.nan, np.float32))
+    gpu.conv2d_backward_data(dp(t), dp(w), dptr(gdx), Cin_l, H, W, Cout_l, 3, 3, 1, 1, 1, 1, H, W, N)
+    got = to_host(gdx)
+    assert np.isfinite(got).all()
+    assert rel_err(got, dx) <= TOL_GEMM
