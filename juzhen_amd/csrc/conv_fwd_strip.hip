@@ -28,7 +28,12 @@ struct FwdStrip {
     static constexpr int NB = BN / 64;               // 32-channel blocks per wave
     static constexpr int CB = 512 / BN;              // input channels per stage: 8 or 4
     static constexpr int KSTEPS = 9 * CB / 2;        // matrix-instruction steps per stage
-    static constexpr int PITCH = W + 2, ROWS = RT + 2, XCS = ROWS * PITCH;
+    // Row pitch of the strip.  A fragment reads 32 pixels at once: one row of 32, two rows of 16 or
+    // four rows of 8.  With pitch 20 rows four apart, and with pitch 12 rows two apart, start 16
+    // (8, 16, 24) banks from each other, so those are the rows a block is made of and its 32 lanes
+    // hit 32 banks; consecutive rows at pitch W + 2 would overlap by two banks and take two cycles.
+    static constexpr int PITCH = W == 16 ? 20 : W == 8 ? 12 : W + 2;
+    static constexpr int ROWS = RT + 2, XCS = ROWS * PITCH;
     static constexpr int XBUF = CB * XCS;
     static constexpr int WBUF = 9 * CB * BN;         // 4608 floats
     static constexpr int XVEC = CB * ROWS * W / 4, XPASS = (XVEC + kBlock - 1) / kBlock;
@@ -138,12 +143,24 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_strip_kernel(const float* 
             if ((b + 1) * kBlock <= S::WVEC || threadIdx.x + b * kBlock < S::WVEC)
                 *reinterpret_cast<floatx4*>(wb + 4 * b * kBlock) = rw[b];
     };
-    // fragment addresses: pixel l32 of block pb (rows of W pixels), channel parity h; output channel l32 of block nb
-    int x_lane[S::PB];
+    // fragment addresses: lane l32 of pixel block pb is pixel (p_row[pb], p_col) of the tile, channel
+    // parity h; output channel l32 of block nb
+    int p_row[S::PB], p_col, x_lane[S::PB];
 #pragma unroll
     for (int pb = 0; pb < S::PB; ++pb) {
-        const int q = wp * (S::BMP / 2) + pb * 32 + l32;
-        x_lane[pb] = (q / W) * S::PITCH + q % W + h * S::XCS;
+        if constexpr (W == 16) {
+            static_assert(W != 16 || (RT == 8 && S::PB == 2), "rows b and b + 4 form a block");
+            p_row[pb] = 2 * wp + pb + 4 * (l32 / 16);
+            p_col = l32 % 16;
+        } else if constexpr (W == 8) {
+            static_assert(W != 8 || (RT == 8 && S::PB == 1), "rows b, b + 2, b + 4, b + 6 form a block");
+            p_row[pb] = wp + 2 * (l32 / 8);
+            p_col = l32 % 8;
+        } else {
+            p_row[pb] = wp * (RT / 2) + pb;
+            p_col = l32;
+        }
+        x_lane[pb] = p_row[pb] * S::PITCH + p_col + h * S::XCS;
     }
     const int w_lane = h * BN + wc * (BN / 2) + l32;
     auto compute = [&](int buf) {
@@ -193,8 +210,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_fwd_strip_kernel(const float* 
         for (int v = 0; v < 16; ++v) bv[v] = bias ? bias[cbase + 8 * (v / 4) + v % 4] : 0.0f;
 #pragma unroll
         for (int pb = 0; pb < S::PB; ++pb) {
-            const int q = wp * (S::BMP / 2) + pb * 32 + l32;
-            float* dst = out + n * CoP + oh0 * W + q;
+            float* dst = out + n * CoP + (oh0 + p_row[pb]) * W + p_col;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 float r = acc[pb][nb][v] + bv[v];
