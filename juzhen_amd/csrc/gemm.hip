@@ -1,7 +1,7 @@
 // fp32 GEMM on CDNA4 matrix cores: C = alpha*op(A)*op(B) + beta*C, column-major,
 // all four transpose variants, arbitrary leading dimensions, plus rank-1
 // products (the layers' bias broadcasts) and a strided-batched form for
-// attention.  Matrix-vector products and products with m or n of at most 8
+// attention.  Matrix-vector products and products with m or n of at most 16
 // are bandwidth-bound and live in gemv.hip.
 //
 // Tiled kernel: a workgroup of four wavefronts owns a BM x BN tile of C and
@@ -867,7 +867,7 @@ JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int
     {
         const long long cus = num_cus();
         const long long t128 = static_cast<long long>((m + 127) / 128) * ((n + 127) / 128);
-        const bool special = k == 1 || m <= 8 || n <= 8 || (t128 * 2 <= cus && k >= 1024);
+        const bool special = k == 1 || m <= 16 || n <= 16 || (t128 * 2 <= cus && k >= 1024);
         const bool flat = ldc == m && (!aux || ld_aux == m) && (!residual || (ldr == m && residual != C));
         if (special && flat) {
             const size_t total = static_cast<size_t>(m) * n;

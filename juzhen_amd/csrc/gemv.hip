@@ -93,21 +93,48 @@ __global__ __launch_bounds__(kGemvCombineBlock) void gemv_n_combine_kernel(float
     }
 }
 
+// The same sum for a few chunks and many outputs (a 10 x 12544 gradient in two chunks): one thread per
+// output, chunks in order.
+__global__ __launch_bounds__(kBlock) void gemv_n_combine_few_kernel(float* y, const float* part, int m, int chunks,
+                                                                    int len, size_t s_in, size_t s_out, float alpha,
+                                                                    float beta) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= m) return;
+    float sum = 0.f;
+    for (int c = 0; c < chunks; ++c) sum += part[static_cast<size_t>(c) * m + i];
+    float* dst = y + static_cast<size_t>(i % len) * s_in + static_cast<size_t>(i / len) * s_out;
+    float r = alpha * sum;
+    if (beta != 0.0f) r += beta * *dst;
+    *dst = r;
+}
+
+void launch_thin_combine(float* y, const float* part, size_t outs, int chunks, int len, size_t s_in, size_t s_out,
+                         float alpha, float beta, hipStream_t s) {
+    if (chunks <= 8)
+        gemv_n_combine_few_kernel<<<static_cast<unsigned>((outs + kBlock - 1) / kBlock), kBlock, 0, s>>>(
+            y, part, static_cast<int>(outs), chunks, len, s_in, s_out, alpha, beta);
+    else
+        gemv_n_combine_kernel<<<static_cast<unsigned>((outs + kWave - 1) / kWave), kGemvCombineBlock, 0, s>>>(
+            y, part, static_cast<int>(outs), chunks, len, s_in, s_out, alpha, beta);
+}
+
 // ── thin products: one extent of C is at most kThinMax ───────────────────
 // C = op(A) op(B) with m or n <= kThinMax (a 3-channel output convolution:
-// 3 x 131072 x 576 forward, 576 x 3 x 131072 for its weight gradient) is a
-// handful of matrix-vector products over one big operand: bound by reading
+// 3 x 131072 x 576 forward, 576 x 3 x 131072 for its weight gradient; a 10-class
+// dense layer: 10 x 128 x 12544) is a handful of matrix-vector products over one big operand: bound by reading
 // that operand once, which an MFMA tile padded to 32 rows cannot approach.
 // The big operand X is L x K (element (l,k) at X[l*xs_l + k*xs_k], one of the
 // strides being 1), the thin one V is T x K (V[t*vs_t + k*vs_k]); output (l,t)
 // goes to C[l*cs_l + t*cs_t].
-constexpr int kThinMax = 8;
+constexpr int kThinMax = 16;
 // rows of X a wavefront walks together in the dot form: two with up to four thin
-// vectors (measured 55 against 58 us at 3 x 131072 x 576), four with more, where
-// each LDS read of V should serve more rows
-template <int TT> constexpr int kThinRows = TT == 1 ? 4 : (TT <= 4 ? 2 : 4);
-constexpr int thin_tt(int T) { return T == 1 ? 1 : (T <= 4 ? 4 : 8); }   // template width serving T vectors
-constexpr int kThinChunkMax = 1024;   // k per workgroup in the other form
+// vectors (measured 55 against 58 us at 3 x 131072 x 576), four with up to eight, where
+// each LDS read of V should serve more rows, two again with sixteen (32 sums per lane)
+template <int TT> constexpr int kThinRows = TT == 1 ? 4 : (TT <= 4 ? 2 : (TT <= 8 ? 4 : 2));
+constexpr int thin_tt(int T) { return T == 1 ? 1 : (T <= 4 ? 4 : (T <= 8 ? 8 : 16)); }   // template width serving T vectors
+constexpr int kThinChunkMax = 1024;   // k per workgroup in the other form (V's slice: 32 KB at eight vectors)
+constexpr int thin_chunk_max(int tt) { return tt <= 8 ? kThinChunkMax : kThinChunkMax / 2; }
+constexpr int kThinDotChunkMax = 512;   // k per workgroup in the chunked dot form: two float4 steps per lane
 
 // Sums NV (a power of two, at most 64) values per lane over the 64 lanes.  On
 // return v[0] of lane i holds the total of value i >> log2(64 / NV); the lane
@@ -138,6 +165,75 @@ __device__ __forceinline__ int wave_sum_many(float (&v)[NV], int lane) {
     return (lane & (rest - 1)) == 0 ? lane / rest : -1;
 }
 
+// Stages V's slice [k_begin, k_begin + len) into LDS as [TT][pitch], zeros for t >= T and k >= len.  When the
+// thin index is the contiguous one in memory (a 10 x K matrix stored by columns) the threads walk the
+// memory order, runs of T floats, instead of gathering one float per 4*vs_k bytes.
+template <int TT>
+__device__ __forceinline__ void stage_thin(float* __restrict__ vl, const float* __restrict__ V, size_t vs_t, size_t vs_k,
+                                           int T, int k_begin, int len, int pitch) {
+    // eight independent loads per thread before their LDS stores: a load per iteration behind a store
+    // the compiler cannot move it past makes every element a full trip to memory
+    constexpr int kBatch = 8;
+    const bool by_t = vs_t == 1 && T > 1;
+    const int n = T * len;
+    const float* block = V + static_cast<size_t>(k_begin) * vs_k;
+    if (by_t && vs_k == static_cast<size_t>(T) && n % 4 == 0 && (reinterpret_cast<uintptr_t>(block) & 15u) == 0) {
+        // the slice is one contiguous block of T*len floats: 16-byte loads, four in flight per thread
+        const float4* b4 = reinterpret_cast<const float4*>(block);
+        const int n4 = n / 4;
+        for (int i0 = threadIdx.x; i0 < n4; i0 += kBlock * 4) {
+            float4 r[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int i = i0 + b * kBlock;
+                r[b] = i < n4 ? b4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int i = i0 + b * kBlock;
+                if (i < n4) {
+                    const float e[4] = {r[b].x, r[b].y, r[b].z, r[b].w};
+                    int kk = (4 * i) / T, t = 4 * i - kk * T;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        vl[t * pitch + kk] = e[q];
+                        if (++t == T) { t = 0; ++kk; }
+                    }
+                }
+            }
+        }
+    } else
+    for (int i0 = threadIdx.x; i0 < n; i0 += kBlock * kBatch) {
+        float r[kBatch];
+        int dst[kBatch];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const int i = i0 + b * kBlock;
+            dst[b] = -1;
+            r[b] = 0.f;
+            if (i < n) {
+                int t, kk;
+                if (by_t) { kk = i / T; t = i - kk * T; }
+                else { t = i / len; kk = i - t * len; }
+                dst[b] = t * pitch + kk;
+                r[b] = V[t * vs_t + static_cast<size_t>(k_begin + kk) * vs_k];
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b)
+            if (dst[b] >= 0) vl[dst[b]] = r[b];
+    }
+    // the rest: rows past T, columns past len (disjoint from the above, no barrier between)
+    for (int i = T * pitch + threadIdx.x; i < TT * pitch; i += kBlock) vl[i] = 0.f;
+    if (len < pitch) {
+        const int tail = pitch - len;
+        for (int i = threadIdx.x; i < T * tail; i += kBlock) {
+            const int t = i / tail;
+            vl[t * pitch + len + (i - t * tail)] = 0.f;
+        }
+    }
+}
+
 // k contiguous in X: a wavefront takes kThinRows<TT> rows, its lanes stride over k
 // in float4 steps against V staged in LDS (each LDS read serves all the rows).
 template <int TT, bool NT>
@@ -146,10 +242,7 @@ __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restric
                                                           float* C, size_t cs_l, size_t cs_t, int L, int K, int T,
                                                           float alpha, float beta) {
     extern __shared__ __attribute__((aligned(16))) float vlds[];   // [TT][K]
-    for (int i = threadIdx.x; i < TT * K; i += kBlock) {
-        const int t = i / K, k = i - t * K;
-        vlds[i] = t < T ? V[t * vs_t + k * vs_k] : 0.f;
-    }
+    stage_thin<TT>(vlds, V, vs_t, vs_k, T, 0, K, K);
     __syncthreads();
     const int lane = threadIdx.x & (kWave - 1);
     const size_t wave0 = (static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x) / kWave;
@@ -199,6 +292,78 @@ __global__ __launch_bounds__(kBlock) void thin_dot_kernel(const float* __restric
     }
 }
 
+// The dot form with K cut into chunks across workgroups: for a short L (a 10 x 128 x 12544
+// product has 128 rows of X: whole-K rows would occupy eight workgroups) or a V that does not
+// fit LDS whole.  A workgroup stages its chunk's slice of V once and walks rows_per_wg rows of
+// X against it, kThinRows<TT> rows per wavefront and pass; the partial sums go to
+// part[chunk][t*L + l] for the combine kernel.
+template <int TT, bool NT>
+__global__ __launch_bounds__(kBlock) void thin_dot_partial_kernel(const float* __restrict__ X, size_t xs_l,
+                                                                  const float* __restrict__ V, size_t vs_t,
+                                                                  size_t vs_k, float* part, int L, int K, int T,
+                                                                  int chunk_len, int rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) float vlds[];   // [TT][chunk_len], chunk_len % 4 == 0
+    const int k_begin = blockIdx.y * chunk_len;
+    const int len = (K - k_begin) < chunk_len ? (K - k_begin) : chunk_len;   // a multiple of 4, as K is
+    const int lane = threadIdx.x & (kWave - 1);
+    constexpr int R = kThinRows<TT>;
+    constexpr int NW = kBlock / kWave;
+    constexpr int kIter = kThinDotChunkMax / 4 / kWave;   // float4 steps a lane takes through the longest chunk
+    const int C4 = chunk_len / 4, len4 = len / 4;
+    const size_t row0 = static_cast<size_t>(blockIdx.x) * rows_per_wg + (threadIdx.x / kWave) * R;
+    float4 x[kIter][R];
+    auto fetch = [&](size_t l0) {
+#pragma unroll
+        for (int it = 0; it < kIter; ++it) {
+            const int k4 = lane + it * kWave;
+#pragma unroll
+            for (int u = 0; u < R; ++u) {
+                const size_t l = l0 + u < static_cast<size_t>(L) ? l0 + u : L - 1;   // clamped, dropped at the store
+                x[it][u] = k4 < len4 ? load4<NT>(X + l * xs_l + k_begin + 4 * static_cast<size_t>(k4))
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    };
+    // the first rows are requested before V is staged, so that the two round trips to memory overlap
+    if (row0 < static_cast<size_t>(L)) fetch(row0);
+    stage_thin<TT>(vlds, V, vs_t, vs_k, T, k_begin, len, chunk_len);
+    __syncthreads();
+    const float4* v4 = reinterpret_cast<const float4*>(vlds);
+    for (int pass = 0; pass * NW * R < rows_per_wg; ++pass) {
+        const size_t l0 = row0 + static_cast<size_t>(pass) * NW * R;
+        if (l0 >= static_cast<size_t>(L)) break;
+        if (pass > 0) fetch(l0);
+        float acc[R][TT];
+#pragma unroll
+        for (int u = 0; u < R; ++u)
+#pragma unroll
+            for (int t = 0; t < TT; ++t) acc[u][t] = 0.f;
+#pragma unroll
+        for (int it = 0; it < kIter; ++it) {
+            const int k4 = lane + it * kWave;
+            if (k4 < len4) {
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    const float4 v = v4[t * C4 + k4];
+#pragma unroll
+                    for (int u = 0; u < R; ++u)
+                        acc[u][t] += x[it][u].x * v.x + x[it][u].y * v.y + x[it][u].z * v.z + x[it][u].w * v.w;
+                }
+            }
+        }
+        constexpr int NV = R * TT;
+        float v[NV];
+#pragma unroll
+        for (int u = 0; u < R; ++u)
+#pragma unroll
+            for (int t = 0; t < TT; ++t) v[u * TT + t] = acc[u][t];
+        const int idx = wave_sum_many<NV>(v, lane);
+        const int u = idx / TT, t = idx - u * TT;
+        if (idx >= 0 && l0 + u < static_cast<size_t>(L) && t < T)
+            part[(static_cast<size_t>(blockIdx.y) * T + t) * L + l0 + u] = v[0];
+    }
+}
+
 // l contiguous in X: lanes hold four rows each (a wavefront reads 1 KB of one
 // column), the block's waves split the k of a chunk eight at a time, and the
 // chunk's slice of V sits in LDS as [t][chunk_len], zero-filled past the end
@@ -211,29 +376,31 @@ __global__ __launch_bounds__(kBlock) void thin_axpy_partial_kernel(const float* 
     constexpr int NW = kBlock / kWave;
     constexpr int U = 8;   // columns in flight per wavefront; chunk_len % U == 0
     extern __shared__ __attribute__((aligned(16))) float vl[];   // [TT][chunk_len]
-    __shared__ float4 red[NW][kWave];
+    __shared__ float4 red[NW][TT < 4 ? TT : 4][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int l = (blockIdx.x * kWave + lane) * 4;
     const bool live = l < L;
     const int k_begin = blockIdx.y * chunk_len;
     const int len = (K - k_begin) < chunk_len ? (K - k_begin) : chunk_len;
-    for (int i = threadIdx.x; i < TT * chunk_len; i += kBlock) {
-        const int t = i / chunk_len, kk = i - t * chunk_len;
-        vl[i] = (t < T && kk < len) ? V[t * vs_t + static_cast<size_t>(k_begin + kk) * vs_k] : 0.f;
-    }
-    __syncthreads();
-    float4 acc[TT];
-#pragma unroll
-    for (int t = 0; t < TT; ++t) acc[t] = make_float4(0.f, 0.f, 0.f, 0.f);
     const float* xp = X + (live ? l : 0) + static_cast<size_t>(k_begin) * xs_k;
-    for (int kk = wave * U; kk < len; kk += NW * U) {
-        float4 x[U];
+    auto fetch = [&](float4 (&x)[U], int kk) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int c = kk + u < len ? kk + u : len - 1;   // clamped; its V entry is zero
             x[u] = load4<NT>(xp + static_cast<size_t>(c) * xs_k);
         }
+    };
+    // the first columns are requested before V is staged, so that the two round trips to memory overlap
+    float4 x[U];
+    int kk = wave * U;
+    if (kk < len) fetch(x, kk);
+    stage_thin<TT>(vl, V, vs_t, vs_k, T, k_begin, len, chunk_len);
+    __syncthreads();
+    float4 acc[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) acc[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    while (kk < len) {
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
 #pragma unroll
@@ -247,17 +414,23 @@ __global__ __launch_bounds__(kBlock) void thin_axpy_partial_kernel(const float* 
                 }
             }
         }
+        kk += NW * U;
+        if (kk < len) fetch(x, kk);
     }
+    // the four waves' sums, four vectors per round: wave w adds vector t0 + w of the four waves in wave order
+    constexpr int G = TT < 4 ? TT : 4;
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-        if (t < T) {   // T is uniform: every thread takes the same barriers
-            red[wave][lane] = acc[t];
+    for (int t0 = 0; t0 < TT; t0 += G) {
+        if (t0 < T) {   // T is uniform: every thread takes the same barriers
+#pragma unroll
+            for (int q = 0; q < G; ++q) red[wave][q][lane] = acc[t0 + q];
             __syncthreads();
-            if (wave == 0 && live) {
-                float4 sum = red[0][lane];
+            const int t = t0 + wave;
+            if (wave < G && t < T && live) {
+                float4 sum = red[0][wave][lane];
 #pragma unroll
                 for (int w = 1; w < NW; ++w) {
-                    const float4 o = red[w][lane];
+                    const float4 o = red[w][wave][lane];
                     sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
                 }
                 *reinterpret_cast<float4*>(part + (static_cast<size_t>(blockIdx.y) * T + t) * L + l) = sum;
@@ -306,11 +479,53 @@ struct ThinArgs {
     float alpha, beta;
 };
 
+// The dot form keeps all of V in LDS and gives a wavefront whole rows when there are rows enough
+// to fill the chip; otherwise K is cut into chunks.
+bool thin_dot_whole_k(const ThinArgs& a) {
+    return a.L >= 256 && static_cast<size_t>(thin_tt(a.T)) * a.K * sizeof(float) <= 64 * 1024;
+}
+int thin_dot_rows_per_wg(const ThinArgs& a, int tt) {
+    const int base = (tt == 1 ? 4 : tt <= 4 ? 2 : tt <= 8 ? 4 : 2) * (kBlock / kWave);   // one pass of the four waves
+    const long long chunks_min = (a.K + kThinDotChunkMax - 1) / kThinDotChunkMax;
+    int rows = base;
+    while (rows < 8 * base && (a.L / (2 * rows)) * chunks_min >= 4ll * num_cus()) rows *= 2;
+    return rows;
+}
+int thin_dot_chunk_len(const ThinArgs& a, int tt, int row_groups) {
+    long long chunks = (2ll * num_cus() + row_groups - 1) / row_groups;
+    if (chunks > a.K / 64) chunks = a.K / 64;
+    if (chunks < 1) chunks = 1;
+    int chunk_len = static_cast<int>(((a.K + chunks - 1) / chunks + 3) / 4 * 4);
+    (void)tt;   // V's slice of a chunk: at most 16 x 512 floats = 32 KB
+    return chunk_len > kThinDotChunkMax ? kThinDotChunkMax : chunk_len;
+}
+
 template <int TT>
 int thin_launch(const ThinArgs& a) {
     hipStream_t s = stream();
     // the big operand is read once: past the cache size with the streaming hint
     const bool nt = streams_past_cache(static_cast<size_t>(a.L) * a.K * sizeof(float));
+    if (a.xs_k == 1 && !thin_dot_whole_k(a)) {
+        // K in chunks: enough of them for two workgroups per CU, V's slice within 32 KB; with many rows a
+        // workgroup walks up to 64 of them against one staged slice
+        const int rows_per_wg = thin_dot_rows_per_wg(a, TT);
+        const int row_groups = (a.L + rows_per_wg - 1) / rows_per_wg;
+        const int chunk_len = thin_dot_chunk_len(a, TT, row_groups);
+        const int chunks = (a.K + chunk_len - 1) / chunk_len;
+        const size_t outs = static_cast<size_t>(a.T) * a.L;
+        if (outs * chunks > kWorkspaceFloats) return -1;            // thin_ok() rules this out
+        float* part = workspace();
+        if (!part) return -2;
+        const size_t lds = static_cast<size_t>(TT) * chunk_len * sizeof(float);
+        if (nt)
+            thin_dot_partial_kernel<TT, true><<<dim3(row_groups, chunks), kBlock, lds, s>>>(a.X, a.xs_l, a.V, a.vs_t, a.vs_k,
+                                                                                         part, a.L, a.K, a.T, chunk_len, rows_per_wg);
+        else
+            thin_dot_partial_kernel<TT, false><<<dim3(row_groups, chunks), kBlock, lds, s>>>(a.X, a.xs_l, a.V, a.vs_t, a.vs_k,
+                                                                                          part, a.L, a.K, a.T, chunk_len, rows_per_wg);
+        launch_thin_combine(a.C, part, outs, chunks, a.L, a.cs_l, a.cs_t, a.alpha, a.beta, s);
+        return launch_rc();
+    }
     if (a.xs_k == 1) {
         const size_t groups = (static_cast<size_t>(a.L) + kThinRows<TT> - 1) / kThinRows<TT>;
         const unsigned grid = grid_for(groups, kBlock / kWave, 8);
@@ -324,10 +539,13 @@ int thin_launch(const ThinArgs& a) {
     }
     const int row_blocks = (a.L / 4 + kWave - 1) / kWave;
     int chunks = static_cast<int>((static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks);
-    if (chunks > a.K / 64) chunks = a.K / 64;
+    // chunks of 64 k and more; of 32 where the rows alone give the chip little to do (a 256 x 16 x 4096
+    // gradient is one row block)
+    const int min_chunk = row_blocks * 8 <= num_cus() ? 32 : 64;
+    if (chunks > a.K / min_chunk) chunks = a.K / min_chunk;
     if (chunks < 1) chunks = 1;
     int chunk_len = ((a.K + chunks - 1) / chunks + 7) / 8 * 8;
-    if (chunk_len > kThinChunkMax) chunk_len = kThinChunkMax;   // V's slice of a chunk stays within 32 KB of LDS
+    if (chunk_len > thin_chunk_max(TT)) chunk_len = thin_chunk_max(TT);   // V's slice of a chunk stays within 32 KB of LDS
     chunks = (a.K + chunk_len - 1) / chunk_len;
     const size_t outs = static_cast<size_t>(a.T) * a.L;
     if (outs * chunks > kWorkspaceFloats) return -1;            // thin_ok() rules this out
@@ -341,8 +559,7 @@ int thin_launch(const ThinArgs& a) {
         thin_axpy_partial_kernel<TT, false><<<dim3(row_blocks, chunks), kBlock,
                                               static_cast<size_t>(TT) * chunk_len * sizeof(float), s>>>(
             a.X, a.xs_k, a.V, a.vs_t, a.vs_k, part, a.L, a.K, a.T, chunk_len);
-    gemv_n_combine_kernel<<<static_cast<unsigned>((outs + kWave - 1) / kWave), kGemvCombineBlock, 0, s>>>(
-        a.C, part, static_cast<int>(outs), chunks, a.L, a.cs_l, a.cs_t, a.alpha, a.beta);
+    launch_thin_combine(a.C, part, outs, chunks, a.L, a.cs_l, a.cs_t, a.alpha, a.beta, s);
     return launch_rc();
 }
 
@@ -350,22 +567,32 @@ int thin_launch(const ThinArgs& a) {
 // V small enough for LDS in the dot form, partial sums that fit the workspace.
 bool thin_ok(const ThinArgs& a) {
     if (a.T > kThinMax || !aligned16(a.X)) return false;
-    if (a.xs_k == 1)
-        return a.L >= 256 && a.K % 4 == 0 && a.xs_l % 4 == 0 && a.K >= 64 &&
-               static_cast<size_t>(thin_tt(a.T)) * a.K * sizeof(float) <= 64 * 1024;
+    if (a.xs_k == 1) {
+        if (!(a.K % 4 == 0 && a.xs_l % 4 == 0 && a.K >= 64)) return false;
+        if (thin_dot_whole_k(a)) return true;
+        // chunked: at least a wavefront's worth of rows, partial sums within the workspace
+        if (a.L < 16) return false;
+        const int tt = thin_tt(a.T);
+        const int per_wg = thin_dot_rows_per_wg(a, tt);
+        const int row_groups = (a.L + per_wg - 1) / per_wg;
+        const int chunk_len = thin_dot_chunk_len(a, tt, row_groups);
+        const size_t chunks = (static_cast<size_t>(a.K) + chunk_len - 1) / chunk_len;
+        return chunks <= 65535 && static_cast<size_t>(a.T) * a.L * chunks <= kWorkspaceFloats;
+    }
     if (a.L < 64) return false;
     // partial sums of every chunk must fit the workspace even at the longest chunk
-    const size_t min_chunks = (static_cast<size_t>(a.K) + kThinChunkMax - 1) / kThinChunkMax;
+    const size_t min_chunks = (static_cast<size_t>(a.K) + thin_chunk_max(thin_tt(a.T)) - 1) / thin_chunk_max(thin_tt(a.T));
     const size_t row_blocks = (static_cast<size_t>(a.L) / 4 + kWave - 1) / kWave;
     const size_t want = (static_cast<size_t>(num_cus()) * 4 + row_blocks - 1) / row_blocks;
     const size_t chunks = want > min_chunks ? want : min_chunks;
-    return a.xs_l == 1 && a.L % 4 == 0 && a.xs_k % 4 == 0 && a.K >= 256 &&
+    return a.xs_l == 1 && a.L % 4 == 0 && a.xs_k % 4 == 0 && a.K >= 64 &&
            static_cast<size_t>(a.T) * a.L * (chunks + 1) <= kWorkspaceFloats;
 }
 
 int thin_impl(const ThinArgs& a) {
     if (a.T == 1) return thin_launch<1>(a);
-    return a.T <= 4 ? thin_launch<4>(a) : thin_launch<kThinMax>(a);
+    if (a.T <= 4) return thin_launch<4>(a);
+    return a.T <= 8 ? thin_launch<8>(a) : thin_launch<16>(a);
 }
 
 }  // namespace

@@ -354,12 +354,16 @@ def test_gemm_variants(gpu, oracle_lib, m, n, k, ta, tb):
             assert np.array_equal(g2[:, m:], C0.reshape(n, ldc)[:, m:])
 
 
-# one extent of at most 8 against a long one: the matrix-vector forms (lanes along
+# one extent of at most 16 against a long one: the matrix-vector forms (lanes along
 # k with the thin operand in LDS, or lanes along the long extent with partial sums
 # over k chunks), in both roles and all four layouts, with and without padded
 # leading dimensions; (64, 1216, 512) and (1216, 64, 512) take full 64 x 64 tiles
 THIN_SHAPES = [(3, 4100, 576), (576, 3, 5000), (8, 2052, 128), (1028, 5, 300), (4, 1024, 64),
-               (1500, 7, 257), (2, 1027, 512), (64, 1216, 512), (1216, 64, 512)]
+               (1500, 7, 257), (2, 1027, 512), (64, 1216, 512), (1216, 64, 512),
+               # nine to sixteen thin vectors; a short long-extent against a very long k (the contraction cut
+               # into chunks in the dot form too): the dense layer of the CNN and the first layer of the MLP
+               (10, 128, 12544), (10, 12544, 128), (12544, 10, 128), (256, 16, 4096), (16, 256, 4096),
+               (12, 260, 1028), (300, 9, 4100), (16, 24, 2048), (13, 64, 640)]
 
 
 @pytest.mark.parametrize("m,n,k", THIN_SHAPES)
