@@ -33,6 +33,12 @@ bool conv_fwd_strip_ok(const float* x, const float* out, int C, int H, int W, in
                        int pad_w, int sh, int sw, int Ho, int Wo, int N);
 int launch_conv_fwd_strip(const float* x, const float* weights, const float* bias, float* out, int C, int H, int W,
                           int Cout, int N, int relu, int flip);
+// conv_few.hip: 3x3 stride-1 layers with at most four input channels, forward and weight gradients
+bool conv_few_ok(const float* x, const float* other, int C, int H, int W, int kH, int kW, int pad_h, int pad_w, int sh,
+                 int sw, int Ho, int Wo);
+int launch_conv_few_fwd(const float* x, const float* Wt, const float* bias, float* out, int C, int H, int W, int Cout,
+                        int N, int relu);
+int launch_conv_few_dw(const float* x, const float* t, float* dW, int C, int H, int W, int Cout, int N);
 namespace {
 
 struct ConvGeom {
@@ -831,6 +837,15 @@ bool data_grad_ok(int C_in, int H_in, int W_in, int C_out, int kH, int kW, int p
 }
 
 // JZHIP_CONV_FWD_STRIP=0 keeps the general forward kernel for every shape (for comparisons)
+// JZHIP_CONV_FEW=0 keeps the general kernels for layers with few input channels (for comparisons)
+bool few_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("JZHIP_CONV_FEW");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 bool fwd_strip_enabled() {
     static const bool on = [] {
         const char* e = std::getenv("JZHIP_CONV_FWD_STRIP");
@@ -1059,6 +1074,9 @@ JZ_API int jzhip_conv2d_forward(const float* input, const float* weights, const 
     if (fwd_strip_enabled() &&
         conv_fwd_strip_ok(input, out, C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N))
         return launch_conv_fwd_strip(input, weights, bias, out, C_in, H_in, W_in, C_out, N, relu ? 1 : 0, 0);
+    if (few_enabled() && C_out >= 8 &&
+        conv_few_ok(input, out, C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out))
+        return launch_conv_few_fwd(input, weights, bias, out, C_in, H_in, W_in, C_out, N, relu ? 1 : 0);
     const ConvGeom g = make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N, C_out);
     return launch_fwd(input, weights, bias, out, g, relu ? 1 : 0);
 }
@@ -1068,6 +1086,9 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
                                          int H_out, int W_out, int N) {
     if (!input || !t || !dW) return -1;
     if (!dims_ok(C_in, H_in, W_in, C_out, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N)) return -1;
+    if (few_enabled() && C_out >= 8 &&
+        conv_few_ok(input, t, C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out))
+        return launch_conv_few_dw(input, t, dW, C_in, H_in, W_in, C_out, N);
     const ConvGeom g = make_geom(C_in, H_in, W_in, kH, kW, pad_h, pad_w, stride_h, stride_w, H_out, W_out, N, C_out);
     if (C_out <= kThinCout && kH == 3 && kW == 3 && C_in <= 65535) {
         // chunks of the patch columns so that channels x chunks gives every CU several workgroups

@@ -381,9 +381,14 @@ def bench_conv_implicit(r):
             jz.col2im(P(col), P(dx), *cargs)
 
         r.run("conv", "forward, patch-matrix route (4 launches)", shape, fwd_patch, flops=fl)
-        r.run("conv", "jzhip_conv2d_forward", shape, lambda: jz.conv2d_forward(P(x), P(w), P(b), P(out), *dims, 1), flops=fl)
+        # with at most four input channels the products are bound by the output (forward) or the upstream
+        # gradient (weight gradients) passing through memory once: those rows are priced in bytes
+        few = Ci <= 4 and s == 1
+        io = 4.0 * (N * Ci * H * H + Co * Pp * N)
+        price = dict(bytes_=io) if few else dict(flops=fl)
+        r.run("conv", "jzhip_conv2d_forward", shape, lambda: jz.conv2d_forward(P(x), P(w), P(b), P(out), *dims, 1), **price)
         r.run("conv", "weight gradients, patch-matrix route (3 launches)", shape, dw_patch, flops=fl)
-        r.run("conv", "jzhip_conv2d_backward_weights", shape, lambda: jz.conv2d_backward_weights(P(x), P(t), P(dW), *dims), flops=fl)
+        r.run("conv", "jzhip_conv2d_backward_weights", shape, lambda: jz.conv2d_backward_weights(P(x), P(t), P(dW), *dims), **price)
         r.run("conv", "input gradients, patch-matrix route (2 launches)", shape, dx_patch, flops=fl)
         if s == 1:
             r.run("conv", "jzhip_conv2d_backward_data", shape, lambda: jz.conv2d_backward_data(P(t), P(w), P(dx), *dims), flops=fl)

@@ -62,6 +62,13 @@ SMALL = [
     (2, 3, 12, 12, 8, 7, 7, 3, 1),    # 7x7 stem, K = 147
     (2, 3, 12, 12, 8, 7, 7, 3, 2),    # the same with stride 2
     (1, 344, 4, 4, 8, 3, 3, 1, 1),    # K = 3096
+    # one to four input channels, rows in multiples of four pixels: the kernels that keep a pixel quad's window
+    # in registers (forward and weight gradients)
+    (3, 1, 28, 28, 32, 3, 3, 1, 1),
+    (2, 3, 8, 12, 20, 3, 3, 1, 1),    # channel groups with a ragged end
+    (2, 4, 4, 4, 9, 3, 3, 1, 1),      # one quad per row, nine output channels
+    (5, 2, 12, 8, 10, 3, 3, 1, 1),
+    (9, 1, 256, 256, 32, 3, 3, 1, 1), # pixel blocks fill the chip: all output channels in one workgroup, several passes per workgroup in the weight gradients
 ]
 
 
