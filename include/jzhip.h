@@ -595,7 +595,10 @@ int jzhip_convtrans_reshape(const float* src, float* dst, int C, int spatial,
  *                                 activation derivative                       (:1679-1696)
  * 3x3, stride-1, pad-1 layers whose shape qualifies (jzhip_conv2d_check with which = 4, 5,
  * 6) run from image strips staged in LDS instead: every pixel is fetched once per stage, the
- * taps are the same strip at another offset.
+ * taps are the same strip at another offset.  The same geometry with one to four input
+ * channels, rows in multiples of four pixels and eight or more output channels (forward and
+ * backward_weights) runs as plain vector kernels bound by the output or the upstream
+ * gradient passing through memory once.
  *   jzhip_conv2d_backward_data    replaces RocmGemm(W t2d) + RocmCol2im for stride 1
  *                                 (returns -1 for other strides: those keep the
  *                                 patch-matrix route); the taps of one input

@@ -499,7 +499,7 @@ __global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restr
     // arithmetic runs in the shadow of the matrix pipe instead of in one burst.
     // QUAD (W_out % 4 == 0): the four patch columns of a thread are consecutive pixels of
     // one output row, so one site and one row test serve all four.
-    const __amdgpu_buffer_rsrc_t in_rsrc = input_resource(in, in_bytes);   // used by the QUAD form
+    const __amdgpu_buffer_rsrc_t in_rsrc = input_resource(in, in_bytes);   // in_bytes == 0: not used
     Site sites[QUAD ? 1 : 4];
     long long jcur = 0;
     bool quad_live = false;   // QUAD: the thread's four columns are inside this workgroup's chunk
@@ -550,9 +550,21 @@ __global__ __launch_bounds__(kBlock, 2) void conv_dw_kernel(const float* __restr
                 r[e] = load_or_zero(in_rsrc, ok ? byte0 + static_cast<unsigned>(e * g.sw) * 4u : kOutside);
             }
         } else {
+            if (in_bytes != 0) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                r[e] = (k_ok[ps] && jcur + e < j_hi) ? patch_value(in, sites[e], tap[ps], g) : 0.0f;
+                for (int e = 0; e < 4; ++e) {
+                    const Site& se = sites[e];
+                    const bool ok = k_ok[ps] && jcur + e < j_hi &&
+                                    static_cast<unsigned>(se.ih0 + tap[ps].ky) < static_cast<unsigned>(g.H) &&
+                                    static_cast<unsigned>(se.iw0 + tap[ps].kx) < static_cast<unsigned>(g.W);
+                    r[e] = load_or_zero(in_rsrc, ok ? (static_cast<unsigned>(se.base) + static_cast<unsigned>(tap[ps].off)) * 4u
+                                                    : kOutside);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    r[e] = (k_ok[ps] && jcur + e < j_hi) ? patch_value(in, sites[e], tap[ps], g) : 0.0f;
+            }
         }
         ra[ps] = r;
     };
@@ -1136,7 +1148,10 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
     long long splits = (per_cu * cus + tiles - 1) / tiles;
     splits = splits <= 2 ? splits : splits <= 4 ? 4 : (splits + 7) / 8 * 8;
     const long long per = static_cast<long long>(g.K) * C_out;
-    while (splits > 1 && (g.J / splits < 16 * BK || per * splits > static_cast<long long>(kWorkspaceFloats)))
+    // at least 16 stages per chunk, 6 where a partial tile set is small (288 x 64: 42 -> 31 us with
+    // the sum of the partial results included; 576 x 128 loses with anything below 16)
+    const int min_stages = per <= 20000 ? 6 : 16;
+    while (splits > 1 && (g.J / splits < min_stages * BK || per * splits > static_cast<long long>(kWorkspaceFloats)))
         splits = splits > 8 ? splits - 8 : splits / 2;
     if (splits < 1) splits = 1;
     long long j_chunk = ((g.J + splits - 1) / splits + BK - 1) / BK * BK;
@@ -1151,8 +1166,10 @@ JZ_API int jzhip_conv2d_backward_weights(const float* input, const float* t, flo
     dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(splits));
     hipStream_t s = stream();
     const long long in_bytes = static_cast<long long>(N) * g.CHW * static_cast<long long>(sizeof(float));
-    const bool quad = W_out % 4 == 0 && in_bytes <= kBufferMaxBytes;
-    const unsigned in_b = quad ? static_cast<unsigned>(in_bytes) : 0u;
+    // inputs of up to 2 GiB are read through a buffer resource (padding by the range check);
+    // larger ones take the loaders with a branch per element
+    const unsigned in_b = in_bytes <= kBufferMaxBytes ? static_cast<unsigned>(in_bytes) : 0u;
+    const bool quad = W_out % 4 == 0 && in_b != 0;
     if (wide && quad) conv_dw_kernel<2, true><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
     else if (wide) conv_dw_kernel<2, false><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
     else if (quad) conv_dw_kernel<1, true><<<grid, kBlock, 0, s>>>(input, t, part, g, tiles_n, j_chunk, t_vec, in_b);
