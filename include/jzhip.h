@@ -334,6 +334,20 @@ int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int n,
                      int k, int trans_a, int trans_b, int lda, int ldb, int ldc,
                      float alpha, float beta, const float* bias, int act,
                      float* aux, int ld_aux, const float* residual, int ldr);
+/* A layer's two parameter gradients from one pass over the upstream gradient
+ * (`gW = t * input.T(); gb = sum(t, 1);`, ml/layer.hpp:99-100; the same pair in
+ * TransformerLayer::backward for Wo / W1 / W2 and their biases): jzhip_gemm as
+ * above plus rowsum[i] = sum_p op(A)(i, p), i < m.  With A plain, B transposed
+ * and every extent a whole number of tiles (16-byte aligned operands, leading
+ * dimensions in multiples of 4) the workgroups of the first tile column add up
+ * their A panel on its way into LDS, so the sums cost no second pass over A;
+ * they are then the sum over K chunks of per-thread partial sums in a fixed
+ * order, equal to jzhip_sum_rows to rounding (<= 1e-5 relative at k = 16384),
+ * not bit for bit.  Every other shape runs jzhip_gemm followed by
+ * jzhip_sum_rows / jzhip_sum_cols.  rowsum must not alias A, B or C. */
+int jzhip_gemm_rowsum(const float* A, const float* B, float* C, float* rowsum, int m,
+                      int n, int k, int trans_a, int trans_b, int lda, int ldb, int ldc,
+                      float alpha, float beta);
 /* Juzhen::RocmGemmNN (cpp/hipbackend.hpp:94-95). */
 int jzhip_gemm_nn(const float* A, const float* B, float* C, int m, int n, int k,
                   float alpha, float beta);
@@ -496,6 +510,22 @@ int jzhip_layernorm_bwd(float* dx, const float* dy, const float* gamma,
 int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float* gamma,
                                  const float* xhat, const float* inv_std,
                                  const float* res, int dim, int N);
+/* Everything a pre-LN block's backward pass sums over the tokens around one
+ * LayerNorm, in the sweep that forms dx: jzhip_layernorm_bwd_residual and
+ * jzhip_layernorm_param_grads (ml/layer.hpp:2674-2686) plus, where asked for
+ * (non-NULL), sum_dx[i] = sum_c dx(i, c) and sum_res[i] = sum_c res(i, c) --
+ * the `sum(t, 1)` bias gradients (ml/layer.hpp:100) of the dense layers that
+ * receive dx and res as their upstream gradients.  dy, xhat and res are read
+ * once instead of two to three times.  dx as jzhip_layernorm_bwd_residual bit
+ * for bit; the sums are added per wave over a run of columns, then over
+ * workgroups in a fixed order: equal to the separate entry points to rounding
+ * (<= 1e-5 relative), not bit for bit.  Takes dim <= 512 in multiples of 4
+ * with 16-byte aligned operands and N >= 1024 in one sweep; other shapes run
+ * the separate entry points.  sum_res needs res; res may alias dx. */
+int jzhip_layernorm_bwd_residual_sums(float* dx, const float* dy, const float* gamma,
+                                      const float* xhat, const float* inv_std,
+                                      const float* res, float* dgamma, float* dbeta,
+                                      float* sum_dx, float* sum_res, int dim, int N);
 /* Tangent through the normalisation at the point cached by the forward call:
  * out = gamma .* inv*(dx - mean(dx) - xhat*mean(dx*xhat)), LayerNorm<D>::jvp
  * (ml/layer.hpp:2690-2702: two sums, three rank-1 products and four Hadamard

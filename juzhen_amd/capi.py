@@ -108,6 +108,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_gemm_nn": (I, [P, P, P, I, I, I, F, F]),
     "jzhip_gemv": (I, [P, P, P, I, I, I, I, I, I, F, F]),
     "jzhip_gemm_fused": (I, [P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P, I, P, I]),
+    "jzhip_gemm_rowsum": (I, [P, P, P, P, I, I, I, I, I, I, I, I, F, F]),
     "jzhip_gemm_strided_batched": (I, [P, P, P, I, I, I, I, I, I, I, I, LL, LL, LL, I, F, F]),
     "jzhip_profile_gemm": (I, [I]),
     "jzhip_profile_gemm_report": (I, [C.c_char_p, Z]),
@@ -131,6 +132,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_layernorm_bwd_residual": (I, [P, P, P, P, P, P, I, I]),
     "jzhip_layernorm_jvp": (I, [P, P, P, P, P, I, I]),
     "jzhip_layernorm_param_grads": (I, [P, P, P, P, I, I]),
+    "jzhip_layernorm_bwd_residual_sums": (I, [P, P, P, P, P, P, P, P, P, P, I, I]),
     "jzhip_adam_update": (I, [P, P, P, Z, F, F, F, F, I]),
     "jzhip_adamw_step": (I, [P, P, P, P, Z, F, F, F, F, F, I]),
     "jzhip_adamw_step_multi": (I, [C.POINTER(AdamTensor), I]),

@@ -252,8 +252,18 @@ inline Matrix<ROCMfloat> Layer<ROCMfloat>::backward(const Matrix<ROCMfloat>& inp
         }
         return hadmd(grad(input), std::move(upstream_grad));
     }();
-    MD gW = t * input.T();
-    MD gb = sum(t, 1);
+    // the two parameter gradients from one pass over t where both operands are stored plainly
+    MD gW = JzRocmFused::make("gW", 0, 0, 0), gb = JzRocmFused::make("gb", 0, 0, 0);
+    if (!t.get_transpose() && !input.get_transpose() && t.num_col() == input.num_col() && t.num_row() > 0 &&
+        input.num_row() > 0 && t.num_col() > 0) {
+        const int m = (int)t.num_row(), n = (int)input.num_row(), k = (int)t.num_col();
+        gW = JzRocmFused::make("gW", m, n, 0);
+        gb = MD("gb", m, 1);
+        must(jzhip_gemm_rowsum(p(t), p(input), p(gW), p(gb), m, n, k, 0, 1, m, n, m, 1.0f, 0.0f), "gemm_rowsum");
+    } else {
+        gW = t * input.T();
+        gb = sum(t, 1);
+    }
     // (Layer::update itself cannot be specialised here: the ROCm ConvLayer bodies earlier in
     // ml/layer.hpp have already instantiated it)
     if (need_update) fused_update({{&weights, &gW, &adamW}, {&bias, &gb, &adamb}});
@@ -433,20 +443,38 @@ inline Matrix<ROCMfloat> stacked_blocks(const char* name, const Matrix<ROCMfloat
     return out;
 }
 
+// sum_dx / sum_res (optional): the row sums of the result and of the residual, i.e. the bias
+// gradients `sum(t, 1)` (ml/layer.hpp:100) of the dense layers those two matrices are the
+// upstream gradients of, formed in the same sweep.
 inline Matrix<ROCMfloat> ln_backward_plus(LayerNorm<ROCMfloat>& ln, Matrix<ROCMfloat>&& dy,
-                                          const Matrix<ROCMfloat>& residual, bool update) {
-    if (dy.get_transpose() || residual.get_transpose()) return ln.backward(std::move(dy), update) + residual;
+                                          const Matrix<ROCMfloat>& residual, bool update,
+                                          Matrix<ROCMfloat>* sum_dx = nullptr, Matrix<ROCMfloat>* sum_res = nullptr) {
+    if (dy.get_transpose() || residual.get_transpose()) {
+        if (sum_res) *sum_res = sum(residual, 1);
+        Matrix<ROCMfloat> dx = ln.backward(std::move(dy), update) + residual;
+        if (sum_dx) *sum_dx = sum(dx, 1);
+        return dx;
+    }
     const int N = (int)dy.num_col();
     Matrix<ROCMfloat> dx("ln_dx", ln.dim, N);
+    if (sum_dx) *sum_dx = Matrix<ROCMfloat>("ln_sum_dx", ln.dim, 1);
+    if (sum_res) *sum_res = Matrix<ROCMfloat>("ln_sum_res", ln.dim, 1);
+    if (update) {
+        // one sweep: dx, the parameter gradients and the row sums; dx reads gamma, so the
+        // parameter step comes after it (ml/layer.hpp:2682-2686)
+        Matrix<ROCMfloat> dg("ln_dgamma", ln.dim, 1), db("ln_dbeta", ln.dim, 1);
+        must(jzhip_layernorm_bwd_residual_sums(p(dx), p(dy), p(ln.gamma), p(ln.cached_xhat), p(ln.cached_inv), p(residual),
+                                               p(dg), p(db), sum_dx ? p(*sum_dx) : nullptr,
+                                               sum_res ? p(*sum_res) : nullptr, ln.dim, N),
+             "layernorm_bwd_residual_sums");
+        fused_update({{&ln.gamma, &dg, &ln.adam_g}, {&ln.beta, &db, &ln.adam_b}});
+        return dx;
+    }
     must(jzhip_layernorm_bwd_residual(p(dx), p(dy), p(ln.gamma), p(ln.cached_xhat), p(ln.cached_inv), p(residual),
                                       ln.dim, N),
          "layernorm_bwd_residual");
-    // dx reads gamma, so the parameter step comes second (ml/layer.hpp:2682-2686)
-    if (update) {
-        Matrix<ROCMfloat> dg("ln_dgamma", ln.dim, 1), db("ln_dbeta", ln.dim, 1);
-        must(jzhip_layernorm_param_grads(p(dg), p(db), p(dy), p(ln.cached_xhat), ln.dim, N), "layernorm_param_grads");
-        fused_update({{&ln.gamma, &dg, &ln.adam_g}, {&ln.beta, &db, &ln.adam_b}});
-    }
+    if (sum_dx) must(jzhip_sum_rows(p(*sum_dx), p(dx), ln.dim, N, ln.dim), "sum_rows");
+    if (sum_res) must(jzhip_sum_rows(p(*sum_res), p(residual), ln.dim, N, ln.dim), "sum_rows");
     return dx;
 }
 }  // namespace rocm_detail
@@ -528,15 +556,16 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
 
     // feed-forward: F = W2 relu(W1 x2 + b1) + b2
     MD dW2 = dout * cached_F1_relu.T();
-    MD db2 = sum(dout, 1);
     MD dF1 = fused_product(W2, true, dout, nullptr, 3, &cached_F1, nullptr);   // (W2^T dout) .* relu'(F1)
     MD dW1 = dF1 * cached_x2.T();
     MD db1 = sum(dF1, 1);
-    MD dR = ln_backward_plus(ln2, W1.T() * dF1, dout, this->need_update);
+    // the sweep that forms dR = LN2'(..) + dout also adds up the rows of dout and of dR: the
+    // bias gradients db2 = sum(dout, 1) and dbo = sum(dR, 1)
+    MD db2 = JzRocmFused::make("db2", 0, 0, 0), dbo = JzRocmFused::make("dbo", 0, 0, 0);
+    MD dR = ln_backward_plus(ln2, W1.T() * dF1, dout, this->need_update, &dbo, &db2);
 
     // output projection: O = Wo H + bo
     MD dWo = dR * cached_H.T();
-    MD dbo = sum(dR, 1);
     MD dH = Wo.T() * dR;
 
     // attention core, all heads and sequences at once, then the three projections

@@ -70,12 +70,18 @@ struct Epilogue {
 };
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
-template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST, bool EPI>
+// RS: the workgroups of the first tile column also add up the rows of their A panel over
+// their K range (A not transposed, unchecked loaders): rs_out[chunk * M + row].  The values
+// are taken from the staging registers on their way to LDS, so the sums cost eight
+// additions per stage and no extra pass over A.
+template <int WGM, int WGN, int TM, int TN, bool TA, bool TB, bool FAST, bool EPI, bool RS = false>
 __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* C, int M, int N, int K,
     size_t lda, size_t ldb, size_t ldc, float alpha, float beta, long long strideA,
     long long strideB, long long strideC, int batch1, long long strideA2, long long strideB2,
-    long long strideC2, int tiles_m, int tiles_n, int k_chunk, long long split_stride, Epilogue ep) {
+    long long strideC2, int tiles_m, int tiles_n, int k_chunk, long long split_stride, Epilogue ep,
+    float* __restrict__ rs_out = nullptr) {
+    static_assert(!RS || (!TA && FAST && !EPI), "row sums ride on the unchecked loaders of a plain A");
     static_assert(WGM * WGN == kBlock / kWave, "four waves per workgroup");
     constexpr int BM = WGM * TM * 32;
     constexpr int BN = WGN * TN * 32;
@@ -181,6 +187,13 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
     load_stage(Set0{}, k_lo);
     LA::store(ra[0], As[odd]);
     LB::store(rb[0], Bs[odd]);
+    // row sums of A: a thread's float4s are the same four rows in every pass and stage
+    floatx4 rs = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (RS) {
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps)
+            if (LA::active(ps)) rs += ra[0][ps];
+    }
     __syncthreads();
     if constexpr (NSET == 2) {
         // stage 1 waits in registers (a single stage is fetched again and dropped)
@@ -248,6 +261,23 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
                 if (kk < LA::kPasses) LA::store_pass(ra[ST], As[cur ^ 1], kk);
                 else if (kk < kStorePasses) LB::store_pass(rb[ST], Bs[cur ^ 1], kk - LA::kPasses);
             }
+            if constexpr (RS) {
+                // (the set holds stage kt+1; past the end it is the last stage fetched again)
+#ifdef JZ_RS_TN0
+                if (kk < LA::kPasses && LA::active(kk) && tile_n == 0) {
+#else
+                if (kk < LA::kPasses && LA::active(kk)) {
+#endif
+#if defined(JZ_RS_NOACC)
+#elif defined(JZ_RS_SUBTRACT)
+                    rs += ra[ST][kk];
+#else
+                    const bool real = kt + 1 < nk;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) rs[e] += real ? ra[ST][kk][e] : 0.0f;
+#endif
+                }
+            }
             if constexpr (NSET == 1) {
                 if (kk == kStorePasses && kt + 2 < nk) load_stage(ld_c, k_lo + (kt + 2) * BK);
             }
@@ -275,6 +305,29 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
         }
     }
 
+    if constexpr (RS) {
+#ifdef JZ_RS_SUBTRACT
+#pragma unroll
+        for (int ps = 0; ps < LA::kPasses; ++ps)
+            if (LA::active(ps)) rs -= ra[0][ps];
+#endif
+        if (tile_n == 0) {
+            // the kBlock / (BM / 4) threads that hold the same four rows meet in LDS and are
+            // added in thread order
+            __syncthreads();   // the last fragment reads of As are done
+            float* red = &As[0][0];
+            static_assert(2 * BK * LDA_S >= 4 * kBlock, "the staging buffers hold one float4 per thread");
+            *reinterpret_cast<floatx4*>(red + 4 * threadIdx.x) = rs;
+            __syncthreads();
+            if (threadIdx.x < BM) {
+                const int xg = threadIdx.x / 4, comp = threadIdx.x % 4;
+                float sum = 0.0f;
+#pragma unroll
+                for (int j = 0; j < kBlock / (BM / 4); ++j) sum += red[4 * (xg + j * (BM / 4)) + comp];
+                rs_out[static_cast<size_t>(chunk) * M + m0 + threadIdx.x] = sum;
+            }
+        }
+    }
     // Epilogue.  Register v of lane (h, l32) holds C(row, col) with
     // row = l32 and col = 8*(v/4) + 4*h + v%4 inside the 32x32 tile.
     if constexpr (!EPI) {
@@ -476,28 +529,37 @@ __global__ __launch_bounds__(kBlock) void add_bias_scalar_kernel(float* y, const
 }
 
 // C = alpha * sum_s part[s] + beta*C for split-K partials (each m x n, ld = m)
+// (rs_part: M further sums per chunk, the row sums a product formed on the side; their
+// total goes to rs_dst as it is)
 __global__ __launch_bounds__(kBlock) void splitk_reduce_kernel(float* C, const float* part, int M, int N,
                                                                size_t ldc, int splits, float alpha,
-                                                               float beta) {
+                                                               float beta, float* rs_dst, const float* rs_part) {
     const size_t total = static_cast<size_t>(M) * N;
+    const size_t all = total + (rs_dst ? M : 0);
     const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
-    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < total; i += stride) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < all; i += stride) {
         // eight partials requested at a time, summed in split order
-        const float* p = part + i;
+        const bool side = i >= total;
+        const float* p = side ? rs_part + (i - total) : part + i;
+        const size_t step = side ? static_cast<size_t>(M) : total;
         float acc = 0.f;
         int s = 0;
         for (; s + 8 <= splits; s += 8) {
             float x[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = p[static_cast<size_t>(s + u) * total];
+            for (int u = 0; u < 8; ++u) x[u] = p[static_cast<size_t>(s + u) * step];
 #pragma unroll
             for (int u = 0; u < 8; ++u) acc += x[u];
         }
-        for (; s < splits; ++s) acc += p[static_cast<size_t>(s) * total];
-        float* dst = C + (i / M) * ldc + (i % M);
-        float r = alpha * acc;
-        if (beta != 0.0f) r += beta * *dst;
-        *dst = r;
+        for (; s < splits; ++s) acc += p[static_cast<size_t>(s) * step];
+        if (side) {
+            rs_dst[i - total] = acc;
+        } else {
+            float* dst = C + (i / M) * ldc + (i % M);
+            float r = alpha * acc;
+            if (beta != 0.0f) r += beta * *dst;
+            *dst = r;
+        }
     }
 }
 
@@ -509,35 +571,43 @@ __global__ __launch_bounds__(kBlock) void splitk_reduce_kernel(float* C, const f
 constexpr int kTallBlock = 1024;
 __global__ __launch_bounds__(kTallBlock) void splitk_reduce_tall_kernel(float* C, const float* part, int M, int N,
                                                                         size_t ldc, int splits, float alpha,
-                                                                        float beta) {
+                                                                        float beta, float* rs_dst,
+                                                                        const float* rs_part) {
     constexpr int NW = kTallBlock / kWave;
     __shared__ float red[NW][kWave];
     const size_t total = static_cast<size_t>(M) * N;
+    const size_t all = total + (rs_dst ? M : 0);
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const size_t i = static_cast<size_t>(blockIdx.x) * kWave + lane;
+    const bool side = i >= total;
     float acc = 0.f;
-    if (i < total) {
-        const float* p = part + i;
+    if (i < all) {
+        const float* p = side ? rs_part + (i - total) : part + i;
+        const size_t step = side ? static_cast<size_t>(M) : total;
         int s = wave;
         for (; s + 3 * NW < splits; s += 4 * NW) {
             float x[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) x[u] = p[static_cast<size_t>(s + u * NW) * total];
+            for (int u = 0; u < 4; ++u) x[u] = p[static_cast<size_t>(s + u * NW) * step];
 #pragma unroll
             for (int u = 0; u < 4; ++u) acc += x[u];
         }
-        for (; s < splits; s += NW) acc += p[static_cast<size_t>(s) * total];
+        for (; s < splits; s += NW) acc += p[static_cast<size_t>(s) * step];
     }
     red[wave][lane] = acc;
     __syncthreads();
-    if (wave == 0 && i < total) {
+    if (wave == 0 && i < all) {
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) sum += red[w][lane];
-        float* dst = C + (i / M) * ldc + (i % M);
-        float r = alpha * sum;
-        if (beta != 0.0f) r += beta * *dst;
-        *dst = r;
+        if (side) {
+            rs_dst[i - total] = sum;
+        } else {
+            float* dst = C + (i / M) * ldc + (i % M);
+            float r = alpha * sum;
+            if (beta != 0.0f) r += beta * *dst;
+            *dst = r;
+        }
     }
 }
 
@@ -551,10 +621,26 @@ void launch_splitk_reduce(float* C, const float* part, int M, int N, size_t ldc,
     hipStream_t s = stream();
     if (splits >= 32 && total <= (size_t(1) << 20))
         splitk_reduce_tall_kernel<<<static_cast<unsigned>((total + kWave - 1) / kWave), kTallBlock, 0, s>>>(
-            C, part, M, N, ldc, splits, alpha, beta);
+            C, part, M, N, ldc, splits, alpha, beta, nullptr, nullptr);
     else
-        splitk_reduce_kernel<<<grid_for(total, kBlock, 4), kBlock, 0, s>>>(C, part, M, N, ldc, splits, alpha, beta);
+        splitk_reduce_kernel<<<grid_for(total, kBlock, 4), kBlock, 0, s>>>(C, part, M, N, ldc, splits, alpha, beta,
+                                                                            nullptr, nullptr);
 }
+
+namespace {
+// The same with the row sums that the product's first tile column left per chunk (M values each).
+void launch_splitk_reduce_rowsum(float* C, const float* part, int M, int N, size_t ldc, int splits, float alpha,
+                                 float beta, float* rs_dst, const float* rs_part) {
+    // (the kernel the plain sum would take for this shape, so that C comes out the same bit for bit)
+    const size_t total = static_cast<size_t>(M) * N, all = total + M;
+    if (splits >= 32 && total <= (size_t(1) << 20))
+        splitk_reduce_tall_kernel<<<static_cast<unsigned>((all + kWave - 1) / kWave), kTallBlock, 0, stream()>>>(
+            C, part, M, N, ldc, splits, alpha, beta, rs_dst, rs_part);
+    else
+        splitk_reduce_kernel<<<grid_for(all, kBlock, 4), kBlock, 0, stream()>>>(C, part, M, N, ldc, splits, alpha,
+                                                                                beta, rs_dst, rs_part);
+}
+}  // namespace
 
 namespace {
 
@@ -571,6 +657,9 @@ struct GemmArgs {
     long long sA2 = 0, sB2 = 0, sC2 = 0;  // outer batch level
     int batch2 = 1;
     Epilogue ep;
+    // row sums of A on the side (jzhip_gemm_rowsum): where to, and whether the launch formed them
+    float* rowsum = nullptr;
+    bool* rowsum_done = nullptr;
 };
 
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB>
@@ -616,7 +705,7 @@ int launch_tile(const GemmArgs& g) {
         // gradients) is still cut, down to four steps, because a handful of
         // workgroups walking it alone only wait for their loads
         const int max_by_k = g.K >= 1024 ? g.K / 256 : g.K / 64;
-        const size_t per = static_cast<size_t>(g.M) * g.N * nb;
+        const size_t per = static_cast<size_t>(g.M) * g.N * nb + (g.rowsum ? g.M : 0);   // partial C (+ row sums) per chunk
         while (splits > 1 && (splits > max_by_k || per * splits > kWorkspaceFloats))
             splits = splits > 8 ? splits - 8 : splits / 2;
         if (splits < 2) splits = 1;
@@ -645,6 +734,13 @@ int launch_tile(const GemmArgs& g) {
                       g.ldb < (1u << 22);
     dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n, splits, g.batch * g.batch2);
     hipStream_t s = stream();
+    // row sums of A on the side: plain A, transposed B (the weight-gradient form), full tiles
+    bool with_rowsum = false;
+    float* rs_part = nullptr;
+    if constexpr (!TA && TB) {
+        with_rowsum = g.rowsum && fast && !g.ep.any && nb == 1;
+        if (with_rowsum) rs_part = splits > 1 ? out + split_stride * splits : g.rowsum;
+    }
     GemmProf& prof = gemm_prof();
     GemmProfRecord rec;
     const bool timing = prof.on;
@@ -663,7 +759,13 @@ int launch_tile(const GemmArgs& g) {
     gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, FASTV, EPIV><<<grid, kBlock, 0, s>>>(                        \
         g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, sC, g.batch, g.sA2, g.sB2, \
         sC2, tiles_m, tiles_n, k_chunk, split_stride, g.ep)
-    if (g.ep.any) {
+    if (with_rowsum) {
+        if constexpr (!TA && TB)
+            gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true, false, true><<<grid, kBlock, 0, s>>>(
+                g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, sC, g.batch, g.sA2, g.sB2,
+                sC2, tiles_m, tiles_n, k_chunk, split_stride, g.ep, rs_part);
+        if (g.rowsum_done) *g.rowsum_done = true;
+    } else if (g.ep.any) {
         if (fast) JZ_LAUNCH_GEMM(true, true); else JZ_LAUNCH_GEMM(false, true);
     } else {
         if (fast) JZ_LAUNCH_GEMM(true, false); else JZ_LAUNCH_GEMM(false, false);
@@ -675,6 +777,10 @@ int launch_tile(const GemmArgs& g) {
         prof.recs.push_back(rec);
     }
     if (splits > 1) {
+        if (with_rowsum) {
+            launch_splitk_reduce_rowsum(g.C, out, g.M, g.N, g.ldc, splits, g.alpha, g.beta, g.rowsum, rs_part);
+            return launch_rc();
+        }
         for (int b = 0; b < nb; ++b) {
             const int b_in = b % g.batch, b_out = b / g.batch;
             launch_splitk_reduce(g.C + b_in * g.sC + b_out * g.sC2, out + b * sC, g.M, g.N, g.ldc, splits, g.alpha,
@@ -847,6 +953,33 @@ JZ_API int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, in
     GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
                static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
     return gemm_dispatch(g, trans_a != 0, trans_b != 0);
+}
+
+JZ_API int jzhip_gemm_rowsum(const float* A, const float* B, float* C, float* rowsum, int m, int n, int k, int trans_a,
+                             int trans_b, int lda, int ldb, int ldc, float alpha, float beta) {
+    if (m <= 0 || n <= 0 || k <= 0) return -1;
+    if (!A || !B || !C || !rowsum) return -1;
+    if (lda < (trans_a ? k : m) || ldb < (trans_b ? n : k) || ldc < m) return -1;
+    // The tiled kernel forms the sums on the side for a plain A against a transposed B in full,
+    // aligned tiles; every other product is the plain entry point followed by the sum kernels.
+    // JZHIP_GEMM_ROWSUM=0 keeps the two separate passes for every shape (for comparisons)
+    static const bool fused_on = [] {
+        const char* e = std::getenv("JZHIP_GEMM_ROWSUM");
+        return !(e && e[0] == '0');
+    }();
+    if (fused_on && !trans_a && trans_b && k > 1 && m > 16 && n > 16) {
+        bool done = false;
+        GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
+                   static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
+        g.rowsum = rowsum;
+        g.rowsum_done = &done;
+        const int rc = gemm_dispatch(g, false, true);
+        if (rc != 0 || done) return rc;
+    } else {
+        const int rc = jzhip_gemm(A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta);
+        if (rc != 0) return rc;
+    }
+    return trans_a ? jzhip_sum_cols(rowsum, A, k, m, lda) : jzhip_sum_rows(rowsum, A, m, k, lda);
 }
 
 JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int n, int k, int trans_a,

@@ -319,6 +319,133 @@ __global__ __launch_bounds__(kCombineThreads) void ln_param_combine_kernel(float
     }
 }
 
+// The backward pass with everything else that is summed over the tokens in the same sweep:
+// dx = P(gamma .* dy) + res as ln_bwd_vec_kernel, and per row the sums over the columns of
+// dy .* xhat (dgamma), dy (dbeta), dx and res (the bias gradients of the dense layers on
+// either side of the residual add).  A wave keeps its rows and walks a run of columns, so
+// the four sums are 4*NV float4 accumulators per lane; the waves of a workgroup meet in LDS
+// (wave w adds up sum w in wave order) and leave part[block][4][dim].
+template <int NV, bool NT>
+__global__ __launch_bounds__(kBlock) void ln_bwd_sums_vec_kernel(float* dx, const float* dy, const float* gamma,
+                                                                 const float* xhat, const float* inv_std,
+                                                                 const float* res, float* part, int dim, int N) {
+    constexpr int NW = kBlock / kWave;
+    static_assert(NW == 4, "one wave per sum in the closing step");
+    __shared__ float4 red[4][NW][NV][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const size_t wave0 = static_cast<size_t>(blockIdx.x) * NW + wave;
+    const size_t nwaves = static_cast<size_t>(gridDim.x) * NW;
+    const float invdim = 1.0f / static_cast<float>(dim);
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 g[NV], acc[4][NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int r = (lane + v * kWave) * 4;
+        g[v] = r < dim ? *reinterpret_cast<const float4*>(gamma + r) : zero;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q][v] = zero;
+    }
+    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
+        const size_t base = col * dim;
+        float4 d[NV], h[NV], rr[NV];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                d[v] = load4<NT>(dy + base + r);
+                h[v] = load4<NT>(xhat + base + r);
+                rr[v] = res ? load4<NT>(res + base + r) : zero;
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                acc[0][v].x += d[v].x * h[v].x; acc[0][v].y += d[v].y * h[v].y;
+                acc[0][v].z += d[v].z * h[v].z; acc[0][v].w += d[v].w * h[v].w;
+                acc[1][v].x += d[v].x; acc[1][v].y += d[v].y; acc[1][v].z += d[v].z; acc[1][v].w += d[v].w;
+                d[v].x *= g[v].x; d[v].y *= g[v].y; d[v].z *= g[v].z; d[v].w *= g[v].w;
+                s1 += (d[v].x + d[v].y) + (d[v].z + d[v].w);
+                s2 += (d[v].x * h[v].x + d[v].y * h[v].y) + (d[v].z * h[v].z + d[v].w * h[v].w);
+            }
+        }
+        const float m1 = wave_sum(s1) * invdim;
+        const float m2 = wave_sum(s2) * invdim;
+        const float inv = inv_std[col];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int r = (lane + v * kWave) * 4;
+            if (r < dim) {
+                float4 o;
+                o.x = inv * (d[v].x - m1 - h[v].x * m2);
+                o.y = inv * (d[v].y - m1 - h[v].y * m2);
+                o.z = inv * (d[v].z - m1 - h[v].z * m2);
+                o.w = inv * (d[v].w - m1 - h[v].w * m2);
+                if (res) {  // rounded like a separate add
+                    o.x += rr[v].x; o.y += rr[v].y; o.z += rr[v].z; o.w += rr[v].w;
+                    acc[3][v].x += rr[v].x; acc[3][v].y += rr[v].y; acc[3][v].z += rr[v].z; acc[3][v].w += rr[v].w;
+                }
+                acc[2][v].x += o.x; acc[2][v].y += o.y; acc[2][v].z += o.z; acc[2][v].w += o.w;
+                store4<NT>(dx + base + r, o);
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) red[q][wave][v][lane] = acc[q][v];
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int r = (lane + v * kWave) * 4;
+        if (r < dim) {
+            float4 sum = red[wave][0][v][lane];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+                const float4 t = red[wave][w][v][lane];
+                sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+            }
+            *reinterpret_cast<float4*>(part + (static_cast<size_t>(blockIdx.x) * 4 + wave) * dim + r) = sum;
+        }
+    }
+}
+
+// part is [chunk][4*dim]; a block owns 64 of the 4*dim outputs, its waves take interleaved
+// chunks and are combined through LDS; a sum nobody asked for (null pointer) is skipped.
+__global__ __launch_bounds__(kCombineThreads) void ln_sums_combine_kernel(float* s0, float* s1, float* s2, float* s3,
+                                                                          const float* part, int dim, int chunks) {
+    constexpr int NW = kCombineThreads / kWave;
+    __shared__ float red[NW][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int i = blockIdx.x * kWave + lane;
+    const int n = 4 * dim;
+    const int which = i < n ? i / dim : 0;
+    float* dst = which == 0 ? s0 : which == 1 ? s1 : which == 2 ? s2 : s3;
+    float acc = 0.f;
+    if (i < n && dst) {
+        int c = wave;
+        for (; c + 3 * NW < chunks; c += 4 * NW) {   // four loads in flight
+            const float a0 = part[static_cast<size_t>(c) * n + i];
+            const float a1 = part[static_cast<size_t>(c + NW) * n + i];
+            const float a2 = part[static_cast<size_t>(c + 2 * NW) * n + i];
+            const float a3 = part[static_cast<size_t>(c + 3 * NW) * n + i];
+            acc += (a0 + a1) + (a2 + a3);
+        }
+        for (; c < chunks; c += NW) acc += part[static_cast<size_t>(c) * n + i];
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && i < n && dst) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += red[w][lane];
+        dst[i - which * dim] = s;
+    }
+}
+
 }  // namespace
 }  // namespace jz
 
@@ -375,6 +502,43 @@ JZ_API int jzhip_layernorm_bwd_residual(float* dx, const float* dy, const float*
                                         const float* xhat, const float* inv_std, const float* res,
                                         int dim, int N) {
     return launch_ln_bwd<false>(dx, dy, gamma, xhat, inv_std, res, dim, N);
+}
+
+JZ_API int jzhip_layernorm_bwd_residual_sums(float* dx, const float* dy, const float* gamma, const float* xhat,
+                                             const float* inv_std, const float* res, float* dgamma, float* dbeta,
+                                             float* sum_dx, float* sum_res, int dim, int N) {
+    if (dim <= 0 || N <= 0 || !dx || !dy || !gamma || !xhat || !inv_std || !dgamma || !dbeta) return -1;
+    if (sum_res && !res) return -1;
+    const bool vec = (dim % 4 == 0) && dim <= 512 && aligned16(dx) && aligned16(dy) && aligned16(xhat) &&
+                     aligned16(gamma) && (!res || aligned16(res));
+    // workgroups: four per CU, each wave a run of columns; the partial sums are 16*dim bytes per workgroup
+    size_t blocks = static_cast<size_t>(num_cus()) * 4;
+    const size_t cover = (static_cast<size_t>(N) + kBlock / kWave - 1) / (kBlock / kWave);
+    if (blocks > cover) blocks = cover;
+    if (vec && N >= 1024 && blocks * 4 * dim <= kWorkspaceFloats) {
+        float* part = workspace();
+        if (!part) return -2;
+        hipStream_t s = stream();
+        const bool nt = streams_past_cache((res ? 4 : 3) * static_cast<size_t>(dim) * N * sizeof(float));
+        const unsigned grid = static_cast<unsigned>(blocks);
+#define JZ_LN_BWD_SUMS(NV_)                                                                                               \
+    do {                                                                                                                  \
+        if (nt) ln_bwd_sums_vec_kernel<NV_, true><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, part, dim, N);   \
+        else ln_bwd_sums_vec_kernel<NV_, false><<<grid, kBlock, 0, s>>>(dx, dy, gamma, xhat, inv_std, res, part, dim, N);     \
+    } while (0)
+        if (dim <= 256) JZ_LN_BWD_SUMS(1);
+        else JZ_LN_BWD_SUMS(2);
+#undef JZ_LN_BWD_SUMS
+        ln_sums_combine_kernel<<<(4 * dim + kWave - 1) / kWave, kCombineThreads, 0, s>>>(dgamma, dbeta, sum_dx, sum_res,
+                                                                                         part, dim, static_cast<int>(blocks));
+        return launch_rc();
+    }
+    // other shapes: the separate passes
+    int rc = jzhip_layernorm_param_grads(dgamma, dbeta, dy, xhat, dim, N);
+    if (rc == 0 && sum_res) rc = jzhip_sum_rows(sum_res, res, dim, N, dim);   // (dx may be res itself)
+    if (rc == 0) rc = jzhip_layernorm_bwd_residual(dx, dy, gamma, xhat, inv_std, res, dim, N);
+    if (rc == 0 && sum_dx) rc = jzhip_sum_rows(sum_dx, dx, dim, N, dim);
+    return rc;
 }
 
 JZ_API int jzhip_layernorm_jvp(float* out, const float* dx, const float* gamma, const float* xhat,

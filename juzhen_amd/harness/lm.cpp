@@ -304,8 +304,7 @@ void backward(Model& M, bool update) {
         float* dy_next = M.dx[(i + 1) % 3];
         // feed-forward
         lanes.fork();
-        gemm(M, dy, false, b.F1a, true, M.t[b.W2].g, d, ff, N);
-        M.ck(jzhip_sum_rows(M.t[b.b2].g, dy, d, N, d));
+        gemm(M, dy, false, b.F1a, true, M.t[b.W2].g, d, ff, N);   // (db2 = row sums of dy: with the LayerNorm sweep below)
         lanes.back();
         // dF1 = (W2^T dy) .* act'(F1)
         gemm_tail(M, M.t[b.W2].w, true, dy, dF1, ff, N, d, nullptr, c.gelu ? 4 : 3, b.F1, nullptr);
@@ -314,15 +313,13 @@ void backward(Model& M, bool update) {
         M.ck(jzhip_sum_rows(M.t[b.b1].g, dF1, ff, N, ff));
         lanes.back();
         gemm(M, M.t[b.W1].w, true, dF1, false, dx2, d, N, ff);
-        lanes.fork();
-        M.ck(jzhip_layernorm_param_grads(M.t[b.g2].g, M.t[b.be2].g, dx2, b.xhat2, d, N));
-        lanes.back();
-        // dR = LN2'(dx2) + dy
-        M.ck(jzhip_layernorm_bwd_residual(dR, dx2, M.t[b.g2].w, b.xhat2, b.inv2, dy, d, N));
+        // dR = LN2'(dx2) + dy, and in the same sweep the LayerNorm's parameter gradients and the
+        // two bias gradients that are row sums of its operands: dbo of dR, db2 of dy
+        M.ck(jzhip_layernorm_bwd_residual_sums(dR, dx2, M.t[b.g2].w, b.xhat2, b.inv2, dy, M.t[b.g2].g, M.t[b.be2].g,
+                                               M.t[b.bo].g, M.t[b.b2].g, d, N));
         // output projection
         lanes.fork();
         gemm(M, dR, false, b.H, true, M.t[b.Wo].g, d, d, N);
-        M.ck(jzhip_sum_rows(M.t[b.bo].g, dR, d, N, d));
         lanes.back();
         gemm(M, M.t[b.Wo].w, true, dR, false, M.dH, d, N, d);
         // attention core, gradients into the stacked (3d x N) buffer
@@ -339,12 +336,12 @@ void backward(Model& M, bool update) {
         gemm(M, dQKV, false, b.x1, true, M.t[b.Wq].g, 3 * d, d, N);          // stacked dWq, dWk, dWv
         lanes.back();
         gemm(M, M.t[b.Wq].w, true, dQKV, false, dx1, d, N, 3 * d);
-        lanes.fork();
-        M.ck(jzhip_layernorm_param_grads(M.t[b.g1].g, M.t[b.be1].g, dx1, b.xhat1, d, N));
-        lanes.back();
         lanes.mark(i);
-        // dx = LN1'(dx1) + dR
-        M.ck(jzhip_layernorm_bwd_residual(dy_next, dx1, M.t[b.g1].w, b.xhat1, b.inv1, dR, d, N));
+        // dx = LN1'(dx1) + dR with the LayerNorm's parameter gradients (and, under the lowest block,
+        // the row sums of dx for the embedding bias)
+        float* sum_dx = (i == L - 1 && M.be >= 0) ? M.t[M.be].g : nullptr;
+        M.ck(jzhip_layernorm_bwd_residual_sums(dy_next, dx1, M.t[b.g1].w, b.xhat1, b.inv1, dR, M.t[b.g1].g,
+                                               M.t[b.be1].g, sum_dx, nullptr, d, N));
         dy = dy_next;
     }
     lanes.join();
@@ -352,7 +349,7 @@ void backward(Model& M, bool update) {
     gemm(M, dy, false, M.oh_tok, true, M.t[M.E].g, d, V, N, c.tied ? 1.0f : 0.0f);
     // (token n = b*S + s: the (d, N) gradient is a (d*S) x B matrix whose row sums are dP)
     M.ck(jzhip_sum_rows(M.t[M.P].g, dy, d * c.seq, c.batch, d * c.seq));
-    if (M.be >= 0) M.ck(jzhip_sum_rows(M.t[M.be].g, dy, d, N, d));
+    if (M.be >= 0 && L == 0) M.ck(jzhip_sum_rows(M.t[M.be].g, dy, d, N, d));
     if (update) {
         step_group(M, kDecay);
         step_group(M, kPlain);

@@ -417,6 +417,72 @@ def test_gemm_with_beta_zero_never_reads_c(gpu, m, n, k, ta, tb):
     assert rel_err(got, exact) <= TOL_GEMM
 
 
+# A layer's two parameter gradients in one call (ml/layer.hpp:99-100).  The first group takes the
+# kernel that adds up A on its way into LDS: 128 x 128 tiles with K cut into chunks, one / two / three
+# K stages, 64 x 64, 32 x 256, 128 x 64, 64 x 128 and 256 x 32 tiles; the second group the plain
+# product followed by the sum kernels (ragged, transposed A, plain B, thin, matrix-vector, rank-1).
+ROWSUM_SHAPES = [(256, 128, 8192, 0, 1), (512, 512, 4096, 0, 1), (256, 256, 16, 0, 1), (256, 256, 32, 0, 1),
+                 (128, 256, 48, 0, 1), (64, 1216, 512, 0, 1), (32, 256, 128, 0, 1), (256, 64, 1024, 0, 1),
+                 (64, 256, 2048, 0, 1), (1024, 32, 512, 0, 1), (256, 128, 80, 0, 1),
+                 (129, 127, 17, 0, 1), (256, 128, 512, 1, 1), (256, 128, 512, 0, 0), (256, 128, 512, 1, 0),
+                 (576, 3, 5000, 0, 1), (300, 1, 70, 0, 0), (1, 300, 70, 1, 0), (40, 50, 1, 0, 1)]
+
+
+@pytest.mark.parametrize("m,n,k,ta,tb", ROWSUM_SHAPES)
+def test_gemm_rowsum(gpu, m, n, k, ta, tb):
+    r = rng(m + 5 * n + 11 * k + ta + 2 * tb)
+    for pad, alpha, beta in ((0, 1.0, 0.0), (4, 0.5, 1.5)):
+        lda, ldb = (k if ta else m) + pad, (n if tb else k) + pad
+        A = r.normal(0.1, 1, lda * (m if ta else k)).astype(np.float32)
+        B = r.normal(0, 1, ldb * (k if tb else n)).astype(np.float32)
+        C0 = r.normal(0, 1, m * n).astype(np.float32) if beta else np.full(m * n, np.nan, np.float32)
+        exact = naive_gemm64(ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, np.nan_to_num(C0), m)
+        Am = A.astype(np.float64).reshape(-1, lda).T
+        want_rs = (Am[:k, :m].T if ta else Am[:m, :k]).sum(axis=1)
+        dC, dR = to_dev(C0), to_dev(np.full(m, np.nan, np.float32))
+        gpu.gemm_rowsum(dp(A), dp(B), dptr(dC), dptr(dR), m, n, k, ta, tb, lda, ldb, m, alpha, beta)
+        got, got_rs = to_host(dC), to_host(dR)
+        assert np.isfinite(got).all() and np.isfinite(got_rs).all()
+        assert rel_err(got, exact) <= TOL_GEMM
+        assert rel_err(got_rs, want_rs) <= TOL_RED
+        # the product itself is the plain entry point's, bit for bit
+        dC2 = to_dev(C0)
+        gpu.gemm(dp(A), dp(B), dptr(dC2), m, n, k, ta, tb, lda, ldb, m, alpha, beta)
+        assert np.array_equal(got, to_host(dC2))
+
+
+def test_gemm_rowsum_at_the_transformer_weight_gradient_shapes(gpu):
+    """512 x 2048, 2048 x 512 and 512 x 512 over 16384 tokens: the sums against jzhip_sum_rows and
+    float64, the product against the plain entry point bit for bit; twice in a row (the
+    partial sums live in the workspace the next call rewrites)."""
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    N = 16384
+    for m, n in ((512, 2048), (2048, 512), (512, 512), (512, 2048)):
+        t = torch.randn(m * N, generator=g, device="cuda") + 0.05
+        x = torch.randn(n * N, generator=g, device="cuda")
+        dW, dW2 = torch.full((m * n,), float("nan"), device="cuda"), torch.empty(m * n, device="cuda")
+        db, db2 = torch.full((m,), float("nan"), device="cuda"), torch.empty(m, device="cuda")
+        gpu.gemm_rowsum(dptr(t), dptr(x), dptr(dW), dptr(db), m, n, N, 0, 1, m, n, m, 1.0, 0.0)
+        gpu.gemm(dptr(t), dptr(x), dptr(dW2), m, n, N, 0, 1, m, n, m, 1.0, 0.0)
+        gpu.sum_rows(dptr(db2), dptr(t), m, N, m)
+        gpu.synchronize()
+        assert torch.equal(dW, dW2)
+        want = t.view(N, m).double().sum(dim=0)
+        assert float((db.double() - want).norm() / want.norm()) <= 1e-5
+        assert float((db - db2).norm() / db2.norm()) <= 1e-5
+
+
+def test_gemm_rowsum_rejects_bad_arguments(gpu):
+    from juzhen_amd import capi
+    lib = capi.load()
+    d = dev_empty(16)
+    assert lib.jzhip_gemm_rowsum(dptr(d), dptr(d), dptr(d), None, 2, 2, 2, 0, 1, 2, 2, 2, 1.0, 0.0) == -1
+    assert lib.jzhip_gemm_rowsum(dptr(d), dptr(d), dptr(d), dptr(d), 2, 0, 2, 0, 1, 2, 2, 2, 1.0, 0.0) == -1
+    assert lib.jzhip_gemm_rowsum(dptr(d), dptr(d), dptr(d), dptr(d), 2, 2, 2, 0, 1, 1, 2, 2, 1.0, 0.0) == -1
+
+
 def test_gemm_thin_products_at_the_output_convolution_size(gpu):
     """3 x 131072 x 576 (forward, TN) and 576 x 3 x 131072 (weight gradient, NT) of a
     64 -> 3 channel 3x3 convolution on 128 images of 32 x 32, against float64."""
@@ -881,6 +947,67 @@ def test_layernorm(gpu, oracle_lib, dim, N):
     assert np.linalg.norm(to_host(og) - (G * XH).sum(0)) <= TOL_RED * sg
     assert np.linalg.norm(to_host(ob) - G.sum(0)) <= TOL_RED * sb
     assert np.linalg.norm(to_host(og) - rg) <= TOL_RED * sg
+
+
+# The backward sweep with the sums over tokens on the side (ml/layer.hpp:2674-2686 and the `sum(t, 1)`
+# bias gradients of the dense layers around the residual add, :100).  (512, 16384) is the transformer
+# configuration's shape; (300, 5000) leaves lanes without rows and waves with ragged runs of columns;
+# the last four take the separate passes (dim > 512, few columns, dim not a multiple of 4).
+@pytest.mark.parametrize("dim,N", [(512, 16384), (256, 2048), (512, 1027), (300, 5000), (64, 4096),
+                                   (1024, 2048), (512, 100), (7, 3000), (513, 1500)])
+@pytest.mark.parametrize("mode", ["res+sums", "res", "plain", "in place"])
+def test_layernorm_backward_with_sums(gpu, oracle_lib, dim, N, mode):
+    r = rng(dim * 3 + N)
+    x = r.normal(0.3, 2, dim * N).astype(np.float32)
+    gamma = r.normal(1, 0.2, dim).astype(np.float32)
+    beta = r.normal(0, 0.2, dim).astype(np.float32)
+    y, xh, inv = (np.empty(dim * N, np.float32), np.empty(dim * N, np.float32), np.empty(N, np.float32))
+    oracle_lib.jzo_layernorm_fwd(hptr(y), hptr(xh), hptr(inv), hptr(x), hptr(gamma), hptr(beta), dim, N)
+    g = r.normal(0.05, 1, dim * N).astype(np.float32)
+    res = r.normal(0.02, 1, dim * N).astype(np.float32)
+    with_res = mode != "plain"
+    dg, dxh, dinv, dgam = to_dev(g), to_dev(xh), to_dev(inv), to_dev(gamma)
+    dres = to_dev(res) if with_res else None
+    pres = dptr(dres) if with_res else None
+    # the separate entry points
+    want_dx = dev_empty(dim * N)
+    gpu.layernorm_bwd_residual(dptr(want_dx), dptr(dg), dptr(dgam), dptr(dxh), dptr(dinv), pres, dim, N)
+    wg, wb = dev_empty(dim), dev_empty(dim)
+    gpu.layernorm_param_grads(dptr(wg), dptr(wb), dptr(dg), dptr(dxh), dim, N)
+    nan = lambda n: to_dev(np.full(n, np.nan, np.float32))
+    og, ob, osx, osr = nan(dim), nan(dim), nan(dim), nan(dim)
+    out = dres if mode == "in place" else nan(dim * N)
+    gpu.layernorm_bwd_residual_sums(dptr(out), dptr(dg), dptr(dgam), dptr(dxh), dptr(dinv), pres, dptr(og), dptr(ob),
+                                    dptr(osx) if mode != "res" else None,
+                                    dptr(osr) if mode in ("res+sums", "in place") else None, dim, N)
+    got = to_host(out)
+    assert np.array_equal(got, to_host(want_dx))
+    G = g.reshape(N, dim).astype(np.float64)
+    XH = xh.reshape(N, dim).astype(np.float64)
+    sg = np.linalg.norm(np.abs(G * XH).sum(0))
+    sb = np.linalg.norm(np.abs(G).sum(0))
+    assert np.linalg.norm(to_host(og) - (G * XH).sum(0)) <= TOL_RED * sg
+    assert np.linalg.norm(to_host(ob) - G.sum(0)) <= TOL_RED * sb
+    assert np.linalg.norm(to_host(og) - to_host(wg)) <= 1e-5 * sg
+    assert np.linalg.norm(to_host(ob) - to_host(wb)) <= 1e-5 * sb
+    if mode != "res":
+        D = got.reshape(N, dim).astype(np.float64)
+        assert np.linalg.norm(to_host(osx) - D.sum(0)) <= 1e-5 * np.linalg.norm(np.abs(D).sum(0))
+    if mode in ("res+sums", "in place"):
+        R = res.reshape(N, dim).astype(np.float64)
+        assert np.linalg.norm(to_host(osr) - R.sum(0)) <= 1e-5 * np.linalg.norm(np.abs(R).sum(0))
+    else:
+        assert np.isnan(to_host(osr)).all()          # not asked for: not written
+
+
+def test_layernorm_backward_with_sums_rejects_bad_arguments(gpu):
+    from juzhen_amd import capi
+    lib = capi.load()
+    d = dev_empty(64)
+    P = dptr(d)
+    assert lib.jzhip_layernorm_bwd_residual_sums(P, P, P, P, P, None, P, P, None, P, 4, 4) == -1   # sum_res without res
+    assert lib.jzhip_layernorm_bwd_residual_sums(P, P, P, P, P, None, None, P, None, None, 4, 4) == -1
+    assert lib.jzhip_layernorm_bwd_residual_sums(P, P, P, P, P, None, P, P, None, None, 0, 4) == -1
 
 
 # ── Adam ─────────────────────────────────────────────────────────────────
