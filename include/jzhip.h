@@ -334,6 +334,19 @@ int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int n,
                      int k, int trans_a, int trans_b, int lda, int ldb, int ldc,
                      float alpha, float beta, const float* bias, int act,
                      float* aux, int ld_aux, const float* residual, int ldr);
+/* jzhip_gemm_fused plus rowsum[i] = sum_j C(i, j) over the values it stores: an
+ * upstream gradient formed as (W^T t) .* act'(pre) and the bias gradient
+ * `sum(., 1)` of the layer below it (ml/layer.hpp:98-100; dF1 and db1 of
+ * TransformerLayer::backward) without a second pass over the (m x n) result.
+ * Each workgroup of the tiled kernel adds up what it stores per row and leaves
+ * one partial sum per tile column; they are summed in a fixed order (equal to
+ * jzhip_sum_rows over C to rounding).  C as jzhip_gemm_fused bit for bit.
+ * Products that take a form without a fused store (see jzhip_gemm_fused) run
+ * jzhip_sum_rows over C afterwards.  rowsum must not alias the other operands. */
+int jzhip_gemm_fused_rowsum(const float* A, const float* B, float* C, float* rowsum,
+                            int m, int n, int k, int trans_a, int trans_b, int lda,
+                            int ldb, int ldc, float alpha, float beta, const float* bias,
+                            int act, float* aux, int ld_aux, const float* residual, int ldr);
 /* A layer's two parameter gradients from one pass over the upstream gradient
  * (`gW = t * input.T(); gb = sum(t, 1);`, ml/layer.hpp:99-100; the same pair in
  * TransformerLayer::backward for Wo / W1 / W2 and their biases): jzhip_gemm as

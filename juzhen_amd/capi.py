@@ -109,6 +109,7 @@ SIGNATURES: dict[str, tuple] = {
     "jzhip_gemv": (I, [P, P, P, I, I, I, I, I, I, F, F]),
     "jzhip_gemm_fused": (I, [P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P, I, P, I]),
     "jzhip_gemm_rowsum": (I, [P, P, P, P, I, I, I, I, I, I, I, I, F, F]),
+    "jzhip_gemm_fused_rowsum": (I, [P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, P, I, P, I]),
     "jzhip_gemm_strided_batched": (I, [P, P, P, I, I, I, I, I, I, I, I, LL, LL, LL, I, F, F]),
     "jzhip_profile_gemm": (I, [I]),
     "jzhip_profile_gemm_report": (I, [C.c_char_p, Z]),

@@ -404,9 +404,10 @@ inline void TransformerLayer<ROCMfloat>::add_bias(Matrix<ROCMfloat>& y, const Ma
 // operator+), so the block computes the same bits as the statement-by-statement form.
 // x, aux and residual must be plain (callers materialise transposed views first).
 namespace rocm_detail {
+// *rowsum (optional) receives sum(out, 1), added up by the workgroups that store out.
 inline Matrix<ROCMfloat> fused_product(const Matrix<ROCMfloat>& W, bool transpose_w, const Matrix<ROCMfloat>& x,
                                        const Matrix<ROCMfloat>* bias, int act, Matrix<ROCMfloat>* aux,
-                                       const Matrix<ROCMfloat>* residual) {
+                                       const Matrix<ROCMfloat>* residual, Matrix<ROCMfloat>* rowsum = nullptr) {
     const bool tw = transpose_w != (bool)W.get_transpose();
     const size_t m = transpose_w ? W.num_col() : W.num_row(), k = transpose_w ? W.num_row() : W.num_col();
     const size_t n = x.num_col();
@@ -415,6 +416,15 @@ inline Matrix<ROCMfloat> fused_product(const Matrix<ROCMfloat>& W, bool transpos
         (residual && (residual->get_transpose() || residual->num_row() != m || residual->num_col() != n)))
         throw std::invalid_argument("Matrix dimensions are not compatible");
     Matrix<ROCMfloat> out = JzRocmFused::make("fused_product", m, n, 0);
+    if (rowsum) {
+        *rowsum = Matrix<ROCMfloat>("fused_product_rowsum", m, 1);
+        must(jzhip_gemm_fused_rowsum(p(W), p(x), p(out), p(*rowsum), (int)m, (int)n, (int)k, tw ? 1 : 0, 0,
+                                     (int)JzRocmFused::phys_rows(W), (int)k, (int)m, 1.0f, 0.0f,
+                                     bias ? p(*bias) : nullptr, act, aux ? p(*aux) : nullptr, (int)m,
+                                     residual ? p(*residual) : nullptr, (int)m),
+             "gemm_fused_rowsum");
+        return out;
+    }
     must(jzhip_gemm_fused(p(W), p(x), p(out), (int)m, (int)n, (int)k, tw ? 1 : 0, 0, (int)JzRocmFused::phys_rows(W),
                           (int)k, (int)m, 1.0f, 0.0f, bias ? p(*bias) : nullptr, act, aux ? p(*aux) : nullptr, (int)m,
                           residual ? p(*residual) : nullptr, (int)m),
@@ -556,9 +566,9 @@ inline Matrix<ROCMfloat> TransformerLayer<ROCMfloat>::backward(const Matrix<ROCM
 
     // feed-forward: F = W2 relu(W1 x2 + b1) + b2
     MD dW2 = dout * cached_F1_relu.T();
-    MD dF1 = fused_product(W2, true, dout, nullptr, 3, &cached_F1, nullptr);   // (W2^T dout) .* relu'(F1)
+    MD db1 = JzRocmFused::make("db1", 0, 0, 0);
+    MD dF1 = fused_product(W2, true, dout, nullptr, 3, &cached_F1, nullptr, &db1);   // (W2^T dout) .* relu'(F1); db1 = sum(dF1, 1)
     MD dW1 = dF1 * cached_x2.T();
-    MD db1 = sum(dF1, 1);
     // the sweep that forms dR = LN2'(..) + dout also adds up the rows of dout and of dR: the
     // bias gradients db2 = sum(dout, 1) and dbo = sum(dR, 1)
     MD db2 = JzRocmFused::make("db2", 0, 0, 0), dbo = JzRocmFused::make("dbo", 0, 0, 0);

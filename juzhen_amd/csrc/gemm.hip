@@ -67,6 +67,8 @@ struct Epilogue {
     size_t ld_aux = 0;
     int act = 0;
     int any = 0;
+    // row sums of the stored values, per tile column: rs_part[tile_n * M + row] (jzhip_gemm_fused_rowsum)
+    float* rs_part = nullptr;
 };
 
 // WGM x WGN waves, each computing TM x TN MFMA tiles of 32x32.
@@ -391,8 +393,11 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
             }
         }
     };
+    float row_acc[TM];   // what this lane stored, added up per row tile
+#pragma unroll
+    for (int i = 0; i < TM; ++i) row_acc[i] = 0.0f;
     auto tail_tile = [&](const floatx16& a, const auto& r, const auto& x, int row0, int col0, float bias,
-                         auto act_c, auto res_c) {
+                         float& stored, auto act_c, auto res_c) {
         constexpr int ACT = decltype(act_c)::value;
         constexpr bool RES = decltype(res_c)::value;
 #pragma unroll
@@ -413,6 +418,7 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
                 }
                 if constexpr (RES) t += r[v];
                 *dst = t;
+                stored += t;
             }
             if (v % 4 == 3) __builtin_amdgcn_sched_barrier(0);
         }
@@ -438,7 +444,8 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
             __builtin_amdgcn_sched_barrier(0);
             const int row = rows(n) + l32;
             const float bias = (ep.bias && (FAST || row < M)) ? ep.bias[row] : 0.0f;
-            tail_tile(acc[n / TN][n % TN], r[n % NBUF], x[n % NBUF], rows(n), cols(n), bias, act_c, res_c);
+            tail_tile(acc[n / TN][n % TN], r[n % NBUF], x[n % NBUF], rows(n), cols(n), bias, row_acc[n / TN], act_c,
+                      res_c);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -455,6 +462,24 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
     case 8: tail_all(integral_constant<int, 4>{}, bool_constant<false>{}); break;
     case 9: tail_all(integral_constant<int, 4>{}, bool_constant<true>{}); break;
     default: tail_all(integral_constant<int, 0>{}, bool_constant<false>{}); break;
+    }
+    if (ep.rs_part) {
+        // a row of the tile lies in two lanes (h = 0, 1) of each of the WGN waves across
+        __syncthreads();   // the staging buffers are free
+        float* red = &As[0][0];
+        static_assert(2 * BK * LDA_S >= WGN * BM, "the staging buffers hold one value per wave column and row");
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const float both = row_acc[i] + __shfl_xor(row_acc[i], 32, kWave);
+            if (h == 0) red[wn_u * BM + (wm_u * TM + i) * 32 + l32] = both;
+        }
+        __syncthreads();
+        if (threadIdx.x < BM && (FAST || m0 + static_cast<int>(threadIdx.x) < M)) {
+            float sum = red[threadIdx.x];
+#pragma unroll
+            for (int w = 1; w < WGN; ++w) sum += red[w * BM + threadIdx.x];
+            ep.rs_part[static_cast<size_t>(tile_n) * M + m0 + threadIdx.x] = sum;
+        }
     }
 }
 
@@ -660,6 +685,9 @@ struct GemmArgs {
     // row sums of A on the side (jzhip_gemm_rowsum): where to, and whether the launch formed them
     float* rowsum = nullptr;
     bool* rowsum_done = nullptr;
+    // row sums of the stored C on the side (jzhip_gemm_fused_rowsum), same pair
+    float* out_rowsum = nullptr;
+    bool* out_rowsum_done = nullptr;
 };
 
 template <int WGM, int WGN, int TM, int TN, bool TA, bool TB>
@@ -755,10 +783,18 @@ int launch_tile(const GemmArgs& g) {
         (void)hipEventCreate(&rec.end);
         (void)hipEventRecord(rec.begin, s);
     }
+    // row sums of the stored values: the fused tail leaves one partial sum per tile column
+    Epilogue ep = g.ep;
+    const bool out_rowsum = g.out_rowsum && g.ep.any && nb == 1 && splits == 1 &&
+                            static_cast<size_t>(tiles_n) * g.M <= kWorkspaceFloats;
+    if (out_rowsum) {
+        ep.rs_part = workspace();
+        if (!ep.rs_part) return -2;
+    }
 #define JZ_LAUNCH_GEMM(FASTV, EPIV)                                                                         \
     gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, FASTV, EPIV><<<grid, kBlock, 0, s>>>(                        \
         g.A, g.B, out, g.M, g.N, g.K, g.lda, g.ldb, ldc, alpha, beta, g.sA, g.sB, sC, g.batch, g.sA2, g.sB2, \
-        sC2, tiles_m, tiles_n, k_chunk, split_stride, g.ep)
+        sC2, tiles_m, tiles_n, k_chunk, split_stride, ep)
     if (with_rowsum) {
         if constexpr (!TA && TB)
             gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, true, false, true><<<grid, kBlock, 0, s>>>(
@@ -775,6 +811,10 @@ int launch_tile(const GemmArgs& g) {
         (void)hipEventRecord(rec.end, s);
         std::lock_guard<std::mutex> lock(prof.mu);
         prof.recs.push_back(rec);
+    }
+    if (out_rowsum) {
+        launch_splitk_reduce(g.out_rowsum, ep.rs_part, g.M, 1, static_cast<size_t>(g.M), tiles_n, 1.0f, 0.0f);
+        if (g.out_rowsum_done) *g.out_rowsum_done = true;
     }
     if (splits > 1) {
         if (with_rowsum) {
@@ -955,6 +995,17 @@ JZ_API int jzhip_gemm(const float* A, const float* B, float* C, int m, int n, in
     return gemm_dispatch(g, trans_a != 0, trans_b != 0);
 }
 
+namespace {
+// JZHIP_GEMM_ROWSUM=0 keeps the separate passes for every shape (for comparisons)
+bool rowsum_fused_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("JZHIP_GEMM_ROWSUM");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+}  // namespace
+
 JZ_API int jzhip_gemm_rowsum(const float* A, const float* B, float* C, float* rowsum, int m, int n, int k, int trans_a,
                              int trans_b, int lda, int ldb, int ldc, float alpha, float beta) {
     if (m <= 0 || n <= 0 || k <= 0) return -1;
@@ -962,12 +1013,7 @@ JZ_API int jzhip_gemm_rowsum(const float* A, const float* B, float* C, float* ro
     if (lda < (trans_a ? k : m) || ldb < (trans_b ? n : k) || ldc < m) return -1;
     // The tiled kernel forms the sums on the side for a plain A against a transposed B in full,
     // aligned tiles; every other product is the plain entry point followed by the sum kernels.
-    // JZHIP_GEMM_ROWSUM=0 keeps the two separate passes for every shape (for comparisons)
-    static const bool fused_on = [] {
-        const char* e = std::getenv("JZHIP_GEMM_ROWSUM");
-        return !(e && e[0] == '0');
-    }();
-    if (fused_on && !trans_a && trans_b && k > 1 && m > 16 && n > 16) {
+    if (rowsum_fused_enabled() && !trans_a && trans_b && k > 1 && m > 16 && n > 16) {
         bool done = false;
         GemmArgs g{A, B, C, m, n, k, static_cast<size_t>(lda), static_cast<size_t>(ldb),
                    static_cast<size_t>(ldc), alpha, beta, 0, 0, 0, 1};
@@ -982,10 +1028,36 @@ JZ_API int jzhip_gemm_rowsum(const float* A, const float* B, float* C, float* ro
     return trans_a ? jzhip_sum_cols(rowsum, A, k, m, lda) : jzhip_sum_rows(rowsum, A, m, k, lda);
 }
 
+namespace {
+int gemm_fused_impl(const float* A, const float* B, float* C, int m, int n, int k, int trans_a, int trans_b, int lda,
+                    int ldb, int ldc, float alpha, float beta, const float* bias, int act, float* aux, int ld_aux,
+                    const float* residual, int ldr, float* rowsum, bool* rowsum_done);
+}
+
 JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int n, int k, int trans_a,
                             int trans_b, int lda, int ldb, int ldc, float alpha, float beta,
                             const float* bias, int act, float* aux, int ld_aux, const float* residual,
                             int ldr) {
+    return gemm_fused_impl(A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, bias, act, aux, ld_aux,
+                           residual, ldr, nullptr, nullptr);
+}
+
+JZ_API int jzhip_gemm_fused_rowsum(const float* A, const float* B, float* C, float* rowsum, int m, int n, int k,
+                                   int trans_a, int trans_b, int lda, int ldb, int ldc, float alpha, float beta,
+                                   const float* bias, int act, float* aux, int ld_aux, const float* residual,
+                                   int ldr) {
+    if (!rowsum) return -1;
+    bool done = false;
+    const int rc = gemm_fused_impl(A, B, C, m, n, k, trans_a, trans_b, lda, ldb, ldc, alpha, beta, bias, act, aux,
+                                   ld_aux, residual, ldr, rowsum_fused_enabled() ? rowsum : nullptr, &done);
+    if (rc != 0 || done) return rc;
+    return jzhip_sum_rows(rowsum, C, m, n, ldc);   // forms without a fused tail
+}
+
+namespace {
+int gemm_fused_impl(const float* A, const float* B, float* C, int m, int n, int k, int trans_a, int trans_b, int lda,
+                    int ldb, int ldc, float alpha, float beta, const float* bias, int act, float* aux, int ld_aux,
+                    const float* residual, int ldr, float* rowsum, bool* rowsum_done) {
     if (m <= 0 || n <= 0 || k <= 0) return -1;
     if (!A || !B || !C) return -1;
     if (lda < (trans_a ? k : m) || ldb < (trans_b ? n : k) || ldc < m) return -1;
@@ -1030,8 +1102,11 @@ JZ_API int jzhip_gemm_fused(const float* A, const float* B, float* C, int m, int
     g.ep.res = residual;
     g.ep.ldr = static_cast<size_t>(ldr);
     g.ep.any = (bias || act || residual) ? 1 : 0;
+    g.out_rowsum = rowsum;
+    g.out_rowsum_done = rowsum_done;
     return gemm_dispatch(g, trans_a != 0, trans_b != 0);
 }
+}  // namespace
 
 JZ_API int jzhip_gemm_nn(const float* A, const float* B, float* C, int m, int n, int k, float alpha,
                          float beta) {

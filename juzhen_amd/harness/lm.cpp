@@ -307,10 +307,11 @@ void backward(Model& M, bool update) {
         gemm(M, dy, false, b.F1a, true, M.t[b.W2].g, d, ff, N);   // (db2 = row sums of dy: with the LayerNorm sweep below)
         lanes.back();
         // dF1 = (W2^T dy) .* act'(F1)
-        gemm_tail(M, M.t[b.W2].w, true, dy, dF1, ff, N, d, nullptr, c.gelu ? 4 : 3, b.F1, nullptr);
+        // (with db1 = row sums of dF1, added up by the workgroups that store it)
+        M.ck(jzhip_gemm_fused_rowsum(M.t[b.W2].w, dy, dF1, M.t[b.b1].g, ff, N, d, 1, 0, d, d, ff, 1.0f, 0.0f, nullptr,
+                                     c.gelu ? 4 : 3, b.F1, ff, nullptr, ff));
         lanes.fork();
         gemm(M, dF1, false, b.x2, true, M.t[b.W1].g, ff, d, N);
-        M.ck(jzhip_sum_rows(M.t[b.b1].g, dF1, ff, N, ff));
         lanes.back();
         gemm(M, M.t[b.W1].w, true, dF1, false, dx2, d, N, ff);
         // dR = LN2'(dx2) + dy, and in the same sweep the LayerNorm's parameter gradients and the

@@ -624,6 +624,59 @@ def test_gemm_more_tiles_than_workgroups(gpu, m, n, k, ta, tb, fused):
     assert rel_err(to_host(whole), to_host(v.T.reshape(-1))) <= TOL_GEMM
 
 
+# The fused store with the row sums of what it stores (upstream gradient times activation derivative and
+# the bias gradient of the layer below): tiled forms of several tile shapes, ragged edges on the checked
+# loaders, and the forms without a fused store (split-K, thin, matrix-vector), which run the sum kernel.
+@pytest.mark.parametrize("m,n,k,ta", [(256, 512, 128, 1), (2048, 1024, 512, 1), (128, 1024, 96, 0), (129, 127, 17, 1),
+                                      (64, 1216, 512, 1), (32, 512, 64, 0), (512, 64, 128, 1), (1024, 32, 64, 0),
+                                      (10, 128, 2560, 1), (5, 300, 64, 0), (300, 1, 70, 0), (256, 128, 4096, 1)])
+@pytest.mark.parametrize("act", [0, 3, 4])
+def test_gemm_fused_rowsum(gpu, m, n, k, ta, act):
+    r = rng(m + 3 * n + 5 * k + act)
+    lda = k if ta else m
+    A = r.normal(0, 1 / math.sqrt(k), m * k).astype(np.float32)
+    B = r.normal(0, 1, k * n).astype(np.float32)
+    pre = r.normal(0.2, 1, m * n).astype(np.float32)
+    bias = r.normal(0.1, 0.5, m).astype(np.float32)
+    dA, dB, dpre, dbias = to_dev(A), to_dev(B), to_dev(pre), to_dev(bias)
+    want = to_dev(np.full(m * n, np.nan, np.float32))
+    got = to_dev(np.full(m * n, np.nan, np.float32))
+    rs = to_dev(np.full(m, np.nan, np.float32))
+    aux = dptr(dpre) if act else None
+    pb = dptr(dbias) if act == 0 else None
+    gpu.gemm_fused(dptr(dA), dptr(dB), dptr(want), m, n, k, ta, 0, lda, k, m, 1.0, 0.0, pb, act, aux, m, None, m)
+    gpu.gemm_fused_rowsum(dptr(dA), dptr(dB), dptr(got), dptr(rs), m, n, k, ta, 0, lda, k, m, 1.0, 0.0, pb, act, aux, m,
+                          None, m)
+    out = to_host(got)
+    assert np.array_equal(out, to_host(want))
+    O = out.reshape(n, m).astype(np.float64)
+    assert np.linalg.norm(to_host(rs) - O.sum(0)) <= 1e-5 * np.linalg.norm(np.abs(O).sum(0))
+
+
+def test_gemm_fused_rowsum_at_the_feed_forward_gradient_shape(gpu):
+    """(W2^T dy) .* gelu'(F1) at 2048 x 16384 x 512 with the row sums: against the plain fused entry
+    point bit for bit and jzhip_sum_rows over its result; twice (the partial sums live in the workspace)."""
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    d, ff, N = 512, 2048, 16384
+    for _ in range(2):
+        W2 = torch.randn(d * ff, generator=g, device="cuda") / math.sqrt(ff)
+        dy = torch.randn(d * N, generator=g, device="cuda")
+        F1 = torch.randn(ff * N, generator=g, device="cuda")
+        a, b = torch.full((ff * N,), float("nan"), device="cuda"), torch.empty(ff * N, device="cuda")
+        rs, rs2 = torch.full((ff,), float("nan"), device="cuda"), torch.empty(ff, device="cuda")
+        gpu.gemm_fused_rowsum(dptr(W2), dptr(dy), dptr(a), dptr(rs), ff, N, d, 1, 0, d, d, ff, 1.0, 0.0, None, 4, dptr(F1), ff,
+                              None, ff)
+        gpu.gemm_fused(dptr(W2), dptr(dy), dptr(b), ff, N, d, 1, 0, d, d, ff, 1.0, 0.0, None, 4, dptr(F1), ff, None, ff)
+        gpu.sum_rows(dptr(rs2), dptr(b), ff, N, ff)
+        gpu.synchronize()
+        assert torch.equal(a, b)
+        want = b.view(N, ff).double().sum(dim=0)
+        assert float((rs.double() - want).norm() / want.norm()) <= 1e-5
+        assert float((rs - rs2).norm() / rs2.norm()) <= 1e-5
+
+
 def test_gemm_fused_rejects_bad_arguments(gpu):
     from juzhen_amd import capi
     lib = capi.load()
