@@ -412,36 +412,44 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_sums_vec_kernel(float* dx, cons
     }
 }
 
-// part is [chunk][4*dim]; a block owns 64 of the 4*dim outputs, its waves take interleaved
-// chunks and are combined through LDS; a sum nobody asked for (null pointer) is skipped.
+// part is [chunk][4*dim]; a block owns 16 of the 4*dim outputs (128 blocks at dim 512, so that
+// the few MB of partial sums are read by half the chip rather than an eighth of it): the four
+// 16-lane groups of a wave and the sixteen waves take interleaved chunks, meet by lane exchange
+// and through LDS, always in the same order; a sum nobody asked for (null pointer) is skipped.
+constexpr int kSumsOutputs = 16;
 __global__ __launch_bounds__(kCombineThreads) void ln_sums_combine_kernel(float* s0, float* s1, float* s2, float* s3,
                                                                           const float* part, int dim, int chunks) {
     constexpr int NW = kCombineThreads / kWave;
-    __shared__ float red[NW][kWave];
+    constexpr int PH = kWave / kSumsOutputs;      // chunk phases inside a wave
+    __shared__ float red[NW][kSumsOutputs];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
-    const int i = blockIdx.x * kWave + lane;
+    const int o = lane % kSumsOutputs, ph = lane / kSumsOutputs;
+    const int i = blockIdx.x * kSumsOutputs + o;
     const int n = 4 * dim;
     const int which = i < n ? i / dim : 0;
     float* dst = which == 0 ? s0 : which == 1 ? s1 : which == 2 ? s2 : s3;
     float acc = 0.f;
     if (i < n && dst) {
-        int c = wave;
-        for (; c + 3 * NW < chunks; c += 4 * NW) {   // four loads in flight
+        constexpr int STEP = NW * PH;
+        int c = wave * PH + ph;
+        for (; c + 3 * STEP < chunks; c += 4 * STEP) {   // four loads in flight
             const float a0 = part[static_cast<size_t>(c) * n + i];
-            const float a1 = part[static_cast<size_t>(c + NW) * n + i];
-            const float a2 = part[static_cast<size_t>(c + 2 * NW) * n + i];
-            const float a3 = part[static_cast<size_t>(c + 3 * NW) * n + i];
+            const float a1 = part[static_cast<size_t>(c + STEP) * n + i];
+            const float a2 = part[static_cast<size_t>(c + 2 * STEP) * n + i];
+            const float a3 = part[static_cast<size_t>(c + 3 * STEP) * n + i];
             acc += (a0 + a1) + (a2 + a3);
         }
-        for (; c < chunks; c += NW) acc += part[static_cast<size_t>(c) * n + i];
+        for (; c < chunks; c += STEP) acc += part[static_cast<size_t>(c) * n + i];
     }
-    red[wave][lane] = acc;
+    acc += __shfl_xor(acc, 16, kWave);
+    acc += __shfl_xor(acc, 32, kWave);
+    if (ph == 0) red[wave][o] = acc;
     __syncthreads();
-    if (wave == 0 && i < n && dst) {
+    if (threadIdx.x < kSumsOutputs && i < n && dst) {
         float s = 0.f;
 #pragma unroll
-        for (int w = 0; w < NW; ++w) s += red[w][lane];
+        for (int w = 0; w < NW; ++w) s += red[w][o];
         dst[i - which * dim] = s;
     }
 }
@@ -529,7 +537,7 @@ JZ_API int jzhip_layernorm_bwd_residual_sums(float* dx, const float* dy, const f
         if (dim <= 256) JZ_LN_BWD_SUMS(1);
         else JZ_LN_BWD_SUMS(2);
 #undef JZ_LN_BWD_SUMS
-        ln_sums_combine_kernel<<<(4 * dim + kWave - 1) / kWave, kCombineThreads, 0, s>>>(dgamma, dbeta, sum_dx, sum_res,
+        ln_sums_combine_kernel<<<(4 * dim + kSumsOutputs - 1) / kSumsOutputs, kCombineThreads, 0, s>>>(dgamma, dbeta, sum_dx, sum_res,
                                                                                          part, dim, static_cast<int>(blocks));
         return launch_rc();
     }
