@@ -143,6 +143,20 @@ def bench_gemm(r):
               lambda: jz.gemm_fused(P(A), P(B), P(Cm), m, n, k, ta, 0, lda, k, m, 1.0, 0.0,
                                     P(bias) if act != 4 else None, act, P(aux) if act else None, m,
                                     P(res) if use_res else None, m), flops=2.0 * m * n * k)
+    # the same store with the row sums of the result (the bias gradient of the layer below) on the side
+    m, n, k = 2048, 16384, 512
+    A, B, Cm, aux, rs = dev(m * k), dev(k * n), dev(m * n, 0), dev(m * n), dev(m, 0)
+    r.run("gemm", "jzhip_gemm_fused_rowsum C4 dF1: .*gelu'(pre) TN + row sums", f"{m}x{n}x{k}",
+          lambda: jz.gemm_fused_rowsum(P(A), P(B), P(Cm), P(rs), m, n, k, 1, 0, k, k, m, 1.0, 0.0, None, 4, P(aux), m, None, m),
+          flops=2.0 * m * n * k)
+    # a dense layer's weight and bias gradients from one pass over the upstream gradient
+    for label, m, n, k in (("C2 dW + db NT", 256, 256, 4096), ("C4 dW1 + db1 NT", 2048, 512, 16384)):
+        A, B, Cm, rs = dev(m * k), dev(n * k), dev(m * n, 0), dev(m, 0)
+        r.run("gemm", f"jzhip_gemm_rowsum {label}", f"{m}x{n}x{k}",
+              lambda: jz.gemm_rowsum(P(A), P(B), P(Cm), P(rs), m, n, k, 0, 1, m, n, m, 1.0, 0.0), flops=2.0 * m * n * k)
+        r.run("gemm", f"jzhip_gemm + jzhip_sum_rows {label}", f"{m}x{n}x{k}",
+              lambda: (jz.gemm(P(A), P(B), P(Cm), m, n, k, 0, 1, m, n, m, 1.0, 0.0), jz.sum_rows(P(rs), P(A), m, k, m)),
+              flops=2.0 * m * n * k)
     # attention-shaped strided batches (C4: 512 blocks of 256x256x64)
     S, dk, nb = 256, 64, 512
     Q, K, A_ = dev(S * dk * nb), dev(S * dk * nb), dev(S * S * nb, 0)
@@ -233,6 +247,17 @@ def bench_fused(r):
               bytes_=4 * (3 * dim * N + N + dim))
         r.run("fused", "jzhip_layernorm_param_grads", s, lambda: jz.layernorm_param_grads(P(dg), P(db), P(x), P(xh), dim, N),
               bytes_=4 * (2 * dim * N + 2 * dim))
+        # the backward sweep with the parameter gradients and two row sums on the side: dy, xhat, res in, dx out
+        res, sx, sr = dev(dim * N), dev(dim, 0), dev(dim, 0)
+        r.run("fused", "jzhip_layernorm_bwd_residual_sums", s,
+              lambda: jz.layernorm_bwd_residual_sums(P(y), P(x), P(g), P(xh), P(inv), P(res), P(dg), P(db), P(sx), P(sr), dim, N),
+              bytes_=4 * (4 * dim * N + N + 5 * dim))
+        r.run("fused", "the same as separate launches (bwd_residual, param_grads, 2 x sum_rows)", s,
+              lambda: (jz.layernorm_bwd_residual(P(y), P(x), P(g), P(xh), P(inv), P(res), dim, N),
+                       jz.layernorm_param_grads(P(dg), P(db), P(x), P(xh), dim, N),
+                       jz.sum_rows(P(sx), P(y), dim, N, dim), jz.sum_rows(P(sr), P(res), dim, N, dim)),
+              bytes_=4 * (4 * dim * N + N + 5 * dim))
+        del res, sx, sr
     for n in (1 << 20, 19_000_000, 1 << 27):
         w, g, m, v = dev(n), dev(n), dev(n, 0), dev(n, 0)
         r.run("fused", "jzhip_adam_update", f"{n}", lambda: jz.adam_update(P(g), P(m), P(v), n, 1e-3, 0.9, 0.999, 1e-8, 3), bytes_=24 * n)
