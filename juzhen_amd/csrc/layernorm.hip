@@ -346,19 +346,31 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_sums_vec_kernel(float* dx, cons
 #pragma unroll
         for (int q = 0; q < 4; ++q) acc[q][v] = zero;
     }
-    for (size_t col = wave_begin(static_cast<size_t>(N), wave0, nwaves), col_end = wave_end(static_cast<size_t>(N), wave0, nwaves); col < col_end; ++col) {
+    // the next column's operands are requested before the current one is worked on
+    const size_t col_begin = wave_begin(static_cast<size_t>(N), wave0, nwaves);
+    const size_t col_end = wave_end(static_cast<size_t>(N), wave0, nwaves);
+    float4 d[NV], h[NV], rr[NV], dn[NV], hn[NV], rn[NV];
+    auto fetch = [&](float4 (&fd)[NV], float4 (&fh)[NV], float4 (&fr)[NV], size_t col) {
         const size_t base = col * dim;
-        float4 d[NV], h[NV], rr[NV];
-        float s1 = 0.f, s2 = 0.f;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int r = (lane + v * kWave) * 4;
             if (r < dim) {
-                d[v] = load4<NT>(dy + base + r);
-                h[v] = load4<NT>(xhat + base + r);
-                rr[v] = res ? load4<NT>(res + base + r) : zero;
+                fd[v] = load4<NT>(dy + base + r);
+                fh[v] = load4<NT>(xhat + base + r);
+                fr[v] = res ? load4<NT>(res + base + r) : zero;
+            } else {
+                fd[v] = zero; fh[v] = zero; fr[v] = zero;
             }
         }
+    };
+    if (col_begin < col_end) fetch(dn, hn, rn, col_begin);
+    for (size_t col = col_begin; col < col_end; ++col) {
+        const size_t base = col * dim;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) { d[v] = dn[v]; h[v] = hn[v]; rr[v] = rn[v]; }
+        if (col + 1 < col_end) fetch(dn, hn, rn, col + 1);
+        float s1 = 0.f, s2 = 0.f;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int r = (lane + v * kWave) * 4;
