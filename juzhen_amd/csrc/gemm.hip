@@ -192,9 +192,11 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
     // row sums of A: a thread's float4s are the same four rows in every pass and stage
     floatx4 rs = {0.f, 0.f, 0.f, 0.f};
     if constexpr (RS) {
+        if (tile_n == 0) {
 #pragma unroll
-        for (int ps = 0; ps < LA::kPasses; ++ps)
-            if (LA::active(ps)) rs += ra[0][ps];
+            for (int ps = 0; ps < LA::kPasses; ++ps)
+                if (LA::active(ps)) rs += ra[0][ps];
+        }
     }
     __syncthreads();
     if constexpr (NSET == 2) {
@@ -265,19 +267,10 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
             }
             if constexpr (RS) {
                 // (the set holds stage kt+1; past the end it is the last stage fetched again)
-#ifdef JZ_RS_TN0
                 if (kk < LA::kPasses && LA::active(kk) && tile_n == 0) {
-#else
-                if (kk < LA::kPasses && LA::active(kk)) {
-#endif
-#if defined(JZ_RS_NOACC)
-#elif defined(JZ_RS_SUBTRACT)
-                    rs += ra[ST][kk];
-#else
                     const bool real = kt + 1 < nk;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) rs[e] += real ? ra[ST][kk][e] : 0.0f;
-#endif
                 }
             }
             if constexpr (NSET == 1) {
@@ -308,11 +301,6 @@ __global__ __launch_bounds__(kBlock, FAST ? JZ_GEMM_OCC : 2) void gemm_mfma_kern
     }
 
     if constexpr (RS) {
-#ifdef JZ_RS_SUBTRACT
-#pragma unroll
-        for (int ps = 0; ps < LA::kPasses; ++ps)
-            if (LA::active(ps)) rs -= ra[0][ps];
-#endif
         if (tile_n == 0) {
             // the kBlock / (BM / 4) threads that hold the same four rows meet in LDS and are
             // added in thread order
