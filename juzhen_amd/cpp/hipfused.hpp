@@ -362,13 +362,17 @@ inline Matrix<ROCMfloat> LayerNorm<ROCMfloat>::backward(Matrix<ROCMfloat>&& dy, 
     if (dy.get_transpose()) return backward(JzRocmFused::materialise(dy), update);
     const int N = (int)dy.num_col();
     Matrix<ROCMfloat> dx("ln_dx", dim, N);
-    must(jzhip_layernorm_bwd(p(dx), p(dy), p(gamma), p(cached_xhat), p(cached_inv), dim, N), "layernorm_bwd");
     // dx reads gamma, so the parameter step comes second (ml/layer.hpp:2682-2686)
     if (update) {
+        // one sweep over dy and xhat for dx and the two parameter gradients
         Matrix<ROCMfloat> dg("ln_dgamma", dim, 1), db("ln_dbeta", dim, 1);
-        must(jzhip_layernorm_param_grads(p(dg), p(db), p(dy), p(cached_xhat), dim, N), "layernorm_param_grads");
+        must(jzhip_layernorm_bwd_residual_sums(p(dx), p(dy), p(gamma), p(cached_xhat), p(cached_inv), nullptr, p(dg),
+                                               p(db), nullptr, nullptr, dim, N),
+             "layernorm_bwd_residual_sums");
         fused_update({{&gamma, &dg, &adam_g}, {&beta, &db, &adam_b}});
+        return dx;
     }
+    must(jzhip_layernorm_bwd(p(dx), p(dy), p(gamma), p(cached_xhat), p(cached_inv), dim, N), "layernorm_bwd");
     return dx;
 }
 
