@@ -757,6 +757,14 @@ int launch_tile(const GemmArgs& g) {
         with_rowsum = g.rowsum && fast && !g.ep.any && nb == 1;
         if (with_rowsum) rs_part = splits > 1 ? out + split_stride * splits : g.rowsum;
     }
+    // row sums of the stored values: the fused tail leaves one partial sum per tile column
+    Epilogue ep = g.ep;
+    const bool out_rowsum = g.out_rowsum && g.ep.any && nb == 1 && splits == 1 &&
+                            static_cast<size_t>(tiles_n) * g.M <= kWorkspaceFloats;
+    if (out_rowsum) {
+        ep.rs_part = workspace();
+        if (!ep.rs_part) return -2;
+    }
     GemmProf& prof = gemm_prof();
     GemmProfRecord rec;
     const bool timing = prof.on;
@@ -770,14 +778,6 @@ int launch_tile(const GemmArgs& g) {
         (void)hipEventCreate(&rec.begin);
         (void)hipEventCreate(&rec.end);
         (void)hipEventRecord(rec.begin, s);
-    }
-    // row sums of the stored values: the fused tail leaves one partial sum per tile column
-    Epilogue ep = g.ep;
-    const bool out_rowsum = g.out_rowsum && g.ep.any && nb == 1 && splits == 1 &&
-                            static_cast<size_t>(tiles_n) * g.M <= kWorkspaceFloats;
-    if (out_rowsum) {
-        ep.rs_part = workspace();
-        if (!ep.rs_part) return -2;
     }
 #define JZ_LAUNCH_GEMM(FASTV, EPIV)                                                                         \
     gemm_mfma_kernel<WGM, WGN, TM, TN, TA, TB, FASTV, EPIV><<<grid, kBlock, 0, s>>>(                        \
